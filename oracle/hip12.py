@@ -1,0 +1,426 @@
+"""CPU oracle driver for ``hip_attention_12`` -- TEST INFRASTRUCTURE ONLY.
+
+Restates the host-side driver of the reference operator
+(``src/hip_attn/v1_2/attention_extend.py:1918-3133``) in NumPy and calls the C restatement of
+the device kernels in ``hip_oracle.c``.  The shipped package never imports this module; tests,
+``__graft_entry__.smoke`` and the benchmark's ``cpu_baseline`` leg do.
+
+Unlike the product, which keeps one chunk list per (batch, query block) when scores are
+max-reduced over heads, this driver keeps the reference's full ``[B, BDST, HEAD, chunks]``
+int64 tensors and performs every glue step (truncate, realign, sort, split, top-k, gather)
+literally, so the product's shortcuts are checked against the long form.
+
+Tie-break rule (the reference leaves ties to ``torch.topk`` / unstable ``sort``): candidates are
+ordered by (score descending, current list position ascending).
+
+bf16 tensors are carried as ``uint16`` bit patterns.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from dataclasses import dataclass, field
+from typing import List, Optional
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+INT64_MAX = np.iinfo(np.int64).max
+
+
+class _Tensors(ctypes.Structure):
+    _fields_ = [
+        ("dtype", ctypes.c_int),
+        ("B", ctypes.c_int),
+        ("TDST", ctypes.c_int),
+        ("HEAD", ctypes.c_int),
+        ("HKV", ctypes.c_int),
+        ("HID", ctypes.c_int),
+        ("q", ctypes.c_void_p),
+        ("pos", ctypes.c_void_p),
+        ("k", ctypes.c_void_p),
+        ("v", ctypes.c_void_p),
+        ("TSRC", ctypes.c_int64),
+        ("k_cache", ctypes.c_void_p),
+        ("v_cache", ctypes.c_void_p),
+        ("page_size", ctypes.c_int),
+        ("block_table", ctypes.c_void_p),
+        ("bt_cols", ctypes.c_int64),
+        ("cache_seq_lens", ctypes.c_void_p),
+        ("MAX_TSRC", ctypes.c_int64),
+    ]
+
+
+def build(force: bool = False) -> str:
+    """Compile ``libhip_oracle.so`` next to this file and return its path."""
+    so = os.path.join(_HERE, "libhip_oracle.so")
+    src = os.path.join(_HERE, "hip_oracle.c")
+    if force or (not os.path.exists(so)) or os.path.getmtime(so) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "libhip_oracle.so"], stdout=subprocess.DEVNULL)
+    return so
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        L = ctypes.CDLL(build())
+        L.hipo_round_bf16.restype = ctypes.c_float
+        L.hipo_round_bf16.argtypes = [ctypes.c_float]
+        L.hipo_dot.restype = ctypes.c_float
+        L.hipo_dot.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int]
+        L.hipo_scale_constants.restype = None
+        L.hipo_mask_stage.restype = ctypes.c_int
+        L.hipo_bsa.restype = ctypes.c_int
+        L.hipo_num_threads.restype = ctypes.c_int
+        _LIB = L
+    return _LIB
+
+
+# ------------------------------------------------------------------ bf16 helpers (uint16 bits)
+
+def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """Round-to-nearest-even float32 -> bf16 bit patterns."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    r = u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))
+    return (r >> np.uint32(16)).astype(np.uint16)
+
+
+def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def scale_constants(hid: int, dtype: str):
+    cq, ck = ctypes.c_float(), ctypes.c_float()
+    lib().hipo_scale_constants(ctypes.c_int(hid), ctypes.c_int(1 if dtype == "bf16" else 0),
+                               ctypes.byref(cq), ctypes.byref(ck))
+    return cq.value, ck.value
+
+
+# ------------------------------------------------------------------ argument containers
+
+@dataclass
+class OStage:
+    """One ScanStage (attention_metadata.py:55-60)."""
+    stage_block_size_q: int
+    stage_block_stride_q: int
+    stage_chunk_size: int
+    stage_k: Optional[int]
+    stage_stride: int = 1
+
+
+def default_stages() -> List[OStage]:
+    return [OStage(64, 4, 256, None, 1), OStage(64, 4, 32, 32768, 1), OStage(64, 1, 8, 8192, 1)]
+
+
+@dataclass
+class OArgs:
+    """The subset of HiPAttentionArgs the oracle models (attention_metadata.py:134-215)."""
+    sink_token_size: int = 256
+    sliding_window_size: int = 512
+    block_size_k: int = 64  # BLOCK_CHUNK
+    second_stage_k: int = 2048
+    stages: List[OStage] = field(default_factory=default_stages)
+    model_context_length: int = 131072
+    extend_context_length: int = 512 * 1024
+    block_sparse_block_size_q: Optional[int] = 64
+    stage_early_terminate: int = 1
+    disable_flashdecode: bool = False
+    head_reduce: bool = True  # env HIP_HEAD_REDUCE, default on (attention_extend.py:2566)
+    mask_only: bool = False
+
+
+@dataclass
+class OInputs:
+    dtype: str  # "f32" | "bf16"
+    q: np.ndarray  # [B,TDST,HEAD,HID] float32, or uint16 bits for bf16
+    pos: np.ndarray  # [B,TDST] int64
+    k: Optional[np.ndarray] = None  # [B,TSRC,HKV,HID]
+    v: Optional[np.ndarray] = None
+    k_cache: Optional[np.ndarray] = None  # [pages,page,HKV,HID]
+    v_cache: Optional[np.ndarray] = None
+    block_table: Optional[np.ndarray] = None  # [B,cols] int64
+    cache_seq_lens: Optional[np.ndarray] = None  # [B] int64
+
+    def c_struct(self, max_tsrc: int):
+        np_t = np.uint16 if self.dtype == "bf16" else np.float32
+        keep = []
+
+        def arr(a, t):
+            if a is None:
+                return None
+            a = np.ascontiguousarray(a, dtype=t)
+            keep.append(a)
+            return a.ctypes.data
+
+        B, TDST, HEAD, HID = self.q.shape
+        S = _Tensors()
+        S.dtype = 1 if self.dtype == "bf16" else 0
+        S.B, S.TDST, S.HEAD, S.HID = B, TDST, HEAD, HID
+        S.q = arr(self.q, np_t)
+        S.pos = arr(self.pos, np.int64)
+        if self.k is not None:
+            S.HKV = self.k.shape[2]
+            S.TSRC = self.k.shape[1]
+            S.k = arr(self.k, np_t)
+            S.v = arr(self.v if self.v is not None else self.k, np_t)
+            S.page_size = 1
+        else:
+            S.HKV = self.k_cache.shape[2]
+            S.TSRC = 0
+            S.k = None
+            S.v = None
+            S.k_cache = arr(self.k_cache, np_t)
+            S.v_cache = arr(self.v_cache if self.v_cache is not None else self.k_cache, np_t)
+            S.page_size = self.k_cache.shape[1]
+            S.block_table = arr(self.block_table, np.int64)
+            S.bt_cols = self.block_table.shape[1]
+            S.cache_seq_lens = arr(self.cache_seq_lens, np.int64)
+        S.MAX_TSRC = max_tsrc
+        return S, keep
+
+
+def cdiv(a, b):
+    return -(-a // b)
+
+
+def npow2(x: int) -> int:
+    return 1 if x <= 1 else 1 << (int(x) - 1).bit_length()
+
+
+def topk_order(scores: np.ndarray, k: int) -> np.ndarray:
+    """Positions of the k best entries along the last axis under (score desc, position asc)."""
+    order = np.argsort(-scores.astype(np.float64), axis=-1, kind="stable")
+    return order[..., :k]
+
+
+# ------------------------------------------------------------------ kernels
+
+def mask_stage(X: OInputs, max_tsrc, left, right, scores, BS, BQ, stride_q, block_chunk,
+               scan_stride, sw_eff, terminate=1):
+    """In-place scan of one stage; arrays as in the reference: int64 [B,BS,HEAD,n], f32 scores."""
+    assert left.dtype == np.int64 and right.dtype == np.int64 and scores.dtype == np.float32
+    assert left.flags.c_contiguous and right.flags.c_contiguous and scores.flags.c_contiguous
+    S, keep = X.c_struct(max_tsrc)
+    n = left.shape[-1]
+    rc = lib().hipo_mask_stage(ctypes.byref(S), ctypes.c_void_p(left.ctypes.data),
+                               ctypes.c_void_p(right.ctypes.data), ctypes.c_void_p(scores.ctypes.data),
+                               ctypes.c_int(n), ctypes.c_int(scores.shape[-1]), ctypes.c_int(BS),
+                               ctypes.c_int(BQ), ctypes.c_int(stride_q), ctypes.c_int(block_chunk),
+                               ctypes.c_int(scan_stride), ctypes.c_int(sw_eff), ctypes.c_int(terminate))
+    if rc != 0:
+        raise RuntimeError(f"hipo_mask_stage failed: {rc}")
+    del keep
+
+
+def bsa(X: OInputs, max_tsrc, indices, ks_start_end, block_size_q, block_size_k, sw, sink,
+        share_first_head=False):
+    """Block-sparse attention given indices; returns context with q's shape and dtype."""
+    S, keep = X.c_struct(max_tsrc)
+    indices = np.ascontiguousarray(indices, dtype=np.int64)
+    kse = np.ascontiguousarray(ks_start_end, dtype=np.int32)
+    out = np.zeros(X.q.shape, dtype=np.uint16 if X.dtype == "bf16" else np.float32)
+    rc = lib().hipo_bsa(ctypes.byref(S), ctypes.c_void_p(indices.ctypes.data), ctypes.c_void_p(kse.ctypes.data),
+                        ctypes.c_int(indices.shape[1]), ctypes.c_int(indices.shape[2]),
+                        ctypes.c_int(block_size_q), ctypes.c_int(block_size_k), ctypes.c_int(sw),
+                        ctypes.c_int(sink), ctypes.c_int(1 if share_first_head else 0),
+                        ctypes.c_void_p(out.ctypes.data))
+    if rc != 0:
+        raise RuntimeError(f"hipo_bsa failed: {rc}")
+    del keep
+    return out
+
+
+# ------------------------------------------------------------------ driver
+
+@dataclass
+class OStageCache:
+    indices_left: Optional[np.ndarray]
+    indices_right: Optional[np.ndarray]
+    out_scores: Optional[np.ndarray]
+
+
+@dataclass
+class OMetadata:
+    indices: Optional[np.ndarray]
+    ks: Optional[np.ndarray]
+    ks_count: Optional[np.ndarray]
+    ks_start_end: Optional[np.ndarray]
+    stage_caches: Optional[List[OStageCache]]
+
+
+def hip_attention_12(X: OInputs, A: OArgs, cached: Optional[OMetadata] = None):
+    """Restatement of dual_stage_quadratic_hip_attention (attention_extend.py:1918-3133)."""
+    B, TDST, HEAD, HID = X.q.shape
+    if X.k is not None:
+        TSRC = X.k.shape[1]
+        MAX_TSRC = TSRC
+    else:
+        MAX_TSRC = A.extend_context_length
+        TSRC = MAX_TSRC
+    stages = A.stages
+    assert len(stages) > 0
+    STAGE_STRIDE = stages[0].stage_stride
+    BQ = stages[0].stage_block_size_q
+    BDST = cdiv(TDST, BQ)
+    BS = cdiv(BDST, STAGE_STRIDE)
+    BLOCK_CHUNK = A.block_size_k
+    chunk = stages[0].stage_chunk_size
+    n = cdiv(max(0, MAX_TSRC - A.sink_token_size - A.sliding_window_size), chunk)  # :1971-1973
+
+    mask_k = stages[0].stage_chunk_size  # :1976
+    sw_orig = A.sliding_window_size
+    sw_eff = max(0, sw_orig - mask_k)  # :1978
+    sink = A.sink_token_size
+    pos = np.ascontiguousarray(X.pos, dtype=np.int64)
+    assert pos.shape == (B, TDST)
+
+    stage_caches = [] if (cached is None or cached.stage_caches is None) else cached.stage_caches
+
+    if cached is None or cached.indices is None:
+        fresh = cached is None or cached.stage_caches is None
+        # A cache holding only the (empty) stage-0 entry carries no tensors: the reference would fail on
+        # None.clone() (attention_extend.py:2052-2056) although its own replay test passes such a list
+        # (tests/v1_2/test_gen3_stage_caching.py:170-181); treated here as a fresh start.
+        if not fresh and stage_caches[-1].indices_left is None:
+            assert len(stage_caches) == 1
+            fresh = True
+        if fresh:
+            left = np.zeros((B, BS, HEAD, n), dtype=np.int64)
+            left[...] = (np.floor(np.arange(n, dtype=np.float64) * chunk + sink)).astype(np.int64)
+            right = np.minimum(left + chunk, MAX_TSRC - sw_eff)
+            scores = np.full((B, BS, HEAD, npow2(n)), -32000.0, dtype=np.float32)
+        else:
+            assert len(stage_caches) <= len(stages)
+            last = stage_caches[-1]
+            left = last.indices_left.copy()
+            right = last.indices_right.copy()
+            scores = last.out_scores.copy()
+
+        for i, st in enumerate(stages):
+            if i < len(stage_caches) - 1:
+                continue
+            elif i == len(stage_caches) - 1:
+                pass
+            elif i > 0:
+                assert st.stage_k % chunk == 0
+                kk = st.stage_k // chunk
+                left = left[..., :kk]
+                left = (left - sink) // chunk * chunk + sink  # realign :2077-2080
+                right = left + chunk
+                scores = scores[..., :kk].copy()
+                scores.fill(-32000.0)
+                order = np.argsort(left, axis=-1, kind="stable")
+                left = np.take_along_axis(left, order, -1)
+                right = np.take_along_axis(right, order, -1)
+                scores = np.take_along_axis(scores, order, -1)
+                if BQ != st.stage_block_size_q:
+                    assert BQ > st.stage_block_size_q and BQ % st.stage_block_size_q == 0
+                    num_split = BQ // st.stage_block_size_q
+                    BQ = st.stage_block_size_q
+                    BDST = cdiv(TDST, BQ)
+                    BS = cdiv(BDST, STAGE_STRIDE)
+                    left = np.repeat(left, num_split, 1)[:, -BDST:]
+                    right = np.repeat(right, num_split, 1)[:, -BDST:]
+                    scores = np.repeat(scores, num_split, 1)[:, -BDST:]
+                if STAGE_STRIDE != st.stage_stride:
+                    assert st.stage_stride < STAGE_STRIDE
+                    rep = STAGE_STRIDE // st.stage_stride
+                    left = np.repeat(left, rep, 1)[:, -BDST:]
+                    right = np.repeat(right, rep, 1)[:, -BDST:]
+                    scores = np.repeat(scores, rep, 1)[:, -BDST:]
+                    STAGE_STRIDE = st.stage_stride
+                    BS = cdiv(BDST, STAGE_STRIDE)
+                assert chunk % st.stage_chunk_size == 0
+                splits = chunk // st.stage_chunk_size
+                w = np.maximum((right - left).astype(np.float32) / np.float32(splits), np.float32(0))
+                ar = np.arange(splits, dtype=np.float32)
+                left = (left[..., None] + np.floor(ar * w[..., None]).astype(np.int64)).reshape(*left.shape[:-1], -1)
+                right = (right[..., None] - np.floor((np.float32(splits - 1) - ar) * w[..., None]).astype(np.int64)
+                         ).reshape(*right.shape[:-1], -1)
+                scores = np.repeat(scores, splits, -1)
+            else:
+                assert st.stage_k is None, "first stage always quadratic"
+                STAGE_STRIDE = st.stage_stride
+
+            if i >= len(stage_caches):
+                if i == 0:
+                    stage_caches.append(OStageCache(None, None, None))
+                else:
+                    stage_caches.append(OStageCache(left.copy(), right.copy(), scores.copy()))
+
+            chunk = st.stage_chunk_size
+            n = left.shape[-1]
+            BLOCK_CHUNK = max(16, npow2(min(n, BLOCK_CHUNK)))  # :2194
+            left = np.ascontiguousarray(left)
+            right = np.ascontiguousarray(right)
+            scores = np.ascontiguousarray(scores)
+            mask_stage(X, MAX_TSRC, left, right, scores, BS=left.shape[1], BQ=BQ,
+                       stride_q=st.stage_block_stride_q, block_chunk=BLOCK_CHUNK,
+                       scan_stride=STAGE_STRIDE, sw_eff=sw_eff, terminate=A.stage_early_terminate)
+            if A.head_reduce:
+                scores = np.broadcast_to(scores.max(axis=2, keepdims=True), scores.shape).copy()
+            if i < len(stages) - 1:
+                kk = min(stages[i + 1].stage_k // st.stage_chunk_size, n)
+                order = topk_order(scores[..., :n], kk)
+            else:
+                order = topk_order(scores[..., :n], n)
+            left = np.take_along_axis(left, order, -1)
+            right = np.take_along_axis(right, order, -1)
+
+        if STAGE_STRIDE > 1:
+            left = np.repeat(left, STAGE_STRIDE, 1)[:, -BDST:]
+            right = np.repeat(right, STAGE_STRIDE, 1)[:, -BDST:]
+
+        assert A.second_stage_k % chunk == 0
+        indices = left[..., : A.second_stage_k // chunk] // chunk * chunk  # :2772-2776
+
+        block_size_q = stages[-1].stage_block_size_q
+        bsbq = min(A.block_sparse_block_size_q, block_size_q) if A.block_sparse_block_size_q is not None else None
+        sw_bsa = sw_eff + mask_k  # :2901
+        block_size_k = chunk
+
+        indices = indices.transpose(0, 2, 1, 3).reshape(B * HEAD, indices.shape[1], -1)  # :2907
+        indices = np.sort(indices, axis=-1)
+        indices = indices // block_size_k * block_size_k
+        uniq = np.roll(indices, 1, axis=-1) != indices  # :2912
+        indices = np.where(uniq, indices, INT64_MAX)
+        indices = np.sort(indices, axis=-1)
+        first_pos = np.repeat(pos[:, ::block_size_q, None], HEAD, axis=0)
+        active = indices < (first_pos + block_size_q)
+        ks = active.astype(np.int32).sum(-1).astype(np.int64)
+        ks_count = ks[..., None]
+        ks_start_end = np.zeros((ks.shape[0], ks.shape[1], 2), dtype=np.int32)
+        ks_start_end[:, :, 1] = ks
+
+        if bsbq is not None and cdiv(TDST, bsbq) != cdiv(TDST, block_size_q):  # :3036-3051
+            assert BQ % bsbq == 0
+            rep = BQ // bsbq
+            indices = np.repeat(indices, rep, 1)
+            ks = np.repeat(ks, rep, 1)
+            ks_count = np.repeat(ks_count, rep, 1)
+            ks_start_end = np.repeat(ks_start_end, rep, 1)
+            block_size_q = bsbq
+        if A.mask_only:
+            return None, None
+    else:
+        sw_bsa = sw_eff + mask_k
+        block_size_k = stages[-1].stage_chunk_size
+        block_size_q = 64  # HiPAttentionArgs.block_size_q default, untouched on this path (:3056-3066)
+        indices = cached.indices.copy()
+        ks = cached.ks.copy()
+        ks_count = cached.ks_count.copy()
+        ks_start_end = cached.ks_start_end.copy()
+
+    block_size_q = min(block_size_q, npow2(TDST))  # :3068
+    if sw_bsa == 777:  # :3070-3076
+        sw_bsa = A.model_context_length - sink - A.second_stage_k - block_size_q
+
+    decode = (TDST == 1) and (not A.disable_flashdecode)
+    context = bsa(X, MAX_TSRC, indices, ks_start_end, block_size_q, block_size_k, sw_bsa, sink,
+                  share_first_head=decode)
+    meta = OMetadata(indices=indices, ks=ks, ks_count=ks_count, ks_start_end=ks_start_end,
+                     stage_caches=stage_caches)
+    return context, meta

@@ -1,0 +1,404 @@
+/*
+ * CPU oracle for HiP / InfiniteHiP attention (v1.2 algorithm).
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file restates, on the CPU, the arithmetic of the
+ * reference's Triton kernels so that the HIP kernels can be checked against it.  Nothing
+ * in the shipped package links, loads or calls it; only tests, the smoke check and the
+ * benchmark's cpu_baseline leg do.
+ *
+ * Reference files restated here (paths relative to the reference repository root):
+ *   mask stage          src/hip_attn/v1_2/attention_extend.py:412-1249
+ *   key row gather      src/hip_attn/v1_2/uvm_gpu_cache.py:843-890,1034-1042
+ *   sparse attention    src/hip_attn/v1_2/attention_extend_bsa.py:496-565,727-795,
+ *                       858-899,1133-1138,1370-1379,1623-1638
+ *   decode head sharing src/hip_attn/v1_2/attention_decode_bsa.py:135-152
+ *
+ * Numeric conventions (the "canonical" arithmetic both sides implement):
+ *   T      = element type of q (f32, or bf16 with round-to-nearest-even)
+ *   c_q    = T( fl(sqrt(HID)) / fl(sqrt(fl(sqrt(HID)))) ),  c_k = T( 1 / fl(sqrt(fl(sqrt(HID)))) )
+ *   q^     = T( q * c_q ),  k^ = T( k * c_k )            (products formed in f32)
+ *   dot    = f32 dot product in a fixed order: HID is cut into 16 contiguous segments, each
+ *            segment is an FMA chain starting from +0, the 16 partial sums are combined by
+ *            a balanced binary tree that adds adjacent partials first.  The reference leaves
+ *            the order to Triton's tl.dot; fixing it makes scores reproducible bit for bit.
+ *   score  = T( dot ) widened back to f32.
+ * Dense key reads at t >= TSRC return a zero row (the reference reads out of bounds there).
+ *
+ * Parity status: the reference ships no golden vectors for this path.  The functions here
+ * are pinned by closed forms and brute-force checks in tests/ (see each function's comment);
+ * hipo_mask_stage on multi-level hierarchies is pinned to this restatement of the source,
+ * not to an execution of the Triton build: parity unpinned against the running reference.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define HIPO_F32 0
+#define HIPO_BF16 1
+
+typedef struct {
+    int dtype;               /* HIPO_F32 / HIPO_BF16 (q, k, v, caches all share it) */
+    int B, TDST, HEAD, HKV, HID;
+    const void *q;           /* [B, TDST, HEAD, HID] contiguous */
+    const int64_t *pos;      /* [B, TDST] 0-based positions */
+    /* dense KV (k == NULL -> paged) */
+    const void *k;           /* [B, TSRC, HKV, HID] */
+    const void *v;
+    int64_t TSRC;
+    /* paged KV */
+    const void *k_cache;     /* [pages, page_size, HKV, HID] */
+    const void *v_cache;
+    int page_size;
+    const int64_t *block_table; /* [B, bt_cols] */
+    int64_t bt_cols;
+    const int64_t *cache_seq_lens; /* [B] */
+    int64_t MAX_TSRC;        /* TSRC (dense) or extend_context_length (paged) */
+} hipo_tensors_t;
+
+/* ---------------------------------------------------------------- scalar helpers */
+
+static inline float bf16_bits_to_f32(uint16_t h) {
+    uint32_t u = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+static inline uint16_t f32_to_bf16_bits(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+static inline float round_T(float f, int dtype) {
+    return dtype == HIPO_BF16 ? bf16_bits_to_f32(f32_to_bf16_bits(f)) : f;
+}
+
+static inline float load_T(const void *base, int64_t i, int dtype) {
+    if (dtype == HIPO_BF16) return bf16_bits_to_f32(((const uint16_t *)base)[i]);
+    return ((const float *)base)[i];
+}
+
+static inline void store_T(void *base, int64_t i, float x, int dtype) {
+    if (dtype == HIPO_BF16) ((uint16_t *)base)[i] = f32_to_bf16_bits(x);
+    else ((float *)base)[i] = x;
+}
+
+/* exported so tests can check the rounding helpers against torch */
+float hipo_round_bf16(float f) { return round_T(f, HIPO_BF16); }
+
+void hipo_scale_constants(int HID, int dtype, float *c_q, float *c_k) {
+    volatile float s = sqrtf((float)HID);
+    volatile float ss = sqrtf(s);
+    volatile float cq = s / ss;
+    volatile float ck = 1.0f / ss;
+    *c_q = round_T(cq, dtype);
+    *c_k = round_T(ck, dtype);
+}
+
+/* canonical f32 dot: 16 segments, FMA chain per segment, balanced adjacent-pair tree */
+float hipo_dot(const float *a, const float *b, int HID) {
+    float part[16];
+    int seg = HID / 16;
+    for (int s = 0; s < 16; s++) {
+        float acc = 0.0f;
+        for (int e = 0; e < seg; e++) acc = fmaf(a[s * seg + e], b[s * seg + e], acc);
+        part[s] = acc;
+    }
+    for (int w = 1; w < 16; w *= 2)
+        for (int i = 0; i < 16; i += 2 * w) part[i] = part[i] + part[i + w];
+    return part[0];
+}
+
+/* fetch one key/value row, already widened to f32 (no scaling) -- uvm_gpu_cache.py:843-890,1034-1042 */
+static void fetch_row(const hipo_tensors_t *X, int want_v, int b, int64_t t, int kvh, float *out) {
+    int HID = X->HID;
+    if (X->k != NULL) {
+        const void *base = want_v ? X->v : X->k;
+        if (t < 0 || t >= X->TSRC) {
+            for (int d = 0; d < HID; d++) out[d] = 0.0f;
+            return;
+        }
+        int64_t off = (((int64_t)b * X->TSRC + t) * X->HKV + kvh) * HID;
+        for (int d = 0; d < HID; d++) out[d] = load_T(base, off + d, X->dtype);
+    } else {
+        const void *base = want_v ? X->v_cache : X->k_cache;
+        int64_t seq_len = X->cache_seq_lens[b];
+        int64_t page = 0;
+        if (t >= 0 && t < seq_len) page = X->block_table[(int64_t)b * X->bt_cols + t / X->page_size];
+        int64_t offp = t % X->page_size;
+        int64_t off = ((page * X->page_size + offp) * X->HKV + kvh) * HID;
+        for (int d = 0; d < HID; d++) out[d] = load_T(base, off + d, X->dtype);
+    }
+}
+
+static void scaled_key(const hipo_tensors_t *X, int b, int64_t t, int kvh, float c_k, float *out) {
+    fetch_row(X, 0, b, t, kvh, out);
+    for (int d = 0; d < X->HID; d++) out[d] = round_T(out[d] * c_k, X->dtype);
+}
+
+/* ---------------------------------------------------------------- mask stage
+ * One call = one launch of the reference's scan kernel for one stage.
+ * left/right: int64 [B, BS, HEAD, n] updated in place; scores: f32 [B, BS, HEAD, score_stride]
+ * updated in place for real lanes of programs that pass the gate.
+ * Pinned by: brute force max-pool for chunk sizes 1 and 2, lane-literal Python version on
+ * random tiny inputs, nesting/width invariants (tests/test_oracle_mask.py).
+ */
+int hipo_mask_stage(const hipo_tensors_t *X, int64_t *left, int64_t *right, float *scores,
+                    int n, int score_stride, int BS, int BQ, int stride_q, int block_chunk,
+                    int scan_stride, int sw_eff, int terminate_size) {
+    const int B = X->B, TDST = X->TDST, HEAD = X->HEAD, HID = X->HID;
+    const int G = HEAD / X->HKV;
+    const int BDST = (TDST + BQ - 1) / BQ;
+    const int nrows = BQ / stride_q;
+    const int ngroups = (n + block_chunk - 1) / block_chunk;
+    if (nrows <= 0 || HID % 16 != 0 || block_chunk > 1024) return -1;
+    float c_q, c_k;
+    hipo_scale_constants(HID, X->dtype, &c_q, &c_k);
+    const int64_t MAXT = X->MAX_TSRC;
+
+    long total = (long)B * HEAD * BS;
+#pragma omp parallel
+    {
+        float *qhat = (float *)malloc(sizeof(float) * nrows * HID);
+        float *kbuf = (float *)malloc(sizeof(float) * HID);
+        int *rowvalid = (int *)malloc(sizeof(int) * nrows);
+        int32_t *l = (int32_t *)malloc(sizeof(int32_t) * block_chunk);
+        int32_t *r = (int32_t *)malloc(sizeof(int32_t) * block_chunk);
+        float *sc = (float *)malloc(sizeof(float) * block_chunk);
+#pragma omp for schedule(dynamic, 1)
+        for (long job = 0; job < total; job++) {
+            int s = (int)(job % BS);
+            int h = (int)((job / BS) % HEAD);
+            int b = (int)(job / ((long)BS * HEAD));
+            /* rows of this program: attention_extend.py:535-552 */
+            int64_t qb = (int64_t)(BDST - 1) - (int64_t)(BS - 1) * scan_stride + (int64_t)s * scan_stride;
+            int64_t pmin = INT64_MAX;
+            int nvalid = 0;
+            for (int j = 0; j < nrows; j++) {
+                int64_t it = qb * BQ + (int64_t)j * stride_q;
+                rowvalid[j] = (it < TDST) && (it >= 0);
+                if (rowvalid[j]) {
+                    int64_t p = X->pos[(int64_t)b * TDST + it];
+                    if (p < pmin) pmin = p;
+                    nvalid++;
+                }
+            }
+            if (nvalid == 0) continue; /* :563-568 */
+            if (pmin < 0) continue;
+            int32_t lim = (int32_t)(pmin - sw_eff);
+            if (lim < 0) lim = 0;
+            /* strided mean of query rows, then scale: :607-734, :924-931 */
+            for (int j = 0; j < nrows; j++) {
+                int64_t it = qb * BQ + (int64_t)j * stride_q;
+                for (int d = 0; d < HID; d++) {
+                    float sum = 0.0f;
+                    int cnt = 0;
+                    for (int o = 0; o < stride_q; o++) {
+                        int64_t iti = it + o;
+                        if (rowvalid[j] && iti < TDST) {
+                            sum += load_T(X->q, (((int64_t)b * TDST + iti) * HEAD + h) * HID + d, X->dtype);
+                            cnt++;
+                        }
+                    }
+                    float mean = sum / ((float)cnt + 1e-12f);
+                    if (!rowvalid[j]) mean = 0.0f;
+                    mean = round_T(mean, X->dtype);
+                    qhat[j * HID + d] = round_T(mean * c_q, X->dtype);
+                }
+            }
+            for (int g = 0; g < ngroups; g++) {
+                int64_t rowoff = (((int64_t)b * BS + s) * HEAD + h);
+                int32_t minl = INT32_MAX;
+                int32_t maxw = INT32_MIN;
+                for (int lane = 0; lane < block_chunk; lane++) {
+                    int c = g * block_chunk + lane;
+                    if (c < n) {
+                        l[lane] = (int32_t)left[rowoff * n + c];
+                        r[lane] = (int32_t)right[rowoff * n + c];
+                    } else {
+                        l[lane] = (int32_t)MAXT;
+                        r[lane] = (int32_t)MAXT;
+                    }
+                    if (l[lane] < minl) minl = l[lane];
+                    if (r[lane] - l[lane] > maxw) maxw = r[lane] - l[lane];
+                    sc[lane] = -32000.0f;
+                }
+                /* gate :595-597 */
+                if (!(pmin + (int64_t)BQ * scan_stride >= (int64_t)minl)) continue;
+                float width = (float)maxw;
+                while (width >= (float)terminate_size) { /* :736-737 */
+                    width /= 2.0f;
+                    for (int lane = 0; lane < block_chunk; lane++) {
+                        int c = g * block_chunk + lane;
+                        int active = (c < n) && (l[lane] < r[lane]) && (l[lane] <= lim) && (l[lane] >= 0);
+                        if (!active) continue;
+                        int32_t ctr = (l[lane] + r[lane]) / 2;
+                        int32_t tl_ = (l[lane] + ctr) / 2;
+                        int32_t tr_ = (ctr + r[lane]) / 2;
+                        float sL = -INFINITY, sR = -INFINITY;
+                        scaled_key(X, b, tl_, h / G, c_k, kbuf);
+                        for (int j = 0; j < nrows; j++) {
+                            if (!rowvalid[j]) continue;
+                            float v = round_T(hipo_dot(qhat + j * HID, kbuf, HID), X->dtype);
+                            if (v > sL) sL = v;
+                        }
+                        scaled_key(X, b, tr_, h / G, c_k, kbuf);
+                        for (int j = 0; j < nrows; j++) {
+                            if (!rowvalid[j]) continue;
+                            float v = round_T(hipo_dot(qhat + j * HID, kbuf, HID), X->dtype);
+                            if (v > sR) sR = v;
+                        }
+                        int win = sL > sR; /* :1183 */
+                        if (win) r[lane] = ctr; else l[lane] = ctr;
+                        float ws = win ? sL : sR;
+                        if (ws > sc[lane]) sc[lane] = ws; /* :1204-1215 */
+                    }
+                }
+                for (int lane = 0; lane < block_chunk; lane++) {
+                    int c = g * block_chunk + lane;
+                    if (c >= n) continue;
+                    left[rowoff * n + c] = l[lane];
+                    right[rowoff * n + c] = r[lane];
+                    scores[rowoff * score_stride + c] = sc[lane];
+                }
+            }
+        }
+        free(qhat); free(kbuf); free(rowvalid); free(l); free(r); free(sc);
+    }
+    return 0;
+}
+
+/* ---------------------------------------------------------------- block sparse attention
+ * Attended set of a query row at position p inside a query block whose largest position+1
+ * is CURR (attention_extend_bsa.py:511-523,881-891,1137,1371-1379):
+ *   selected blocks j < min(BK, ks_end): tokens t with 0<=t<MAX_TSRC, sink<=t<CURR, t+sw<=p
+ *   sink:   t < min(CURR, sink), t+sw<=p
+ *   window: max(0,CURR-sw-BQ) <= t < CURR,  t<=p<t+sw
+ * Softmax in base 2 over f32 logits, probabilities rounded to T before the value product
+ * (:531-558).  Rows with an empty set give 0 (l stays at its initial 1.0, :764,1625).
+ * share_first_head != 0 uses, for every head of a GQA group, the index row of the group's
+ * first head, as the decode kernel does (attention_decode_bsa.py:150).
+ * Pinned by: dense masked softmax in f64 built from the set definition above
+ * (tests/test_oracle_bsa.py), StreamingLLM and plain-causal special cases.
+ */
+int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_start_end,
+             int NBQ_rows /* rows of indices per (b,h) */, int BK, int block_size_q,
+             int block_size_k, int sw, int sink, int share_first_head, void *out) {
+    const int B = X->B, TDST = X->TDST, HEAD = X->HEAD, HID = X->HID;
+    const int G = HEAD / X->HKV;
+    const int NBQ = (TDST + block_size_q - 1) / block_size_q;
+    if (NBQ > NBQ_rows) return -2;
+    float c_q, c_k;
+    hipo_scale_constants(HID, X->dtype, &c_q, &c_k);
+    const int64_t MAXT = X->MAX_TSRC;
+    long total = (long)B * HEAD * NBQ;
+    int cap = BK * block_size_k + sink + sw + block_size_q + 8;
+#pragma omp parallel
+    {
+        int64_t *tok = (int64_t *)malloc(sizeof(int64_t) * cap);
+        int *kind = (int *)malloc(sizeof(int) * cap); /* 0: excluded-window rule, 1: window rule */
+        float *khat = (float *)malloc(sizeof(float) * (size_t)cap * HID);
+        float *vrow = (float *)malloc(sizeof(float) * (size_t)cap * HID);
+        float *qhat = (float *)malloc(sizeof(float) * HID);
+        float *logit = (float *)malloc(sizeof(float) * cap);
+        double *acc = (double *)malloc(sizeof(double) * HID);
+#pragma omp for schedule(dynamic, 1)
+        for (long job = 0; job < total; job++) {
+            int qb = (int)(job % NBQ);
+            int h = (int)((job / NBQ) % HEAD);
+            int b = (int)(job / ((long)NBQ * HEAD));
+            int kvh = h / G;
+            int hrow = share_first_head ? (h / G) * G : h;
+            int64_t irow = ((int64_t)b * HEAD + hrow) * NBQ_rows + qb;
+            int64_t curr = 0;
+            for (int j = 0; j < block_size_q; j++) {
+                int64_t it = (int64_t)qb * block_size_q + j;
+                if (it < TDST) {
+                    int64_t sl = X->pos[(int64_t)b * TDST + it] + 1;
+                    if (sl > curr) curr = sl;
+                }
+            }
+            int nt = 0;
+            int rs = ks_start_end[irow * 2 + 0], re = ks_start_end[irow * 2 + 1];
+            if (BK <= 0) { rs = 0; re = 0; }
+            for (int j = rs; j < rs + BK && j < re; j++) {
+                int64_t st = indices[irow * BK + j];
+                for (int e = 0; e < block_size_k; e++) {
+                    int64_t t = st + e;
+                    if (t < 0 || t >= MAXT) continue;
+                    if (!(t < curr && t >= sink)) continue;
+                    tok[nt] = t; kind[nt] = 0; nt++;
+                }
+            }
+            int64_t sink_end = curr < sink ? curr : sink;
+            for (int64_t t = 0; t < sink_end; t++) { tok[nt] = t; kind[nt] = 0; nt++; }
+            if (sw > 0) {
+                int64_t ws = curr - sw - block_size_q;
+                if (ws < 0) ws = 0;
+                for (int64_t t = ws; t < curr; t++) { tok[nt] = t; kind[nt] = 1; nt++; }
+            }
+            for (int i = 0; i < nt; i++) {
+                scaled_key(X, b, tok[i], kvh, c_k, khat + (size_t)i * HID);
+                fetch_row(X, 1, b, tok[i], kvh, vrow + (size_t)i * HID);
+            }
+            for (int j = 0; j < block_size_q; j++) {
+                int64_t it = (int64_t)qb * block_size_q + j;
+                if (it >= TDST) continue;
+                int64_t p = X->pos[(int64_t)b * TDST + it];
+                int64_t qoff = (((int64_t)b * TDST + it) * HEAD + h) * HID;
+                for (int d = 0; d < HID; d++)
+                    qhat[d] = round_T(load_T(X->q, qoff + d, X->dtype) * c_q, X->dtype);
+                float m = -INFINITY;
+                for (int i = 0; i < nt; i++) {
+                    int64_t t = tok[i];
+                    int att = kind[i] == 0 ? (t + sw <= p) : (t <= p && p < t + sw);
+                    if (!att) { logit[i] = -INFINITY; continue; }
+                    logit[i] = hipo_dot(qhat, khat + (size_t)i * HID, HID) * 1.44269504f;
+                    if (logit[i] > m) m = logit[i];
+                }
+                double lsum = 0.0;
+                for (int d = 0; d < HID; d++) acc[d] = 0.0;
+                if (m > -INFINITY) {
+                    for (int i = 0; i < nt; i++) {
+                        if (logit[i] == -INFINITY) continue;
+                        float pr = exp2f(logit[i] - m);
+                        lsum += (double)pr;
+                        float prT = round_T(pr, X->dtype);
+                        const float *vr = vrow + (size_t)i * HID;
+                        for (int d = 0; d < HID; d++) acc[d] += (double)prT * (double)vr[d];
+                    }
+                } else {
+                    lsum = 1.0;
+                }
+                if (lsum == 0.0) lsum = 1e-20;
+                for (int d = 0; d < HID; d++) store_T(out, qoff + d, (float)(acc[d] / lsum), X->dtype);
+            }
+        }
+        free(tok); free(kind); free(khat); free(vrow); free(qhat); free(logit); free(acc);
+    }
+    return 0;
+}
+
+int hipo_num_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+void hipo_set_num_threads(int n) {
+#ifdef _OPENMP
+    omp_set_num_threads(n);
+#else
+    (void)n;
+#endif
+}

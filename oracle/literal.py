@@ -1,0 +1,138 @@
+"""Lane-literal, pure-Python restatement of one scan stage -- TEST INFRASTRUCTURE ONLY.
+
+A second, independently written form of ``hipo_mask_stage`` (hip_oracle.c) that walks the
+reference's program/lane structure one lane at a time
+(``src/hip_attn/v1_2/attention_extend.py:516-1249``).  It is slow and meant for tiny shapes;
+tests use it to pin the C oracle.
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+from . import hip12 as O
+
+F = np.float32
+
+
+def _round(x, dtype):
+    x = F(x)
+    if dtype == "bf16":
+        return O.bf16_bits_to_f32(O.f32_to_bf16_bits(np.array([x], dtype=F)))[0]
+    return x
+
+
+def _widen(a, dtype):
+    return O.bf16_bits_to_f32(a) if dtype == "bf16" else np.asarray(a, dtype=F)
+
+
+def dot_canonical(a, b):
+    """16 segments, sequential FMA chain per segment, adjacent-pair tree."""
+    hid = len(a)
+    seg = hid // 16
+    part = []
+    for s in range(16):
+        acc = F(0.0)
+        for e in range(seg):
+            # float64 holds the exact product of two float32 values, so rounding the sum once
+            # to float32 reproduces a fused multiply-add
+            acc = F(np.float64(a[s * seg + e]) * np.float64(b[s * seg + e]) + np.float64(acc))
+        part.append(acc)
+    w = 1
+    while w < 16:
+        for i in range(0, 16, 2 * w):
+            part[i] = F(part[i] + part[i + w])
+        w *= 2
+    return part[0]
+
+
+def key_row(X: O.OInputs, b, t, kvh, max_tsrc):
+    if X.k is not None:
+        if t < 0 or t >= X.k.shape[1]:
+            return np.zeros(X.k.shape[-1], dtype=F)
+        return _widen(X.k[b, t, kvh], X.dtype)
+    P = X.k_cache.shape[1]
+    page = 0
+    if 0 <= t < int(X.cache_seq_lens[b]):
+        page = int(X.block_table[b, t // P])
+    return _widen(X.k_cache[page, t % P, kvh], X.dtype)
+
+
+def mask_stage(X: O.OInputs, max_tsrc, left, right, scores, BQ, stride_q, block_chunk, scan_stride,
+               sw_eff, terminate=1):
+    B, TDST, HEAD, HID = X.q.shape
+    HKV = X.k.shape[2] if X.k is not None else X.k_cache.shape[2]
+    G = HEAD // HKV
+    BS = left.shape[1]
+    n = left.shape[-1]
+    BDST = O.cdiv(TDST, BQ)
+    s_ = F(math.sqrt(HID))
+    s_ = F(np.sqrt(F(HID)))
+    ss = F(np.sqrt(s_))
+    c_q = _round(F(s_ / ss), X.dtype)
+    c_k = _round(F(F(1.0) / ss), X.dtype)
+    qf = _widen(X.q, X.dtype)
+    nrows = BQ // stride_q
+    for b in range(B):
+        for h in range(HEAD):
+            for s in range(BS):
+                qb = (BDST - 1) - (BS - 1) * scan_stride + s * scan_stride
+                rows = [qb * BQ + j * stride_q for j in range(nrows)]
+                valid = [0 <= r < TDST for r in rows]
+                if not any(valid):
+                    continue
+                pmin = min(int(X.pos[b, r]) for r, ok in zip(rows, valid) if ok)
+                if pmin < 0:
+                    continue
+                lim = max(pmin - sw_eff, 0)
+                qhat = []
+                for r, ok in zip(rows, valid):
+                    if not ok:
+                        qhat.append(None)
+                        continue
+                    acc = np.zeros(HID, dtype=F)
+                    cnt = 0
+                    for o in range(stride_q):
+                        if r + o < TDST:
+                            acc = (acc + qf[b, r + o, h]).astype(F)
+                            cnt += 1
+                    mean = (acc / F(F(cnt) + F(1e-12))).astype(F)
+                    mean = np.array([_round(x, X.dtype) for x in mean], dtype=F)
+                    qhat.append(np.array([_round(F(x * c_q), X.dtype) for x in mean], dtype=F))
+                for g in range(O.cdiv(n, block_chunk)):
+                    lanes = list(range(g * block_chunk, (g + 1) * block_chunk))
+                    l = [int(left[b, s, h, c]) if c < n else max_tsrc for c in lanes]
+                    r_ = [int(right[b, s, h, c]) if c < n else max_tsrc for c in lanes]
+                    if not (pmin + BQ * scan_stride >= min(l)):
+                        continue
+                    width = F(max(rr - ll for ll, rr in zip(l, r_)))
+                    sc = [F(-32000.0)] * block_chunk
+                    while width >= terminate:
+                        width = F(width / F(2.0))
+                        for i, c in enumerate(lanes):
+                            if not (c < n and l[i] < r_[i] and l[i] <= lim and l[i] >= 0):
+                                continue
+                            ctr = (l[i] + r_[i]) // 2
+                            res = []
+                            for t in ((l[i] + ctr) // 2, (ctr + r_[i]) // 2):
+                                kk = key_row(X, b, t, h // G, max_tsrc)
+                                kh = np.array([_round(F(x * c_k), X.dtype) for x in kk], dtype=F)
+                                best = F(-np.inf)
+                                for qh in qhat:
+                                    if qh is None:
+                                        continue
+                                    best = max(best, _round(dot_canonical(qh, kh), X.dtype))
+                                res.append(best)
+                            if res[0] > res[1]:
+                                r_[i] = ctr
+                                w = res[0]
+                            else:
+                                l[i] = ctr
+                                w = res[1]
+                            sc[i] = max(sc[i], w)
+                    for i, c in enumerate(lanes):
+                        if c < n:
+                            left[b, s, h, c] = l[i]
+                            right[b, s, h, c] = r_[i]
+                            scores[b, s, h, c] = sc[i]

@@ -1,0 +1,139 @@
+"""Pins hipo_bsa against dense masked softmax in float64 and against textbook special cases."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import hip12 as O
+from helpers import make_inputs, to_paged, widen
+
+
+def dense_reference(X, indices, ks, bq, bk, sw, sink, max_tsrc, share_first_head=False):
+    """softmax over the attended set written as an explicit boolean mask, float64 arithmetic.
+
+    Built from the set definition only (no tiling): sink tokens and selected-block tokens at
+    distance >= sw from the query, window tokens at distance < sw, everything clipped by the
+    query block's largest position.
+    """
+    B, TQ, H, D = X.q.shape
+    k = widen(X.k, X.dtype).astype(np.float64)
+    v = widen(X.v, X.dtype).astype(np.float64)
+    TK = k.shape[1]
+    G = H // k.shape[2]
+    cq, ck = O.scale_constants(D, X.dtype)
+    rnd = (lambda a: O.bf16_bits_to_f32(O.f32_to_bf16_bits(a.astype(np.float32))).astype(np.float64)) \
+        if X.dtype == "bf16" else (lambda a: a.astype(np.float32).astype(np.float64))
+    qh = rnd(widen(X.q, X.dtype) * np.float32(cq))
+    kh = rnd(widen(X.k, X.dtype) * np.float32(ck))
+    out = np.zeros((B, TQ, H, D))
+    t = np.arange(TK)
+    for b in range(B):
+        for h in range(H):
+            hrow = (h // G) * G if share_first_head else h
+            for qb in range(O.cdiv(TQ, bq)):
+                rows = np.arange(qb * bq, min(TQ, (qb + 1) * bq))
+                p = X.pos[b, rows]
+                curr = p.max() + 1
+                sel = np.zeros(TK, dtype=bool)
+                for j in range(int(ks[b * H + hrow, qb])):
+                    st = int(indices[b * H + hrow, qb, j])
+                    sel[max(st, 0): max(min(st + bk, TK, max_tsrc), 0)] = True
+                sel &= (t >= sink)
+                far = (t[None, :] + sw <= p[:, None]) & (t[None, :] < curr)
+                near = (t[None, :] <= p[:, None]) & (t[None, :] + sw > p[:, None]) & \
+                       (t[None, :] >= max(0, curr - sw - bq)) & (sw > 0)
+                mask = (far & (sel | (t < sink))[None, :]) | near
+                logits = qh[b, rows, h] @ kh[b, :, h // G].T
+                logits = np.where(mask, logits, -np.inf)
+                m = logits.max(axis=1, keepdims=True)
+                m = np.where(np.isfinite(m), m, 0.0)
+                pr = np.exp(logits - m)
+                den = pr.sum(axis=1, keepdims=True)
+                den = np.where(den == 0, 1.0, den)
+                out[b, rows, h] = (pr / den) @ v[b, :, h // G]
+    return out
+
+
+def random_indices(rng, B, H, nbq, BK, bk, tk, same_heads=True):
+    idx = np.full((B * H, nbq, BK), O.INT64_MAX, dtype=np.int64)
+    ks = np.zeros((B * H, nbq), dtype=np.int64)
+    for b in range(B):
+        for qb in range(nbq):
+            for h in range(H):
+                if same_heads and h > 0:
+                    idx[b * H + h, qb] = idx[b * H, qb]; ks[b * H + h, qb] = ks[b * H, qb]
+                    continue
+                n = int(rng.integers(0, BK + 1))
+                st = np.sort(rng.choice(tk // bk, size=n, replace=False)) * bk
+                idx[b * H + h, qb, :n] = st
+                ks[b * H + h, qb] = n
+    kse = np.zeros((B * H, nbq, 2), dtype=np.int32)
+    kse[..., 1] = ks
+    return idx, ks, kse
+
+
+@pytest.mark.parametrize("dtype,tol", [("f32", 2e-5), ("bf16", 1.5e-2)])
+@pytest.mark.parametrize("bq,TQ", [(16, 40), (1, 1), (64, 64)])
+def test_bsa_equals_dense_masked_softmax(dtype, tol, bq, TQ):
+    rng = np.random.default_rng(2)
+    TK, H, HKV, D, bk, BK, sw, sink = 192, 4, 2, 32, 4, 12, 24, 8
+    X = make_inputs(4, B=2, TQ=TQ, TK=TK, H=H, HKV=HKV, D=D, dtype=dtype, scale=0.3)
+    nbq = O.cdiv(TQ, bq)
+    idx, ks, kse = random_indices(rng, 2, H, nbq, BK, bk, TK, same_heads=False)
+    got = widen(O.bsa(X, TK, idx, kse, bq, bk, sw, sink), dtype)
+    ref = dense_reference(X, idx, ks, bq, bk, sw, sink, TK)
+    assert np.abs(got - ref).max() < tol
+    # decode flavour: every head of a GQA group reads the first head's index row
+    got2 = widen(O.bsa(X, TK, idx, kse, bq, bk, sw, sink, share_first_head=True), dtype)
+    ref2 = dense_reference(X, idx, ks, bq, bk, sw, sink, TK, share_first_head=True)
+    assert np.abs(got2 - ref2).max() < tol
+    assert np.abs(ref2 - ref).max() > 1e-3  # the two flavours really differ on this input
+
+
+def test_no_selected_blocks_is_streaming_attention():
+    # ks = 0 everywhere -> sink + sliding window (StreamingLLM)
+    TK, TQ, H, D, sw, sink, bq = 160, 48, 2, 32, 32, 4, 16
+    X = make_inputs(6, B=1, TQ=TQ, TK=TK, H=H, HKV=2, D=D, dtype="f32", scale=0.3)
+    idx = np.full((H, 3, 4), O.INT64_MAX, dtype=np.int64)
+    kse = np.zeros((H, 3, 2), dtype=np.int32)
+    got = O.bsa(X, TK, idx, kse, bq, 4, sw, sink)
+    q = torch.from_numpy(X.q).permute(0, 2, 1, 3).double()
+    k = torch.from_numpy(X.k).permute(0, 2, 1, 3).double()
+    v = torch.from_numpy(X.v).permute(0, 2, 1, 3).double()
+    p = torch.from_numpy(X.pos[0])[:, None]; t = torch.arange(TK)[None, :]
+    mask = ((t <= p) & (t > p - sw)) | ((t < sink) & (t <= p - sw))
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask[None, None], scale=1.0)
+    assert np.abs(got - ref.permute(0, 2, 1, 3).numpy()).max() < 2e-5
+
+
+def test_huge_window_is_plain_causal_attention():
+    TK, TQ, H, D = 96, 96, 2, 64
+    X = make_inputs(8, B=1, TQ=TQ, TK=TK, H=H, HKV=1, D=D, dtype="f32", scale=0.3)
+    idx = np.full((H, 6, 2), O.INT64_MAX, dtype=np.int64)
+    kse = np.zeros((H, 6, 2), dtype=np.int32)
+    got = O.bsa(X, TK, idx, kse, 16, 2, 4096, 0)
+    q = torch.from_numpy(X.q).permute(0, 2, 1, 3).double()
+    k = torch.from_numpy(X.k).permute(0, 2, 1, 3).double().repeat(1, 2, 1, 1)
+    v = torch.from_numpy(X.v).permute(0, 2, 1, 3).double().repeat(1, 2, 1, 1)
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, scale=1.0)
+    assert np.abs(got - ref.permute(0, 2, 1, 3).numpy()).max() < 2e-5
+
+
+def test_empty_row_gives_zero_and_sink_only_rows():
+    # sw = 0, sink = 0, no blocks: nothing attended -> output 0 (l keeps its initial 1.0)
+    X = make_inputs(9, B=1, TQ=8, TK=32, H=1, HKV=1, D=16, dtype="f32")
+    idx = np.full((1, 1, 1), O.INT64_MAX, dtype=np.int64)
+    kse = np.zeros((1, 1, 2), dtype=np.int32)
+    got = O.bsa(X, 32, idx, kse, 8, 2, 0, 0)
+    assert (got == 0).all()
+
+
+@pytest.mark.parametrize("page_size", [1, 2, 4, 8, 16, 32])
+def test_paged_equals_dense_bit_exact(page_size):
+    rng = np.random.default_rng(3)
+    TK, TQ, H, HKV, D, bk, BK = 128, 32, 4, 2, 32, 4, 6
+    X = make_inputs(10, B=2, TQ=TQ, TK=TK, H=H, HKV=HKV, D=D, dtype="bf16", scale=0.3)
+    idx, ks, kse = random_indices(rng, 2, H, 2, BK, bk, TK)
+    dense = O.bsa(X, TK, idx, kse, 16, bk, 16, 4)
+    XP = to_paged(X, page_size, seed=page_size)
+    paged = O.bsa(XP, 4096, idx, kse, 16, bk, 16, 4)
+    assert np.array_equal(dense, paged)
