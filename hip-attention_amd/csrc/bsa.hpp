@@ -1,0 +1,31 @@
+// Parameter block shared by the block-sparse attention kernels.
+#pragma once
+
+#include "common.hpp"
+
+namespace hipattn {
+
+struct BsaParams {
+    const void *q;
+    int64_t q_sb, q_st, q_sh;
+    const int64_t *pos;
+    int64_t pos_sb, pos_st;
+    KVView kv;
+    const int64_t *indices;
+    const int32_t *kse;
+    int idx_rows, BK, bq, bk, sw, sink, share_first_head;
+    int B, TDST, HEAD, G, NBQ;
+    float c_q, c_k;
+    void *out;
+    int64_t o_sb, o_st, o_sh;
+};
+
+// validates arguments and fills the parameter block (host)
+int bsa_fill_params(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t *indices, const int32_t *kse,
+                    int idx_rows, int BK, int bq, int bk, int sw, int sink, int share_first_head, void *out,
+                    int64_t o_sb, int64_t o_st, int64_t o_sh, BsaParams *p);
+int bsa_simple_launch(const BsaParams &p, int dtype, int HID, hipStream_t st);
+// returns HIPATTN_E_UNSUPPORTED (without setting an error) when the tile kernel does not cover the case
+int bsa_mfma_launch(const BsaParams &p, int dtype, int HID, hipStream_t st);
+
+}  // namespace hipattn

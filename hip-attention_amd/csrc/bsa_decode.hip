@@ -1,0 +1,286 @@
+// Decode (one query token per sequence) block-sparse attention: split-KV partials + merge.
+//
+// A workgroup owns one (sequence, kv head, split) and all G query heads of the GQA group, so every
+// gathered K/V row is read once for the whole group.  Sixteen lanes share a token row (HID/16
+// contiguous elements each: one coalesced 16-lane load per row, four rows per load instruction per
+// wave); each 16-lane group keeps its own online-softmax state and output slice, and the sixteen
+// states of a workgroup are merged through LDS before the partial is written.
+#include "bsa.hpp"
+
+namespace hipattn {
+
+struct DecodeParams {
+    BsaParams a;
+    int nsplits;
+    float *ws;  // [B, HEAD, nsplits, HID + 4]: acc / l, then m + log2(l)
+};
+
+template <typename T, int HID, int G>
+__global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParams dp) {
+    constexpr int SEG = HID / 16;
+    const BsaParams &p = dp.a;
+    __shared__ float s_m[16][G];
+    __shared__ float s_l[16][G];
+    __shared__ float s_acc[16][G][HID];
+
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    const int sub = lane >> 4, dl = lane & 15;
+    const int grp = wid * 4 + sub;  // 16-lane group id inside the workgroup
+    const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+    const int h0 = kvh * G;
+    const int64_t irow = ((int64_t)b * p.HEAD + h0) * p.idx_rows;  // query block 0, first head of the group
+
+    const long long ppos = p.pos[(int64_t)b * p.pos_sb];
+    const long long curr = ppos + 1;
+    int rs = p.kse[irow * 2 + 0], re = p.kse[irow * 2 + 1];
+    if (p.BK <= 0) { rs = 0; re = 0; }
+    const int jend = rs + p.BK < re ? rs + p.BK : re;
+    const int nsel = jend > rs ? jend - rs : 0;
+    const long long n_sel_tok = (long long)nsel * p.bk;
+    const long long sink_end = curr < p.sink ? curr : p.sink;
+    long long ws0 = curr - p.sw - 1;  // block_size_q = 1 for decode
+    if (ws0 < 0) ws0 = 0;
+    const long long n_win = p.sw > 0 ? curr - ws0 : 0;
+    const long long total = n_sel_tok + sink_end + n_win;
+    long long per = (total + dp.nsplits - 1) / dp.nsplits;
+    per = (per + 15) / 16 * 16;
+    const long long o_begin = (long long)split * per;
+    const long long o_end = o_begin + per < total ? o_begin + per : total;
+
+    const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
+    const T *kbase = reinterpret_cast<const T *>(p.kv.k);
+    const T *vbase = reinterpret_cast<const T *>(p.kv.v);
+
+    float qh[G][SEG];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        const T *qrow = reinterpret_cast<const T *>(p.q) + (int64_t)b * p.q_sb + (int64_t)(h0 + g) * p.q_sh;
+        load_elems<T, SEG>(qrow + dl * SEG, qh[g]);
+#pragma unroll
+        for (int e = 0; e < SEG; e++) qh[g][e] = Elem<T>::round(qh[g][e] * p.c_q);
+    }
+    float m[G], l[G], acc[G][SEG];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        m[g] = -INFINITY;
+        l[g] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < SEG; e++) acc[g][e] = 0.0f;
+    }
+
+    for (long long base = o_begin; base < o_end; base += 16) {
+        const long long o = base + grp;
+        long long t = -1;
+        int kind = 0;
+        bool valid = false;
+        if (o < o_end) {
+            if (o < n_sel_tok) {
+                const long long st = p.indices[irow * p.BK + rs + o / p.bk];
+                t = st + o % p.bk;
+                valid = (t >= 0) && (t < p.kv.max_tsrc) && (t < curr) && (t >= p.sink);
+            } else if (o < n_sel_tok + sink_end) {
+                t = o - n_sel_tok;
+                valid = true;
+            } else {
+                t = ws0 + (o - n_sel_tok - sink_end);
+                kind = 1;
+                valid = true;
+            }
+        }
+        const bool att = valid && (kind == 0 ? (t + p.sw <= ppos) : (t <= ppos && ppos < t + p.sw));
+        if (!att) continue;  // uniform inside the 16-lane group; shuffles below stay inside the group
+        const int64_t koff = p.kv.k_row(b, t, kvh, seqlen);
+        const int64_t voff = p.kv.v_row(b, t, kvh, seqlen);
+        float kh[SEG], vv[SEG];
+        if (koff >= 0) {
+            load_elems<T, SEG>(kbase + koff + dl * SEG, kh);
+        } else {
+#pragma unroll
+            for (int e = 0; e < SEG; e++) kh[e] = 0.0f;
+        }
+        if (voff >= 0) {
+            load_elems<T, SEG>(vbase + voff + dl * SEG, vv);
+        } else {
+#pragma unroll
+            for (int e = 0; e < SEG; e++) vv[e] = 0.0f;
+        }
+#pragma unroll
+        for (int e = 0; e < SEG; e++) kh[e] = Elem<T>::round(kh[e] * p.c_k);
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float d = 0.0f;
+#pragma unroll
+            for (int e = 0; e < SEG; e++) d = __fmaf_rn(qh[g][e], kh[e], d);
+            d += __shfl_xor(d, 1);
+            d += __shfl_xor(d, 2);
+            d += __shfl_xor(d, 4);
+            d += __shfl_xor(d, 8);
+            const float x = d * 1.44269504f;
+            const float m_new = fmaxf(m[g], x);
+            const float alpha = exp2f(m[g] - m_new);
+            const float pr = exp2f(x - m_new);
+            l[g] = l[g] * alpha + pr;
+            const float prT = Elem<T>::round(pr);
+#pragma unroll
+            for (int e = 0; e < SEG; e++) acc[g][e] = __fmaf_rn(prT, vv[e], acc[g][e] * alpha);
+            m[g] = m_new;
+        }
+    }
+
+    // merge the 16 group states
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        if (dl == 0) {
+            s_m[grp][g] = m[g];
+            s_l[grp][g] = l[g];
+        }
+#pragma unroll
+        for (int e = 0; e < SEG; e++) s_acc[grp][g][dl * SEG + e] = acc[g][e];
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < G * HID; idx += 256) {
+        const int g = idx / HID, d = idx % HID;
+        float mm = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; i++) mm = fmaxf(mm, s_m[i][g]);
+        float ll = 0.0f, aa = 0.0f;
+        if (mm > -INFINITY) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const float w = exp2f(s_m[i][g] - mm);
+                ll += s_l[i][g] * w;
+                aa += s_acc[i][g][d] * w;
+            }
+        }
+        float *wrow = dp.ws + (((int64_t)b * p.HEAD + h0 + g) * dp.nsplits + split) * (HID + 4);
+        wrow[d] = ll > 0.0f ? aa / ll : 0.0f;
+        if (d == 0) wrow[HID] = ll > 0.0f ? mm + log2f(ll) : -INFINITY;
+    }
+}
+
+template <typename T, int HID>
+__global__ void bsa_decode_merge_kernel(const float *ws, int HEAD, int nsplits, T *out, int64_t o_sb, int64_t o_sh) {
+    const int h = blockIdx.x, b = blockIdx.y;
+    const float *base = ws + ((int64_t)b * HEAD + h) * nsplits * (HID + 4);
+    float mm = -INFINITY;
+    for (int s = 0; s < nsplits; s++) mm = fmaxf(mm, base[(int64_t)s * (HID + 4) + HID]);
+    for (int d = threadIdx.x; d < HID; d += blockDim.x) {
+        float num = 0.0f, den = 0.0f;
+        if (mm > -INFINITY) {
+            for (int s = 0; s < nsplits; s++) {
+                const float w = exp2f(base[(int64_t)s * (HID + 4) + HID] - mm);
+                num += w * base[(int64_t)s * (HID + 4) + d];
+                den += w;
+            }
+        }
+        out[(int64_t)b * o_sb + (int64_t)h * o_sh + d] = Elem<T>::narrow(den > 0.0f ? num / den : 0.0f);
+    }
+}
+
+template <typename T, int HID>
+static int launch_partial(const DecodeParams &dp, hipStream_t st) {
+    dim3 grid((unsigned)dp.nsplits, (unsigned)dp.a.kv.HKV, (unsigned)dp.a.B), block(256);
+    bool launched = false;
+#define DEC_CASE(GG)                                                                                   \
+    if constexpr (GG * HID <= 512) {                                                                   \
+        if (dp.a.G == GG) {                                                                            \
+            hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG>), grid, block, 0, st, dp);       \
+            launched = true;                                                                           \
+        }                                                                                              \
+    }
+    DEC_CASE(1) DEC_CASE(2) DEC_CASE(4) DEC_CASE(8)
+#undef DEC_CASE
+    if (!launched) {
+        set_error("decode: GQA group size %d with head dim %d is not built", dp.a.G, HID);
+        return HIPATTN_E_UNSUPPORTED;
+    }
+    HIPATTN_CHECK_HIP(hipGetLastError());
+    return 0;
+}
+
+}  // namespace hipattn
+
+using namespace hipattn;
+
+extern "C" int64_t hipattn_bsa_decode_workspace_bytes(int32_t B, int32_t HEAD, int32_t HID, int32_t nsplits) {
+    if (B <= 0 || HEAD <= 0 || HID <= 0 || nsplits <= 0) return 0;
+    return (int64_t)B * HEAD * nsplits * (HID + 4) * (int64_t)sizeof(float);
+}
+
+extern "C" int32_t hipattn_bsa_decode_default_splits(int32_t B, int32_t HKV, int32_t tokens) {
+    if (B <= 0 || HKV <= 0) return 1;
+    int64_t groups = (int64_t)B * HKV;
+    int64_t s = (1024 + groups - 1) / groups;  // aim at ~4 workgroups per compute unit
+    int64_t by_tokens = (tokens + 63) / 64;
+    if (s > by_tokens) s = by_tokens;
+    if (s > 64) s = 64;
+    if (s < 1) s = 1;
+    return (int32_t)s;
+}
+
+extern "C" int hipattn_bsa_decode_partial(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t *indices,
+                                          const int32_t *ks_start_end, int32_t idx_rows, int32_t BK,
+                                          int32_t block_size_k, int32_t sliding_window, int32_t sink, int32_t nsplits,
+                                          void *workspace, void *stream) {
+    DecodeParams dp;
+    HIPATTN_CHECK_ARG(workspace, HIPATTN_E_ARG, "decode: null workspace");
+    HIPATTN_CHECK_ARG(nsplits >= 1 && nsplits <= 1024, HIPATTN_E_ARG, "decode: nsplits %d out of range", nsplits);
+    int rc = bsa_fill_params(q, kv, indices, ks_start_end, idx_rows, BK, 1, block_size_k, sliding_window, sink, 1,
+                             workspace, 0, 0, 0, &dp.a);
+    if (rc) return rc;
+    HIPATTN_CHECK_ARG(q->TDST == 1, HIPATTN_E_ARG, "decode: TDST must be 1, got %d", q->TDST);
+    dp.nsplits = nsplits;
+    dp.ws = reinterpret_cast<float *>(workspace);
+    hipStream_t st = (hipStream_t)stream;
+    if (q->dtype == HIPATTN_BF16) {
+        switch (q->HID) {
+            case 32: return launch_partial<bf16_t, 32>(dp, st);
+            case 64: return launch_partial<bf16_t, 64>(dp, st);
+            case 128: return launch_partial<bf16_t, 128>(dp, st);
+            case 256: return launch_partial<bf16_t, 256>(dp, st);
+        }
+    } else {
+        switch (q->HID) {
+            case 32: return launch_partial<float, 32>(dp, st);
+            case 64: return launch_partial<float, 64>(dp, st);
+            case 128: return launch_partial<float, 128>(dp, st);
+        }
+    }
+    set_error("decode: head dim %d with dtype %d is not built", q->HID, q->dtype);
+    return HIPATTN_E_UNSUPPORTED;
+}
+
+extern "C" int hipattn_bsa_decode_merge(const void *workspace, int32_t B, int32_t HEAD, int32_t HID, int32_t nsplits,
+                                        int32_t dtype, void *out, int64_t out_stride_b, int64_t out_stride_h,
+                                        void *stream) {
+    HIPATTN_CHECK_ARG(workspace && out, HIPATTN_E_ARG, "decode merge: null pointer");
+    HIPATTN_CHECK_ARG(B > 0 && HEAD > 0 && nsplits > 0, HIPATTN_E_ARG, "decode merge: non-positive size");
+    dim3 grid((unsigned)HEAD, (unsigned)B), block(HID < 64 ? 64 : (HID > 256 ? 256 : HID));
+    const float *ws = reinterpret_cast<const float *>(workspace);
+    hipStream_t st = (hipStream_t)stream;
+#define MERGE_CASE(TT, HH)                                                                                         \
+    hipLaunchKernelGGL((bsa_decode_merge_kernel<TT, HH>), grid, block, 0, st, ws, HEAD, nsplits, (TT *)out, \
+                       out_stride_b, out_stride_h)
+    if (dtype == HIPATTN_BF16) {
+        switch (HID) {
+            case 32: MERGE_CASE(bf16_t, 32); break;
+            case 64: MERGE_CASE(bf16_t, 64); break;
+            case 128: MERGE_CASE(bf16_t, 128); break;
+            case 256: MERGE_CASE(bf16_t, 256); break;
+            default: set_error("decode merge: head dim %d", HID); return HIPATTN_E_UNSUPPORTED;
+        }
+    } else if (dtype == HIPATTN_F32) {
+        switch (HID) {
+            case 32: MERGE_CASE(float, 32); break;
+            case 64: MERGE_CASE(float, 64); break;
+            case 128: MERGE_CASE(float, 128); break;
+            default: set_error("decode merge: head dim %d", HID); return HIPATTN_E_UNSUPPORTED;
+        }
+    } else {
+        set_error("decode merge: dtype %d", dtype);
+        return HIPATTN_E_UNSUPPORTED;
+    }
+#undef MERGE_CASE
+    HIPATTN_CHECK_HIP(hipGetLastError());
+    return 0;
+}

@@ -1,0 +1,220 @@
+// Shared device/host helpers for the hipattn kernels (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/hipattn.h"
+
+namespace hipattn {
+
+constexpr int WAVE = 64;
+
+// ---------------------------------------------------------------- host-side error plumbing
+void set_error(const char *fmt, ...);
+
+#define HIPATTN_CHECK_ARG(cond, code, ...)  \
+    do {                                    \
+        if (!(cond)) {                      \
+            ::hipattn::set_error(__VA_ARGS__); \
+            return (code);                  \
+        }                                   \
+    } while (0)
+
+#define HIPATTN_CHECK_HIP(expr)                                                       \
+    do {                                                                              \
+        hipError_t _e = (expr);                                                       \
+        if (_e != hipSuccess) {                                                       \
+            ::hipattn::set_error("%s failed: %s", #expr, hipGetErrorString(_e));      \
+            return (int)_e;                                                           \
+        }                                                                             \
+    } while (0)
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---------------------------------------------------------------- element types
+// bf16 is carried as raw 16-bit patterns; all arithmetic happens in f32.
+struct bf16_t {
+    uint16_t bits;
+};
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+
+// round-to-nearest-even f32 -> bf16, result widened back to f32 (NaN inputs are not expected)
+__device__ __forceinline__ float round_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return __uint_as_float(u & 0xffff0000u);
+}
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+template <typename T>
+struct Elem;
+
+template <>
+struct Elem<float> {
+    static constexpr int dtype = HIPATTN_F32;
+    __device__ static __forceinline__ float widen(float x) { return x; }
+    __device__ static __forceinline__ float round(float x) { return x; }
+    __device__ static __forceinline__ float narrow(float x) { return x; }
+};
+
+template <>
+struct Elem<bf16_t> {
+    static constexpr int dtype = HIPATTN_BF16;
+    __device__ static __forceinline__ float widen(bf16_t x) { return bf16_to_f32(x.bits); }
+    __device__ static __forceinline__ float round(float x) { return round_bf16(x); }
+    __device__ static __forceinline__ bf16_t narrow(float x) { return bf16_t{f32_to_bf16_bits(x)}; }
+};
+
+// scale constants: c_q = T(sqrt(HID)/sqrt(sqrt(HID))), c_k = T(1/sqrt(sqrt(HID))), f32 IEEE ops.
+// Computed on the host (correctly rounded sqrtf and division) and passed to kernels.
+void scale_constants(int hid, int dtype, float *c_q, float *c_k);
+
+// ---------------------------------------------------------------- vector row loads
+// A row slice of N elements of T kept as raw dwords (N*sizeof(T) is a multiple of 4 bytes and the
+// address is aligned to min(16, N*sizeof(T)) bytes).
+template <typename T, int N>
+struct RawSlice {
+    static constexpr int BYTES = N * (int)sizeof(T);
+    static_assert(BYTES % 4 == 0, "row slices are whole dwords");
+    static_assert(BYTES < 16 || BYTES % 16 == 0, "wide slices are whole 16-byte packs");
+    uint32_t w[BYTES / 4];
+
+    __device__ __forceinline__ void zero() {
+#pragma unroll
+        for (int i = 0; i < BYTES / 4; i++) w[i] = 0u;
+    }
+    __device__ __forceinline__ void load(const T *p) {
+        if constexpr (BYTES >= 16) {
+            const uint4 *pp = reinterpret_cast<const uint4 *>(p);
+#pragma unroll
+            for (int i = 0; i < BYTES / 16; i++) {
+                uint4 v = pp[i];
+                w[i * 4 + 0] = v.x; w[i * 4 + 1] = v.y; w[i * 4 + 2] = v.z; w[i * 4 + 3] = v.w;
+            }
+        } else if constexpr (BYTES == 8) {
+            uint2 v = *reinterpret_cast<const uint2 *>(p);
+            w[0] = v.x; w[1] = v.y;
+        } else {
+            w[0] = *reinterpret_cast<const uint32_t *>(p);
+        }
+    }
+    __device__ __forceinline__ void widen(float (&out)[N]) const {
+#pragma unroll
+        for (int i = 0; i < BYTES / 4; i++) {
+            if constexpr (sizeof(T) == 4) {
+                out[i] = __uint_as_float(w[i]);
+            } else {
+                out[i * 2] = __uint_as_float(w[i] << 16);
+                out[i * 2 + 1] = __uint_as_float(w[i] & 0xffff0000u);
+            }
+        }
+    }
+};
+
+template <typename T, int N>
+__device__ __forceinline__ void load_elems(const T *p, float (&out)[N]) {
+    RawSlice<T, N> r;
+    r.load(p);
+    r.widen(out);
+}
+
+// ---------------------------------------------------------------- KV addressing (device copy of hipattn_kv_t)
+struct KVView {
+    const void *k;
+    const void *v;
+    int64_t k_stride_b, k_stride_t, k_stride_h;
+    int64_t v_stride_b, v_stride_t, v_stride_h;
+    int64_t tsrc;
+    int64_t max_tsrc;
+    const void *block_table;
+    const void *cache_seq_lens;
+    int64_t bt_stride_b;
+    int bt_is64, sl_is64, paged, page_size, HKV;
+
+    __device__ __forceinline__ int64_t seq_len(int b) const {
+        return sl_is64 ? reinterpret_cast<const int64_t *>(cache_seq_lens)[b]
+                       : (int64_t) reinterpret_cast<const int32_t *>(cache_seq_lens)[b];
+    }
+    // element offset of the K row of token t (kv head h) or -1 for "zero row"
+    __device__ __forceinline__ int64_t k_row(int b, int64_t t, int h, int64_t seqlen) const {
+        if (!paged) {
+            if (t < 0 || t >= tsrc) return -1;
+            return (int64_t)b * k_stride_b + t * k_stride_t + (int64_t)h * k_stride_h;
+        }
+        int64_t page = 0;
+        if (t >= 0 && t < seqlen) {
+            int64_t i = (int64_t)b * bt_stride_b + t / page_size;
+            page = bt_is64 ? reinterpret_cast<const int64_t *>(block_table)[i]
+                           : (int64_t) reinterpret_cast<const int32_t *>(block_table)[i];
+        }
+        if (t < 0) return -1;
+        return page * k_stride_b + (t % page_size) * k_stride_t + (int64_t)h * k_stride_h;
+    }
+    // same page arithmetic for V given the K offset's (page, in-page) decomposition is not shared:
+    __device__ __forceinline__ int64_t v_row(int b, int64_t t, int h, int64_t seqlen) const {
+        if (!paged) {
+            if (t < 0 || t >= tsrc) return -1;
+            return (int64_t)b * v_stride_b + t * v_stride_t + (int64_t)h * v_stride_h;
+        }
+        int64_t page = 0;
+        if (t >= 0 && t < seqlen) {
+            int64_t i = (int64_t)b * bt_stride_b + t / page_size;
+            page = bt_is64 ? reinterpret_cast<const int64_t *>(block_table)[i]
+                           : (int64_t) reinterpret_cast<const int32_t *>(block_table)[i];
+        }
+        if (t < 0) return -1;
+        return page * v_stride_b + (t % page_size) * v_stride_t + (int64_t)h * v_stride_h;
+    }
+};
+
+int make_kv_view(const hipattn_kv_t *kv, int B, int HID, int dtype, KVView *out);
+int check_q(const hipattn_q_t *q);
+
+// ---------------------------------------------------------------- wave helpers
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+__device__ __forceinline__ int wave_min_i(int v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ int wave_max_i(int v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ long long wave_min_ll(long long v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        long long w = __shfl_xor(v, o);
+        v = w < v ? w : v;
+    }
+    return v;
+}
+
+// XCD-aware remap: consecutive workgroup ids are dealt round-robin to the 8 XCDs (each with its
+// own L2), so give every XCD one contiguous range of logical work ids.
+__device__ __forceinline__ long long xcd_remap(long long bid, long long total) {
+    constexpr long long NX = 8;
+    long long per = total / NX;
+    long long main = per * NX;
+    if (bid >= main) return bid;  // tail that does not divide evenly keeps its id
+    return (bid % NX) * per + bid / NX;
+}
+
+}  // namespace hipattn

@@ -1,0 +1,343 @@
+// Mask-estimation scan stage: per (batch, scan row, head, chunk) binary-search refinement + score.
+//
+// One wavefront plays one program of the reference kernel (a group of `block_chunk` <= 64 chunks
+// of one (batch, head, scan row)), because the reference's gate and iteration count are
+// program-level quantities.  Inside the wave, 16 lanes share one sampled key row (each lane owns
+// HID/16 contiguous head-dim elements, so a row is one fully coalesced 16-lane load), four key
+// rows are in flight per load instruction, and the dot product is reduced across the 16 lanes in
+// the fixed order  [FMA chain over the lane's elements] -> [adjacent-pair tree over lanes],
+// which makes scores reproducible bit for bit on any implementation that follows the same order.
+#include "common.hpp"
+
+namespace hipattn {
+
+struct MaskParams {
+    const void *q;
+    int64_t q_sb, q_st, q_sh;
+    const int64_t *pos;
+    int64_t pos_sb, pos_st;
+    KVView kv;
+    const int32_t *chunk_left;
+    int hg, n, chunk;
+    int64_t right_clamp;
+    int B, TDST, HEAD, G, BS, BDST, BQ, stride_q, nrows, block_chunk, scan_stride, sw_eff;
+    float terminate;
+    int ngroups;
+    long long total;
+    float c_q, c_k;
+    float *scores;
+    int32_t *left_out;
+};
+
+template <int N>
+__device__ __forceinline__ void rs_step(const float (&in)[N], float (&out)[N / 2], bool hi, int xmask) {
+#pragma unroll
+    for (int i = 0; i < N / 2; i++) {
+        float a = in[2 * i], b = in[2 * i + 1];
+        float keep = hi ? b : a;
+        float send = hi ? a : b;
+        out[i] = keep + __shfl_xor(send, xmask);
+    }
+}
+
+// Sum part[r] over the 16 lanes of a row group in adjacent-pair tree order.  Returns, in lane dl,
+// the total for row (dl & (ROWS-1)).
+template <int ROWS>
+__device__ __forceinline__ float reduce16(const float (&part)[ROWS], int dl) {
+    if constexpr (ROWS == 16) {
+        float a[8], b[4], c[2], d[1];
+        rs_step<16>(part, a, dl & 1, 1);
+        rs_step<8>(a, b, dl & 2, 2);
+        rs_step<4>(b, c, dl & 4, 4);
+        rs_step<2>(c, d, dl & 8, 8);
+        return d[0];
+    } else if constexpr (ROWS == 4) {
+        float a[2], b[1];
+        rs_step<4>(part, a, dl & 1, 1);
+        rs_step<2>(a, b, dl & 2, 2);
+        float v = b[0];
+        v += __shfl_xor(v, 4);
+        v += __shfl_xor(v, 8);
+        return v;
+    } else {
+        static_assert(ROWS == 1, "ROWS is 1, 4 or 16");
+        float v = part[0];
+        v += __shfl_xor(v, 1);
+        v += __shfl_xor(v, 2);
+        v += __shfl_xor(v, 4);
+        v += __shfl_xor(v, 8);
+        return v;
+    }
+}
+
+template <typename T, int HID, int ROWS, int MAXROWS, int STEPS>
+__global__ __launch_bounds__(64) void mask_stage_kernel(MaskParams p) {
+    constexpr int SEG = HID / 16;
+    __shared__ int64_t s_koff[128];
+    __shared__ float s_sc[128];
+    __shared__ __align__(16) T s_q[MAXROWS * HID];
+
+    const int lane = threadIdx.x;
+    const int sub = lane >> 4;
+    const int dl = lane & 15;
+
+    long long L = xcd_remap((long long)blockIdx.x, p.total);
+    const int hin = (int)(L % p.G);
+    L /= p.G;
+    const int s = (int)(L % p.BS);
+    L /= p.BS;
+    const int g = (int)(L % p.ngroups);
+    L /= p.ngroups;
+    const int kvh = (int)(L % p.kv.HKV);
+    const int b = (int)(L / p.kv.HKV);
+    const int h = kvh * p.G + hin;
+
+    const int BC = p.block_chunk;
+    const int ci = g * BC + lane;
+    const bool real = (lane < BC) && (ci < p.n);
+    const int hgi = p.hg == 1 ? 0 : h;
+    const int64_t row_in = (((int64_t)b * p.BS + s) * p.hg + hgi) * p.n;
+    const int64_t row_out = (((int64_t)b * p.BS + s) * p.HEAD + h) * p.n;
+
+    int l = (int)p.kv.max_tsrc, r = (int)p.kv.max_tsrc;
+    if (real) {
+        l = p.chunk_left[row_in + ci];
+        int64_t rr = (int64_t)l + p.chunk;
+        r = (int)(rr < p.right_clamp ? rr : p.right_clamp);
+    }
+    float score = -32000.0f;
+
+    // rows of this program
+    const long long qb = (long long)(p.BDST - 1) - (long long)(p.BS - 1) * p.scan_stride + (long long)s * p.scan_stride;
+    long long myrow = qb * p.BQ + (long long)lane * p.stride_q;
+    bool rv = (lane < p.nrows) && (myrow >= 0) && (myrow < p.TDST);
+    const unsigned long long rowmask = __ballot(rv);
+    long long mypos = rv ? p.pos[(int64_t)b * p.pos_sb + myrow * p.pos_st] : 0x7fffffffffffffffLL;
+    const long long pmin = wave_min_ll(mypos);
+
+    bool run = (rowmask != 0ull) && (pmin >= 0);
+    int lim = 0;
+    float width = 0.0f;
+    if (run) {
+        long long lm = pmin - p.sw_eff;
+        lim = (int)(lm < 0 ? 0 : lm);
+        const int minl = wave_min_i(l);
+        run = (pmin + (long long)p.BQ * p.scan_stride >= (long long)minl);
+        width = (float)wave_max_i(r - l);
+    }
+    if (!run || !(width >= p.terminate)) {
+        if (real) {
+            p.scores[row_out + ci] = score;
+            if (p.left_out) p.left_out[row_out + ci] = l;
+        }
+        return;
+    }
+
+    // q^ rows: strided mean -> T -> *c_q -> T, staged in LDS
+    const T *qbase = reinterpret_cast<const T *>(p.q) + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
+    const int rows_here = p.nrows < MAXROWS ? p.nrows : MAXROWS;
+    for (int idx = lane; idx < rows_here * HID; idx += 64) {
+        const int j = idx / HID, d = idx % HID;
+        float qh = 0.0f;
+        if ((rowmask >> j) & 1ull) {
+            const long long it = qb * p.BQ + (long long)j * p.stride_q;
+            float sum = 0.0f;
+            int cnt = 0;
+            for (int o = 0; o < p.stride_q; o++) {
+                if (it + o < p.TDST) {
+                    sum += Elem<T>::widen(qbase[(it + o) * p.q_st + d]);
+                    cnt++;
+                }
+            }
+            float mean = Elem<T>::round(__fdiv_rn(sum, (float)cnt + 1e-12f));
+            qh = Elem<T>::round(mean * p.c_q);
+        }
+        s_q[idx] = Elem<T>::narrow(qh);
+    }
+    __syncthreads();
+
+    const int npass = (rows_here + ROWS - 1) / ROWS;
+    float qh[ROWS][SEG];
+    auto load_q_pass = [&](int pass) {
+#pragma unroll
+        for (int rr = 0; rr < ROWS; rr++) {
+            const int j = pass * ROWS + rr;
+            if (j < rows_here) {
+                load_elems<T, SEG>(&s_q[j * HID + dl * SEG], qh[rr]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < SEG; e++) qh[rr][e] = 0.0f;
+            }
+        }
+    };
+    if (npass == 1) load_q_pass(0);
+
+    const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
+    const T *kbase = reinterpret_cast<const T *>(p.kv.k);
+    const int nsteps = BC / 2;
+
+    while (width >= p.terminate) {
+        width *= 0.5f;
+        const bool active = real && (l < r) && (l <= lim) && (l >= 0);
+        const int c = (l + r) >> 1;
+        if (lane < BC) {
+            int64_t o0 = -1, o1 = -1;
+            if (active) {
+                o0 = p.kv.k_row(b, (l + c) >> 1, kvh, seqlen);
+                o1 = p.kv.k_row(b, (c + r) >> 1, kvh, seqlen);
+            }
+            s_koff[2 * lane] = o0;
+            s_koff[2 * lane + 1] = o1;
+            s_sc[2 * lane] = -INFINITY;
+            s_sc[2 * lane + 1] = -INFINITY;
+        }
+        __syncthreads();
+
+        for (int cs = 0; cs < nsteps; cs += STEPS) {
+            RawSlice<T, SEG> raw[STEPS];
+#pragma unroll
+            for (int st = 0; st < STEPS; st++) {
+                const int krow = (cs + st) * 4 + sub;
+                const int64_t off = (cs + st) < nsteps ? s_koff[krow] : -1;
+                if (off >= 0) raw[st].load(kbase + off + dl * SEG);
+                else raw[st].zero();
+            }
+            for (int pass = 0; pass < npass; pass++) {
+                if (npass > 1) load_q_pass(pass);
+                const int j = pass * ROWS + (dl & (ROWS - 1));
+                const bool jvalid = (j < p.nrows) && ((rowmask >> j) & 1ull);
+#pragma unroll
+                for (int st = 0; st < STEPS; st++) {
+                    if ((cs + st) < nsteps) {
+                        float kh[SEG];
+                        raw[st].widen(kh);
+#pragma unroll
+                        for (int e = 0; e < SEG; e++) kh[e] = Elem<T>::round(kh[e] * p.c_k);
+                        float part[ROWS];
+#pragma unroll
+                        for (int rr = 0; rr < ROWS; rr++) {
+                            float acc = 0.0f;
+#pragma unroll
+                            for (int e = 0; e < SEG; e++) acc = __fmaf_rn(qh[rr][e], kh[e], acc);
+                            part[rr] = acc;
+                        }
+                        float v = Elem<T>::round(reduce16<ROWS>(part, dl));
+                        v = jvalid ? v : -INFINITY;
+                        if constexpr (ROWS > 1) {
+                            v = fmaxf(v, __shfl_xor(v, 1));
+                            if constexpr (ROWS > 2) v = fmaxf(v, __shfl_xor(v, 2));
+                            if constexpr (ROWS > 4) {
+                                v = fmaxf(v, __shfl_xor(v, 4));
+                                v = fmaxf(v, __shfl_xor(v, 8));
+                            }
+                        }
+                        if (dl == 0) {
+                            const int krow = (cs + st) * 4 + sub;
+                            s_sc[krow] = fmaxf(s_sc[krow], v);
+                        }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        if (active) {
+            const float sL = s_sc[2 * lane], sR = s_sc[2 * lane + 1];
+            const bool win = sL > sR;
+            if (win) r = c; else l = c;
+            score = fmaxf(score, win ? sL : sR);
+        }
+        __syncthreads();
+    }
+    if (real) {
+        p.scores[row_out + ci] = score;
+        if (p.left_out) p.left_out[row_out + ci] = l;
+    }
+}
+
+template <typename T, int HID>
+static int launch_mask(const MaskParams &p, int rows_eff, hipStream_t stream) {
+    dim3 grid((unsigned)p.total), block(64);
+    if (rows_eff <= 1) {
+        if (p.block_chunk == 64)
+            hipLaunchKernelGGL((mask_stage_kernel<T, HID, 1, 1, 32>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((mask_stage_kernel<T, HID, 1, 1, 8>), grid, block, 0, stream, p);
+    } else if (rows_eff <= 4) {
+        hipLaunchKernelGGL((mask_stage_kernel<T, HID, 4, 4, 8>), grid, block, 0, stream, p);
+    } else if (rows_eff <= 16) {
+        hipLaunchKernelGGL((mask_stage_kernel<T, HID, 16, 16, 8>), grid, block, 0, stream, p);
+    } else if (rows_eff <= 64) {
+        hipLaunchKernelGGL((mask_stage_kernel<T, HID, 16, 64, 8>), grid, block, 0, stream, p);
+    } else {
+        set_error("mask stage: %d query rows per program exceed the supported 64", rows_eff);
+        return HIPATTN_E_UNSUPPORTED;
+    }
+    HIPATTN_CHECK_HIP(hipGetLastError());
+    return 0;
+}
+
+}  // namespace hipattn
+
+using namespace hipattn;
+
+extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, const int32_t *chunk_left,
+                                  int32_t hg, int32_t n, int32_t chunk_size, int64_t right_clamp,
+                                  int32_t bs, int32_t bq, int32_t stride_q, int32_t block_chunk,
+                                  int32_t scan_stride, int32_t sw_eff, int32_t terminate_size,
+                                  float *scores, int32_t *left_out, void *stream) {
+    int rc = check_q(q);
+    if (rc) return rc;
+    HIPATTN_CHECK_ARG(kv && chunk_left && scores, HIPATTN_E_ARG, "mask stage: null pointer");
+    HIPATTN_CHECK_ARG(n >= 0 && chunk_size > 0 && bs > 0 && bq > 0 && stride_q > 0 && scan_stride > 0,
+                      HIPATTN_E_ARG, "mask stage: non-positive size");
+    HIPATTN_CHECK_ARG(hg == 1 || hg == q->HEAD, HIPATTN_E_ARG, "mask stage: hg must be 1 or HEAD");
+    HIPATTN_CHECK_ARG(block_chunk == 16 || block_chunk == 32 || block_chunk == 64, HIPATTN_E_UNSUPPORTED,
+                      "mask stage: block_chunk %d not in {16,32,64}", block_chunk);
+    HIPATTN_CHECK_ARG(bq % stride_q == 0 || bq / stride_q > 0, HIPATTN_E_ARG, "mask stage: bad stride_q");
+    HIPATTN_CHECK_ARG(terminate_size >= 1, HIPATTN_E_ARG, "mask stage: terminate_size < 1");
+    if (n == 0) return 0;
+    MaskParams p;
+    rc = make_kv_view(kv, q->B, q->HID, q->dtype, &p.kv);
+    if (rc) return rc;
+    HIPATTN_CHECK_ARG(q->HEAD % p.kv.HKV == 0, HIPATTN_E_ARG, "mask stage: HEAD %% HKV != 0");
+    p.q = q->ptr; p.q_sb = q->stride_b; p.q_st = q->stride_t; p.q_sh = q->stride_h;
+    p.pos = q->pos; p.pos_sb = q->pos_stride_b; p.pos_st = q->pos_stride_t;
+    p.chunk_left = chunk_left; p.hg = hg; p.n = n; p.chunk = chunk_size; p.right_clamp = right_clamp;
+    p.B = q->B; p.TDST = q->TDST; p.HEAD = q->HEAD; p.G = q->HEAD / p.kv.HKV;
+    p.BQ = bq; p.BDST = (q->TDST + bq - 1) / bq; p.BS = bs; p.stride_q = stride_q;
+    p.nrows = bq / stride_q;
+    HIPATTN_CHECK_ARG(p.nrows >= 1, HIPATTN_E_ARG, "mask stage: stride_q larger than block");
+    HIPATTN_CHECK_ARG(bs == (p.BDST + scan_stride - 1) / scan_stride, HIPATTN_E_ARG,
+                      "mask stage: bs %d does not match cdiv(BDST %d, scan_stride %d)", bs, p.BDST, scan_stride);
+    p.block_chunk = block_chunk; p.scan_stride = scan_stride; p.sw_eff = sw_eff;
+    p.terminate = (float)terminate_size;
+    p.ngroups = (n + block_chunk - 1) / block_chunk;
+    p.total = (long long)q->B * q->HEAD * bs * p.ngroups;
+    HIPATTN_CHECK_ARG(p.total < 0x7fffffffLL, HIPATTN_E_UNSUPPORTED, "mask stage: grid too large");
+    scale_constants(q->HID, q->dtype, &p.c_q, &p.c_k);
+    p.scores = scores; p.left_out = left_out;
+    int rows_max = (q->TDST + stride_q - 1) / stride_q;
+    int rows_eff = p.nrows < rows_max ? p.nrows : rows_max;
+    if (p.nrows > 64) {
+        set_error("mask stage: %d query rows per program exceed the supported 64", p.nrows);
+        return HIPATTN_E_UNSUPPORTED;
+    }
+    // the kernel indexes rows up to nrows; MAXROWS must cover every row that can be valid
+    hipStream_t st = (hipStream_t)stream;
+    if (q->dtype == HIPATTN_BF16) {
+        switch (q->HID) {
+            case 32: return launch_mask<bf16_t, 32>(p, rows_eff, st);
+            case 64: return launch_mask<bf16_t, 64>(p, rows_eff, st);
+            case 128: return launch_mask<bf16_t, 128>(p, rows_eff, st);
+            case 256: return launch_mask<bf16_t, 256>(p, rows_eff, st);
+        }
+    } else if (q->dtype == HIPATTN_F32) {
+        switch (q->HID) {
+            case 32: return launch_mask<float, 32>(p, rows_eff, st);
+            case 64: return launch_mask<float, 64>(p, rows_eff, st);
+            case 128: return launch_mask<float, 128>(p, rows_eff, st);
+        }
+    }
+    set_error("mask stage: head dim %d with dtype %d is not built", q->HID, q->dtype);
+    return HIPATTN_E_UNSUPPORTED;
+}

@@ -1,0 +1,292 @@
+// Selection between scan stages and the final metadata layout.
+//
+// One workgroup owns one (batch, output scan row, head group).  Chunk lists are kept ascending by
+// start position at every stage, so "gather the top-k, then sort by position" is a stream
+// compaction in position order: no sort is needed.  The top-k set is found by an exact radix
+// select on order-preserving integer keys; ties at the threshold are broken by position, which
+// is the fixed tie-break rule (score descending, position ascending).
+#include "common.hpp"
+
+namespace hipattn {
+
+constexpr int SEL_THREADS = 256;
+constexpr int SEL_MAX_N = 16384;
+
+__device__ __forceinline__ uint32_t score_key(float f) {
+    if (f == 0.0f) f = 0.0f;  // -0 and +0 tie
+    uint32_t u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// block-wide exclusive scan of one int per thread; returns the exclusive prefix, total in *total
+__device__ __forceinline__ int block_excl_scan(int v, int *s_tmp, int *total) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wid = tid >> 6;
+    int incl = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        int t = __shfl_up(incl, o);
+        if (lane >= o) incl += t;
+    }
+    if (lane == 63) s_tmp[wid] = incl;
+    __syncthreads();
+    int base = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < SEL_THREADS / 64; w++) {
+        int x = s_tmp[w];
+        if (w < wid) base += x;
+        tot += x;
+    }
+    __syncthreads();
+    *total = tot;
+    return base + incl - v;
+}
+
+// Shared front end: keys[c] = max over the heads of the group, then the k-th largest key.
+// On return s_keys holds the keys, *thr the threshold key and *need how many entries equal to the
+// threshold are taken (in position order).
+__device__ void topk_threshold(const float *scores_row /* [nheads, n] with stride n */, int nheads, int n, int k,
+                               uint32_t *s_keys, int *s_hist, int *s_misc, uint32_t *thr, int *need_out) {
+    const int tid = threadIdx.x;
+    for (int c = tid; c < n; c += SEL_THREADS) {
+        float m = scores_row[c];
+        for (int hh = 1; hh < nheads; hh++) m = fmaxf(m, scores_row[(int64_t)hh * n + c]);
+        s_keys[c] = score_key(m);
+    }
+    __syncthreads();
+    uint32_t prefix = 0, mask = 0;
+    int need = k;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        for (int i = tid; i < 256; i += SEL_THREADS) s_hist[i] = 0;
+        __syncthreads();
+        for (int c = tid; c < n; c += SEL_THREADS) {
+            uint32_t key = s_keys[c];
+            if ((key & mask) == prefix) atomicAdd(&s_hist[(key >> shift) & 255u], 1);
+        }
+        __syncthreads();
+        if (tid == 0) {
+            int cum = 0, digit = 0, nd = need;
+            for (int bin = 255; bin >= 0; bin--) {
+                int hcount = s_hist[bin];
+                if (cum + hcount >= need) {
+                    digit = bin;
+                    nd = need - cum;
+                    break;
+                }
+                cum += hcount;
+            }
+            s_misc[0] = digit;
+            s_misc[1] = nd;
+        }
+        __syncthreads();
+        prefix |= ((uint32_t)s_misc[0]) << shift;
+        mask |= 255u << shift;
+        need = s_misc[1];
+        __syncthreads();
+    }
+    *thr = prefix;
+    *need_out = need;
+}
+
+// Marks the selected entries and returns, per thread, the output rank of the first selected entry
+// of its contiguous segment.  seg = entries per thread.
+struct SegScan {
+    int seg, begin, end, out_base, eq_base;
+};
+
+__device__ __forceinline__ SegScan selection_scan(const uint32_t *s_keys, int n, uint32_t thr, int need, int *s_tmp) {
+    SegScan r;
+    r.seg = (n + SEL_THREADS - 1) / SEL_THREADS;
+    r.begin = threadIdx.x * r.seg;
+    r.end = r.begin + r.seg < n ? r.begin + r.seg : n;
+    int eq = 0, gt = 0;
+    for (int c = r.begin; c < r.end; c++) {
+        uint32_t key = s_keys[c];
+        eq += (key == thr);
+        gt += (key > thr);
+    }
+    int tot;
+    r.eq_base = block_excl_scan(eq, s_tmp, &tot);
+    // selected in this segment = gt + clamp(need - eq_base, 0, eq)
+    int take = need - r.eq_base;
+    take = take < 0 ? 0 : (take > eq ? eq : take);
+    r.out_base = block_excl_scan(gt + take, s_tmp, &tot);
+    return r;
+}
+
+__global__ __launch_bounds__(SEL_THREADS) void select_stage_kernel(const float *scores, const int32_t *chunk_left,
+                                                                  int bs_in, int bs_out, int row_rep, int HEAD, int hg,
+                                                                  int n, int k, int sub_chunk, int splits,
+                                                                  int32_t *next_left) {
+    __shared__ uint32_t s_keys[SEL_MAX_N];
+    __shared__ int s_hist[256];
+    __shared__ int s_misc[2];
+    __shared__ int s_tmp[SEL_THREADS / 64];
+
+    const int hgi = blockIdx.x % hg;
+    const int o = (blockIdx.x / hg) % bs_out;
+    const int b = blockIdx.x / (hg * bs_out);
+    const int i = (o + row_rep * bs_in - bs_out) / row_rep;
+    const int nheads = HEAD / hg;
+    const float *srow = scores + (((int64_t)b * bs_in + i) * HEAD + (int64_t)hgi * nheads) * n;
+    const int32_t *lrow = chunk_left + (((int64_t)b * bs_in + i) * hg + hgi) * n;
+    int32_t *orow = next_left + (((int64_t)b * bs_out + o) * hg + hgi) * ((int64_t)k * splits);
+
+    uint32_t thr;
+    int need;
+    if (k >= n) {
+        thr = 0;
+        need = 0;
+        for (int c = threadIdx.x; c < n; c += SEL_THREADS) s_keys[c] = 1u;  // everything > thr
+        __syncthreads();
+    } else {
+        topk_threshold(srow, nheads, n, k, s_keys, s_hist, s_misc, &thr, &need);
+    }
+    SegScan sc = selection_scan(s_keys, n, thr, need, s_tmp);
+    int out = sc.out_base, eqr = sc.eq_base;
+    for (int c = sc.begin; c < sc.end; c++) {
+        uint32_t key = s_keys[c];
+        bool sel = key > thr;
+        if (key == thr) {
+            sel = eqr < need;
+            eqr++;
+        }
+        if (sel) {
+            const int left = lrow[c];
+            for (int j = 0; j < splits; j++) orow[(int64_t)out * splits + j] = left + j * sub_chunk;
+            out++;
+        }
+    }
+}
+
+__global__ __launch_bounds__(SEL_THREADS) void finalize_kernel(const float *scores, const int32_t *left_out,
+                                                               const int64_t *pos, int64_t pos_sb, int64_t pos_st,
+                                                               int bs, int bdst, int scan_stride, int HEAD, int hg,
+                                                               int n, int K, int chunk, int bq, int64_t *indices,
+                                                               int64_t *ks, int32_t *ks_start_end) {
+    __shared__ uint32_t s_keys[SEL_MAX_N];
+    __shared__ int s_hist[256];
+    __shared__ int s_misc[2];
+    __shared__ int s_tmp[SEL_THREADS / 64];
+    int *s_sel = reinterpret_cast<int *>(s_keys);  // reused after selection: positions of selected chunks
+
+    const int hgi = blockIdx.x % hg;
+    const int qb = (blockIdx.x / hg) % bdst;
+    const int b = blockIdx.x / (hg * bdst);
+    const int i = (qb + scan_stride * bs - bdst) / scan_stride;
+    const int nheads = HEAD / hg;
+    const int BK = K < n ? K : n;
+    const float *srow = scores + (((int64_t)b * bs + i) * HEAD + (int64_t)hgi * nheads) * n;
+
+    uint32_t thr;
+    int need;
+    if (BK >= n) {
+        thr = 0;
+        need = 0;
+        for (int c = threadIdx.x; c < n; c += SEL_THREADS) s_keys[c] = 1u;
+        __syncthreads();
+    } else {
+        topk_threshold(srow, nheads, n, BK, s_keys, s_hist, s_misc, &thr, &need);
+    }
+    SegScan sc = selection_scan(s_keys, n, thr, need, s_tmp);
+    // each thread lists its selected positions in registers first (keys are still being read by others)
+    int out = sc.out_base, eqr = sc.eq_base;
+    unsigned long long selbits = 0ull;  // seg <= 64 since n <= 16384
+    for (int c = sc.begin; c < sc.end; c++) {
+        uint32_t key = s_keys[c];
+        bool sel = key > thr;
+        if (key == thr) {
+            sel = eqr < need;
+            eqr++;
+        }
+        if (sel) selbits |= 1ull << (c - sc.begin);
+    }
+    __syncthreads();
+    for (int c = sc.begin; c < sc.end; c++) {
+        if ((selbits >> (c - sc.begin)) & 1ull) s_sel[out++] = c;
+    }
+    __syncthreads();
+
+    const int64_t first_pos = pos[(int64_t)b * pos_sb + (int64_t)qb * bq * pos_st];
+    const int64_t limit = first_pos + bq;
+    const int per = (BK + SEL_THREADS - 1) / SEL_THREADS;
+    const int o0 = threadIdx.x * per;
+    const int o1 = o0 + per < BK ? o0 + per : BK;
+    for (int hh = 0; hh < nheads; hh++) {
+        const int h = hgi * nheads + hh;
+        const int32_t *lrow = left_out + (((int64_t)b * bs + i) * HEAD + h) * n;
+        int64_t *irow = indices + (((int64_t)b * HEAD + h) * bdst + qb) * BK;
+        // value of entry o: refined left edge aligned down to the block grid
+        auto val = [&](int o) -> int64_t {
+            int64_t v = lrow[s_sel[o]];
+            return v / chunk * chunk;
+        };
+        int uniq = 0, act = 0;
+        for (int o = o0; o < o1; o++) {
+            const int64_t v = val(o);
+            const int64_t prev = val(o == 0 ? BK - 1 : o - 1);  // roll(1): entry 0 is compared with the last
+            if (v != prev) {
+                uniq++;
+                act += (v < limit);
+            }
+        }
+        int tot_u, tot_a;
+        int ubase = block_excl_scan(uniq, s_tmp, &tot_u);
+        (void)block_excl_scan(act, s_tmp, &tot_a);
+        for (int o = o0; o < o1; o++) {
+            const int64_t v = val(o);
+            const int64_t prev = val(o == 0 ? BK - 1 : o - 1);
+            if (v != prev) irow[ubase++] = v;
+        }
+        for (int o = tot_u + threadIdx.x; o < BK; o += SEL_THREADS) irow[o] = 0x7fffffffffffffffLL;
+        if (threadIdx.x == 0) {
+            const int64_t r = ((int64_t)b * HEAD + h) * bdst + qb;
+            ks[r] = tot_a;
+            ks_start_end[r * 2 + 0] = 0;
+            ks_start_end[r * 2 + 1] = tot_a;
+        }
+    }
+}
+
+}  // namespace hipattn
+
+using namespace hipattn;
+
+extern "C" int hipattn_select_stage(const float *scores, const int32_t *chunk_left, int32_t B, int32_t bs_in,
+                                    int32_t bs_out, int32_t row_rep, int32_t HEAD, int32_t hg, int32_t n,
+                                    int32_t k, int32_t chunk_size, int32_t splits, int32_t *next_left,
+                                    void *stream) {
+    HIPATTN_CHECK_ARG(scores && chunk_left && next_left, HIPATTN_E_ARG, "select stage: null pointer");
+    HIPATTN_CHECK_ARG(B > 0 && bs_in > 0 && bs_out > 0 && row_rep > 0 && HEAD > 0 && n > 0 && k > 0 && splits > 0,
+                      HIPATTN_E_ARG, "select stage: non-positive size");
+    HIPATTN_CHECK_ARG(hg == 1 || hg == HEAD, HIPATTN_E_ARG, "select stage: hg must be 1 or HEAD");
+    HIPATTN_CHECK_ARG(k <= n, HIPATTN_E_ARG, "select stage: k %d > n %d", k, n);
+    HIPATTN_CHECK_ARG(chunk_size % splits == 0, HIPATTN_E_ARG, "select stage: chunk %d %% splits %d", chunk_size, splits);
+    HIPATTN_CHECK_ARG(bs_out <= row_rep * bs_in, HIPATTN_E_ARG, "select stage: bs_out > row_rep*bs_in");
+    HIPATTN_CHECK_ARG(n <= SEL_MAX_N, HIPATTN_E_UNSUPPORTED, "select stage: %d chunks exceed the limit %d", n, SEL_MAX_N);
+    dim3 grid((unsigned)(B * bs_out * hg)), block(SEL_THREADS);
+    hipLaunchKernelGGL(select_stage_kernel, grid, block, 0, (hipStream_t)stream, scores, chunk_left, bs_in, bs_out,
+                       row_rep, HEAD, hg, n, k, chunk_size / splits, splits, next_left);
+    HIPATTN_CHECK_HIP(hipGetLastError());
+    return 0;
+}
+
+extern "C" int hipattn_finalize_indices(const float *scores, const int32_t *left_out, const int64_t *pos,
+                                        int64_t pos_stride_b, int64_t pos_stride_t, int32_t B, int32_t bs,
+                                        int32_t bdst, int32_t scan_stride, int32_t HEAD, int32_t hg, int32_t n,
+                                        int32_t K, int32_t chunk_size, int32_t bq, int64_t *indices, int64_t *ks,
+                                        int32_t *ks_start_end, void *stream) {
+    HIPATTN_CHECK_ARG(scores && left_out && pos && indices && ks && ks_start_end, HIPATTN_E_ARG,
+                      "finalize: null pointer");
+    HIPATTN_CHECK_ARG(B > 0 && bs > 0 && bdst > 0 && scan_stride > 0 && HEAD > 0 && n > 0 && K > 0 && chunk_size > 0 &&
+                          bq > 0,
+                      HIPATTN_E_ARG, "finalize: non-positive size");
+    HIPATTN_CHECK_ARG(hg == 1 || hg == HEAD, HIPATTN_E_ARG, "finalize: hg must be 1 or HEAD");
+    HIPATTN_CHECK_ARG(bdst <= scan_stride * bs, HIPATTN_E_ARG, "finalize: bdst > scan_stride*bs");
+    HIPATTN_CHECK_ARG(n <= SEL_MAX_N, HIPATTN_E_UNSUPPORTED, "finalize: %d chunks exceed the limit %d", n, SEL_MAX_N);
+    dim3 grid((unsigned)(B * bdst * hg)), block(SEL_THREADS);
+    hipLaunchKernelGGL(finalize_kernel, grid, block, 0, (hipStream_t)stream, scores, left_out, pos, pos_stride_b,
+                       pos_stride_t, bs, bdst, scan_stride, HEAD, hg, n, K, chunk_size, bq, indices, ks, ks_start_end);
+    HIPATTN_CHECK_HIP(hipGetLastError());
+    return 0;
+}

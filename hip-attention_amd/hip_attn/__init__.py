@@ -1,0 +1,28 @@
+"""HiP / InfiniteHiP attention for AMD Instinct MI355X (gfx950).
+
+Import surface of the reference package for the v1.2 operator (``src/hip_attn/__init__.py:30-45``):
+``hip_attention_12(q, k, v, args=HiPAttentionArgs12()) -> (context, metadata)`` plus the paged entry
+points.  Everything executes in hand-written HIP kernels behind ``libhipattn.so``.
+"""
+from .metadata import HiPAttentionArgs as HiPAttentionArgs12
+from .metadata import HiPAttentionCacheAccessStatistics as HiPAttentionCacheAccessStatistics12
+from .metadata import HiPAttentionOutputMetadata as HiPAttentionOutputMetadata12
+from .metadata import ScanStage as ScanStage12
+from .operator import dual_stage_quadratic_hip_attention as hip_attention_12
+
+hip_attention = hip_attention_12
+HiPAttentionArgs = HiPAttentionArgs12
+HiPAttentionOutputMetadata = HiPAttentionOutputMetadata12
+
+__version__ = "1.2.0+mi355x"
+
+__all__ = [
+    "hip_attention_12",
+    "HiPAttentionArgs12",
+    "HiPAttentionOutputMetadata12",
+    "HiPAttentionCacheAccessStatistics12",
+    "ScanStage12",
+    "hip_attention",
+    "HiPAttentionArgs",
+    "HiPAttentionOutputMetadata",
+]

@@ -1,0 +1,211 @@
+"""ctypes binding of ``libhipattn.so`` (the C ABI declared in ``include/hipattn.h``).
+
+PyTorch is used only for device memory and the current HIP stream; every kernel is entered
+through the plain-C entry points.  Loading fails loudly when the library is missing: there is
+no CPU or eager fallback behind this module.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libhipattn.so")
+_lib = None
+
+F32, BF16 = 0, 1
+
+
+class HipAttnError(RuntimeError):
+    pass
+
+
+class QStruct(ctypes.Structure):
+    _fields_ = [
+        ("ptr", ctypes.c_void_p),
+        ("stride_b", ctypes.c_int64), ("stride_t", ctypes.c_int64), ("stride_h", ctypes.c_int64),
+        ("pos", ctypes.c_void_p),
+        ("pos_stride_b", ctypes.c_int64), ("pos_stride_t", ctypes.c_int64),
+        ("B", ctypes.c_int32), ("TDST", ctypes.c_int32), ("HEAD", ctypes.c_int32), ("HID", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+    ]
+
+
+class KVStruct(ctypes.Structure):
+    _fields_ = [
+        ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
+        ("k_stride_b", ctypes.c_int64), ("k_stride_t", ctypes.c_int64), ("k_stride_h", ctypes.c_int64),
+        ("v_stride_b", ctypes.c_int64), ("v_stride_t", ctypes.c_int64), ("v_stride_h", ctypes.c_int64),
+        ("tsrc", ctypes.c_int64), ("max_tsrc", ctypes.c_int64),
+        ("block_table", ctypes.c_void_p), ("cache_seq_lens", ctypes.c_void_p),
+        ("bt_stride_b", ctypes.c_int64),
+        ("bt_is64", ctypes.c_int32), ("sl_is64", ctypes.c_int32),
+        ("paged", ctypes.c_int32), ("page_size", ctypes.c_int32),
+        ("HKV", ctypes.c_int32),
+    ]
+
+
+def lib_path() -> str:
+    return _LIB_PATH
+
+
+def lib():
+    """Load the shared library once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise HipAttnError(
+                f"{_LIB_PATH} is missing: build it with `make -C hip-attention_amd/csrc` "
+                "(or `python -c 'import __graft_entry__ as g; g.build()'`). There is no fallback path.")
+        L = ctypes.CDLL(_LIB_PATH)
+        L.hipattn_version.restype = ctypes.c_char_p
+        L.hipattn_last_error.restype = ctypes.c_char_p
+        L.hipattn_bsa_decode_workspace_bytes.restype = ctypes.c_int64
+        L.hipattn_bsa_decode_default_splits.restype = ctypes.c_int32
+        for name in ("hipattn_mask_stage", "hipattn_select_stage", "hipattn_finalize_indices",
+                     "hipattn_bsa_prefill", "hipattn_bsa_decode_partial", "hipattn_bsa_decode_merge"):
+            getattr(L, name).restype = ctypes.c_int
+        _lib = L
+    return _lib
+
+
+def check(rc: int, what: str):
+    if rc != 0:
+        msg = lib().hipattn_last_error().decode()
+        kind = "argument error" if rc < 0 else "HIP error"
+        raise HipAttnError(f"{what}: {kind} {rc}: {msg}")
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return BF16
+    if t.dtype == torch.float32:
+        return F32
+    raise HipAttnError(f"unsupported dtype {t.dtype}: the kernels take float32 or bfloat16")
+
+
+def stream_ptr(device) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _p(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def make_q(q: torch.Tensor, pos: torch.Tensor) -> QStruct:
+    assert q.ndim == 4 and q.stride(3) == 1
+    assert pos.dtype == torch.int64 and pos.ndim == 2
+    s = QStruct()
+    s.ptr = q.data_ptr()
+    s.stride_b, s.stride_t, s.stride_h = q.stride(0), q.stride(1), q.stride(2)
+    s.pos = pos.data_ptr()
+    s.pos_stride_b, s.pos_stride_t = pos.stride(0), pos.stride(1)
+    s.B, s.TDST, s.HEAD, s.HID = q.shape
+    s.dtype = dtype_code(q)
+    return s
+
+
+def make_kv_dense(k: torch.Tensor, v: torch.Tensor) -> KVStruct:
+    assert k.ndim == 4 and k.stride(3) == 1 and v.stride(3) == 1
+    s = KVStruct()
+    s.k, s.v = k.data_ptr(), v.data_ptr()
+    s.k_stride_b, s.k_stride_t, s.k_stride_h = k.stride(0), k.stride(1), k.stride(2)
+    s.v_stride_b, s.v_stride_t, s.v_stride_h = v.stride(0), v.stride(1), v.stride(2)
+    s.tsrc = k.shape[1]
+    s.max_tsrc = k.shape[1]
+    s.paged = 0
+    s.page_size = 1
+    s.HKV = k.shape[2]
+    return s
+
+
+def make_kv_paged(k_cache, v_cache, block_table, cache_seq_lens, max_tsrc: int) -> KVStruct:
+    assert k_cache.ndim == 4 and k_cache.stride(3) == 1 and v_cache.stride(3) == 1
+    assert block_table.ndim == 2 and block_table.stride(1) == 1
+    assert cache_seq_lens.ndim == 1 and cache_seq_lens.stride(0) == 1
+    assert block_table.dtype in (torch.int32, torch.int64)
+    assert cache_seq_lens.dtype in (torch.int32, torch.int64)
+    s = KVStruct()
+    s.k, s.v = k_cache.data_ptr(), v_cache.data_ptr()
+    s.k_stride_b, s.k_stride_t, s.k_stride_h = k_cache.stride(0), k_cache.stride(1), k_cache.stride(2)
+    s.v_stride_b, s.v_stride_t, s.v_stride_h = v_cache.stride(0), v_cache.stride(1), v_cache.stride(2)
+    s.tsrc = 0
+    s.max_tsrc = max_tsrc
+    s.block_table = block_table.data_ptr()
+    s.cache_seq_lens = cache_seq_lens.data_ptr()
+    s.bt_stride_b = block_table.stride(0)
+    s.bt_is64 = int(block_table.dtype == torch.int64)
+    s.sl_is64 = int(cache_seq_lens.dtype == torch.int64)
+    s.paged = 1
+    s.page_size = k_cache.shape[1]
+    s.HKV = k_cache.shape[2]
+    return s
+
+
+# ------------------------------------------------------------------ thin wrappers, one per entry point
+
+def mask_stage(qs, kvs, chunk_left, hg, n, chunk, right_clamp, bs, bq, stride_q, block_chunk, scan_stride,
+               sw_eff, terminate, scores, left_out, device):
+    rc = lib().hipattn_mask_stage(
+        ctypes.byref(qs), ctypes.byref(kvs), _p(chunk_left), ctypes.c_int32(hg), ctypes.c_int32(n),
+        ctypes.c_int32(chunk), ctypes.c_int64(right_clamp), ctypes.c_int32(bs), ctypes.c_int32(bq),
+        ctypes.c_int32(stride_q), ctypes.c_int32(block_chunk), ctypes.c_int32(scan_stride),
+        ctypes.c_int32(sw_eff), ctypes.c_int32(terminate), _p(scores), _p(left_out), stream_ptr(device))
+    check(rc, "hipattn_mask_stage")
+
+
+def select_stage(scores, chunk_left, B, bs_in, bs_out, row_rep, HEAD, hg, n, k, chunk, splits, next_left, device):
+    rc = lib().hipattn_select_stage(
+        _p(scores), _p(chunk_left), ctypes.c_int32(B), ctypes.c_int32(bs_in), ctypes.c_int32(bs_out),
+        ctypes.c_int32(row_rep), ctypes.c_int32(HEAD), ctypes.c_int32(hg), ctypes.c_int32(n), ctypes.c_int32(k),
+        ctypes.c_int32(chunk), ctypes.c_int32(splits), _p(next_left), stream_ptr(device))
+    check(rc, "hipattn_select_stage")
+
+
+def finalize_indices(scores, left_out, pos, B, bs, bdst, scan_stride, HEAD, hg, n, K, chunk, bq,
+                     indices, ks, ks_start_end, device):
+    rc = lib().hipattn_finalize_indices(
+        _p(scores), _p(left_out), _p(pos), ctypes.c_int64(pos.stride(0)), ctypes.c_int64(pos.stride(1)),
+        ctypes.c_int32(B), ctypes.c_int32(bs), ctypes.c_int32(bdst), ctypes.c_int32(scan_stride),
+        ctypes.c_int32(HEAD), ctypes.c_int32(hg), ctypes.c_int32(n), ctypes.c_int32(K), ctypes.c_int32(chunk),
+        ctypes.c_int32(bq), _p(indices), _p(ks), _p(ks_start_end), stream_ptr(device))
+    check(rc, "hipattn_finalize_indices")
+
+
+def bsa_prefill(qs, kvs, indices, ks_start_end, BK, bq, bk, sw, sink, share_first_head, impl, out, device):
+    assert indices.dtype == torch.int64 and indices.is_contiguous()
+    assert ks_start_end.dtype == torch.int32 and ks_start_end.is_contiguous()
+    rc = lib().hipattn_bsa_prefill(
+        ctypes.byref(qs), ctypes.byref(kvs), _p(indices), _p(ks_start_end), ctypes.c_int32(indices.shape[1]),
+        ctypes.c_int32(BK), ctypes.c_int32(bq), ctypes.c_int32(bk), ctypes.c_int32(sw), ctypes.c_int32(sink),
+        ctypes.c_int32(int(share_first_head)), ctypes.c_int32(impl), _p(out), ctypes.c_int64(out.stride(0)),
+        ctypes.c_int64(out.stride(1)), ctypes.c_int64(out.stride(2)), stream_ptr(device))
+    check(rc, "hipattn_bsa_prefill")
+
+
+def bsa_decode(qs, kvs, indices, ks_start_end, BK, bk, sw, sink, out, device, nsplits=0, workspace=None):
+    assert indices.dtype == torch.int64 and indices.is_contiguous()
+    assert ks_start_end.dtype == torch.int32 and ks_start_end.is_contiguous()
+    L = lib()
+    B, HEAD, HID = qs.B, qs.HEAD, qs.HID
+    if nsplits <= 0:
+        nsplits = L.hipattn_bsa_decode_default_splits(ctypes.c_int32(B), ctypes.c_int32(kvs.HKV),
+                                                      ctypes.c_int32(BK * bk + sink + sw + 1))
+    need = L.hipattn_bsa_decode_workspace_bytes(ctypes.c_int32(B), ctypes.c_int32(HEAD), ctypes.c_int32(HID),
+                                                ctypes.c_int32(nsplits))
+    if workspace is None or workspace.numel() * workspace.element_size() < need:
+        workspace = torch.empty(need // 4, dtype=torch.float32, device=out.device)
+    rc = L.hipattn_bsa_decode_partial(
+        ctypes.byref(qs), ctypes.byref(kvs), _p(indices), _p(ks_start_end), ctypes.c_int32(indices.shape[1]),
+        ctypes.c_int32(BK), ctypes.c_int32(bk), ctypes.c_int32(sw), ctypes.c_int32(sink), ctypes.c_int32(nsplits),
+        _p(workspace), stream_ptr(device))
+    check(rc, "hipattn_bsa_decode_partial")
+    rc = L.hipattn_bsa_decode_merge(
+        _p(workspace), ctypes.c_int32(B), ctypes.c_int32(HEAD), ctypes.c_int32(HID), ctypes.c_int32(nsplits),
+        ctypes.c_int32(qs.dtype), _p(out), ctypes.c_int64(out.stride(0)), ctypes.c_int64(out.stride(2)),
+        stream_ptr(device))
+    check(rc, "hipattn_bsa_decode_merge")
+    return workspace

@@ -1,0 +1,382 @@
+"""``hip_attention_12``: hierarchical mask estimation followed by block-sparse attention.
+
+Host-side driver with the call signature and result layout of the reference operator
+``dual_stage_quadratic_hip_attention`` (``src/hip_attn/v1_2/attention_extend.py:1918-3133``).
+All arithmetic runs in ``libhipattn.so``; this module only sizes buffers and sequences launches
+on the current stream.  No host synchronisation happens inside a call.
+
+Differences in representation (not in results):
+  * with head reduction on (the default, env ``HIP_HEAD_REDUCE``), every head of a batch item
+    works on the same candidate chunk list, so one ``int32 [B, BDST, 1, chunks]`` list is kept
+    instead of the reference's ``int64 [B, BDST, HEAD, chunks]`` left/right pair; chunk lists stay
+    ascending, which turns the reference's topk + sort + gather into a compaction;
+  * stage caches are materialised in the reference layout only as expanded views.
+"""
+from __future__ import annotations
+
+import os
+from typing import List, Optional
+
+import torch
+from torch import Tensor
+
+from . import _native as N
+from .metadata import (
+    HiPAttentionArgs,
+    HiPAttentionCacheAccessStatistics,
+    HiPAttentionOutputMetadata,
+    HiPAttentionStageInputCache,
+    NopStage,
+    ScanStage,
+)
+
+_BIG = (1 << 62)
+
+
+def _cdiv(a: int, b: int) -> int:
+    return -(-a // b)
+
+
+def _npow2(x: int) -> int:
+    return 1 if x <= 1 else 1 << (int(x) - 1).bit_length()
+
+
+def _head_reduce_enabled() -> bool:
+    return os.getenv("HIP_HEAD_REDUCE", "1") == "1"
+
+
+def _reject_unsupported(args: HiPAttentionArgs):
+    if args.using_extend or args.need_apply_rope:
+        raise NotImplementedError("RoPE 'extend' modes (using_extend / need_apply_rope) are not built yet")
+    if args.logit_softcap is not None:
+        raise NotImplementedError("logit_softcap is not built yet")
+    if not args.is_causal:
+        raise NotImplementedError("is_causal=False is not built")
+    if args.sliding_window_indices is not None:
+        raise NotImplementedError("sliding_window_indices is a research switch and is not built")
+    if args.online_update_cache:
+        raise NotImplementedError("online_update_cache (in-kernel cache fill) is not built")
+    if (args.low_percent > 0) and (args.low_k_ratio < 1):
+        raise NotImplementedError("low_percent / low_k_ratio pruning is dead code in the reference and not built")
+
+
+def _kv_struct(args: HiPAttentionArgs, k: Optional[Tensor], v: Optional[Tensor], max_tsrc: int):
+    """Returns (struct, keepalive) describing where K/V rows live."""
+    if k is not None:
+        kk = k if k.stride(-1) == 1 else k.contiguous()
+        vv = v if v.stride(-1) == 1 else v.contiguous()
+        return N.make_kv_dense(kk, vv), (kk, vv)
+    if args.offload_cache is not None:
+        return args.offload_cache.kv_struct(max_tsrc)
+    bt = args.block_table
+    sl = args.cache_seq_lens
+    assert args.k_cache is not None and args.v_cache is not None, "paged mode needs k_cache and v_cache"
+    assert bt is not None and bt.ndim == 2, "paged mode needs block_table [B, pages]"
+    assert sl is not None and sl.ndim == 1, "paged mode needs cache_seq_lens [B]"
+    assert args.k_cache.ndim == 4 and args.v_cache.ndim == 4
+    if bt.dtype not in (torch.int32, torch.int64):
+        bt = bt.to(torch.int64)
+    if bt.stride(1) != 1:
+        bt = bt.contiguous()
+    if sl.dtype not in (torch.int32, torch.int64):
+        sl = sl.to(torch.int64)
+    if sl.stride(0) != 1:
+        sl = sl.contiguous()
+    return N.make_kv_paged(args.k_cache, args.v_cache, bt, sl, max_tsrc), (bt, sl)
+
+
+def _stage_cache_views(chunk_left: Tensor, HEAD: int, chunk: int) -> HiPAttentionStageInputCache:
+    """Reference-layout view of a stage's inputs: int64 left/right and the reset scores."""
+    B, BS, hg, n = chunk_left.shape
+    left = chunk_left.to(torch.int64)
+    if hg == 1:
+        left = left.expand(B, BS, HEAD, n)
+    right = left + chunk
+    scores = torch.full((1, 1, 1, 1), -32000.0, dtype=torch.float32, device=chunk_left.device).expand(B, BS, HEAD, n)
+    return HiPAttentionStageInputCache(indices_left=left, indices_right=right, out_scores=scores)
+
+
+def _chunk_list_from_cache(cache: HiPAttentionStageInputCache, hg: int) -> Tensor:
+    left = cache.indices_left
+    if hg == 1:
+        left = left[:, :, :1, :]
+    return left.to(torch.int32).contiguous()
+
+
+@torch.no_grad()
+def dual_stage_quadratic_hip_attention(
+    q: Tensor,
+    k: Optional[Tensor],
+    v: Optional[Tensor],
+    args: HiPAttentionArgs,
+    cached_metadata: Optional[HiPAttentionOutputMetadata] = None,
+):
+    """HiP attention: returns ``(context, HiPAttentionOutputMetadata)``.
+
+    ``q [B, TDST, HEAD, HID]``; ``k, v [B, TSRC, HEAD_KV, HID]`` or ``None`` with a paged cache in
+    ``args``.  ``q`` is used as given: no softmax scale is applied (callers pre-scale).
+    Passing ``cached_metadata`` with ``indices`` skips mask estimation; with only
+    ``stage_caches`` it resumes estimation from the last cached stage.  Returns ``(None, None)``
+    when ``args.mask_only``.
+    """
+    N.lib()
+    if not q.is_cuda:
+        raise N.HipAttnError("hip_attention_12 runs on the GPU only: q must be a device tensor")
+    _reject_unsupported(args)
+    device = q.device
+
+    q_bsa = q
+    if args.q_mask is not None:
+        q = args.q_mask
+    k_mask = k if args.k_mask is None else args.k_mask
+
+    BSZ, TDST, HEAD, HID = q.shape
+    if k is not None:
+        _, TSRC, HEAD_KV, _ = k.shape
+        assert v is not None and v.shape == k.shape
+        MAX_TSRC = TSRC
+    else:
+        MAX_TSRC = args.extend_context_length
+        TSRC = MAX_TSRC
+        HEAD_KV = args.k_cache.shape[-2] if args.k_cache is not None else args.offload_cache.head_kv
+
+    stages = args.stages
+    assert len(stages) > 0
+    STAGE_STRIDE = stages[0].stage_stride
+    BLOCK_SIZE_Q = stages[0].stage_block_size_q
+    BDST = _cdiv(TDST, BLOCK_SIZE_Q)
+    BDST_SCAN = _cdiv(BDST, STAGE_STRIDE)
+    BLOCK_CHUNK = args.block_size_k
+    chunk_size = stages[0].stage_chunk_size
+    chunk_count = _cdiv(max(0, MAX_TSRC - args.sink_token_size - args.sliding_window_size), chunk_size)
+
+    args = args.clone()
+    args.mask_k = stages[0].stage_chunk_size
+    args.sliding_window_size = max(0, args.sliding_window_size - args.mask_k)
+    sw_eff = args.sliding_window_size
+    sink = args.sink_token_size
+
+    if args.position_ids is not None:
+        position_ids = args.position_ids
+        if position_ids.dtype != torch.int64:
+            position_ids = position_ids.to(torch.int64)
+    else:
+        position_ids = (torch.arange(0, TDST, device=device, dtype=torch.int64) + (TSRC - TDST))[None, :].expand(BSZ, TDST)
+    assert position_ids.shape == (BSZ, TDST), position_ids.shape
+
+    stage_caches: Optional[List[HiPAttentionStageInputCache]] = (
+        [] if (cached_metadata is None) or (cached_metadata.stage_caches is None) else cached_metadata.stage_caches
+    )
+    if not args.require_stage_caches:
+        stage_caches = None
+
+    qq = q if q.stride(-1) == 1 else q.contiguous()
+    mask_kv, keep_mask_kv = _kv_struct(args, k_mask, k_mask, MAX_TSRC)
+    hg = 1 if _head_reduce_enabled() else HEAD
+
+    if (cached_metadata is None) or (cached_metadata.indices is None):
+        fresh = (cached_metadata is None) or (cached_metadata.stage_caches is None) or (stage_caches is None)
+        if (not fresh) and stage_caches[-1].indices_left is None:
+            # only the empty stage-0 entry is cached: nothing to resume from
+            assert len(stage_caches) == 1
+            fresh = True
+        if fresh:
+            chunk_left = (torch.arange(0, chunk_count, device=device, dtype=torch.int32) * chunk_size + sink)
+            chunk_left = chunk_left[None, None, None, :].expand(BSZ, BDST_SCAN, hg, chunk_count).contiguous()
+            right_clamp = MAX_TSRC - sw_eff
+        else:
+            assert len(stage_caches) <= len(stages)
+            chunk_left = _chunk_list_from_cache(stage_caches[-1], hg)
+            right_clamp = _BIG
+
+        scores = None
+        left_out = None
+        prev_n = None
+        n_cached = len(stage_caches) if stage_caches is not None else 0
+        for i_stage, stage in enumerate(stages):
+            if i_stage < n_cached - 1:
+                continue
+            elif i_stage == n_cached - 1:
+                pass
+            elif i_stage > 0:
+                # truncate / realign / sort / re-tile / split (:2072-2165) folded into one selection pass
+                assert isinstance(stage, (ScanStage, NopStage)), f"stage type {type(stage).__name__} is not executable"
+                if not stage.require_realign_index or not stage.require_reset_score:
+                    raise NotImplementedError("stages with require_realign_index/require_reset_score off are not built")
+                assert (stage.stage_k % chunk_size) == 0, f"{stage.stage_k} % {chunk_size}"
+                keep = min(stage.stage_k // chunk_size, prev_n)
+                row_rep = 1
+                bs_in = chunk_left.shape[1]
+                if BLOCK_SIZE_Q != stage.stage_block_size_q:
+                    assert stage.stage_block_size_q > 0 and BLOCK_SIZE_Q > stage.stage_block_size_q
+                    assert (BLOCK_SIZE_Q % stage.stage_block_size_q) == 0
+                    row_rep *= BLOCK_SIZE_Q // stage.stage_block_size_q
+                    BLOCK_SIZE_Q = stage.stage_block_size_q
+                    BDST = _cdiv(TDST, BLOCK_SIZE_Q)
+                    BDST_SCAN = _cdiv(BDST, STAGE_STRIDE)
+                if row_rep != 1 and STAGE_STRIDE != 1:
+                    raise NotImplementedError("a stage may shrink its query block only when stage_stride is 1")
+                if STAGE_STRIDE != stage.stage_stride:
+                    assert stage.stage_stride < STAGE_STRIDE and STAGE_STRIDE > 0
+                    if stage.stage_stride != 1:
+                        raise NotImplementedError("stage_stride may only drop to 1 between stages")
+                    row_rep *= STAGE_STRIDE // stage.stage_stride
+                    STAGE_STRIDE = stage.stage_stride
+                    BDST_SCAN = _cdiv(BDST, STAGE_STRIDE)
+                bs_out = BDST_SCAN if row_rep == 1 else min(BDST, row_rep * bs_in)
+                assert (chunk_size % stage.stage_chunk_size) == 0
+                splits = chunk_size // stage.stage_chunk_size
+                next_left = torch.empty((BSZ, bs_out, hg, keep * splits), dtype=torch.int32, device=device)
+                N.select_stage(scores, chunk_left, BSZ, bs_in, bs_out, row_rep, HEAD, hg, prev_n, keep,
+                               chunk_size, splits, next_left, device)
+                chunk_left = next_left
+                right_clamp = _BIG
+            else:
+                assert stage.stage_k is None, "first stage always quadratic"
+                assert isinstance(stage, ScanStage), f"first stage always scan {stage}"
+                STAGE_STRIDE = stage.stage_stride
+
+            if (stage_caches is not None) and (i_stage >= len(stage_caches)):
+                if i_stage == 0:
+                    stage_caches.append(HiPAttentionStageInputCache(None, None, None))
+                else:
+                    stage_caches.append(_stage_cache_views(chunk_left, HEAD, stage.stage_chunk_size))
+
+            chunk_size = stage.stage_chunk_size
+            chunk_count = chunk_left.shape[-1]
+            BLOCK_CHUNK = max(16, _npow2(min(chunk_count, BLOCK_CHUNK)))
+            if BLOCK_CHUNK > 64:
+                raise NotImplementedError(f"block_size_k (chunks per scan program) above 64 is not built: {BLOCK_CHUNK}")
+            bs = chunk_left.shape[1]
+            last = i_stage == len(stages) - 1
+
+            if isinstance(stage, ScanStage):
+                scores = torch.empty((BSZ, bs, HEAD, chunk_count), dtype=torch.float32, device=device)
+                left_out = torch.empty((BSZ, bs, HEAD, chunk_count), dtype=torch.int32, device=device) if last else None
+                if chunk_count > 0:
+                    qs = N.make_q(qq, position_ids)
+                    N.mask_stage(qs, mask_kv, chunk_left, hg, chunk_count, chunk_size, right_clamp, bs,
+                                 BLOCK_SIZE_Q, stage.stage_block_stride_q, BLOCK_CHUNK, STAGE_STRIDE, sw_eff,
+                                 args.stage_early_terminate, scores, left_out, device)
+            elif isinstance(stage, NopStage):
+                scores = torch.full((BSZ, bs, HEAD, chunk_count), -32000.0, dtype=torch.float32, device=device)
+                left_out = chunk_left.expand(BSZ, bs, HEAD, chunk_count).contiguous() if last else None
+            else:
+                raise NotImplementedError(f"stage type {type(stage).__name__} raises in the reference as well")
+            if not stage.require_post_sort:
+                raise NotImplementedError("stages without require_post_sort are not built")
+            prev_n = chunk_count
+
+        assert (args.second_stage_k % chunk_size) == 0
+        K = args.second_stage_k // chunk_size
+        BK = min(K, chunk_count)
+        indices = torch.empty((BSZ * HEAD, BDST, max(BK, 1)), dtype=torch.int64, device=device)
+        ks = torch.empty((BSZ * HEAD, BDST), dtype=torch.int64, device=device)
+        ks_start_end = torch.empty((BSZ * HEAD, BDST, 2), dtype=torch.int32, device=device)
+        if BK > 0:
+            N.finalize_indices(scores, left_out, position_ids, BSZ, chunk_left.shape[1], BDST, STAGE_STRIDE, HEAD, hg,
+                               chunk_count, K, chunk_size, stages[-1].stage_block_size_q, indices, ks, ks_start_end,
+                               device)
+        else:
+            indices = indices[:, :, :0]
+            ks.zero_()
+            ks_start_end.zero_()
+        ks_count = ks.unsqueeze(-1)
+
+        args = args.clone()
+        args.block_size_q = stages[-1].stage_block_size_q
+        block_sparse_block_size_q = (
+            min(args.block_sparse_block_size_q, args.block_size_q) if args.block_sparse_block_size_q is not None else None
+        )
+        args.sliding_window_size += args.mask_k
+        args.block_size_k = chunk_size
+        args.mask_k = args.second_stage_k
+
+        if (block_sparse_block_size_q is not None) and (
+            _cdiv(TDST, block_sparse_block_size_q) != _cdiv(TDST, args.block_size_q)
+        ):
+            assert (BLOCK_SIZE_Q % block_sparse_block_size_q) == 0
+            rep = BLOCK_SIZE_Q // block_sparse_block_size_q
+            indices = indices.repeat_interleave(rep, 1)
+            ks = ks.repeat_interleave(rep, 1)
+            ks_count = ks_count.repeat_interleave(rep, 1)
+            ks_start_end = ks_start_end.repeat_interleave(rep, 1)
+            args.block_size_q = block_sparse_block_size_q
+
+        if args.mask_only:
+            return None, None
+        fresh_mask = True
+    else:
+        args = args.clone()
+        args.sliding_window_size += args.mask_k
+        args.block_size_k = stages[-1].stage_chunk_size
+        args.mask_k = args.second_stage_k
+        indices = cached_metadata.indices.clone()
+        ks = cached_metadata.ks.clone()
+        ks_count = cached_metadata.ks_count.clone()
+        ks_start_end = cached_metadata.ks_start_end.clone()
+        fresh_mask = False
+
+    args.block_size_q = min(args.block_size_q, _npow2(TDST))
+    if args.sliding_window_size == 777:
+        args.sliding_window_size = (
+            args.model_context_length - args.sink_token_size - args.second_stage_k - args.block_size_q
+        )
+
+    use_decode = (
+        (TDST == 1) and (os.environ.get("HIP_DISABLE_FLASHDECODE", "0") != "1") and (not args.disable_flashdecode)
+    )
+    seq_pos = position_ids[:, -q_bsa.shape[1]:]
+    context = block_sparse_attention(
+        q_bsa, k, v, seq_pos, indices, ks_start_end, args, MAX_TSRC, decode=use_decode,
+    )
+
+    return context, HiPAttentionOutputMetadata(
+        indices=indices,
+        ks=ks,
+        ks_count=ks_count,
+        ks_start_end=ks_start_end,
+        mask_cache_statistics=(HiPAttentionCacheAccessStatistics(None, None) if fresh_mask else None),
+        sa_cache_statistics=HiPAttentionCacheAccessStatistics(None, None),
+        stage_caches=stage_caches,
+    )
+
+
+@torch.no_grad()
+def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], position_ids: Tensor, indices: Tensor,
+                           ks_start_end: Tensor, args: HiPAttentionArgs, max_tsrc: int, decode: bool = False,
+                           impl: int = 0) -> Tensor:
+    """Sparse attention over (selected blocks, sink, sliding window) given the metadata tensors.
+
+    ``position_ids`` are 0-based (the reference passes ``seq_lens = position_ids + 1``,
+    attention_extend.py:3092).  ``args.block_size_q / block_size_k / sliding_window_size`` must
+    already hold the values the operator derives for this step.  ``decode`` selects the split-KV
+    path, which, like the reference's decode kernel, lets every head of a GQA group read the
+    index row of the group's first head.
+    """
+    device = q.device
+    qq = q if q.stride(-1) == 1 else q.contiguous()
+    kvs, keep = _kv_struct(args, k, v, max_tsrc)
+    if position_ids.dtype != torch.int64:
+        position_ids = position_ids.to(torch.int64)
+    qs = N.make_q(qq, position_ids)
+    if not indices.is_contiguous():
+        indices = indices.contiguous()
+    if not ks_start_end.is_contiguous():
+        ks_start_end = ks_start_end.contiguous()
+    BK = indices.shape[-1]
+    out = torch.empty(q.shape, dtype=q.dtype, device=device)
+    if BK == 0:
+        indices = torch.zeros((indices.shape[0], indices.shape[1], 1), dtype=torch.int64, device=device)
+    if decode:
+        try:
+            N.bsa_decode(qs, kvs, indices, ks_start_end, BK, args.block_size_k, args.sliding_window_size,
+                         args.sink_token_size, out, device)
+            return out
+        except N.HipAttnError as e:
+            if "is not built" not in str(e):
+                raise
+    N.bsa_prefill(qs, kvs, indices, ks_start_end, BK, args.block_size_q, args.block_size_k,
+                  args.sliding_window_size, args.sink_token_size, decode, impl, out, device)
+    del keep
+    return out

@@ -1,0 +1,144 @@
+/*
+ * hipattn -- MI355X (gfx950) kernels for HiP / InfiniteHiP attention, C ABI.
+ *
+ * The reference operator is Python + Triton and has no C interface of its own; each entry
+ * point below names the reference function or kernel launch it stands in for (paths relative
+ * to the reference repository root).  Conventions:
+ *   - extern "C", plain pointers and sizes only; every pointer is a DEVICE pointer unless the
+ *     comment says host; strides are in ELEMENTS; the innermost (head-dim) stride is 1.
+ *   - the caller owns every buffer; nothing here allocates device memory.
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*); nothing synchronises.
+ *   - return value: 0 = ok, negative = argument error (HIPATTN_E_*), positive = hipError_t.
+ *     hipattn_last_error() returns a host string describing the last failure of this thread.
+ */
+#ifndef HIPATTN_H
+#define HIPATTN_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HIPATTN_F32 0
+#define HIPATTN_BF16 1
+
+#define HIPATTN_E_ARG (-1)       /* null pointer / negative size / inconsistent shapes */
+#define HIPATTN_E_UNSUPPORTED (-2) /* valid request the kernels do not cover (head dim, limits) */
+#define HIPATTN_E_ALIGN (-3)     /* pointer or stride not aligned for 16-byte row loads */
+
+/* Query tensor q[B, TDST, HEAD, HID] and its token positions (0-based, int64)
+ * -- the (q, position_ids) pair of dual_stage_quadratic_hip_attention,
+ * src/hip_attn/v1_2/attention_extend.py:1918-1987. */
+typedef struct hipattn_q {
+    const void *ptr;
+    int64_t stride_b, stride_t, stride_h;
+    const int64_t *pos; /* [B, TDST] */
+    int64_t pos_stride_b, pos_stride_t;
+    int32_t B, TDST, HEAD, HID;
+    int32_t dtype; /* HIPATTN_F32 / HIPATTN_BF16; K and V share it */
+} hipattn_q_t;
+
+/* Key/value storage: dense k,v[B, TSRC, HKV, HID] or a paged cache [pages, page_size, HKV, HID]
+ * addressed through block_table[B, cols] -- HiPAttentionArgs.args_paged_kv_cache,
+ * src/hip_attn/v1_2/attention_metadata.py:282-330, and load_tokens,
+ * src/hip_attn/v1_2/uvm_gpu_cache.py:843-890,1034-1042.
+ * Row address: dense  ptr + b*stride_b + t*stride_t + h*stride_h
+ *              paged  ptr + page*stride_b + (t % page_size)*stride_t + h*stride_h,
+ *                     page = (0 <= t < cache_seq_lens[b]) ? block_table[b][t / page_size] : 0
+ * Dense reads at t >= tsrc return zeros. */
+typedef struct hipattn_kv {
+    const void *k;
+    const void *v;
+    int64_t k_stride_b, k_stride_t, k_stride_h;
+    int64_t v_stride_b, v_stride_t, v_stride_h;
+    int64_t tsrc;     /* dense only */
+    int64_t max_tsrc; /* TSRC, or extend_context_length when paged */
+    const void *block_table;    /* int32 or int64 [B, cols] */
+    const void *cache_seq_lens; /* int32 or int64 [B] */
+    int64_t bt_stride_b;
+    int32_t bt_is64, sl_is64;
+    int32_t paged, page_size;
+    int32_t HKV;
+} hipattn_kv_t;
+
+const char *hipattn_version(void);
+const char *hipattn_last_error(void);
+
+/* One scan stage of mask estimation: per (batch, scan row, head, chunk) binary-search refinement
+ * and score.  Replaces the launch of chunk_controllable_sampling_mask_cuda,
+ * src/hip_attn/v1_2/attention_extend.py:412-1249 (launch :2516-2563).
+ *   chunk_left  int32 [B, BS, HG, n]   start of every candidate chunk, ascending; HG = 1 when
+ *                                      scores are max-reduced over heads, else HEAD
+ *   right = min(left + chunk_size, right_clamp)
+ *   scores      f32   [B, BS, HEAD, n] written for every chunk (-32000 where not scored)
+ *   left_out    int32 [B, BS, HEAD, n] refined left edge per head, or NULL
+ *   block_chunk = chunks per reference program (16/32/64): fixes the program-level gate and
+ *   iteration count (:595-601,736-737). */
+int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, const int32_t *chunk_left,
+                       int32_t hg, int32_t n, int32_t chunk_size, int64_t right_clamp,
+                       int32_t bs, int32_t bq, int32_t stride_q, int32_t block_chunk,
+                       int32_t scan_stride, int32_t sw_eff, int32_t terminate_size,
+                       float *scores, int32_t *left_out, void *stream);
+
+/* Between two stages: max over heads, top-k under (score desc, position asc), realign, split.
+ * Replaces the ATen glue at src/hip_attn/v1_2/attention_extend.py:2566-2570 (head reduce),
+ * :2710-2728 (topk + gather) and :2072-2165 (truncate, realign, sort, re-tile, split).
+ *   scores      f32   [B, BS_in, HEAD, n]
+ *   chunk_left  int32 [B, BS_in, HG, n]
+ *   next_left   int32 [B, BS_out, HG, k*splits]; chunk j of a kept parent starts at
+ *               left + j*(chunk_size/splits)
+ *   output row o reads input row (o + row_rep*BS_in - BS_out) / row_rep
+ *   (repeat_interleave(row_rep, 1)[:, -BS_out:], :2092-2123). */
+int hipattn_select_stage(const float *scores, const int32_t *chunk_left, int32_t B, int32_t bs_in,
+                         int32_t bs_out, int32_t row_rep, int32_t HEAD, int32_t hg, int32_t n,
+                         int32_t k, int32_t chunk_size, int32_t splits, int32_t *next_left,
+                         void *stream);
+
+/* After the last stage: top-K chunks, block alignment, de-duplication, active count, in the
+ * reference's metadata layout.  Replaces src/hip_attn/v1_2/attention_extend.py:2757-2776 and
+ * :2906-2924.
+ *   left_out    int32 [B, BS, HEAD, n]  refined left edges from the last hipattn_mask_stage
+ *   indices     int64 [B*HEAD, BDST, BK] ascending unique block starts then INT64_MAX
+ *   ks          int64 [B*HEAD, BDST]     entries below pos[b, qb*bq] + bq
+ *   ks_start_end int32 [B*HEAD, BDST, 2] = (0, ks)
+ *   BK = min(K, n); output row qb reads scan row (qb + scan_stride*BS - BDST) / scan_stride. */
+int hipattn_finalize_indices(const float *scores, const int32_t *left_out, const int64_t *pos,
+                             int64_t pos_stride_b, int64_t pos_stride_t, int32_t B, int32_t bs,
+                             int32_t bdst, int32_t scan_stride, int32_t HEAD, int32_t hg, int32_t n,
+                             int32_t K, int32_t chunk_size, int32_t bq, int64_t *indices,
+                             int64_t *ks, int32_t *ks_start_end, void *stream);
+
+/* Block-sparse flash attention over selected blocks + sink + sliding window.  Replaces
+ * block_sparse_attention, src/hip_attn/v1_2/attention_extend_bsa.py:1641-1777 (kernel :607-1638).
+ *   indices int64 [B*HEAD, idx_rows, BK], ks_start_end int32 [B*HEAD, idx_rows, 2]
+ *   out has q's dtype; out strides in elements.
+ *   share_first_head != 0: every head of a GQA group reads the index row of the group's first
+ *   head (decode kernel behaviour, src/hip_attn/v1_2/attention_decode_bsa.py:150).
+ *   impl: 0 = pick automatically, 1 = portable row-at-a-time kernel, 2 = MFMA tile kernel. */
+int hipattn_bsa_prefill(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t *indices,
+                        const int32_t *ks_start_end, int32_t idx_rows, int32_t BK,
+                        int32_t block_size_q, int32_t block_size_k, int32_t sliding_window,
+                        int32_t sink, int32_t share_first_head, int32_t impl, void *out,
+                        int64_t out_stride_b, int64_t out_stride_t, int64_t out_stride_h,
+                        void *stream);
+
+/* Decode (TDST == 1) split-KV attention.  Replaces decode_block_sparse_attention,
+ * src/hip_attn/v1_2/attention_decode_bsa.py:1331-1435: _fwd_kernel_stage1 (:22-1045) writes
+ * per-split partials, _fwd_kernel_stage2 (:1148-1226) merges them by log-sum-exp.
+ *   workspace: f32, hipattn_bsa_decode_workspace_bytes(...) bytes, caller-allocated.
+ *   nsplits: 0 = choose from the device size. */
+int64_t hipattn_bsa_decode_workspace_bytes(int32_t B, int32_t HEAD, int32_t HID, int32_t nsplits);
+int32_t hipattn_bsa_decode_default_splits(int32_t B, int32_t HKV, int32_t tokens);
+int hipattn_bsa_decode_partial(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t *indices,
+                               const int32_t *ks_start_end, int32_t idx_rows, int32_t BK,
+                               int32_t block_size_k, int32_t sliding_window, int32_t sink,
+                               int32_t nsplits, void *workspace, void *stream);
+int hipattn_bsa_decode_merge(const void *workspace, int32_t B, int32_t HEAD, int32_t HID,
+                             int32_t nsplits, int32_t dtype, void *out, int64_t out_stride_b,
+                             int64_t out_stride_h, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HIPATTN_H */
