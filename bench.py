@@ -1,0 +1,259 @@
+#!/usr/bin/env python3
+"""Benchmark of the HiP attention hot path on one MI355X.
+
+Primary workload (BASELINE.json configs[1], the README shape): one ``hip_attention_12`` prefill call
+with B=1, 32768 queries against 131072 keys, 32 query heads over 8 KV heads, head dim 128, bf16,
+default stages, sink 256, window 1024.  A "step" is one full call (mask estimation + block-sparse
+attention) on synthetic inputs already resident in HBM.  ``value`` = queries / second.
+
+Also reported in the same JSON line:
+  * ``decode``: a 1M-token KV decode loop (configs[3] phase B: mask refreshed every 8 steps),
+    microseconds per step and the HBM roofline fraction of a refresh step;
+  * ``roofline``: the dominant kernel of the prefill step, timed with HIP events inside the timed
+    region, against its algorithmic bytes (mask stage: sampled key rows) or flops (attention);
+  * ``cpu_baseline``: the CPU oracle (a port of the reference algorithm, OpenMP) on a bounded sample
+    of the same workload (the last two query blocks against the full 128k keys), threads stated.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "hip-attention_amd"), os.path.join(ROOT, "tests")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def cdiv(a, b):
+    return -(-a // b)
+
+
+def mask_stage_bytes(B, TDST, HEAD, HID, esz, stage_shapes):
+    """Algorithmic bytes of mask estimation: every sampled key row, per (batch, q-block, head, chunk, iteration)."""
+    out = []
+    for (bq, n, chunk) in stage_shapes:
+        iters = chunk.bit_length()  # floor(log2(chunk)) + 1
+        rows = B * cdiv(TDST, bq) * HEAD * n * iters * 2
+        out.append(rows * HID * esz)
+    return out
+
+
+def prefill_workload(device, seed=1, TQ=32768, TK=131072, H=32, HKV=8, D=128):
+    import torch
+
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    q = torch.randn((1, TQ, H, D), generator=g, dtype=torch.float32).to(torch.bfloat16).to(device)
+    k = torch.randn((1, TK, HKV, D), generator=g, dtype=torch.float32).to(torch.bfloat16).to(device)
+    v = k.clone()
+    return q, k, v
+
+
+def run_prefill(args, device):
+    import torch
+    from hip_attn import HiPAttentionArgs12, hip_attention_12
+    from hip_attn import _native as N
+
+    TQ, TK, H, HKV, D = 32768, 131072, 32, 8, 128
+    q, k, v = prefill_workload(device, 1, TQ, TK, H, HKV, D)
+    hargs = HiPAttentionArgs12(sliding_window_size=1024)
+    for _ in range(args.warmup):
+        hip_attention_12(q, k, v, hargs)
+    torch.cuda.synchronize()
+    N.profile_begin()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        ctx, meta = hip_attention_12(q, k, v, hargs)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    prof = N.profile_end()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+
+    # per-kernel averages over the timed region
+    agg = {}
+    for name, ms in prof:
+        a = agg.setdefault(name, [0.0, 0])
+        a[0] += ms
+        a[1] += 1
+    kern = {name: tot / cnt for name, (tot, cnt) in agg.items()}
+    launches_per_step = {name: cnt / args.steps for name, (tot, cnt) in agg.items()}
+
+    sink, sw, K2 = 256, 1024, 2048
+    n0 = cdiv(TK - sink - sw, 256)
+    n1 = min(32768 // 256, n0) * 8
+    n2 = min(8192 // 32, n1) * 4
+    stage_bytes = mask_stage_bytes(1, TQ, H, D, 2, [(64, n0, 256), (64, n1, 32), (64, n2, 8)])
+    names = [f"mask_stage[n={n0},chunk=256,rows=16]", f"mask_stage[n={n1},chunk=32,rows=16]",
+             f"mask_stage[n={n2},chunk=8,rows=64]"]
+    attended = K2 + sink + sw
+    bsa_flops = 4.0 * D * TQ * H * attended
+    rooflines = []
+    for nm, by in zip(names, stage_bytes):
+        if nm in kern:
+            gbs = by / (kern[nm] * 1e-3) / 1e9
+            rooflines.append({"kernel": nm, "bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                              "frac": gbs / HBM_PEAK_GBS, "traffic": None, "ms": kern[nm],
+                              "algorithmic_bytes": by})
+    if "bsa_prefill" in kern:
+        tf = bsa_flops / (kern["bsa_prefill"] * 1e-3) / 1e12
+        rooflines.append({"kernel": "bsa_prefill", "bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS,
+                          "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                          "ms": kern["bsa_prefill"], "algorithmic_flops": bsa_flops})
+    dominant = max(rooflines, key=lambda r: r["ms"]) if rooflines else None
+    del q, k, v, ctx, meta
+    torch.cuda.empty_cache()
+    return {
+        "ms_per_step": ms_per_step,
+        "tok_per_s": TQ / (ms_per_step * 1e-3),
+        "kernels_ms": kern,
+        "launches_per_step": launches_per_step,
+        "rooflines": rooflines,
+        "dominant": dominant,
+    }
+
+
+def run_decode(args, device, TK=1 << 20, steps=64, refresh_every=8):
+    """configs[3] phase B: single sequence, 1M keys, q_len 1, mask refreshed every 8 steps."""
+    import torch
+    from hip_attn import HiPAttentionArgs12, hip_attention_12
+    from hip_attn import _native as N
+
+    H, HKV, D = 32, 8, 128
+    g = torch.Generator(device="cpu").manual_seed(3)
+    k = torch.empty((1, TK, HKV, D), dtype=torch.bfloat16, device=device)
+    step = 1 << 17
+    for s in range(0, TK, step):
+        k[:, s:s + step] = torch.randn((1, step, HKV, D), generator=g, dtype=torch.float32).to(torch.bfloat16).to(device)
+    v = k.clone()
+    q = torch.randn((1, 1, H, D), generator=g, dtype=torch.float32).to(torch.bfloat16).to(device)
+    hargs = HiPAttentionArgs12(sliding_window_size=1024,
+                               position_ids=torch.full((1, 1), TK - 1, dtype=torch.int64, device=device))
+    meta = None
+    for i in range(16):
+        _, meta = hip_attention_12(q, k, v, hargs, cached_metadata=None if i % refresh_every == 0 else meta)
+    torch.cuda.synchronize()
+
+    def timed(n, cached_fn):
+        s_ev = torch.cuda.Event(enable_timing=True)
+        e_ev = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        s_ev.record()
+        m = meta
+        for i in range(n):
+            _, m = hip_attention_12(q, k, v, hargs, cached_metadata=cached_fn(i, m))
+        e_ev.record()
+        torch.cuda.synchronize()
+        return s_ev.elapsed_time(e_ev) * 1e3 / n
+
+    us_mixed = timed(steps, lambda i, m: None if i % refresh_every == 0 else m)
+    us_refresh = timed(16, lambda i, m: None)
+    us_cached = timed(64, lambda i, m: m)
+    # wall-clock per step including host launch overhead
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    m = meta
+    for i in range(steps):
+        _, m = hip_attention_12(q, k, v, hargs, cached_metadata=None if i % refresh_every == 0 else m)
+    torch.cuda.synchronize()
+    wall_us = (time.perf_counter() - t0) * 1e6 / steps
+
+    sink, sw = 256, 1024
+    n0 = cdiv(TK - sink - sw, 256)
+    n1 = min(32768 // 256, n0) * 8
+    n2 = min(8192 // 32, n1) * 4
+    mb = sum(mask_stage_bytes(1, 1, H, D, 2, [(64, n0, 256), (64, n1, 32), (64, n2, 8)]))
+    attn_bytes = HKV * (2048 + sink + sw) * 2 * D * 2
+    refresh_bytes = mb + attn_bytes
+    gbs_refresh = refresh_bytes / (us_refresh * 1e-6) / 1e9
+    gbs_cached = attn_bytes / (us_cached * 1e-6) / 1e9
+    N.profile_begin()
+    hip_attention_12(q, k, v, hargs)
+    prof = N.profile_end()
+    del k, v
+    torch.cuda.empty_cache()
+    return {
+        "kv_len": TK, "us_per_step_mixed": us_mixed, "us_per_step_refresh": us_refresh,
+        "us_per_step_cached": us_cached, "wall_us_per_step_mixed": wall_us, "refresh_every": refresh_every,
+        "refresh_algorithmic_bytes": refresh_bytes, "cached_algorithmic_bytes": attn_bytes,
+        "hbm_frac_refresh": gbs_refresh / HBM_PEAK_GBS, "hbm_frac_cached": gbs_cached / HBM_PEAK_GBS,
+        "refresh_GBps": gbs_refresh, "cached_GBps": gbs_cached,
+        "refresh_kernels_us": [(n, round(ms * 1e3, 1)) for n, ms in prof],
+    }
+
+
+def run_cpu_baseline(args):
+    """The CPU oracle on a bounded sample of the prefill workload: last 128 queries, all heads, full keys."""
+    import numpy as np
+    import torch
+    from oracle import hip12 as O
+
+    TQ_full, TK, H, HKV, D = 32768, 131072, 32, 8, 128
+    TQs = 128
+    g = torch.Generator(device="cpu").manual_seed(1)
+    q = torch.randn((1, TQ_full, H, D), generator=g, dtype=torch.float32).to(torch.bfloat16)[:, -TQs:]
+    k = torch.randn((1, TK, HKV, D), generator=g, dtype=torch.float32).to(torch.bfloat16)
+    qb = q.contiguous().view(torch.int16).numpy().view(np.uint16)
+    kb = k.contiguous().view(torch.int16).numpy().view(np.uint16)
+    pos = (np.arange(TQs) + TK - TQs)[None].astype(np.int64)
+    X = O.OInputs("bf16", qb, pos, k=kb, v=kb)
+    A = O.OArgs(sliding_window_size=1024)
+    threads = O.lib().hipo_num_threads()
+    t0 = time.perf_counter()
+    O.hip_attention_12(X, A)
+    dt = time.perf_counter() - t0
+    return {"value": TQs / dt, "unit": "tok/s", "cores": int(threads), "kind": "port",
+            "sample": f"last {TQs} of 32768 queries (2 query blocks) x 32 heads against all 131072 keys, "
+                      f"{dt:.1f} s of CPU time; throughput is per query token, so it compares directly"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--skip-decode", action="store_true")
+    ap.add_argument("--skip-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; every figure is one MI355X's throughput (--gpus 1).",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    pre = run_prefill(args, device)
+    dec = None if args.skip_decode else run_decode(args, device)
+    cpu = None if args.skip_cpu else run_cpu_baseline(args)
+    dom = pre["dominant"] or {}
+    line = {
+        "metric": "prefill tok/s at 128k KV (hip_attention_12, mask estimation + block-sparse attention)",
+        "value": pre["tok_per_s"],
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": pre["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: B=1, q_len=32768, kv_len=131072, 32 q heads / 8 kv heads, head_dim=128, "
+                               "bf16, HiPAttentionArgs12 defaults with sliding_window_size=1024"},
+        "roofline": {k2: dom.get(k2) for k2 in ("bound", "achieved", "peak", "unit", "frac", "traffic")} | {
+            "kernel": dom.get("kernel")},
+        "roofline_all": pre["rooflines"],
+        "kernels_ms": pre["kernels_ms"],
+        "decode": dec,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -145,11 +145,48 @@ def make_kv_paged(k_cache, v_cache, block_table, cache_seq_lens, max_tsrc: int) 
     return s
 
 
+# ------------------------------------------------------------------ optional per-launch timing
+_profile = None
+
+
+def profile_begin():
+    """Start recording a (name, start_event, end_event) triple around every kernel entry point."""
+    global _profile
+    _profile = []
+
+
+def profile_end():
+    """Stop recording and return ``[(name, milliseconds), ...]`` in launch order (synchronises)."""
+    global _profile
+    rec, _profile = _profile, None
+    torch.cuda.synchronize()
+    return [(name, s.elapsed_time(e)) for name, s, e in (rec or [])]
+
+
+class _timed:
+    def __init__(self, name):
+        self.name = name
+
+    def __enter__(self):
+        if _profile is not None:
+            self.s = torch.cuda.Event(enable_timing=True)
+            self.e = torch.cuda.Event(enable_timing=True)
+            self.s.record()
+        return self
+
+    def __exit__(self, *exc):
+        if _profile is not None and exc[0] is None:
+            self.e.record()
+            _profile.append((self.name, self.s, self.e))
+        return False
+
+
 # ------------------------------------------------------------------ thin wrappers, one per entry point
 
 def mask_stage(qs, kvs, chunk_left, hg, n, chunk, right_clamp, bs, bq, stride_q, block_chunk, scan_stride,
                sw_eff, terminate, scores, left_out, device):
-    rc = lib().hipattn_mask_stage(
+    with _timed(f"mask_stage[n={n},chunk={chunk},rows={bq // stride_q}]"):
+      rc = lib().hipattn_mask_stage(
         ctypes.byref(qs), ctypes.byref(kvs), _p(chunk_left), ctypes.c_int32(hg), ctypes.c_int32(n),
         ctypes.c_int32(chunk), ctypes.c_int64(right_clamp), ctypes.c_int32(bs), ctypes.c_int32(bq),
         ctypes.c_int32(stride_q), ctypes.c_int32(block_chunk), ctypes.c_int32(scan_stride),
@@ -158,7 +195,8 @@ def mask_stage(qs, kvs, chunk_left, hg, n, chunk, right_clamp, bs, bq, stride_q,
 
 
 def select_stage(scores, chunk_left, B, bs_in, bs_out, row_rep, HEAD, hg, n, k, chunk, splits, next_left, device):
-    rc = lib().hipattn_select_stage(
+    with _timed("select_stage"):
+      rc = lib().hipattn_select_stage(
         _p(scores), _p(chunk_left), ctypes.c_int32(B), ctypes.c_int32(bs_in), ctypes.c_int32(bs_out),
         ctypes.c_int32(row_rep), ctypes.c_int32(HEAD), ctypes.c_int32(hg), ctypes.c_int32(n), ctypes.c_int32(k),
         ctypes.c_int32(chunk), ctypes.c_int32(splits), _p(next_left), stream_ptr(device))
@@ -167,7 +205,8 @@ def select_stage(scores, chunk_left, B, bs_in, bs_out, row_rep, HEAD, hg, n, k, 
 
 def finalize_indices(scores, left_out, pos, B, bs, bdst, scan_stride, HEAD, hg, n, K, chunk, bq,
                      indices, ks, ks_start_end, device):
-    rc = lib().hipattn_finalize_indices(
+    with _timed("finalize_indices"):
+      rc = lib().hipattn_finalize_indices(
         _p(scores), _p(left_out), _p(pos), ctypes.c_int64(pos.stride(0)), ctypes.c_int64(pos.stride(1)),
         ctypes.c_int32(B), ctypes.c_int32(bs), ctypes.c_int32(bdst), ctypes.c_int32(scan_stride),
         ctypes.c_int32(HEAD), ctypes.c_int32(hg), ctypes.c_int32(n), ctypes.c_int32(K), ctypes.c_int32(chunk),
@@ -178,7 +217,8 @@ def finalize_indices(scores, left_out, pos, B, bs, bdst, scan_stride, HEAD, hg, 
 def bsa_prefill(qs, kvs, indices, ks_start_end, BK, bq, bk, sw, sink, share_first_head, impl, out, device):
     assert indices.dtype == torch.int64 and indices.is_contiguous()
     assert ks_start_end.dtype == torch.int32 and ks_start_end.is_contiguous()
-    rc = lib().hipattn_bsa_prefill(
+    with _timed("bsa_prefill"):
+      rc = lib().hipattn_bsa_prefill(
         ctypes.byref(qs), ctypes.byref(kvs), _p(indices), _p(ks_start_end), ctypes.c_int32(indices.shape[1]),
         ctypes.c_int32(BK), ctypes.c_int32(bq), ctypes.c_int32(bk), ctypes.c_int32(sw), ctypes.c_int32(sink),
         ctypes.c_int32(int(share_first_head)), ctypes.c_int32(impl), _p(out), ctypes.c_int64(out.stride(0)),
@@ -198,7 +238,8 @@ def bsa_decode(qs, kvs, indices, ks_start_end, BK, bk, sw, sink, out, device, ns
                                                 ctypes.c_int32(nsplits))
     if workspace is None or workspace.numel() * workspace.element_size() < need:
         workspace = torch.empty(need // 4, dtype=torch.float32, device=out.device)
-    rc = L.hipattn_bsa_decode_partial(
+    with _timed("bsa_decode"):
+      rc = L.hipattn_bsa_decode_partial(
         ctypes.byref(qs), ctypes.byref(kvs), _p(indices), _p(ks_start_end), ctypes.c_int32(indices.shape[1]),
         ctypes.c_int32(BK), ctypes.c_int32(bk), ctypes.c_int32(sw), ctypes.c_int32(sink), ctypes.c_int32(nsplits),
         _p(workspace), stream_ptr(device))

@@ -227,8 +227,9 @@ def dual_stage_quadratic_hip_attention(
                 assert (chunk_size % stage.stage_chunk_size) == 0
                 splits = chunk_size // stage.stage_chunk_size
                 next_left = torch.empty((BSZ, bs_out, hg, keep * splits), dtype=torch.int32, device=device)
-                N.select_stage(scores, chunk_left, BSZ, bs_in, bs_out, row_rep, HEAD, hg, prev_n, keep,
-                               chunk_size, splits, next_left, device)
+                if keep > 0:
+                    N.select_stage(scores, chunk_left, BSZ, bs_in, bs_out, row_rep, HEAD, hg, prev_n, keep,
+                                   chunk_size, splits, next_left, device)
                 chunk_left = next_left
                 right_clamp = _BIG
             else:
@@ -306,6 +307,7 @@ def dual_stage_quadratic_hip_attention(
         if args.mask_only:
             return None, None
         fresh_mask = True
+        rows_shared = hg == 1  # every head of a batch item carries the same index row
     else:
         args = args.clone()
         args.sliding_window_size += args.mask_k
@@ -316,6 +318,7 @@ def dual_stage_quadratic_hip_attention(
         ks_count = cached_metadata.ks_count.clone()
         ks_start_end = cached_metadata.ks_start_end.clone()
         fresh_mask = False
+        rows_shared = bool(getattr(cached_metadata, "_rows_shared", False))
 
     args.block_size_q = min(args.block_size_q, _npow2(TDST))
     if args.sliding_window_size == 777:
@@ -328,10 +331,10 @@ def dual_stage_quadratic_hip_attention(
     )
     seq_pos = position_ids[:, -q_bsa.shape[1]:]
     context = block_sparse_attention(
-        q_bsa, k, v, seq_pos, indices, ks_start_end, args, MAX_TSRC, decode=use_decode,
+        q_bsa, k, v, seq_pos, indices, ks_start_end, args, MAX_TSRC, decode=use_decode, rows_shared=rows_shared,
     )
 
-    return context, HiPAttentionOutputMetadata(
+    metadata = HiPAttentionOutputMetadata(
         indices=indices,
         ks=ks,
         ks_count=ks_count,
@@ -340,19 +343,25 @@ def dual_stage_quadratic_hip_attention(
         sa_cache_statistics=HiPAttentionCacheAccessStatistics(None, None),
         stage_caches=stage_caches,
     )
+    # private hint for later calls that reuse this metadata: index rows are identical across heads,
+    # so the tile kernel may serve a whole GQA group from one gathered K/V tile
+    metadata._rows_shared = rows_shared
+    return context, metadata
 
 
 @torch.no_grad()
 def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], position_ids: Tensor, indices: Tensor,
                            ks_start_end: Tensor, args: HiPAttentionArgs, max_tsrc: int, decode: bool = False,
-                           impl: int = 0) -> Tensor:
+                           impl: int = 0, rows_shared: bool = False) -> Tensor:
     """Sparse attention over (selected blocks, sink, sliding window) given the metadata tensors.
 
     ``position_ids`` are 0-based (the reference passes ``seq_lens = position_ids + 1``,
     attention_extend.py:3092).  ``args.block_size_q / block_size_k / sliding_window_size`` must
     already hold the values the operator derives for this step.  ``decode`` selects the split-KV
     path, which, like the reference's decode kernel, lets every head of a GQA group read the
-    index row of the group's first head.
+    index row of the group's first head.  ``rows_shared`` promises that all heads of a GQA group hold
+    identical index rows (true for masks estimated with head reduction), which lets one gathered
+    K/V tile serve the whole group.
     """
     device = q.device
     qq = q if q.stride(-1) == 1 else q.contiguous()
@@ -377,6 +386,6 @@ def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], 
             if "is not built" not in str(e):
                 raise
     N.bsa_prefill(qs, kvs, indices, ks_start_end, BK, args.block_size_q, args.block_size_k,
-                  args.sliding_window_size, args.sink_token_size, decode, impl, out, device)
+                  args.sliding_window_size, args.sink_token_size, decode or rows_shared, impl, out, device)
     del keep
     return out

@@ -1,0 +1,92 @@
+"""GPU parity of the block-sparse attention kernels given indices (tile kernel, portable kernel, decode)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import hip12 as O
+from helpers import make_inputs, to_paged
+from gpu_utils import assert_context_close, to_torch
+from test_oracle_bsa import random_indices
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(X, max_tsrc, idx, kse, bq, bk, sw, sink, impl, share=False, decode=False):
+    from hip_attn import HiPAttentionArgs12
+    from hip_attn.operator import block_sparse_attention
+
+    dev = "cuda"
+    q = to_torch(X.q, X.dtype, dev)
+    kw = {}
+    if X.k is None:
+        kw = dict(k_cache=to_torch(X.k_cache, X.dtype, dev), v_cache=to_torch(X.v_cache, X.dtype, dev),
+                  block_table=torch.from_numpy(X.block_table).to(dev),
+                  cache_seq_lens=torch.from_numpy(X.cache_seq_lens).to(dev))
+    args = HiPAttentionArgs12(sink_token_size=sink, sliding_window_size=sw, **kw)
+    args.block_size_q, args.block_size_k = bq, bk
+    out = block_sparse_attention(q, to_torch(X.k, X.dtype, dev), to_torch(X.v, X.dtype, dev),
+                                 torch.from_numpy(X.pos.copy()).to(dev), torch.from_numpy(idx).to(dev),
+                                 torch.from_numpy(kse).to(dev), args, max_tsrc, decode=decode, impl=impl,
+                                 rows_shared=share)
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("bq,TQ,bk", [(64, 200, 8), (32, 96, 2), (16, 40, 16)])
+@pytest.mark.parametrize("paged", [False, True])
+def test_tile_kernel_matches_oracle_and_portable_kernel(D, bq, TQ, bk, paged):
+    print(f"[case] bsa mfma D={D} bq={bq} TQ={TQ} bk={bk} paged={paged}", flush=True)
+    rng = np.random.default_rng(D + bq + bk)
+    TK, H, HKV, BK, sw, sink = 1536, 8, 2, 24, 100, 24
+    X = make_inputs(12, B=2, TQ=TQ, TK=TK, H=H, HKV=HKV, D=D, dtype="bf16", scale=0.5)
+    nbq = O.cdiv(TQ, bq)
+    idx, ks, kse = random_indices(rng, 2, H, nbq, BK, bk, TK, same_heads=True)
+    max_tsrc = TK
+    if paged:
+        X = to_paged(X, 16, seed=7)
+        max_tsrc = 4096
+    ref = O.bsa(X, max_tsrc, idx, kse, bq, bk, sw, sink)
+    out_tile = _run(X, max_tsrc, idx, kse, bq, bk, sw, sink, impl=2, share=True)
+    out_port = _run(X, max_tsrc, idx, kse, bq, bk, sw, sink, impl=1, share=True)
+    assert_context_close(out_tile, ref, "bf16")
+    assert_context_close(out_port, ref, "bf16")
+
+
+def test_tile_kernel_per_head_rows():
+    print("[case] bsa mfma per-head rows", flush=True)
+    rng = np.random.default_rng(5)
+    TK, TQ, H, HKV, D, bq, bk, BK, sw, sink = 1024, 128, 8, 2, 128, 64, 8, 20, 64, 16
+    X = make_inputs(13, B=1, TQ=TQ, TK=TK, H=H, HKV=HKV, D=D, dtype="bf16", scale=0.5)
+    idx, ks, kse = random_indices(rng, 1, H, 2, BK, bk, TK, same_heads=False)
+    ref = O.bsa(X, TK, idx, kse, bq, bk, sw, sink)
+    out = _run(X, TK, idx, kse, bq, bk, sw, sink, impl=2, share=False)
+    assert_context_close(out, ref, "bf16")
+    ref_shared = O.bsa(X, TK, idx, kse, bq, bk, sw, sink, share_first_head=True)
+    out_shared = _run(X, TK, idx, kse, bq, bk, sw, sink, impl=2, share=True)
+    assert_context_close(out_shared, ref_shared, "bf16")
+
+
+def test_tile_kernel_empty_rows_and_early_positions():
+    print("[case] bsa mfma early positions", flush=True)
+    # queries at the very start of the sequence: window and sink are clipped by the position, ks = 0
+    X = make_inputs(14, B=1, TQ=64, TK=64, H=4, HKV=1, D=64, dtype="bf16", scale=0.5)
+    idx = np.full((4, 1, 4), O.INT64_MAX, dtype=np.int64)
+    kse = np.zeros((4, 1, 2), dtype=np.int32)
+    ref = O.bsa(X, 64, idx, kse, 64, 8, 16, 4)
+    out = _run(X, 64, idx, kse, 64, 8, 16, 4, impl=2, share=True)
+    assert_context_close(out, ref, "bf16")
+
+
+@pytest.mark.parametrize("dtype,D,G", [("bf16", 128, 4), ("bf16", 64, 2), ("f32", 64, 4), ("bf16", 128, 1)])
+def test_decode_kernel_matches_oracle(dtype, D, G):
+    print(f"[case] decode {dtype} D={D} G={G}", flush=True)
+    rng = np.random.default_rng(D + G)
+    B, HKV, TK, bk, BK, sw, sink = 3, 2, 3000, 8, 40, 200, 32
+    H = HKV * G
+    lens = np.array([3000, 1500, 257])
+    X = make_inputs(15, B=B, TQ=1, TK=TK, H=H, HKV=HKV, D=D, dtype=dtype, scale=0.5, pos=(lens - 1)[:, None])
+    idx, ks, kse = random_indices(rng, B, H, 1, BK, bk, 1400, same_heads=True)
+    ref = O.bsa(X, TK, idx, kse, 1, bk, sw, sink, share_first_head=True)
+    out = _run(X, TK, idx, kse, 1, bk, sw, sink, impl=0, decode=True)
+    assert_context_close(out, ref, dtype)
