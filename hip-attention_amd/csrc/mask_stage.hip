@@ -7,27 +7,9 @@
 // rows are in flight per load instruction, and the dot product is reduced across the 16 lanes in
 // the fixed order  [FMA chain over the lane's elements] -> [adjacent-pair tree over lanes],
 // which makes scores reproducible bit for bit on any implementation that follows the same order.
-#include "common.hpp"
+#include "mask_common.hpp"
 
 namespace hipattn {
-
-struct MaskParams {
-    const void *q;
-    int64_t q_sb, q_st, q_sh;
-    const int64_t *pos;
-    int64_t pos_sb, pos_st;
-    KVView kv;
-    const int32_t *chunk_left;
-    int hg, n, chunk;
-    int64_t right_clamp;
-    int B, TDST, HEAD, G, BS, BDST, BQ, stride_q, nrows, block_chunk, scan_stride, sw_eff;
-    float terminate;
-    int ngroups;
-    long long total;
-    float c_q, c_k;
-    float *scores;
-    int32_t *left_out;
-};
 
 template <int N>
 __device__ __forceinline__ void rs_step(const float (&in)[N], float (&out)[N / 2], bool hi, int xmask) {
@@ -284,7 +266,7 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
                                   int32_t hg, int32_t n, int32_t chunk_size, int64_t right_clamp,
                                   int32_t bs, int32_t bq, int32_t stride_q, int32_t block_chunk,
                                   int32_t scan_stride, int32_t sw_eff, int32_t terminate_size,
-                                  float *scores, int32_t *left_out, void *stream) {
+                                  int32_t k_prescaled, float *scores, int32_t *left_out, void *stream) {
     int rc = check_q(q);
     if (rc) return rc;
     HIPATTN_CHECK_ARG(kv && chunk_left && scores, HIPATTN_E_ARG, "mask stage: null pointer");
@@ -325,13 +307,9 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
     // the kernel indexes rows up to nrows; MAXROWS must cover every row that can be valid
     hipStream_t st = (hipStream_t)stream;
     if (q->dtype == HIPATTN_BF16) {
-        switch (q->HID) {
-            case 32: return launch_mask<bf16_t, 32>(p, rows_eff, st);
-            case 64: return launch_mask<bf16_t, 64>(p, rows_eff, st);
-            case 128: return launch_mask<bf16_t, 128>(p, rows_eff, st);
-            case 256: return launch_mask<bf16_t, 256>(p, rows_eff, st);
-        }
+        return mask_stage_mfma_launch(p, q->HID, rows_eff, k_prescaled, st);
     } else if (q->dtype == HIPATTN_F32) {
+        HIPATTN_CHECK_ARG(!k_prescaled, HIPATTN_E_ARG, "mask stage: prescaled keys are a bf16-only option");
         switch (q->HID) {
             case 32: return launch_mask<float, 32>(p, rows_eff, st);
             case 64: return launch_mask<float, 64>(p, rows_eff, st);

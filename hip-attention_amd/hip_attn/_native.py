@@ -65,7 +65,7 @@ def lib():
         L.hipattn_last_error.restype = ctypes.c_char_p
         L.hipattn_bsa_decode_workspace_bytes.restype = ctypes.c_int64
         L.hipattn_bsa_decode_default_splits.restype = ctypes.c_int32
-        for name in ("hipattn_mask_stage", "hipattn_select_stage", "hipattn_finalize_indices",
+        for name in ("hipattn_mask_stage", "hipattn_prescale_k", "hipattn_select_stage", "hipattn_finalize_indices",
                      "hipattn_bsa_prefill", "hipattn_bsa_decode_partial", "hipattn_bsa_decode_merge"):
             getattr(L, name).restype = ctypes.c_int
         _lib = L
@@ -183,14 +183,28 @@ class _timed:
 
 # ------------------------------------------------------------------ thin wrappers, one per entry point
 
+def prescale_k(k: torch.Tensor, device) -> torch.Tensor:
+    """``bf16(k * c_k)`` for a whole 4-D bf16 key tensor (dense ``[B,T,HKV,D]`` or a paged cache)."""
+    assert k.ndim == 4 and k.dtype == torch.bfloat16 and k.stride(3) == 1
+    out = torch.empty(k.shape, dtype=k.dtype, device=k.device)
+    with _timed("prescale_k"):
+      rc = lib().hipattn_prescale_k(
+        _p(k), ctypes.c_int64(k.stride(0)), ctypes.c_int64(k.stride(1)), ctypes.c_int64(k.stride(2)),
+        ctypes.c_int64(k.shape[0]), ctypes.c_int32(k.shape[1]), ctypes.c_int32(k.shape[2]),
+        ctypes.c_int32(k.shape[3]), _p(out), stream_ptr(device))
+    check(rc, "hipattn_prescale_k")
+    return out
+
+
 def mask_stage(qs, kvs, chunk_left, hg, n, chunk, right_clamp, bs, bq, stride_q, block_chunk, scan_stride,
-               sw_eff, terminate, scores, left_out, device):
+               sw_eff, terminate, scores, left_out, device, k_prescaled=False):
     with _timed(f"mask_stage[n={n},chunk={chunk},rows={bq // stride_q}]"):
       rc = lib().hipattn_mask_stage(
         ctypes.byref(qs), ctypes.byref(kvs), _p(chunk_left), ctypes.c_int32(hg), ctypes.c_int32(n),
         ctypes.c_int32(chunk), ctypes.c_int64(right_clamp), ctypes.c_int32(bs), ctypes.c_int32(bq),
         ctypes.c_int32(stride_q), ctypes.c_int32(block_chunk), ctypes.c_int32(scan_stride),
-        ctypes.c_int32(sw_eff), ctypes.c_int32(terminate), _p(scores), _p(left_out), stream_ptr(device))
+        ctypes.c_int32(sw_eff), ctypes.c_int32(terminate), ctypes.c_int32(int(k_prescaled)), _p(scores),
+        _p(left_out), stream_ptr(device))
     check(rc, "hipattn_mask_stage")
 
 

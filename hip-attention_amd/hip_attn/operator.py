@@ -85,6 +85,30 @@ def _kv_struct(args: HiPAttentionArgs, k: Optional[Tensor], v: Optional[Tensor],
     return N.make_kv_paged(args.k_cache, args.v_cache, bt, sl, max_tsrc), (bt, sl)
 
 
+def _mask_kv(args: HiPAttentionArgs, k_mask: Optional[Tensor], max_tsrc: int, q: Tensor, programs_rows: int,
+             chunk_count: int, device):
+    """KV description for the scan kernels, with keys pre-scaled when that saves work."""
+    stage0 = args.stages[0]
+    iters = max(1, int(stage0.stage_chunk_size).bit_length())
+    sampled_rows = 2 * iters * programs_rows * chunk_count  # stage 0 alone
+    if q.dtype == torch.bfloat16 and args.offload_cache is None:
+        src = k_mask if k_mask is not None else args.k_cache
+        if src is not None and src.dtype == torch.bfloat16 and src.ndim == 4 and src.stride(-1) == 1:
+            rows_total = src.shape[0] * src.shape[1] * src.shape[2]
+            force = os.getenv("HIP_ATTN_PRESCALE_K", "")  # "0" / "1" override the heuristic (testing)
+            if force == "1" or (force != "0" and sampled_rows >= 4 * rows_total):
+                khat = N.prescale_k(src, device)
+                if k_mask is not None:
+                    st, keep = _kv_struct(args, khat, khat, max_tsrc)
+                else:
+                    a2 = args.clone()
+                    a2.k_cache, a2.v_cache = khat, khat
+                    st, keep = _kv_struct(a2, None, None, max_tsrc)
+                return st, (keep, khat), True
+    st, keep = _kv_struct(args, k_mask, k_mask, max_tsrc)
+    return st, keep, False
+
+
 def _stage_cache_views(chunk_left: Tensor, HEAD: int, chunk: int) -> HiPAttentionStageInputCache:
     """Reference-layout view of a stage's inputs: int64 left/right and the reset scores."""
     B, BS, hg, n = chunk_left.shape
@@ -171,8 +195,9 @@ def dual_stage_quadratic_hip_attention(
         stage_caches = None
 
     qq = q if q.stride(-1) == 1 else q.contiguous()
-    mask_kv, keep_mask_kv = _kv_struct(args, k_mask, k_mask, MAX_TSRC)
     hg = 1 if _head_reduce_enabled() else HEAD
+    mask_kv = None  # built lazily: cached-mask steps never touch the estimation path
+    k_prescaled = False
 
     if (cached_metadata is None) or (cached_metadata.indices is None):
         fresh = (cached_metadata is None) or (cached_metadata.stage_caches is None) or (stage_caches is None)
@@ -188,6 +213,10 @@ def dual_stage_quadratic_hip_attention(
             assert len(stage_caches) <= len(stages)
             chunk_left = _chunk_list_from_cache(stage_caches[-1], hg)
             right_clamp = _BIG
+
+        # Keys are scaled by c_k and re-rounded every time they are sampled.  When the scan will sample
+        # far more rows than the key tensor holds (prefill), scale the whole tensor once instead.
+        mask_kv, keep_mask_kv, k_prescaled = _mask_kv(args, k_mask, MAX_TSRC, q, BSZ * HEAD * BDST_SCAN, chunk_count, device)
 
         scores = None
         left_out = None
@@ -258,7 +287,7 @@ def dual_stage_quadratic_hip_attention(
                     qs = N.make_q(qq, position_ids)
                     N.mask_stage(qs, mask_kv, chunk_left, hg, chunk_count, chunk_size, right_clamp, bs,
                                  BLOCK_SIZE_Q, stage.stage_block_stride_q, BLOCK_CHUNK, STAGE_STRIDE, sw_eff,
-                                 args.stage_early_terminate, scores, left_out, device)
+                                 args.stage_early_terminate, scores, left_out, device, k_prescaled=k_prescaled)
             elif isinstance(stage, NopStage):
                 scores = torch.full((BSZ, bs, HEAD, chunk_count), -32000.0, dtype=torch.float32, device=device)
                 left_out = chunk_left.expand(BSZ, bs, HEAD, chunk_count).contiguous() if last else None

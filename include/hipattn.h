@@ -74,12 +74,20 @@ const char *hipattn_last_error(void);
  *   scores      f32   [B, BS, HEAD, n] written for every chunk (-32000 where not scored)
  *   left_out    int32 [B, BS, HEAD, n] refined left edge per head, or NULL
  *   block_chunk = chunks per reference program (16/32/64): fixes the program-level gate and
- *   iteration count (:595-601,736-737). */
+ *   iteration count (:595-601,736-737).
+ *   k_prescaled != 0: kv->k already holds bf16(K * c_k) (see hipattn_prescale_k). */
 int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, const int32_t *chunk_left,
                        int32_t hg, int32_t n, int32_t chunk_size, int64_t right_clamp,
                        int32_t bs, int32_t bq, int32_t stride_q, int32_t block_chunk,
                        int32_t scan_stride, int32_t sw_eff, int32_t terminate_size,
-                       float *scores, int32_t *left_out, void *stream);
+                       int32_t k_prescaled, float *scores, int32_t *left_out, void *stream);
+
+/* K^ = bf16(K * c_k) for a whole bf16 key tensor viewed as [n0, n1, n2, HID] with element strides
+ * (stride0, stride1, stride2, 1); `out` is contiguous [n0, n1, n2, HID].  Passing `out` as kv->k
+ * with k_prescaled = 1 lets hipattn_mask_stage skip the per-sample scaling the reference performs on
+ * every loaded key (src/hip_attn/v1_2/attention_extend.py:932-937); results are identical. */
+int hipattn_prescale_k(const void *k, int64_t stride0, int64_t stride1, int64_t stride2, int64_t n0,
+                       int32_t n1, int32_t n2, int32_t HID, void *out, void *stream);
 
 /* Between two stages: max over heads, top-k under (score desc, position asc), realign, split.
  * Replaces the ATen glue at src/hip_attn/v1_2/attention_extend.py:2566-2570 (head reduce),

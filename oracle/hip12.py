@@ -71,6 +71,8 @@ def lib():
         L.hipo_round_bf16.argtypes = [ctypes.c_float]
         L.hipo_dot.restype = ctypes.c_float
         L.hipo_dot.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int]
+        L.hipo_dot_mfma.restype = ctypes.c_float
+        L.hipo_dot_mfma.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int]
         L.hipo_scale_constants.restype = None
         L.hipo_mask_stage.restype = ctypes.c_int
         L.hipo_bsa.restype = ctypes.c_int

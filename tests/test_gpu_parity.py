@@ -85,6 +85,22 @@ def test_batched_paged_decode(page_size):
     assert_context_close(ctx3, octx, "bf16")
 
 
+@pytest.mark.parametrize("force", ["0", "1"])
+def test_prescaled_keys_give_identical_masks(force, monkeypatch):
+    _case(f"prescale forced {force}")
+    monkeypatch.setenv("HIP_ATTN_PRESCALE_K", force)
+    X = make_inputs(9, B=1, TQ=300, TK=8192, H=8, HKV=2, D=128, dtype="bf16")
+    A = O.OArgs(sliding_window_size=512)
+    octx, ometa = O.hip_attention_12(X, A)
+    ctx, meta = run_product(X, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, "bf16")
+    XP = to_paged(X, 8, seed=11)
+    A.extend_context_length = 8192
+    ctx, meta = run_product(XP, A)
+    assert_metadata_equal(meta, ometa)
+
+
 def test_stage_cache_replay_reproduces_output():
     _case("stage cache replay")
     from hip_attn import HiPAttentionOutputMetadata12
