@@ -9,6 +9,9 @@ from .metadata import HiPAttentionCacheAccessStatistics as HiPAttentionCacheAcce
 from .metadata import HiPAttentionOutputMetadata as HiPAttentionOutputMetadata12
 from .metadata import ScanStage as ScanStage12
 from .operator import dual_stage_quadratic_hip_attention as hip_attention_12
+from .config import HiPAttentionConfig, HiPAttentionPerLayerConfig
+from .refresh import HiPMaskRefreshState
+from .paged import forward_paged_hip
 
 hip_attention = hip_attention_12
 HiPAttentionArgs = HiPAttentionArgs12
@@ -25,4 +28,8 @@ __all__ = [
     "hip_attention",
     "HiPAttentionArgs",
     "HiPAttentionOutputMetadata",
+    "HiPAttentionConfig",
+    "HiPAttentionPerLayerConfig",
+    "HiPMaskRefreshState",
+    "forward_paged_hip",
 ]

@@ -1,0 +1,105 @@
+"""GPU parity of forward_paged_hip (the serving entry point) against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import hip12 as O
+from helpers import make_inputs
+from gpu_utils import assert_context_close, assert_metadata_equal, from_torch, to_torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _pool(X, seed):
+    """Token-granular KV pool + req_to_tokens as a serving framework keeps them (page size 1)."""
+    B, TK, HKV, D = X.k.shape
+    rng = np.random.default_rng(seed)
+    slots = rng.permutation(np.arange(1, B * TK + 8))[: B * TK].reshape(B, TK)
+    kc = np.zeros((B * TK + 8, HKV, D), dtype=X.k.dtype)
+    vc = np.zeros_like(kc)
+    for b in range(B):
+        kc[slots[b]] = X.k[b]
+        vc[slots[b]] = X.v[b]
+    req_to_tokens = np.zeros((B + 3, TK), dtype=np.int32)
+    pool_idx = np.array([2, 0, 4][:B])
+    req_to_tokens[pool_idx] = slots
+    return kc, vc, req_to_tokens, pool_idx
+
+
+def _config(sw):
+    from hip_attn import HiPAttentionConfig
+
+    spec = ('{"using_extend": false, "dense_layers": [0], "layers": [{"second_stage_k": 256, "sliding_window_size": %d},'
+            '{"second_stage_k": 128, "sliding_window_size": %d}], "prefill_layers": [{"second_stage_k": 256, '
+            '"sliding_window_size": %d}, {"second_stage_k": 128, "sliding_window_size": %d}]}') % (sw, sw, sw, sw)
+    return HiPAttentionConfig(json_or_path=spec)
+
+
+def _oracle(X, kc, vc, r2t, pool_idx, lens, sm_scale, second_k, sw, max_ctx, disable_flashdecode, model_ctx=131072):
+    qs = O.bf16_bits_to_f32(X.q) * np.float32(sm_scale)
+    XP = O.OInputs("bf16", O.f32_to_bf16_bits(qs), X.pos, k_cache=kc[:, None], v_cache=vc[:, None],
+                   block_table=r2t[pool_idx].astype(np.int64), cache_seq_lens=lens.astype(np.int64))
+    A = O.OArgs(sliding_window_size=sw, second_stage_k=second_k, extend_context_length=max_ctx,
+                model_context_length=model_ctx, disable_flashdecode=disable_flashdecode)
+    return XP, A
+
+
+def test_forward_paged_hip_decode_and_short_prefill():
+    from hip_attn import forward_paged_hip
+
+    print("[case] forward_paged_hip decode", flush=True)
+    B, TK, H, HKV, D, sw = 2, 3072, 8, 2, 128, 512
+    lens = np.array([3072, 2000])
+    X = make_inputs(21, B=B, TQ=1, TK=TK, H=H, HKV=HKV, D=D, dtype="bf16", pos=(lens - 1)[:, None])
+    kc, vc, r2t, pool_idx = _pool(X, 1)
+    cfg = _config(sw)
+    sm = D ** -0.5
+    dev = "cuda"
+    common = dict(sm_scale=sm, batch_size=B, k_cache=to_torch(kc, "bf16", dev), v_cache=to_torch(vc, "bf16", dev),
+                  offload_cache=None, seq_lens=torch.from_numpy(lens).to(dev), req_to_tokens=torch.from_numpy(r2t).to(dev),
+                  req_pool_indices=torch.from_numpy(pool_idx).to(dev), rope_cos=None, rope_sin=None, logit_cap=0.0,
+                  orig_context_len=131072, max_context_len=TK, hip_config=cfg)
+    q = to_torch(X.q, "bf16", dev).view(B, H, D)
+    for layer_id, second_k in ((0, 256), (5, 128)):
+        out, meta = forward_paged_hip(q, positions=torch.from_numpy(X.pos.reshape(-1)).to(dev), layer_id=layer_id,
+                                      is_prefill=False, is_decode=True, **common)
+        XP, A = _oracle(X, kc, vc, r2t, pool_idx, lens, sm, second_k, sw, TK, False)
+        octx, ometa = O.hip_attention_12(XP, A)
+        assert out.shape == (B, H, D)
+        assert_metadata_equal(meta, ometa)
+        assert_context_close(out.view(B, 1, H, D), octx, "bf16")
+        out2, meta2 = forward_paged_hip(q, positions=torch.from_numpy(X.pos.reshape(-1)).to(dev), layer_id=layer_id,
+                                        is_prefill=False, is_decode=True, cached_metadata=meta, **common)
+        assert_context_close(out2.view(B, 1, H, D), octx, "bf16")
+
+
+def test_forward_paged_hip_long_prefill_splits_off_last_64_queries():
+    from hip_attn import forward_paged_hip
+
+    print("[case] forward_paged_hip prefill", flush=True)
+    B, TK, TQ, H, HKV, D, sw = 1, 2048, 192, 4, 2, 64, 256
+    X = make_inputs(22, B=B, TQ=TQ, TK=TK, H=H, HKV=HKV, D=D, dtype="bf16")
+    kc, vc, r2t, pool_idx = _pool(X, 2)
+    lens = np.array([TK])
+    cfg = _config(sw)
+    sm = D ** -0.5
+    dev = "cuda"
+    out, meta = forward_paged_hip(
+        to_torch(X.q, "bf16", dev).view(B * TQ, H, D), sm_scale=sm, batch_size=B, k_cache=to_torch(kc, "bf16", dev),
+        v_cache=to_torch(vc, "bf16", dev), offload_cache=None, positions=torch.from_numpy(X.pos.reshape(-1)).to(dev),
+        seq_lens=torch.from_numpy(lens).to(dev), req_to_tokens=torch.from_numpy(r2t).to(dev),
+        req_pool_indices=torch.from_numpy(pool_idx).to(dev), rope_cos=None, rope_sin=None, layer_id=7, logit_cap=0.0,
+        orig_context_len=4096, max_context_len=TK, is_prefill=True, hip_config=cfg)
+    # oracle: same two calls
+    XP, A = _oracle(X, kc, vc, r2t, pool_idx, lens, sm, 128, sw, TK, True, model_ctx=4096)
+    first = O.OInputs("bf16", XP.q[:, :-64], XP.pos[:, :-64], k_cache=XP.k_cache, v_cache=XP.v_cache,
+                      block_table=XP.block_table, cache_seq_lens=XP.cache_seq_lens)
+    octx1, _ = O.hip_attention_12(first, A)
+    last = O.OInputs("bf16", XP.q[:, -64:], XP.pos[:, -64:], k_cache=XP.k_cache, v_cache=XP.v_cache,
+                     block_table=XP.block_table, cache_seq_lens=XP.cache_seq_lens)
+    A2 = O.OArgs(**{**A.__dict__, "sliding_window_size": 777})
+    octx2, ometa2 = O.hip_attention_12(last, A2)
+    assert_metadata_equal(meta, ometa2)
+    got = out.view(B, TQ, H, D)
+    assert_context_close(got[:, :-64], octx1, "bf16")
+    assert_context_close(got[:, -64:], octx2, "bf16")
