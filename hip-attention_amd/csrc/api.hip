@@ -90,7 +90,8 @@ extern "C" const char *hipattn_last_error(void) { return g_err; }
 extern "C" int hipattn_bsa_prefill(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t *indices,
                                    const int32_t *ks_start_end, int32_t idx_rows, int32_t BK, int32_t block_size_q,
                                    int32_t block_size_k, int32_t sliding_window, int32_t sink,
-                                   int32_t share_first_head, int32_t impl, void *out, int64_t out_stride_b,
+                                   int32_t share_first_head, int32_t impl, const void *k_prescaled, void *out,
+                                   int64_t out_stride_b,
                                    int64_t out_stride_t, int64_t out_stride_h, void *stream) {
     BsaParams p;
     int rc = bsa_fill_params(q, kv, indices, ks_start_end, idx_rows, BK, block_size_q, block_size_k, sliding_window,
@@ -99,7 +100,13 @@ extern "C" int hipattn_bsa_prefill(const hipattn_q_t *q, const hipattn_kv_t *kv,
     HIPATTN_CHECK_ARG(impl >= 0 && impl <= 2, HIPATTN_E_ARG, "bsa: impl %d not in {0,1,2}", impl);
     hipStream_t st = (hipStream_t)stream;
     if (impl != 1) {
-        rc = bsa_mfma_launch(p, q->dtype, q->HID, st);
+        BsaParams pm = p;
+        if (k_prescaled) {  // same layout and strides as kv->k
+            HIPATTN_CHECK_ARG(aligned16(k_prescaled), HIPATTN_E_ALIGN, "bsa: k_prescaled must be 16-byte aligned");
+            pm.kv.k = k_prescaled;
+            pm.k_prescaled = 1;
+        }
+        rc = bsa_mfma_launch(pm, q->dtype, q->HID, st);
         if (rc != HIPATTN_E_UNSUPPORTED) return rc;
         if (impl == 2) {
             set_error("bsa: the MFMA tile kernel does not cover dtype %d, head dim %d, block_size_q %d, block_size_k %d",

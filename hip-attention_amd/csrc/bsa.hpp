@@ -14,6 +14,7 @@ struct BsaParams {
     const int64_t *indices;
     const int32_t *kse;
     int idx_rows, BK, bq, bk, sw, sink, share_first_head;
+    int k_prescaled;  // kv.k already holds bf16(K * c_k) (tile kernel only)
     int B, TDST, HEAD, G, NBQ;
     float c_q, c_k;
     void *out;

@@ -1,7 +1,9 @@
 // MFMA tile kernel for block-sparse attention (bf16, head dim 64 / 128, query block <= 64 rows).
 //
-// One workgroup = one (batch, kv head, query block) and up to four query heads of the GQA group,
-// one head per wavefront, so every gathered K/V tile in LDS is consumed by the whole group.
+// One workgroup = one (batch, kv head, query block) and up to four query heads of the GQA group;
+// a wavefront owns one head and one 32-row half of the query block, so every gathered K/V tile in
+// LDS is consumed by the whole group (eight waves, two per SIMD: while one wave of a SIMD runs its
+// softmax on the vector unit the other keeps the matrix unit busy).
 // Per 64-token tile:   S^T[token, query] = K^ . Q^^T      (v_mfma_f32_32x32x16_bf16, K^ from LDS,
 //                                                           Q^ resident in registers)
 //                      online softmax down the token axis  (a lane owns one query column)
@@ -9,21 +11,28 @@
 //                                                           taken straight from the S^T registers)
 // Working on the transposed problem keeps the softmax statistics lane-local and lets P feed the
 // second MFMA without a trip through LDS.  Global loads of tile i+1 are issued before the math of
-// tile i; LDS is double-buffered so one barrier per tile suffices.
+// tile i; LDS is double-buffered so one barrier per tile suffices.  The running maximum is only
+// raised when it grows by more than 2^8, so the accumulator is rescaled a handful of times per row.
 #include "bsa.hpp"
 
 namespace hipattn {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 constexpr int TN = 64;        // tokens per tile
 constexpr int KPAD = 8;       // bf16 elements of row padding for the K^ tile
 constexpr int VPAD = 4;       // bf16 elements of row padding for the V^T tile
+constexpr int NTHREADS = 512;
+constexpr int MAX_LDS_IDX = 1024;  // selected-block starts kept in LDS
 constexpr float LOG2E = 1.44269504f;
+constexpr float RESCALE_STEP = 8.0f;  // raise the running max only when it grows by more than this (log2 units)
 
-__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
-    return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+__device__ __forceinline__ uint32_t cvt_pk_bf16(float a, float b) {  // one v_cvt_pk_bf16_f32
+    f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
 
 union Frag {
@@ -38,18 +47,20 @@ struct MfmaSmem {
     uint16_t k[2][TN][HID + KPAD];
     uint16_t vt[2][HID][TN + VPAD];
     int tok[2][TN];
+    int idx[MAX_LDS_IDX];
 };
 
-template <int HID>
-__global__ __launch_bounds__(256) void bsa_mfma_kernel(BsaParams p, int hgroups, int hpw, long long total_wg) {
+template <int HID, bool KSCALED>
+__global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParams p, int hgroups, int hpw, long long total_wg) {
     constexpr int KS = HID / 16;   // k-steps of the first product
     constexpr int DB = HID / 32;   // 32-row blocks of O^T
-    constexpr int CPT = TN * (HID / 8) / 256;  // 16-byte chunks per thread per tile
+    constexpr int CPT = TN * (HID / 8) / NTHREADS;  // 16-byte chunks per thread per tile
     extern __shared__ __align__(16) unsigned char smem_raw[];
     MfmaSmem<HID> &sm = *reinterpret_cast<MfmaSmem<HID> *>(smem_raw);
 
     const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
     const int col = lane & 31, hh = lane >> 5;
+    const int whead = wid >> 1, half = wid & 1;
 
     long long L = xcd_remap((long long)blockIdx.x, total_wg);
     const int qb = (int)(L % p.NBQ);
@@ -58,16 +69,15 @@ __global__ __launch_bounds__(256) void bsa_mfma_kernel(BsaParams p, int hgroups,
     L /= hgroups;
     const int kvh = (int)(L % p.kv.HKV);
     const int b = (int)(L / p.kv.HKV);
-    const int hin = hgrp * hpw + wid;
-    const bool head_ok = (wid < hpw) && (hin < p.G);
-    const int h = kvh * p.G + (head_ok ? hin : 0);
+    const int hin = hgrp * hpw + whead;
+    const bool head_ok = (whead < hpw) && (hin < p.G) && (half * 32 < p.bq);
+    const int h = kvh * p.G + ((whead < hpw && hin < p.G) ? hin : 0);
     // index row: the group's first head when rows are shared, else the single head this workgroup serves
     const int hrow = p.share_first_head ? kvh * p.G : kvh * p.G + hgrp * hpw;
     const int64_t irow = ((int64_t)b * p.HEAD + hrow) * p.idx_rows + qb;
 
     // ---- query block geometry
-    int pm[2];
-    int pmin_blk = 0x7fffffff, pmax_blk = -1;
+    int pmin_blk, pmax_blk;
     {
         long long cur = -1, mn = 0x7fffffff;
         for (int j = lane; j < p.bq; j += 64) {
@@ -87,13 +97,12 @@ __global__ __launch_bounds__(256) void bsa_mfma_kernel(BsaParams p, int hgroups,
         }
         pmax_blk = (int)cur;
         pmin_blk = (int)mn;
-#pragma unroll
-        for (int mb = 0; mb < 2; mb++) {
-            const int j = mb * 32 + col;
-            const long long it = (long long)qb * p.bq + j;
-            pm[mb] = (j < p.bq && it < p.TDST) ? (int)p.pos[(int64_t)b * p.pos_sb + it * p.pos_st] : -0x40000000;
-        }
     }
+    const int myj = half * 32 + col;                       // this lane's query row inside the block
+    const long long myit = (long long)qb * p.bq + myj;
+    const bool row_ok = (myj < p.bq) && (myit < p.TDST);
+    const int pq = row_ok ? (int)p.pos[(int64_t)b * p.pos_sb + myit * p.pos_st] : -0x40000000;
+
     const int curr = pmax_blk + 1;
     int rs = p.kse[irow * 2 + 0], re = p.kse[irow * 2 + 1];
     if (p.BK <= 0) { rs = 0; re = 0; }
@@ -109,35 +118,37 @@ __global__ __launch_bounds__(256) void bsa_mfma_kernel(BsaParams p, int hgroups,
     const int tiles_win = (n_win + TN - 1) / TN;
     const int ntiles = tiles_sel + tiles_sink + tiles_win;
 
-    // ---- Q^ fragments (B operand of the first product), resident for the whole kernel
-    Frag qf[2][KS];
-    {
-        const uint16_t *qbase = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
-#pragma unroll
-        for (int mb = 0; mb < 2; mb++) {
-            const int j = mb * 32 + col;
-            const long long it = (long long)qb * p.bq + j;
-            const bool ok = head_ok && (j < p.bq) && (it < p.TDST);
-#pragma unroll
-            for (int ks = 0; ks < KS; ks++) {
-                uint4 raw = make_uint4(0, 0, 0, 0);
-                if (ok) raw = *reinterpret_cast<const uint4 *>(qbase + it * p.q_st + ks * 16 + hh * 8);
-                const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const float lo = __uint_as_float(w[e] << 16) * p.c_q;
-                    const float hi = __uint_as_float(w[e] & 0xffff0000u) * p.c_q;
-                    qf[mb][ks].u[e] = pack_bf16(lo, hi);
-                }
-            }
+    // selected block starts -> LDS (removes a dependent global load from every tile's prefetch)
+    const bool idx_in_lds = nsel <= MAX_LDS_IDX;
+    if (idx_in_lds) {
+        for (int i = tid; i < nsel; i += NTHREADS) {
+            const long long st = p.indices[irow * p.BK + rs + i];
+            sm.idx[i] = (st >= 0 && st < 0x7fffffffLL) ? (int)st : -0x40000000;
         }
     }
+
+    // ---- Q^ fragments (B operand of the first product), resident for the whole kernel
+    Frag qf[KS];
+    {
+        const uint16_t *qbase = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
+        const bool ok = head_ok && row_ok;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            uint4 raw = make_uint4(0, 0, 0, 0);
+            if (ok) raw = *reinterpret_cast<const uint4 *>(qbase + myit * p.q_st + ks * 16 + hh * 8);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                qf[ks].u[e] = cvt_pk_bf16(__uint_as_float(w[e] << 16) * p.c_q, __uint_as_float(w[e] & 0xffff0000u) * p.c_q);
+        }
+    }
+    __syncthreads();  // sm.idx visible
 
     const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
     const uint16_t *kbase = reinterpret_cast<const uint16_t *>(p.kv.k);
     const uint16_t *vbase = reinterpret_cast<const uint16_t *>(p.kv.v);
 
-    // ---- staging: thread handles chunks c = tid + 256*j: token slot c / (HID/8), 16-byte piece c % (HID/8)
+    // ---- staging: thread handles chunks c = tid + NTHREADS*j: token slot c / (HID/8), 16-byte piece c % (HID/8)
     uint4 kreg[CPT], vreg[CPT];
     int treg[CPT];
     auto prefetch = [&](int tile) {
@@ -147,13 +158,14 @@ __global__ __launch_bounds__(256) void bsa_mfma_kernel(BsaParams p, int hgroups,
         else { kind = 2; base = (tile - tiles_sel - tiles_sink) * TN; }
 #pragma unroll
         for (int j = 0; j < CPT; j++) {
-            const int c = tid + 256 * j;
+            const int c = tid + NTHREADS * j;
             const int slot = c / (HID / 8), piece = c % (HID / 8);
             const int o = base + slot;
             long long t = -1;
             if (kind == 0) {
                 if (o < n_sel_tok) {
-                    const long long st = p.indices[irow * p.BK + rs + o / p.bk];
+                    const int bi = o / p.bk;
+                    const long long st = idx_in_lds ? (long long)sm.idx[bi] : p.indices[irow * p.BK + rs + bi];
                     t = st + o % p.bk;
                     if (!(t >= 0 && t < p.kv.max_tsrc && t < curr && t >= p.sink)) t = -1;
                 }
@@ -176,17 +188,16 @@ __global__ __launch_bounds__(256) void bsa_mfma_kernel(BsaParams p, int hgroups,
     auto commit = [&](int buf) {
 #pragma unroll
         for (int j = 0; j < CPT; j++) {
-            const int c = tid + 256 * j;
+            const int c = tid + NTHREADS * j;
             const int slot = c / (HID / 8), piece = c % (HID / 8);
-            const uint32_t kw[4] = {kreg[j].x, kreg[j].y, kreg[j].z, kreg[j].w};
-            uint32_t ko[4];
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const float lo = __uint_as_float(kw[e] << 16) * p.c_k;
-                const float hi = __uint_as_float(kw[e] & 0xffff0000u) * p.c_k;
-                ko[e] = pack_bf16(lo, hi);
+            uint4 kq = kreg[j];
+            if (!KSCALED) {
+                kq.x = cvt_pk_bf16(__uint_as_float(kq.x << 16) * p.c_k, __uint_as_float(kq.x & 0xffff0000u) * p.c_k);
+                kq.y = cvt_pk_bf16(__uint_as_float(kq.y << 16) * p.c_k, __uint_as_float(kq.y & 0xffff0000u) * p.c_k);
+                kq.z = cvt_pk_bf16(__uint_as_float(kq.z << 16) * p.c_k, __uint_as_float(kq.z & 0xffff0000u) * p.c_k);
+                kq.w = cvt_pk_bf16(__uint_as_float(kq.w << 16) * p.c_k, __uint_as_float(kq.w & 0xffff0000u) * p.c_k);
             }
-            *reinterpret_cast<uint4 *>(&sm.k[buf][slot][piece * 8]) = make_uint4(ko[0], ko[1], ko[2], ko[3]);
+            *reinterpret_cast<uint4 *>(&sm.k[buf][slot][piece * 8]) = kq;
             const uint32_t vw[4] = {vreg[j].x, vreg[j].y, vreg[j].z, vreg[j].w};
 #pragma unroll
             for (int e = 0; e < 4; e++) {
@@ -197,16 +208,14 @@ __global__ __launch_bounds__(256) void bsa_mfma_kernel(BsaParams p, int hgroups,
         }
     };
 
-    // ---- running state (per lane: two query columns)
-    f32x16 oacc[DB][2];
+    // ---- running state (a lane owns one query column)
+    f32x16 oacc[DB];
 #pragma unroll
     for (int db = 0; db < DB; db++)
 #pragma unroll
-        for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) oacc[db][mb][i] = 0.0f;
-    float m_run[2] = {-INFINITY, -INFINITY};
-    float l_run[2] = {0.0f, 0.0f};
+        for (int i = 0; i < 16; i++) oacc[db][i] = 0.0f;
+    float m_run = -INFINITY;   // in log2 units, already multiplied by log2(e)
+    float l_run = 0.0f;
 
     if (ntiles > 0) prefetch(0);
     for (int tile = 0; tile < ntiles; tile++) {
@@ -225,91 +234,80 @@ __global__ __launch_bounds__(256) void bsa_mfma_kernel(BsaParams p, int hgroups,
         bool full;  // every (valid row, token) pair of the tile is attended
         if (!window) full = all_valid && ((long long)tmax + p.sw <= pmin_blk);
         else full = all_valid && (tmax <= pmin_blk) && ((long long)pmax_blk < (long long)tmin + p.sw);
-        if (tmax < 0) continue;  // nothing valid in this tile (uniform)
+        if (tmax < 0 || !head_ok) continue;  // nothing valid in this tile, or an idle wave (both wave-uniform)
 
         // ---- S^T = K^ Q^^T
-        f32x16 sacc[2][2];
+        f32x16 sacc[2];
 #pragma unroll
         for (int nb = 0; nb < 2; nb++)
 #pragma unroll
-            for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) sacc[nb][mb][i] = 0.0f;
+            for (int i = 0; i < 16; i++) sacc[nb][i] = 0.0f;
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
             Frag a0, a1;
             a0.q = *reinterpret_cast<const uint4 *>(&sm.k[buf][col][ks * 16 + hh * 8]);
             a1.q = *reinterpret_cast<const uint4 *>(&sm.k[buf][32 + col][ks * 16 + hh * 8]);
-            sacc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0.v, qf[0][ks].v, sacc[0][0], 0, 0, 0);
-            sacc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0.v, qf[1][ks].v, sacc[0][1], 0, 0, 0);
-            sacc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1.v, qf[0][ks].v, sacc[1][0], 0, 0, 0);
-            sacc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1.v, qf[1][ks].v, sacc[1][1], 0, 0, 0);
-            if (ks % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+            sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0.v, qf[ks].v, sacc[0], 0, 0, 0);
+            sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1.v, qf[ks].v, sacc[1], 0, 0, 0);
         }
 
         // ---- mask + online softmax; element (nb, i) of a lane is token slot nb*32 + (i/4)*8 + hh*4 + i%4
-        Frag pf[2][4];
-        float alpha[2];
-#pragma unroll
-        for (int mb = 0; mb < 2; mb++) {
-            float mx = -INFINITY;
-            if (full) {
-#pragma unroll
-                for (int nb = 0; nb < 2; nb++)
-#pragma unroll
-                    for (int i = 0; i < 16; i++) {
-                        sacc[nb][mb][i] *= LOG2E;
-                        mx = fmaxf(mx, sacc[nb][mb][i]);
-                    }
-            } else {
-                const int pq = pm[mb];
-#pragma unroll
-                for (int nb = 0; nb < 2; nb++)
-#pragma unroll
-                    for (int i4 = 0; i4 < 4; i4++) {
-                        const int4 tt = *reinterpret_cast<const int4 *>(&sm.tok[buf][nb * 32 + i4 * 8 + hh * 4]);
-                        const int ts[4] = {tt.x, tt.y, tt.z, tt.w};
-#pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            const int t = ts[e];
-                            bool att;
-                            if (!window) att = (t >= 0) && ((long long)t + p.sw <= pq);
-                            else att = (t >= 0) && (t <= pq) && ((long long)pq < (long long)t + p.sw);
-                            const float s = att ? sacc[nb][mb][i4 * 4 + e] * LOG2E : -INFINITY;
-                            sacc[nb][mb][i4 * 4 + e] = s;
-                            mx = fmaxf(mx, s);
-                        }
-                    }
-            }
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float m_new = fmaxf(m_run[mb], mx);
-            const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-            alpha[mb] = __builtin_amdgcn_exp2f(m_run[mb] - m_use);  // m_run = -inf -> 0
-            float lsum = 0.0f;
+        float mx = -INFINITY;
+        if (full) {
 #pragma unroll
             for (int nb = 0; nb < 2; nb++)
 #pragma unroll
-                for (int u = 0; u < 2; u++)
+                for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[nb][i]);
+        } else {
+#pragma unroll
+            for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+                for (int i4 = 0; i4 < 4; i4++) {
+                    const int4 tt = *reinterpret_cast<const int4 *>(&sm.tok[buf][nb * 32 + i4 * 8 + hh * 4]);
+                    const int ts[4] = {tt.x, tt.y, tt.z, tt.w};
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        const float p0 = __builtin_amdgcn_exp2f(sacc[nb][mb][u * 8 + 2 * e] - m_use);
-                        const float p1 = __builtin_amdgcn_exp2f(sacc[nb][mb][u * 8 + 2 * e + 1] - m_use);
-                        lsum += p0 + p1;
-                        pf[mb][nb * 2 + u].u[e] = pack_bf16(p0, p1);
+                        const int t = ts[e];
+                        bool att;
+                        if (!window) att = (t >= 0) && ((long long)t + p.sw <= pq);
+                        else att = (t >= 0) && (t <= pq) && ((long long)pq < (long long)t + p.sw);
+                        const float s = att ? sacc[nb][i4 * 4 + e] : -INFINITY;
+                        sacc[nb][i4 * 4 + e] = s;
+                        mx = fmaxf(mx, s);
                     }
-            l_run[mb] = l_run[mb] * alpha[mb] + lsum;
-            m_run[mb] = m_new;
+                }
         }
+        mx = fmaxf(mx, __shfl_xor(mx, 32)) * LOG2E;
+        // raise the reference point only when the maximum grew noticeably
+        float m_use = m_run;
+        float alpha = 1.0f;
+        if (mx > m_run + RESCALE_STEP || m_run == -INFINITY) {
+            m_use = fmaxf(m_run, mx);
+            alpha = (m_use == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_use);  // m_run = -inf -> 0
+        }
+        const float m_sub = (m_use == -INFINITY) ? 0.0f : m_use;
+        Frag pf[4];
+        float lsum = 0.0f;
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+            for (int u = 0; u < 2; u++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[nb][u * 8 + 2 * e], LOG2E, -m_sub));
+                    const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[nb][u * 8 + 2 * e + 1], LOG2E, -m_sub));
+                    lsum += p0 + p1;
+                    pf[nb * 2 + u].u[e] = cvt_pk_bf16(p0, p1);
+                }
+        l_run = l_run * alpha + lsum;
+        m_run = m_use;
 
         // ---- O^T += V^T P^T
-        const bool rescale = __any((alpha[0] != 1.0f) || (alpha[1] != 1.0f));
-        if (rescale) {
+        if (__any(alpha != 1.0f)) {
 #pragma unroll
             for (int db = 0; db < DB; db++)
 #pragma unroll
-                for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-                    for (int i = 0; i < 16; i++) oacc[db][mb][i] *= alpha[mb];
+                for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
         }
 #pragma unroll
         for (int db = 0; db < DB; db++) {
@@ -318,37 +316,30 @@ __global__ __launch_bounds__(256) void bsa_mfma_kernel(BsaParams p, int hgroups,
                 Frag a;
                 a.d[0] = *reinterpret_cast<const uint2 *>(&sm.vt[buf][db * 32 + col][j * 16 + hh * 4]);
                 a.d[1] = *reinterpret_cast<const uint2 *>(&sm.vt[buf][db * 32 + col][j * 16 + 8 + hh * 4]);
-                oacc[db][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pf[0][j].v, oacc[db][0], 0, 0, 0);
-                oacc[db][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pf[1][j].v, oacc[db][1], 0, 0, 0);
-                if (j % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pf[j].v, oacc[db], 0, 0, 0);
             }
         }
     }
 
     // ---- epilogue: O^T[d, m] / l -> out[b, m, h, d]
     if (!head_ok) return;
-    uint16_t *obase = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
+    const float l = l_run + __shfl_xor(l_run, 32);
+    if (!row_ok) return;
+    const float inv = 1.0f / (l == 0.0f ? 1.0f : l);
+    uint16_t *obase = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + myit * p.o_st;
 #pragma unroll
-    for (int mb = 0; mb < 2; mb++) {
-        const int j = mb * 32 + col;
-        const long long it = (long long)qb * p.bq + j;
-        float l = l_run[mb] + __shfl_xor(l_run[mb], 32);
-        if (!(j < p.bq && it < p.TDST)) continue;
-        const float inv = 1.0f / (l == 0.0f ? 1.0f : l);
+    for (int db = 0; db < DB; db++)
 #pragma unroll
-        for (int db = 0; db < DB; db++)
-#pragma unroll
-            for (int i4 = 0; i4 < 4; i4++) {
-                const int d = db * 32 + i4 * 8 + hh * 4;
-                uint2 o;
-                o.x = pack_bf16(oacc[db][mb][i4 * 4 + 0] * inv, oacc[db][mb][i4 * 4 + 1] * inv);
-                o.y = pack_bf16(oacc[db][mb][i4 * 4 + 2] * inv, oacc[db][mb][i4 * 4 + 3] * inv);
-                *reinterpret_cast<uint2 *>(obase + it * p.o_st + d) = o;
-            }
-    }
+        for (int i4 = 0; i4 < 4; i4++) {
+            const int d = db * 32 + i4 * 8 + hh * 4;
+            uint2 o;
+            o.x = cvt_pk_bf16(oacc[db][i4 * 4 + 0] * inv, oacc[db][i4 * 4 + 1] * inv);
+            o.y = cvt_pk_bf16(oacc[db][i4 * 4 + 2] * inv, oacc[db][i4 * 4 + 3] * inv);
+            *reinterpret_cast<uint2 *>(obase + d) = o;
+        }
 }
 
-template <int HID>
+template <int HID, bool KSCALED>
 static int launch_mfma(const BsaParams &p, hipStream_t st) {
     const int hpw = p.share_first_head ? 4 : 1;  // per-head index rows: one head per workgroup
     const int hgroups = (p.G + hpw - 1) / hpw;
@@ -357,11 +348,12 @@ static int launch_mfma(const BsaParams &p, hipStream_t st) {
     const size_t smem = sizeof(MfmaSmem<HID>);
     static bool attr_set = false;
     if (!attr_set) {
-        HIPATTN_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&bsa_mfma_kernel<HID>),
+        HIPATTN_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&bsa_mfma_kernel<HID, KSCALED>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
-    hipLaunchKernelGGL((bsa_mfma_kernel<HID>), dim3((unsigned)total), dim3(256), smem, st, p, hgroups, hpw, total);
+    hipLaunchKernelGGL((bsa_mfma_kernel<HID, KSCALED>), dim3((unsigned)total), dim3(NTHREADS), smem, st, p, hgroups,
+                       hpw, total);
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
 }
@@ -370,9 +362,16 @@ int bsa_mfma_launch(const BsaParams &p, int dtype, int HID, hipStream_t st) {
     if (dtype != HIPATTN_BF16) return HIPATTN_E_UNSUPPORTED;
     if (p.bq > 64) return HIPATTN_E_UNSUPPORTED;
     if ((p.o_st % 4) != 0 || (p.o_sh % 4) != 0 || (p.o_sb % 4) != 0) return HIPATTN_E_UNSUPPORTED;
-    switch (HID) {
-        case 64: return launch_mfma<64>(p, st);
-        case 128: return launch_mfma<128>(p, st);
+    if (p.k_prescaled) {
+        switch (HID) {
+            case 64: return launch_mfma<64, true>(p, st);
+            case 128: return launch_mfma<128, true>(p, st);
+        }
+    } else {
+        switch (HID) {
+            case 64: return launch_mfma<64, false>(p, st);
+            case 128: return launch_mfma<128, false>(p, st);
+        }
     }
     return HIPATTN_E_UNSUPPORTED;
 }

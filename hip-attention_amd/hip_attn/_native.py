@@ -13,7 +13,7 @@ from typing import Optional
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "libhipattn.so")
+_LIB_PATH = os.environ.get("HIPATTN_LIBRARY", os.path.join(_HERE, "libhipattn.so"))
 _lib = None
 
 F32, BF16 = 0, 1
@@ -228,14 +228,16 @@ def finalize_indices(scores, left_out, pos, B, bs, bdst, scan_stride, HEAD, hg, 
     check(rc, "hipattn_finalize_indices")
 
 
-def bsa_prefill(qs, kvs, indices, ks_start_end, BK, bq, bk, sw, sink, share_first_head, impl, out, device):
+def bsa_prefill(qs, kvs, indices, ks_start_end, BK, bq, bk, sw, sink, share_first_head, impl, out, device,
+                k_prescaled=None):
     assert indices.dtype == torch.int64 and indices.is_contiguous()
     assert ks_start_end.dtype == torch.int32 and ks_start_end.is_contiguous()
     with _timed("bsa_prefill"):
       rc = lib().hipattn_bsa_prefill(
         ctypes.byref(qs), ctypes.byref(kvs), _p(indices), _p(ks_start_end), ctypes.c_int32(indices.shape[1]),
         ctypes.c_int32(BK), ctypes.c_int32(bq), ctypes.c_int32(bk), ctypes.c_int32(sw), ctypes.c_int32(sink),
-        ctypes.c_int32(int(share_first_head)), ctypes.c_int32(impl), _p(out), ctypes.c_int64(out.stride(0)),
+        ctypes.c_int32(int(share_first_head)), ctypes.c_int32(impl), _p(k_prescaled), _p(out),
+        ctypes.c_int64(out.stride(0)),
         ctypes.c_int64(out.stride(1)), ctypes.c_int64(out.stride(2)), stream_ptr(device))
     check(rc, "hipattn_bsa_prefill")
 

@@ -104,9 +104,9 @@ def _mask_kv(args: HiPAttentionArgs, k_mask: Optional[Tensor], max_tsrc: int, q:
                     a2 = args.clone()
                     a2.k_cache, a2.v_cache = khat, khat
                     st, keep = _kv_struct(a2, None, None, max_tsrc)
-                return st, (keep, khat), True
+                return st, (keep, khat), khat
     st, keep = _kv_struct(args, k_mask, k_mask, max_tsrc)
-    return st, keep, False
+    return st, keep, None
 
 
 def _stage_cache_views(chunk_left: Tensor, HEAD: int, chunk: int) -> HiPAttentionStageInputCache:
@@ -198,6 +198,7 @@ def dual_stage_quadratic_hip_attention(
     hg = 1 if _head_reduce_enabled() else HEAD
     mask_kv = None  # built lazily: cached-mask steps never touch the estimation path
     k_prescaled = False
+    khat = None
 
     if (cached_metadata is None) or (cached_metadata.indices is None):
         fresh = (cached_metadata is None) or (cached_metadata.stage_caches is None) or (stage_caches is None)
@@ -216,7 +217,8 @@ def dual_stage_quadratic_hip_attention(
 
         # Keys are scaled by c_k and re-rounded every time they are sampled.  When the scan will sample
         # far more rows than the key tensor holds (prefill), scale the whole tensor once instead.
-        mask_kv, keep_mask_kv, k_prescaled = _mask_kv(args, k_mask, MAX_TSRC, q, BSZ * HEAD * BDST_SCAN, chunk_count, device)
+        mask_kv, keep_mask_kv, khat = _mask_kv(args, k_mask, MAX_TSRC, q, BSZ * HEAD * BDST_SCAN, chunk_count, device)
+        k_prescaled = khat is not None
 
         scores = None
         left_out = None
@@ -361,6 +363,7 @@ def dual_stage_quadratic_hip_attention(
     seq_pos = position_ids[:, -q_bsa.shape[1]:]
     context = block_sparse_attention(
         q_bsa, k, v, seq_pos, indices, ks_start_end, args, MAX_TSRC, decode=use_decode, rows_shared=rows_shared,
+        khat=khat if (args.k_mask is None) else None,
     )
 
     metadata = HiPAttentionOutputMetadata(
@@ -381,7 +384,7 @@ def dual_stage_quadratic_hip_attention(
 @torch.no_grad()
 def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], position_ids: Tensor, indices: Tensor,
                            ks_start_end: Tensor, args: HiPAttentionArgs, max_tsrc: int, decode: bool = False,
-                           impl: int = 0, rows_shared: bool = False) -> Tensor:
+                           impl: int = 0, rows_shared: bool = False, khat: Optional[Tensor] = None) -> Tensor:
     """Sparse attention over (selected blocks, sink, sliding window) given the metadata tensors.
 
     ``position_ids`` are 0-based (the reference passes ``seq_lens = position_ids + 1``,
@@ -390,7 +393,8 @@ def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], 
     path, which, like the reference's decode kernel, lets every head of a GQA group read the
     index row of the group's first head.  ``rows_shared`` promises that all heads of a GQA group hold
     identical index rows (true for masks estimated with head reduction), which lets one gathered
-    K/V tile serve the whole group.
+    K/V tile serve the whole group.  ``khat`` is an optional ``bf16(k * c_k)`` tensor with the shape and
+    strides of the key storage (dense ``k`` or ``args.k_cache``).
     """
     device = q.device
     qq = q if q.stride(-1) == 1 else q.contiguous()
@@ -414,7 +418,11 @@ def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], 
         except N.HipAttnError as e:
             if "is not built" not in str(e):
                 raise
+    ksrc = k if k is not None else args.k_cache
+    if khat is not None and (ksrc is None or khat.shape != ksrc.shape or khat.stride() != ksrc.stride()):
+        khat = None
     N.bsa_prefill(qs, kvs, indices, ks_start_end, BK, args.block_size_q, args.block_size_k,
-                  args.sliding_window_size, args.sink_token_size, decode or rows_shared, impl, out, device)
+                  args.sliding_window_size, args.sink_token_size, decode or rows_shared, impl, out, device,
+                  k_prescaled=khat)
     del keep
     return out

@@ -123,11 +123,14 @@ int hipattn_finalize_indices(const float *scores, const int32_t *left_out, const
  *   out has q's dtype; out strides in elements.
  *   share_first_head != 0: every head of a GQA group reads the index row of the group's first
  *   head (decode kernel behaviour, src/hip_attn/v1_2/attention_decode_bsa.py:150).
- *   impl: 0 = pick automatically, 1 = portable row-at-a-time kernel, 2 = MFMA tile kernel. */
+ *   impl: 0 = pick automatically, 1 = portable row-at-a-time kernel, 2 = MFMA tile kernel.
+ *   k_prescaled: NULL, or bf16(K * c_k) with exactly the layout and strides of kv->k (the buffer
+ *   hipattn_prescale_k fills when K itself is contiguous); only the tile kernel reads it. */
 int hipattn_bsa_prefill(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t *indices,
                         const int32_t *ks_start_end, int32_t idx_rows, int32_t BK,
                         int32_t block_size_q, int32_t block_size_k, int32_t sliding_window,
-                        int32_t sink, int32_t share_first_head, int32_t impl, void *out,
+                        int32_t sink, int32_t share_first_head, int32_t impl,
+                        const void *k_prescaled, void *out,
                         int64_t out_stride_b, int64_t out_stride_t, int64_t out_stride_h,
                         void *stream);
 
