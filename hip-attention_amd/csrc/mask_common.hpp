@@ -21,6 +21,7 @@ struct MaskParams {
     float c_q, c_k;
     float *scores;
     int32_t *left_out;
+    const uint16_t *qhat;  // bf16 path: workspace [B, BS, HEAD, nrows, HID] filled by the entry point
 };
 
 // bf16 path on the matrix cores (mask_stage_mfma.hip)

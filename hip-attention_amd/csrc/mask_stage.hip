@@ -266,7 +266,7 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
                                   int32_t hg, int32_t n, int32_t chunk_size, int64_t right_clamp,
                                   int32_t bs, int32_t bq, int32_t stride_q, int32_t block_chunk,
                                   int32_t scan_stride, int32_t sw_eff, int32_t terminate_size,
-                                  int32_t k_prescaled, float *scores, int32_t *left_out, void *stream) {
+                                  int32_t k_prescaled, void *workspace, float *scores, int32_t *left_out, void *stream) {
     int rc = check_q(q);
     if (rc) return rc;
     HIPATTN_CHECK_ARG(kv && chunk_left && scores, HIPATTN_E_ARG, "mask stage: null pointer");
@@ -307,6 +307,9 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
     // the kernel indexes rows up to nrows; MAXROWS must cover every row that can be valid
     hipStream_t st = (hipStream_t)stream;
     if (q->dtype == HIPATTN_BF16) {
+        HIPATTN_CHECK_ARG(workspace && aligned16(workspace), HIPATTN_E_ARG,
+                          "mask stage: bf16 inputs need a 16-byte aligned workspace (hipattn_mask_stage_workspace_bytes)");
+        p.qhat = reinterpret_cast<const uint16_t *>(workspace);
         return mask_stage_mfma_launch(p, q->HID, rows_eff, k_prescaled, st);
     } else if (q->dtype == HIPATTN_F32) {
         HIPATTN_CHECK_ARG(!k_prescaled, HIPATTN_E_ARG, "mask stage: prescaled keys are a bf16-only option");
@@ -318,4 +321,10 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
     }
     set_error("mask stage: head dim %d with dtype %d is not built", q->HID, q->dtype);
     return HIPATTN_E_UNSUPPORTED;
+}
+
+extern "C" int64_t hipattn_mask_stage_workspace_bytes(int32_t dtype, int32_t B, int32_t bs, int32_t HEAD, int32_t HID,
+                                                      int32_t bq, int32_t stride_q) {
+    if (dtype != HIPATTN_BF16 || B <= 0 || bs <= 0 || HEAD <= 0 || HID <= 0 || bq <= 0 || stride_q <= 0) return 0;
+    return (int64_t)B * bs * HEAD * (bq / stride_q) * HID * 2;
 }

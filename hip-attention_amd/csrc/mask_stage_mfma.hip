@@ -3,8 +3,9 @@
 // Scores of a binary-search iteration are S[query row, sampled token] = q^ . k^.  One
 // v_mfma_f32_32x32x16_bf16 covers 32 query rows x 32 sampled tokens x 16 head-dim elements with
 //   A = Q^ rows     (resident in registers for the whole kernel),
-//   B = K^ rows     (lane n%32 <-> token, loaded straight from global memory: a lane reads one half
-//                    of its token's row, HID bytes contiguous, no LDS staging and no barriers),
+//   B = K^ rows     (lane n%32 <-> token; rows are fetched with fully coalesced 16-lane-per-row loads,
+//                    parked in a per-wave LDS tile with an XOR swizzle of the 16-byte pieces, and read
+//                    back in operand layout without bank conflicts),
 //   D[row, token]   (a lane ends up with 16 query rows of ITS token: the max over rows is in-lane).
 // A wave owns NB blocks of 32 tokens = 16*NB chunks (left and right sample of a chunk sit in
 // adjacent lanes); the program-level gate and iteration count of the reference (a "program" is a
@@ -14,6 +15,8 @@
 // Accumulation order of the dot product is the hardware's: two groups of 8 per instruction,
 // instructions chained through the f32 accumulator; head-dim element of (instruction ks, lane half
 // hh, i) is  hh*HID/2 + ks*8 + i.  The order is part of the operator's numeric definition.
+#include <stdlib.h>
+
 #include "mask_common.hpp"
 
 namespace hipattn {
@@ -27,16 +30,30 @@ union BFrag {
     uint4 q;
 };
 
-__device__ __forceinline__ uint32_t scale_pack(uint32_t w, float c) {
-    const float lo = __uint_as_float(w << 16) * c;
-    const float hi = __uint_as_float(w & 0xffff0000u) * c;
-    return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+
+// two f32 -> packed bf16 pair with round-to-nearest-even (one v_cvt_pk_bf16_f32)
+__device__ __forceinline__ uint32_t cvt_pk_bf16(float a, float b) {
+    f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
 
-template <int HID, int MB, int NB, bool PRESCALED>
+__device__ __forceinline__ uint32_t scale_pack(uint32_t w, float c) {
+    return cvt_pk_bf16(__uint_as_float(w << 16) * c, __uint_as_float(w & 0xffff0000u) * c);
+}
+
+template <int HID, int MB, int NB, bool PRESCALED, bool VIA_LDS>
 __global__ __launch_bounds__(64) void mask_stage_mfma_kernel(MaskParams p, int nsub) {
     constexpr int KS = HID / 16;
     constexpr int HALF = HID / 2;
+    constexpr int PPR = HID / 8;                  // 16-byte pieces per key row
+    constexpr int RPI = 64 / PPR;                 // rows fetched per load instruction
+    constexpr int NROWS = NB * 32;                // sampled rows per iteration of this wave
+    constexpr int SWZ = (PPR < 16 ? PPR : 16) - 1;
+    constexpr int SWZ_DIV = PPR < 16 ? 16 / PPR : 1;
+    __shared__ __align__(16) uint4 s_rows[VIA_LDS ? NROWS * PPR : 1];
+    __shared__ int64_t s_off[VIA_LDS ? NROWS : 1];
     const int lane = threadIdx.x;
     const int n = lane & 31, hh = lane >> 5;
     const int side = n & 1;
@@ -120,42 +137,19 @@ __global__ __launch_bounds__(64) void mask_stage_mfma_kernel(MaskParams p, int n
         return;
     }
 
-    // ---- Q^ fragments: lane (row = mb*32 + n, half hh) holds elements hh*HALF + ks*8 .. +8
+    // ---- Q^ fragments: lane (row = mb*32 + n, half hh) holds elements hh*HALF + ks*8 .. +8.
+    // Rows were averaged, rounded and scaled once per stage by qhat_kernel: [B, BS, HEAD, nrows, HID].
     BFrag qf[MB][KS];
     {
-        const uint16_t *qbase = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
+        const uint16_t *qh = p.qhat + ((((int64_t)b * p.BS + s) * p.HEAD + h) * p.nrows) * HID;
 #pragma unroll
         for (int mb = 0; mb < MB; mb++) {
             const int j = mb * 32 + n;
             const bool jv = (j < p.nrows) && ((rowmask >> j) & 1ull);
-            const long long it = qb * p.BQ + (long long)j * p.stride_q;
 #pragma unroll
             for (int ks = 0; ks < KS; ks++) {
-                float sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-                int cnt = 0;
-                if (jv) {
-                    for (int o = 0; o < p.stride_q; o++) {
-                        if (it + o < p.TDST) {
-                            const uint4 raw = *reinterpret_cast<const uint4 *>(qbase + (it + o) * p.q_st + hh * HALF + ks * 8);
-                            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-                            for (int e = 0; e < 4; e++) {
-                                sum[2 * e] += __uint_as_float(w[e] << 16);
-                                sum[2 * e + 1] += __uint_as_float(w[e] & 0xffff0000u);
-                            }
-                            cnt++;
-                        }
-                    }
-                }
-                const float den = (float)cnt + 1e-12f;
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const float m0 = round_bf16(__fdiv_rn(sum[2 * e], den));
-                    const float m1 = round_bf16(__fdiv_rn(sum[2 * e + 1], den));
-                    qf[mb][ks].u[e] = jv ? ((uint32_t)f32_to_bf16_bits(m0 * p.c_q) |
-                                            ((uint32_t)f32_to_bf16_bits(m1 * p.c_q) << 16))
-                                         : 0u;
-                }
+                qf[mb][ks].q = make_uint4(0, 0, 0, 0);
+                if (jv) qf[mb][ks].q = *reinterpret_cast<const uint4 *>(qh + (int64_t)j * HID + hh * HALF + ks * 8);
             }
         }
     }
@@ -181,11 +175,12 @@ __global__ __launch_bounds__(64) void mask_stage_mfma_kernel(MaskParams p, int n
     const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
     const uint16_t *kbase = reinterpret_cast<const uint16_t *>(p.kv.k);
 
+    const int lrow = lane / PPR, lpos = lane % PPR;  // loader role: row within an instruction, piece slot
     while (width >= p.terminate) {
         width *= 0.5f;
         bool active[NB];
         int ctr[NB];
-        uint4 raw[NB][KS];
+        uint4 raw[VIA_LDS ? 1 : NB][VIA_LDS ? 1 : KS];
 #pragma unroll
         for (int tb = 0; tb < NB; tb++) {
             active[tb] = real[tb] && (cl[tb] < cr[tb]) && (cl[tb] <= lim) && (cl[tb] >= 0);
@@ -195,11 +190,35 @@ __global__ __launch_bounds__(64) void mask_stage_mfma_kernel(MaskParams p, int n
                 const int t = side ? ((ctr[tb] + cr[tb]) >> 1) : ((cl[tb] + ctr[tb]) >> 1);
                 off = p.kv.k_row(b, t, kvh, seqlen);
             }
+            if constexpr (VIA_LDS) {
+                if (hh == 0) s_off[tb * 32 + n] = off;
+            } else {
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) {
-                raw[tb][ks] = make_uint4(0, 0, 0, 0);
-                if (off >= 0) raw[tb][ks] = *reinterpret_cast<const uint4 *>(kbase + off + hh * HALF + ks * 8);
+                for (int ks = 0; ks < KS; ks++) {
+                    raw[tb][ks] = make_uint4(0, 0, 0, 0);
+                    if (off >= 0) raw[tb][ks] = *reinterpret_cast<const uint4 *>(kbase + off + hh * HALF + ks * 8);
+                }
             }
+        }
+        if constexpr (VIA_LDS) {
+            __syncthreads();
+            // coalesced fetch: PPR lanes cover one row; piece q of row r is parked at slot q ^ swz(r)
+#pragma unroll
+            for (int i = 0; i < NROWS / RPI; i++) {
+                const int r = i * RPI + lrow;
+                const int64_t off = s_off[r];
+                const int q = lpos ^ ((r / SWZ_DIV) & SWZ);
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (off >= 0) v = *reinterpret_cast<const uint4 *>(kbase + off + q * 8);
+                if (!PRESCALED) {
+                    v.x = scale_pack(v.x, p.c_k);
+                    v.y = scale_pack(v.y, p.c_k);
+                    v.z = scale_pack(v.z, p.c_k);
+                    v.w = scale_pack(v.w, p.c_k);
+                }
+                s_rows[r * PPR + lpos] = v;
+            }
+            __syncthreads();
         }
 #pragma unroll
         for (int tb = 0; tb < NB; tb++) {
@@ -208,10 +227,14 @@ __global__ __launch_bounds__(64) void mask_stage_mfma_kernel(MaskParams p, int n
             for (int mb = 0; mb < MB; mb++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) acc[mb][i] = 0.0f;
+            const int r = tb * 32 + n;
+            const int sw = (r / SWZ_DIV) & SWZ;
 #pragma unroll
             for (int ks = 0; ks < KS; ks++) {
                 BFrag kf;
-                if (PRESCALED) {
+                if constexpr (VIA_LDS) {
+                    kf.q = s_rows[r * PPR + ((hh * (PPR / 2) + ks) ^ sw)];
+                } else if constexpr (PRESCALED) {
                     kf.q = raw[tb][ks];
                 } else {
                     kf.u[0] = scale_pack(raw[tb][ks].x, p.c_k);
@@ -256,31 +279,91 @@ __global__ __launch_bounds__(64) void mask_stage_mfma_kernel(MaskParams p, int n
     store_out();
 }
 
+// Q^ rows of every scan program: strided mean of stride_q query rows in f32, rounded to bf16, scaled
+// by c_q, rounded again (attention_extend.py:607-734,924-931).  One thread makes 8 elements.
+__global__ void qhat_kernel(MaskParams p, int hid, uint16_t *out) {
+    const int per_row = hid / 8;
+    const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long total = (long long)p.B * p.BS * p.HEAD * p.nrows * per_row;
+    if (gid >= total) return;
+    const int piece = (int)(gid % per_row);
+    long long r = gid / per_row;
+    const int j = (int)(r % p.nrows);
+    r /= p.nrows;
+    const int h = (int)(r % p.HEAD);
+    r /= p.HEAD;
+    const int s = (int)(r % p.BS);
+    const int b = (int)(r / p.BS);
+    const long long qb = (long long)(p.BDST - 1) - (long long)(p.BS - 1) * p.scan_stride + (long long)s * p.scan_stride;
+    const long long it = qb * p.BQ + (long long)j * p.stride_q;
+    uint4 o = make_uint4(0, 0, 0, 0);
+    if (it >= 0 && it < p.TDST) {
+        const uint16_t *qbase = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
+        float sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        int cnt = 0;
+        for (int oo = 0; oo < p.stride_q; oo++) {
+            if (it + oo < p.TDST) {
+                const uint4 raw = *reinterpret_cast<const uint4 *>(qbase + (it + oo) * p.q_st + piece * 8);
+                const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    sum[2 * e] += __uint_as_float(w[e] << 16);
+                    sum[2 * e + 1] += __uint_as_float(w[e] & 0xffff0000u);
+                }
+                cnt++;
+            }
+        }
+        const float den = (float)cnt + 1e-12f;
+        uint32_t ow[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const float m0 = round_bf16(__fdiv_rn(sum[2 * e], den));
+            const float m1 = round_bf16(__fdiv_rn(sum[2 * e + 1], den));
+            ow[e] = cvt_pk_bf16(m0 * p.c_q, m1 * p.c_q);
+        }
+        o = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+    }
+    *reinterpret_cast<uint4 *>(out + gid * 8) = o;
+}
+
+static int g_mask_via_lds = -1;  // -1: decide per shape; 0 / 1: forced through HIPATTN_MASK_VIA_LDS (tuning aid)
+
 template <int HID>
 static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hipStream_t st) {
     MaskParams p = p0;
     const int BC = p.block_chunk;
     const bool two = rows_eff > 32;
-    // one wave per program (4 token blocks) when programs are plentiful, else one block per wave
+    // two token blocks (32 chunks) per wave when programs are plentiful, else one block per wave
     const long long programs = (long long)p.B * p.HEAD * p.BS * p.ngroups;
-    const bool wide = (BC == 64) && (programs >= 16384);
-    const int nb = wide ? 4 : 1;
+    const bool wide = (BC >= 32) && (programs >= 16384);
+    const int nb = wide ? 2 : 1;
     const int nsub = (BC / 16) / nb;
     p.total = programs * nsub;
     if (p.total >= 0x7fffffffLL) {
         set_error("mask stage: grid too large");
         return HIPATTN_E_UNSUPPORTED;
     }
-    dim3 grid((unsigned)p.total), block(64);
-#define MS_LAUNCH(MBv, NBv, PSv) \
-    hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, NBv, PSv>), grid, block, 0, st, p, nsub)
-    if (two) {
-        if (wide) { if (prescaled) MS_LAUNCH(2, 4, true); else MS_LAUNCH(2, 4, false); }
-        else { if (prescaled) MS_LAUNCH(2, 1, true); else MS_LAUNCH(2, 1, false); }
-    } else {
-        if (wide) { if (prescaled) MS_LAUNCH(1, 4, true); else MS_LAUNCH(1, 4, false); }
-        else { if (prescaled) MS_LAUNCH(1, 1, true); else MS_LAUNCH(1, 1, false); }
+    {
+        const long long work = (long long)p.B * p.BS * p.HEAD * p.nrows * (HID / 8);
+        const long long blocks = (work + 255) / 256;
+        hipLaunchKernelGGL(qhat_kernel, dim3((unsigned)blocks), dim3(256), 0, st, p, HID, const_cast<uint16_t *>(p.qhat));
     }
+    if (g_mask_via_lds < 0) {
+        const char *e = getenv("HIPATTN_MASK_VIA_LDS");
+        g_mask_via_lds = e ? (e[0] == '1' ? 1 : 0) : 2;
+    }
+    const bool via_lds = g_mask_via_lds == 2 ? !wide : (g_mask_via_lds == 1);
+    dim3 grid((unsigned)p.total), block(64);
+#define MS_LAUNCH(MBv, NBv, PSv, VLv) \
+    hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, NBv, PSv, VLv>), grid, block, 0, st, p, nsub)
+#define MS_PICK(MBv, NBv)                                                \
+    do {                                                                  \
+        if (prescaled) { if (via_lds) MS_LAUNCH(MBv, NBv, true, true); else MS_LAUNCH(MBv, NBv, true, false); } \
+        else { if (via_lds) MS_LAUNCH(MBv, NBv, false, true); else MS_LAUNCH(MBv, NBv, false, false); }        \
+    } while (0)
+    if (two) { if (wide) MS_PICK(2, 2); else MS_PICK(2, 1); }
+    else { if (wide) MS_PICK(1, 2); else MS_PICK(1, 1); }
+#undef MS_PICK
 #undef MS_LAUNCH
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;

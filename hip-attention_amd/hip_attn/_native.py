@@ -64,6 +64,7 @@ def lib():
         L.hipattn_version.restype = ctypes.c_char_p
         L.hipattn_last_error.restype = ctypes.c_char_p
         L.hipattn_bsa_decode_workspace_bytes.restype = ctypes.c_int64
+        L.hipattn_mask_stage_workspace_bytes.restype = ctypes.c_int64
         L.hipattn_bsa_decode_default_splits.restype = ctypes.c_int32
         for name in ("hipattn_mask_stage", "hipattn_prescale_k", "hipattn_select_stage", "hipattn_finalize_indices",
                      "hipattn_bsa_prefill", "hipattn_bsa_decode_partial", "hipattn_bsa_decode_merge"):
@@ -198,12 +199,17 @@ def prescale_k(k: torch.Tensor, device) -> torch.Tensor:
 
 def mask_stage(qs, kvs, chunk_left, hg, n, chunk, right_clamp, bs, bq, stride_q, block_chunk, scan_stride,
                sw_eff, terminate, scores, left_out, device, k_prescaled=False):
+    need = lib().hipattn_mask_stage_workspace_bytes(
+        ctypes.c_int32(qs.dtype), ctypes.c_int32(qs.B), ctypes.c_int32(bs), ctypes.c_int32(qs.HEAD),
+        ctypes.c_int32(qs.HID), ctypes.c_int32(bq), ctypes.c_int32(stride_q))
+    workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=scores.device) if need > 0 else None
     with _timed(f"mask_stage[n={n},chunk={chunk},rows={bq // stride_q}]"):
       rc = lib().hipattn_mask_stage(
         ctypes.byref(qs), ctypes.byref(kvs), _p(chunk_left), ctypes.c_int32(hg), ctypes.c_int32(n),
         ctypes.c_int32(chunk), ctypes.c_int64(right_clamp), ctypes.c_int32(bs), ctypes.c_int32(bq),
         ctypes.c_int32(stride_q), ctypes.c_int32(block_chunk), ctypes.c_int32(scan_stride),
-        ctypes.c_int32(sw_eff), ctypes.c_int32(terminate), ctypes.c_int32(int(k_prescaled)), _p(scores),
+        ctypes.c_int32(sw_eff), ctypes.c_int32(terminate), ctypes.c_int32(int(k_prescaled)), _p(workspace),
+        _p(scores),
         _p(left_out), stream_ptr(device))
     check(rc, "hipattn_mask_stage")
 

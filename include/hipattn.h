@@ -75,12 +75,19 @@ const char *hipattn_last_error(void);
  *   left_out    int32 [B, BS, HEAD, n] refined left edge per head, or NULL
  *   block_chunk = chunks per reference program (16/32/64): fixes the program-level gate and
  *   iteration count (:595-601,736-737).
- *   k_prescaled != 0: kv->k already holds bf16(K * c_k) (see hipattn_prescale_k). */
+ *   k_prescaled != 0: kv->k already holds bf16(K * c_k) (see hipattn_prescale_k).
+ *   workspace: device scratch of hipattn_mask_stage_workspace_bytes(...) bytes. */
 int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, const int32_t *chunk_left,
                        int32_t hg, int32_t n, int32_t chunk_size, int64_t right_clamp,
                        int32_t bs, int32_t bq, int32_t stride_q, int32_t block_chunk,
                        int32_t scan_stride, int32_t sw_eff, int32_t terminate_size,
-                       int32_t k_prescaled, float *scores, int32_t *left_out, void *stream);
+                       int32_t k_prescaled, void *workspace, float *scores, int32_t *left_out,
+                       void *stream);
+
+/* Bytes of caller-allocated scratch hipattn_mask_stage needs (bf16: the averaged, scaled query rows
+ * of every scan program, [B, BS, HEAD, bq/stride_q, HID]; f32: 0, workspace may be NULL). */
+int64_t hipattn_mask_stage_workspace_bytes(int32_t dtype, int32_t B, int32_t bs, int32_t HEAD, int32_t HID,
+                                           int32_t bq, int32_t stride_q);
 
 /* K^ = bf16(K * c_k) for a whole bf16 key tensor viewed as [n0, n1, n2, HID] with element strides
  * (stride0, stride1, stride2, 1); `out` is contiguous [n0, n1, n2, HID].  Passing `out` as kv->k
