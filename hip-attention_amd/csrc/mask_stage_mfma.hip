@@ -44,7 +44,7 @@ __device__ __forceinline__ uint32_t scale_pack(uint32_t w, float c) {
 }
 
 template <int HID, int MB, int NB, bool PRESCALED, bool VIA_LDS>
-__global__ __launch_bounds__(64) void mask_stage_mfma_kernel(MaskParams p, int nsub) {
+__global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(MaskParams p, int nsub, int hpw) {
     constexpr int KS = HID / 16;
     constexpr int HALF = HID / 2;
     constexpr int PPR = HID / 8;                  // 16-byte pieces per key row
@@ -54,13 +54,17 @@ __global__ __launch_bounds__(64) void mask_stage_mfma_kernel(MaskParams p, int n
     constexpr int SWZ_DIV = PPR < 16 ? 16 / PPR : 1;
     __shared__ __align__(16) uint4 s_rows[VIA_LDS ? NROWS * PPR : 1];
     __shared__ int64_t s_off[VIA_LDS ? NROWS : 1];
-    const int lane = threadIdx.x;
+    // a workgroup holds `hpw` waves = `hpw` query heads of one GQA group working on the same chunks:
+    // their early-iteration samples coincide, so they share cache lines in the CU's L1
+    const int lane = threadIdx.x & 63;
     const int n = lane & 31, hh = lane >> 5;
     const int side = n & 1;
 
     long long L = xcd_remap((long long)blockIdx.x, p.total);
-    const int hin = (int)(L % p.G);
-    L /= p.G;
+    const int hblocks = (p.G + hpw - 1) / hpw;
+    const int hin = (int)(L % hblocks) * hpw + (int)(threadIdx.x >> 6);
+    L /= hblocks;
+    if (hin >= p.G) return;
     const int sub = (int)(L % nsub);
     L /= nsub;
     const int s = (int)(L % p.BS);
@@ -338,7 +342,16 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
     const bool wide = (BC >= 32) && (programs >= 16384);
     const int nb = wide ? 2 : 1;
     const int nsub = (BC / 16) / nb;
-    p.total = programs * nsub;
+    // LDS path: one wave per workgroup (it uses workgroup barriers); direct path: up to 4 heads per workgroup
+    // (measured: sharing pays with one query-row block per program, not with two)
+    if (g_mask_via_lds < 0) {
+        const char *e = getenv("HIPATTN_MASK_VIA_LDS");
+        g_mask_via_lds = e ? (e[0] == '1' ? 1 : 0) : 2;
+    }
+    const bool via_lds = g_mask_via_lds == 2 ? !wide : (g_mask_via_lds == 1);
+    const int hpw = (via_lds || two) ? 1 : (p.G < 4 ? p.G : 4);
+    const int hblocks = (p.G + hpw - 1) / hpw;
+    p.total = (long long)p.B * p.kv.HKV * hblocks * p.BS * p.ngroups * nsub;
     if (p.total >= 0x7fffffffLL) {
         set_error("mask stage: grid too large");
         return HIPATTN_E_UNSUPPORTED;
@@ -348,14 +361,9 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
         const long long blocks = (work + 255) / 256;
         hipLaunchKernelGGL(qhat_kernel, dim3((unsigned)blocks), dim3(256), 0, st, p, HID, const_cast<uint16_t *>(p.qhat));
     }
-    if (g_mask_via_lds < 0) {
-        const char *e = getenv("HIPATTN_MASK_VIA_LDS");
-        g_mask_via_lds = e ? (e[0] == '1' ? 1 : 0) : 2;
-    }
-    const bool via_lds = g_mask_via_lds == 2 ? !wide : (g_mask_via_lds == 1);
-    dim3 grid((unsigned)p.total), block(64);
+    dim3 grid((unsigned)p.total), block(64 * hpw);
 #define MS_LAUNCH(MBv, NBv, PSv, VLv) \
-    hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, NBv, PSv, VLv>), grid, block, 0, st, p, nsub)
+    hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, NBv, PSv, VLv>), grid, block, 0, st, p, nsub, hpw)
 #define MS_PICK(MBv, NBv)                                                \
     do {                                                                  \
         if (prescaled) { if (via_lds) MS_LAUNCH(MBv, NBv, true, true); else MS_LAUNCH(MBv, NBv, true, false); } \
