@@ -77,6 +77,13 @@ int make_kv_view(const hipattn_kv_t *kv, int B, int HID, int dtype, KVView *o) {
     o->block_table = kv->block_table; o->cache_seq_lens = kv->cache_seq_lens; o->bt_stride_b = kv->bt_stride_b;
     o->bt_is64 = kv->bt_is64; o->sl_is64 = kv->sl_is64; o->paged = kv->paged; o->page_size = kv->page_size ? kv->page_size : 1;
     o->HKV = kv->HKV;
+    o->cached = 0;
+    memset(&o->cache, 0, sizeof(o->cache));
+    o->access_flags = kv->access_flags;
+    o->miss_flags = kv->miss_flags;
+    o->flags_stride_b = kv->flags_stride_b;
+    o->flags_stride_h = kv->flags_stride_h;
+    if (kv->cache) return cache_view_for(kv->cache, kv, HID, dtype, o);
     return 0;
 }
 
@@ -102,6 +109,7 @@ extern "C" int hipattn_bsa_prefill(const hipattn_q_t *q, const hipattn_kv_t *kv,
     if (impl != 1) {
         BsaParams pm = p;
         if (k_prescaled) {  // same layout and strides as kv->k
+            HIPATTN_CHECK_ARG(!kv->cache, HIPATTN_E_ARG, "bsa: k_prescaled cannot be combined with an offload cache");
             HIPATTN_CHECK_ARG(aligned16(k_prescaled), HIPATTN_E_ALIGN, "bsa: k_prescaled must be 16-byte aligned");
             pm.kv.k = k_prescaled;
             pm.k_prescaled = 1;

@@ -15,7 +15,7 @@ struct DecodeParams {
     float *ws;  // [B, HEAD, nsplits, HID + 4]: acc / l, then m + log2(l)
 };
 
-template <typename T, int HID, int G>
+template <typename T, int HID, int G, bool EXT>
 __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParams dp) {
     constexpr int SEG = HID / 16;
     const BsaParams &p = dp.a;
@@ -89,16 +89,16 @@ __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParams dp
         }
         const bool att = valid && (kind == 0 ? (t + p.sw <= ppos) : (t <= ppos && ppos < t + p.sw));
         if (!att) continue;  // uniform inside the 16-lane group; shuffles below stay inside the group
-        const int64_t koff = p.kv.k_row(b, t, kvh, seqlen);
-        const int64_t voff = p.kv.v_row(b, t, kvh, seqlen);
+        int64_t koff, voff;
+        p.kv.rows<true, EXT>(b, t, kvh, seqlen, koff, voff);
         float kh[SEG], vv[SEG];
-        if (koff >= 0) {
+        if (koff != NO_ROW) {
             load_elems<T, SEG>(kbase + koff + dl * SEG, kh);
         } else {
 #pragma unroll
             for (int e = 0; e < SEG; e++) kh[e] = 0.0f;
         }
-        if (voff >= 0) {
+        if (voff != NO_ROW) {
             load_elems<T, SEG>(vbase + voff + dl * SEG, vv);
         } else {
 #pragma unroll
@@ -184,7 +184,10 @@ static int launch_partial(const DecodeParams &dp, hipStream_t st) {
 #define DEC_CASE(GG)                                                                                   \
     if constexpr (GG * HID <= 512) {                                                                   \
         if (dp.a.G == GG) {                                                                            \
-            hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG>), grid, block, 0, st, dp);       \
+            if (dp.a.kv.extended())                                                                    \
+                hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG, true>), grid, block, 0, st, dp);  \
+            else                                                                                       \
+                hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG, false>), grid, block, 0, st, dp); \
             launched = true;                                                                           \
         }                                                                                              \
     }

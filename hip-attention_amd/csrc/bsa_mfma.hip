@@ -50,7 +50,7 @@ struct MfmaSmem {
     int idx[MAX_LDS_IDX];
 };
 
-template <int HID, bool KSCALED>
+template <int HID, bool KSCALED, bool EXT>
 __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParams p, int hgroups, int hpw, long long total_wg) {
     constexpr int KS = HID / 16;   // k-steps of the first product
     constexpr int DB = HID / 32;   // 32-row blocks of O^T
@@ -178,10 +178,10 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParams p, int hgr
             kreg[j] = make_uint4(0, 0, 0, 0);
             vreg[j] = make_uint4(0, 0, 0, 0);
             if (t >= 0) {
-                const int64_t ko = p.kv.k_row(b, t, kvh, seqlen);
-                const int64_t vo = p.kv.v_row(b, t, kvh, seqlen);
-                if (ko >= 0) kreg[j] = *reinterpret_cast<const uint4 *>(kbase + ko + piece * 8);
-                if (vo >= 0) vreg[j] = *reinterpret_cast<const uint4 *>(vbase + vo + piece * 8);
+                int64_t ko, vo;
+                p.kv.rows<true, EXT>(b, t, kvh, seqlen, ko, vo);
+                if (ko != NO_ROW) kreg[j] = *reinterpret_cast<const uint4 *>(kbase + ko + piece * 8);
+                if (vo != NO_ROW) vreg[j] = *reinterpret_cast<const uint4 *>(vbase + vo + piece * 8);
             }
         }
     };
@@ -339,7 +339,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParams p, int hgr
         }
 }
 
-template <int HID, bool KSCALED>
+template <int HID, bool KSCALED, bool EXT>
 static int launch_mfma(const BsaParams &p, hipStream_t st) {
     const int hpw = p.share_first_head ? 4 : 1;  // per-head index rows: one head per workgroup
     const int hgroups = (p.G + hpw - 1) / hpw;
@@ -348,11 +348,11 @@ static int launch_mfma(const BsaParams &p, hipStream_t st) {
     const size_t smem = sizeof(MfmaSmem<HID>);
     static bool attr_set = false;
     if (!attr_set) {
-        HIPATTN_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&bsa_mfma_kernel<HID, KSCALED>),
+        HIPATTN_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&bsa_mfma_kernel<HID, KSCALED, EXT>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
-    hipLaunchKernelGGL((bsa_mfma_kernel<HID, KSCALED>), dim3((unsigned)total), dim3(NTHREADS), smem, st, p, hgroups,
+    hipLaunchKernelGGL((bsa_mfma_kernel<HID, KSCALED, EXT>), dim3((unsigned)total), dim3(NTHREADS), smem, st, p, hgroups,
                        hpw, total);
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
@@ -362,17 +362,16 @@ int bsa_mfma_launch(const BsaParams &p, int dtype, int HID, hipStream_t st) {
     if (dtype != HIPATTN_BF16) return HIPATTN_E_UNSUPPORTED;
     if (p.bq > 64) return HIPATTN_E_UNSUPPORTED;
     if ((p.o_st % 4) != 0 || (p.o_sh % 4) != 0 || (p.o_sb % 4) != 0) return HIPATTN_E_UNSUPPORTED;
-    if (p.k_prescaled) {
-        switch (HID) {
-            case 64: return launch_mfma<64, true>(p, st);
-            case 128: return launch_mfma<128, true>(p, st);
-        }
-    } else {
-        switch (HID) {
-            case 64: return launch_mfma<64, false>(p, st);
-            case 128: return launch_mfma<128, false>(p, st);
-        }
+    const bool ext = p.kv.extended();
+#define BSA_PICK(H)                                                                  \
+    case H:                                                                          \
+        if (p.k_prescaled) return ext ? launch_mfma<H, true, true>(p, st) : launch_mfma<H, true, false>(p, st); \
+        return ext ? launch_mfma<H, false, true>(p, st) : launch_mfma<H, false, false>(p, st);
+    switch (HID) {
+        BSA_PICK(64)
+        BSA_PICK(128)
     }
+#undef BSA_PICK
     return HIPATTN_E_UNSUPPORTED;
 }
 

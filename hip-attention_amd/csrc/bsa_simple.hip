@@ -82,12 +82,12 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
             }
             const bool att = valid && (kind == 0 ? (t + p.sw <= ppos) : (t <= ppos && ppos < t + p.sw));
             float logit = -INFINITY;
-            int64_t voff = -1;
+            int64_t voff = NO_ROW;
             if (att) {
-                const int64_t koff = p.kv.k_row(b, t, kvh, seqlen);
-                voff = p.kv.v_row(b, t, kvh, seqlen);
+                int64_t koff;
+                p.kv.rows<true, true>(b, t, kvh, seqlen, koff, voff);
                 float dot = 0.0f;
-                if (koff >= 0) {
+                if (koff != NO_ROW) {
                     constexpr int CH = 16 / (int)sizeof(T) < HID ? 16 / (int)sizeof(T) : HID;
                     for (int d0 = 0; d0 < HID; d0 += CH) {
                         float kk[CH];
@@ -114,7 +114,7 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
                     live &= live - 1;
                     const float pj = __shfl(prT, src);
                     const long long vo = __shfl((long long)voff, src);
-                    if (vo >= 0) {
+                    if (vo != (long long)NO_ROW) {
 #pragma unroll
                         for (int e = 0; e < DPL; e++) {
                             const int d = lane + e * 64;

@@ -126,6 +126,29 @@ __device__ __forceinline__ void load_elems(const T *p, float (&out)[N]) {
 }
 
 // ---------------------------------------------------------------- KV addressing (device copy of hipattn_kv_t)
+// Block cache in front of a host-resident pool: what the kernels need of a hipattn_cache_t.
+// "no such row" marker for row offsets.  Offsets are relative to the K / V base pointer and may be negative
+// when they lead into an offload cache's bank, so the marker is not simply "below zero".
+constexpr int64_t NO_ROW = INT64_MIN;
+
+struct CacheView {
+    const int32_t *table;   // [HKV, n_blocks] slot or -1
+    int32_t *last_use;      // [slots] step of the last read
+    uint8_t *miss;          // [HKV, n_blocks] set when a read went to the host pool
+    const int32_t *step;    // current step counter
+    int64_t k_delta;        // element offset from KVView::k to the K part of slot 0
+    int64_t v_delta;        // element offset from KVView::v to the V part of slot 0
+    int64_t slot_stride;    // elements per slot
+    int64_t n_blocks;
+    int32_t shift;          // log2(block_tokens)
+    int32_t row_elems;      // HID
+    int32_t with_v;         // slots hold V rows too
+};
+
+__device__ __forceinline__ void mark_flag(int32_t *f) {
+    if (*f == 0) *f = 1;  // racing lanes store the same value; a stale read only repeats the store
+}
+
 struct KVView {
     const void *k;
     const void *v;
@@ -137,44 +160,77 @@ struct KVView {
     const void *cache_seq_lens;
     int64_t bt_stride_b;
     int bt_is64, sl_is64, paged, page_size, HKV;
+    int cached;
+    CacheView cache;
+    int32_t *access_flags, *miss_flags;
+    int64_t flags_stride_b, flags_stride_h;
 
     __device__ __forceinline__ int64_t seq_len(int b) const {
         return sl_is64 ? reinterpret_cast<const int64_t *>(cache_seq_lens)[b]
                        : (int64_t) reinterpret_cast<const int32_t *>(cache_seq_lens)[b];
     }
-    // element offset of the K row of token t (kv head h) or -1 for "zero row"
+    __device__ __forceinline__ int64_t page_of(int b, int64_t t, int64_t seqlen) const {
+        int64_t page = 0;
+        if (t >= 0 && t < seqlen) {
+            int64_t i = (int64_t)b * bt_stride_b + t / page_size;
+            page = bt_is64 ? reinterpret_cast<const int64_t *>(block_table)[i]
+                           : (int64_t) reinterpret_cast<const int32_t *>(block_table)[i];
+        }
+        return page;
+    }
+    // Element offsets (from k and v) of the rows of token t, kv head h; NO_ROW = "zero row".
+    // WANT_V = false skips the V side.  EXT = true also records the access and consults the block cache;
+    // kernels are built both ways so that the plain path does not carry the extra arguments.
+    template <bool WANT_V, bool EXT>
+    __device__ __forceinline__ void rows(int b, int64_t t, int h, int64_t seqlen, int64_t &ko, int64_t &vo) const {
+        ko = NO_ROW;
+        vo = NO_ROW;
+        if (!paged) {
+            if (t < 0 || t >= tsrc) return;
+            if (EXT && access_flags)
+                mark_flag(access_flags + (int64_t)b * flags_stride_b + (int64_t)h * flags_stride_h + t);
+            ko = (int64_t)b * k_stride_b + t * k_stride_t + (int64_t)h * k_stride_h;
+            if (WANT_V) vo = (int64_t)b * v_stride_b + t * v_stride_t + (int64_t)h * v_stride_h;
+            return;
+        }
+        if (t < 0) return;
+        const int64_t page = page_of(b, t, seqlen);
+        const int64_t inpage = t % page_size;
+        if (EXT && access_flags)
+            mark_flag(access_flags + (int64_t)b * flags_stride_b + (int64_t)h * flags_stride_h + page);
+        if (EXT && cached) {
+            const int64_t row = page * page_size + inpage;
+            const int64_t e = (int64_t)h * cache.n_blocks + (row >> cache.shift);
+            const int32_t slot = cache.table[e];
+            if (slot >= 0) {
+                const int32_t now = *cache.step;
+                if (cache.last_use[slot] != now) cache.last_use[slot] = now;
+                const int64_t o = (int64_t)slot * cache.slot_stride +
+                                  (row & ((1LL << cache.shift) - 1)) * cache.row_elems;
+                ko = cache.k_delta + o;
+                if (WANT_V)
+                    vo = cache.with_v ? cache.v_delta + o
+                                      : page * v_stride_b + inpage * v_stride_t + (int64_t)h * v_stride_h;
+                return;
+            }
+            if (cache.miss[e] == 0) cache.miss[e] = 1;
+            if (miss_flags) mark_flag(miss_flags + (int64_t)b * flags_stride_b + (int64_t)h * flags_stride_h + page);
+        }
+        ko = page * k_stride_b + inpage * k_stride_t + (int64_t)h * k_stride_h;
+        if (WANT_V) vo = page * v_stride_b + inpage * v_stride_t + (int64_t)h * v_stride_h;
+    }
+    template <bool EXT>
     __device__ __forceinline__ int64_t k_row(int b, int64_t t, int h, int64_t seqlen) const {
-        if (!paged) {
-            if (t < 0 || t >= tsrc) return -1;
-            return (int64_t)b * k_stride_b + t * k_stride_t + (int64_t)h * k_stride_h;
-        }
-        int64_t page = 0;
-        if (t >= 0 && t < seqlen) {
-            int64_t i = (int64_t)b * bt_stride_b + t / page_size;
-            page = bt_is64 ? reinterpret_cast<const int64_t *>(block_table)[i]
-                           : (int64_t) reinterpret_cast<const int32_t *>(block_table)[i];
-        }
-        if (t < 0) return -1;
-        return page * k_stride_b + (t % page_size) * k_stride_t + (int64_t)h * k_stride_h;
+        int64_t ko, vo;
+        rows<false, EXT>(b, t, h, seqlen, ko, vo);
+        return ko;
     }
-    // same page arithmetic for V given the K offset's (page, in-page) decomposition is not shared:
-    __device__ __forceinline__ int64_t v_row(int b, int64_t t, int h, int64_t seqlen) const {
-        if (!paged) {
-            if (t < 0 || t >= tsrc) return -1;
-            return (int64_t)b * v_stride_b + t * v_stride_t + (int64_t)h * v_stride_h;
-        }
-        int64_t page = 0;
-        if (t >= 0 && t < seqlen) {
-            int64_t i = (int64_t)b * bt_stride_b + t / page_size;
-            page = bt_is64 ? reinterpret_cast<const int64_t *>(block_table)[i]
-                           : (int64_t) reinterpret_cast<const int32_t *>(block_table)[i];
-        }
-        if (t < 0) return -1;
-        return page * v_stride_b + (t % page_size) * v_stride_t + (int64_t)h * v_stride_h;
-    }
+    // host: does a launch need the EXT build of its kernel
+    bool extended() const { return cached || access_flags || miss_flags; }
 };
 
 int make_kv_view(const hipattn_kv_t *kv, int B, int HID, int dtype, KVView *out);
+int cache_view_for(const hipattn_cache *c, const hipattn_kv_t *kv, int HID, int dtype, KVView *out);
 int check_q(const hipattn_q_t *q);
 
 // ---------------------------------------------------------------- wave helpers

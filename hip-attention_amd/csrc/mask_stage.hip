@@ -163,10 +163,10 @@ __global__ __launch_bounds__(64) void mask_stage_kernel(MaskParams p) {
         const bool active = real && (l < r) && (l <= lim) && (l >= 0);
         const int c = (l + r) >> 1;
         if (lane < BC) {
-            int64_t o0 = -1, o1 = -1;
+            int64_t o0 = NO_ROW, o1 = NO_ROW;
             if (active) {
-                o0 = p.kv.k_row(b, (l + c) >> 1, kvh, seqlen);
-                o1 = p.kv.k_row(b, (c + r) >> 1, kvh, seqlen);
+                o0 = p.kv.k_row<true>(b, (l + c) >> 1, kvh, seqlen);
+                o1 = p.kv.k_row<true>(b, (c + r) >> 1, kvh, seqlen);
             }
             s_koff[2 * lane] = o0;
             s_koff[2 * lane + 1] = o1;
@@ -181,7 +181,7 @@ __global__ __launch_bounds__(64) void mask_stage_kernel(MaskParams p) {
             for (int st = 0; st < STEPS; st++) {
                 const int krow = (cs + st) * 4 + sub;
                 const int64_t off = (cs + st) < nsteps ? s_koff[krow] : -1;
-                if (off >= 0) raw[st].load(kbase + off + dl * SEG);
+                if (off != NO_ROW) raw[st].load(kbase + off + dl * SEG);
                 else raw[st].zero();
             }
             for (int pass = 0; pass < npass; pass++) {

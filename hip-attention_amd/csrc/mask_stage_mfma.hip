@@ -43,7 +43,7 @@ __device__ __forceinline__ uint32_t scale_pack(uint32_t w, float c) {
     return cvt_pk_bf16(__uint_as_float(w << 16) * c, __uint_as_float(w & 0xffff0000u) * c);
 }
 
-template <int HID, int MB, int NB, bool PRESCALED, bool VIA_LDS>
+template <int HID, int MB, int NB, bool PRESCALED, bool VIA_LDS, bool EXT>
 __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(MaskParams p, int nsub, int hpw) {
     constexpr int KS = HID / 16;
     constexpr int HALF = HID / 2;
@@ -189,10 +189,10 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
         for (int tb = 0; tb < NB; tb++) {
             active[tb] = real[tb] && (cl[tb] < cr[tb]) && (cl[tb] <= lim) && (cl[tb] >= 0);
             ctr[tb] = (cl[tb] + cr[tb]) >> 1;
-            int64_t off = -1;
+            int64_t off = NO_ROW;
             if (active[tb]) {
                 const int t = side ? ((ctr[tb] + cr[tb]) >> 1) : ((cl[tb] + ctr[tb]) >> 1);
-                off = p.kv.k_row(b, t, kvh, seqlen);
+                off = p.kv.k_row<EXT>(b, t, kvh, seqlen);
             }
             if constexpr (VIA_LDS) {
                 if (hh == 0) s_off[tb * 32 + n] = off;
@@ -200,7 +200,7 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
 #pragma unroll
                 for (int ks = 0; ks < KS; ks++) {
                     raw[tb][ks] = make_uint4(0, 0, 0, 0);
-                    if (off >= 0) raw[tb][ks] = *reinterpret_cast<const uint4 *>(kbase + off + hh * HALF + ks * 8);
+                    if (off != NO_ROW) raw[tb][ks] = *reinterpret_cast<const uint4 *>(kbase + off + hh * HALF + ks * 8);
                 }
             }
         }
@@ -213,7 +213,7 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
                 const int64_t off = s_off[r];
                 const int q = lpos ^ ((r / SWZ_DIV) & SWZ);
                 uint4 v = make_uint4(0, 0, 0, 0);
-                if (off >= 0) v = *reinterpret_cast<const uint4 *>(kbase + off + q * 8);
+                if (off != NO_ROW) v = *reinterpret_cast<const uint4 *>(kbase + off + q * 8);
                 if (!PRESCALED) {
                     v.x = scale_pack(v.x, p.c_k);
                     v.y = scale_pack(v.y, p.c_k);
@@ -348,7 +348,8 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
         const char *e = getenv("HIPATTN_MASK_VIA_LDS");
         g_mask_via_lds = e ? (e[0] == '1' ? 1 : 0) : 2;
     }
-    const bool via_lds = g_mask_via_lds == 2 ? !wide : (g_mask_via_lds == 1);
+    const bool ext = p.kv.extended();  // statistics / offload cache: built for the direct path only
+    const bool via_lds = !ext && (g_mask_via_lds == 2 ? !wide : (g_mask_via_lds == 1));
     const int hpw = (via_lds || two) ? 1 : (p.G < 4 ? p.G : 4);
     const int hblocks = (p.G + hpw - 1) / hpw;
     p.total = (long long)p.B * p.kv.HKV * hblocks * p.BS * p.ngroups * nsub;
@@ -362,8 +363,13 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
         hipLaunchKernelGGL(qhat_kernel, dim3((unsigned)blocks), dim3(256), 0, st, p, HID, const_cast<uint16_t *>(p.qhat));
     }
     dim3 grid((unsigned)p.total), block(64 * hpw);
-#define MS_LAUNCH(MBv, NBv, PSv, VLv) \
-    hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, NBv, PSv, VLv>), grid, block, 0, st, p, nsub, hpw)
+#define MS_LAUNCH(MBv, NBv, PSv, VLv)                                                                                 \
+    do {                                                                                                              \
+        if (ext && !VLv)                                                                                              \
+            hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, NBv, PSv, false, true>), grid, block, 0, st, p, nsub, hpw); \
+        else                                                                                                          \
+            hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, NBv, PSv, VLv, false>), grid, block, 0, st, p, nsub, hpw);  \
+    } while (0)
 #define MS_PICK(MBv, NBv)                                                \
     do {                                                                  \
         if (prescaled) { if (via_lds) MS_LAUNCH(MBv, NBv, true, true); else MS_LAUNCH(MBv, NBv, true, false); } \

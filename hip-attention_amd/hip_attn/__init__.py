@@ -12,6 +12,7 @@ from .operator import dual_stage_quadratic_hip_attention as hip_attention_12
 from .config import HiPAttentionConfig, HiPAttentionPerLayerConfig
 from .refresh import HiPMaskRefreshState
 from .paged import forward_paged_hip
+from .offload import HiPOffloadCache
 
 hip_attention = hip_attention_12
 HiPAttentionArgs = HiPAttentionArgs12
@@ -32,4 +33,5 @@ __all__ = [
     "HiPAttentionPerLayerConfig",
     "HiPMaskRefreshState",
     "forward_paged_hip",
+    "HiPOffloadCache",
 ]

@@ -45,6 +45,29 @@ class KVStruct(ctypes.Structure):
         ("bt_is64", ctypes.c_int32), ("sl_is64", ctypes.c_int32),
         ("paged", ctypes.c_int32), ("page_size", ctypes.c_int32),
         ("HKV", ctypes.c_int32),
+        ("cache", ctypes.c_void_p),
+        ("access_flags", ctypes.c_void_p), ("miss_flags", ctypes.c_void_p),
+        ("flags_stride_b", ctypes.c_int64), ("flags_stride_h", ctypes.c_int64),
+    ]
+
+
+class CacheDesc(ctypes.Structure):
+    _fields_ = [
+        ("dtype", ctypes.c_int32), ("HKV", ctypes.c_int32), ("HID", ctypes.c_int32),
+        ("block_tokens", ctypes.c_int32), ("with_v", ctypes.c_int32),
+        ("pool_rows", ctypes.c_int64), ("slots", ctypes.c_int64),
+        ("host_k", ctypes.c_void_p), ("host_v", ctypes.c_void_p),
+        ("host_stride_row", ctypes.c_int64), ("host_stride_h", ctypes.c_int64),
+        ("bank", ctypes.c_void_p), ("table", ctypes.c_void_p), ("last_use", ctypes.c_void_p),
+        ("backref", ctypes.c_void_p), ("miss", ctypes.c_void_p), ("workspace", ctypes.c_void_p),
+    ]
+
+
+class CacheSizes(ctypes.Structure):
+    _fields_ = [
+        ("n_blocks", ctypes.c_int64), ("bank_bytes", ctypes.c_int64), ("table_bytes", ctypes.c_int64),
+        ("last_use_bytes", ctypes.c_int64), ("backref_bytes", ctypes.c_int64), ("miss_bytes", ctypes.c_int64),
+        ("workspace_bytes", ctypes.c_int64),
     ]
 
 
@@ -67,8 +90,14 @@ def lib():
         L.hipattn_mask_stage_workspace_bytes.restype = ctypes.c_int64
         L.hipattn_bsa_decode_default_splits.restype = ctypes.c_int32
         for name in ("hipattn_mask_stage", "hipattn_prescale_k", "hipattn_select_stage", "hipattn_finalize_indices",
-                     "hipattn_bsa_prefill", "hipattn_bsa_decode_partial", "hipattn_bsa_decode_merge"):
+                     "hipattn_bsa_prefill", "hipattn_bsa_decode_partial", "hipattn_bsa_decode_merge",
+                     "hipattn_cache_sizes", "hipattn_cache_create", "hipattn_cache_flush",
+                     "hipattn_cache_lookup_and_schedule", "hipattn_cache_commit", "hipattn_cache_write_rows",
+                     "hipattn_cache_stats", "hipattn_pool_write_rows", "hipattn_host_device_pointer",
+                     "hipattn_host_alloc", "hipattn_host_free"):
             getattr(L, name).restype = ctypes.c_int
+        L.hipattn_cache_destroy.restype = None
+        L.hipattn_cache_destroy.argtypes = [ctypes.c_void_p]
         _lib = L
     return _lib
 
@@ -121,6 +150,19 @@ def make_kv_dense(k: torch.Tensor, v: torch.Tensor) -> KVStruct:
     s.page_size = 1
     s.HKV = k.shape[2]
     return s
+
+
+def set_flags(s: KVStruct, access: Optional[torch.Tensor], miss: Optional[torch.Tensor]) -> KVStruct:
+    """Attach ``int32 [B, HKV, pages]`` access / miss flag tensors to a KV description (returns a copy)."""
+    out = KVStruct.from_buffer_copy(s)
+    if access is not None:
+        assert access.dtype == torch.int32 and access.ndim == 3 and access.stride(2) == 1
+        out.access_flags = access.data_ptr()
+        out.flags_stride_b, out.flags_stride_h = access.stride(0), access.stride(1)
+        if miss is not None:
+            assert miss.shape == access.shape and miss.stride() == access.stride() and miss.dtype == torch.int32
+            out.miss_flags = miss.data_ptr()
+    return out
 
 
 def make_kv_paged(k_cache, v_cache, block_table, cache_seq_lens, max_tsrc: int) -> KVStruct:
@@ -272,3 +314,97 @@ def bsa_decode(qs, kvs, indices, ks_start_end, BK, bk, sw, sink, out, device, ns
         stream_ptr(device))
     check(rc, "hipattn_bsa_decode_merge")
     return workspace
+
+
+# ------------------------------------------------------------------ offload cache
+
+class HostPool:
+    """Pinned host memory from ``hipattn_host_alloc`` exposed as a CPU tensor; freed with the object."""
+
+    def __init__(self, shape, dtype: torch.dtype, coherent: bool = True):
+        n = 1
+        for d in shape:
+            n *= int(d)
+        self.nbytes = max(16, n * torch.empty((), dtype=dtype).element_size())
+        out = ctypes.c_void_p(0)
+        check(lib().hipattn_host_alloc(ctypes.c_int64(self.nbytes), ctypes.c_int32(int(coherent)), ctypes.byref(out)),
+              "hipattn_host_alloc")
+        self.ptr = int(out.value)
+        buf = (ctypes.c_uint8 * self.nbytes).from_address(self.ptr)
+        self.tensor = torch.frombuffer(buf, dtype=dtype, count=n).view(*shape)
+
+    def __del__(self):
+        p, self.ptr = getattr(self, "ptr", 0), 0
+        try:
+            if p and _lib is not None:
+                self.tensor = None
+                _lib.hipattn_host_free(ctypes.c_void_p(p))
+        except Exception:  # interpreter shutdown
+            pass
+
+
+def host_device_pointer(t: torch.Tensor) -> int:
+    """Device-visible address of a pinned host tensor."""
+    assert not t.is_cuda, "the host pool must live in pinned host memory"
+    out = ctypes.c_void_p(0)
+    rc = lib().hipattn_host_device_pointer(ctypes.c_void_p(t.data_ptr()), ctypes.byref(out))
+    check(rc, "hipattn_host_device_pointer")
+    return int(out.value)
+
+
+def cache_sizes(desc: CacheDesc, max_fetch: int) -> CacheSizes:
+    out = CacheSizes()
+    check(lib().hipattn_cache_sizes(ctypes.byref(desc), ctypes.c_int64(max_fetch), ctypes.byref(out)),
+          "hipattn_cache_sizes")
+    return out
+
+
+def cache_create(desc: CacheDesc, max_fetch: int, device) -> int:
+    handle = ctypes.c_void_p(0)
+    check(lib().hipattn_cache_create(ctypes.byref(desc), ctypes.c_int64(max_fetch), ctypes.byref(handle),
+                                     stream_ptr(device)), "hipattn_cache_create")
+    return int(handle.value)
+
+
+def cache_destroy(handle: int):
+    if _lib is not None and handle and ctypes is not None:
+        _lib.hipattn_cache_destroy(ctypes.c_void_p(handle))
+
+
+def cache_flush(handle: int, device):
+    check(lib().hipattn_cache_flush(ctypes.c_void_p(handle), stream_ptr(device)), "hipattn_cache_flush")
+
+
+def cache_schedule(handle: int, device):
+    with _timed("cache_lookup_and_schedule"):
+        rc = lib().hipattn_cache_lookup_and_schedule(ctypes.c_void_p(handle), stream_ptr(device))
+    check(rc, "hipattn_cache_lookup_and_schedule")
+
+
+def cache_commit(handle: int, device):
+    with _timed("cache_commit"):
+        rc = lib().hipattn_cache_commit(ctypes.c_void_p(handle), stream_ptr(device))
+    check(rc, "hipattn_cache_commit")
+
+
+def cache_write_rows(handle: int, rows: torch.Tensor, k_rows: torch.Tensor, v_rows: Optional[torch.Tensor], device):
+    assert rows.dtype == torch.int64 and rows.is_cuda and rows.is_contiguous()
+    assert k_rows.is_cuda and k_rows.is_contiguous() and (v_rows is None or (v_rows.is_cuda and v_rows.is_contiguous()))
+    check(lib().hipattn_cache_write_rows(ctypes.c_void_p(handle), _p(rows), ctypes.c_int64(rows.numel()), _p(k_rows),
+                                         _p(v_rows), stream_ptr(device)), "hipattn_cache_write_rows")
+
+
+def cache_stats(handle: int, device) -> list:
+    out = (ctypes.c_int64 * 8)()
+    check(lib().hipattn_cache_stats(ctypes.c_void_p(handle), out, stream_ptr(device)), "hipattn_cache_stats")
+    return list(out)
+
+
+def pool_write_rows(pool_ptr: int, stride_row: int, stride_h: int, HKV: int, HID: int, dtype: int,
+                    rows: torch.Tensor, src: torch.Tensor, device):
+    """Scatter device rows ``src [n, HKV, HID]`` into the pinned host pool at ``rows``."""
+    assert rows.dtype == torch.int64 and rows.is_cuda and rows.is_contiguous() and src.is_cuda and src.is_contiguous()
+    check(lib().hipattn_pool_write_rows(ctypes.c_void_p(pool_ptr), ctypes.c_int64(stride_row), ctypes.c_int64(stride_h),
+                                        ctypes.c_int32(HKV), ctypes.c_int32(HID), ctypes.c_int32(dtype), _p(rows),
+                                        ctypes.c_int64(rows.numel()), _p(src), stream_ptr(device)),
+          "hipattn_pool_write_rows")

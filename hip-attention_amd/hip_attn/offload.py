@@ -1,0 +1,230 @@
+"""KV offloading: keys and values live in pinned host memory, a block cache in HBM serves the kernels.
+
+Takes the place of ``UVMCache`` / ``GPUCache`` / ``HiPOffloadCache`` of the reference
+(``src/hip_attn/v1_2/uvm_gpu_cache.py:72-117,204-566,569-700``) with the same constructor arguments and
+methods, re-designed for this hardware:
+
+* the host pool is ordinary pinned memory that the GPU reads in place over the host link (the reference
+  uses managed memory advised to stay on the CPU);
+* the cache is block granular (``block_tokens`` consecutive pool rows of one kv head per slot) instead
+  of token granular, so one table lookup covers a whole 16-token attention block;
+* there are two caches as in the reference -- a large key-only one for mask estimation and a key+value
+  one for sparse attention -- and replacement is exact LRU by the step of the last read;
+* misses do not stall anything: the reading kernel takes the row from the host pool and flags the block;
+  ``handle_cache_miss`` brings the flagged blocks in afterwards with device-side kernels (no host round
+  trip), optionally on a side stream so that the copy overlaps whatever runs next.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from . import _native as N
+
+
+class UVMCache:
+    """Host pool ``[max_token_size, head_num, head_dim]`` in pinned memory (``uvm_gpu_cache.py:72-117``)."""
+
+    def __init__(self, layer_id: int, max_token_size: int, head_num: int, head_dim: int, dtype: torch.dtype,
+                 device: torch.device):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise NotImplementedError(f"offload pool dtype {dtype}: only bfloat16 and float32 are built")
+        self.layer_id = layer_id
+        self.max_token_size = max_token_size
+        self.head_num = head_num
+        self.head_dim = head_dim
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.bank_cpu = torch.zeros((max_token_size, head_num, head_dim), dtype=dtype, pin_memory=True)
+        self.device_ptr = N.host_device_pointer(self.bank_cpu)
+        # per-token generation, bumped on every overwrite (uvm_gpu_cache.py:109-114,681-688)
+        self.metadata = torch.zeros((max_token_size, 1), dtype=torch.int32, device=self.device)
+
+    def gather_cpu(self, table: Tensor, pin_memory: bool = False) -> Tensor:
+        out = torch.empty((table.numel(), self.head_num, self.head_dim), dtype=self.dtype, pin_memory=pin_memory)
+        torch.index_select(self.bank_cpu, 0, table.reshape(-1).to(torch.int64), out=out)
+        return out
+
+
+class GPUCache:
+    """Block cache in device memory over one or two host pools (``uvm_gpu_cache.py:204-566``)."""
+
+    def __init__(self, k_uvm: UVMCache, v_uvm: Optional[UVMCache], max_cache_token_size: int,
+                 online_cache_update: bool = False, block_tokens: int = 16, max_fetch: Optional[int] = None):
+        if online_cache_update:
+            raise NotImplementedError("online_cache_update (cache fill inside the attention kernel) is not built")
+        self.k_uvm = k_uvm
+        self.v_uvm = v_uvm
+        self.kv_packed = v_uvm is not None
+        self.device = k_uvm.device
+        self.block_tokens = block_tokens
+        self.max_cache_token_size = max_cache_token_size
+        self.slots = max(1, max_cache_token_size // block_tokens)
+        self.max_fetch = int(max_fetch if max_fetch is not None else min(self.slots, 65536))
+
+        d = N.CacheDesc()
+        d.dtype = N.dtype_code(k_uvm.bank_cpu)
+        d.HKV, d.HID = k_uvm.head_num, k_uvm.head_dim
+        d.block_tokens = block_tokens
+        d.with_v = int(self.kv_packed)
+        d.pool_rows = k_uvm.max_token_size
+        d.slots = self.slots
+        d.host_k = k_uvm.device_ptr
+        d.host_v = v_uvm.device_ptr if v_uvm is not None else 0
+        d.host_stride_row, d.host_stride_h = k_uvm.bank_cpu.stride(0), k_uvm.bank_cpu.stride(1)
+        if v_uvm is not None:
+            assert v_uvm.bank_cpu.shape == k_uvm.bank_cpu.shape and v_uvm.bank_cpu.stride() == k_uvm.bank_cpu.stride()
+        sz = N.cache_sizes(d, self.max_fetch)
+        self.n_blocks = sz.n_blocks
+        dev = self.device
+        esz = k_uvm.bank_cpu.element_size()
+        self.bank = torch.empty(sz.bank_bytes // esz, dtype=k_uvm.dtype, device=dev)
+        self.table = torch.empty((k_uvm.head_num, sz.n_blocks), dtype=torch.int32, device=dev)
+        self.last_use = torch.empty(self.slots, dtype=torch.int32, device=dev)
+        self.backref = torch.empty(self.slots, dtype=torch.int32, device=dev)
+        self.miss = torch.empty((k_uvm.head_num, sz.n_blocks), dtype=torch.uint8, device=dev)
+        self.workspace = torch.empty(sz.workspace_bytes, dtype=torch.uint8, device=dev)
+        d.bank, d.table, d.last_use = self.bank.data_ptr(), self.table.data_ptr(), self.last_use.data_ptr()
+        d.backref, d.miss, d.workspace = self.backref.data_ptr(), self.miss.data_ptr(), self.workspace.data_ptr()
+        self._desc = d
+        self.handle = N.cache_create(d, self.max_fetch, dev)
+        self._ready: Optional[torch.cuda.Event] = None
+
+    def __del__(self):
+        h, self.handle = getattr(self, "handle", 0), 0
+        try:
+            if h:
+                N.cache_destroy(h)
+        except Exception:  # interpreter shutdown: the module may already be torn down
+            pass
+
+    def flush(self):
+        self.wait()
+        N.cache_flush(self.handle, self.device)
+
+    def wait(self):
+        """Order the current stream after the last ``handle_cache_miss`` issued on another stream."""
+        if self._ready is not None:
+            torch.cuda.current_stream(self.device).wait_event(self._ready)
+            self._ready = None
+
+    def handle_cache_miss(self, metadata=None, stats=None, stream: Optional[torch.cuda.Stream] = None):
+        """Bring the blocks flagged during the last step into the cache (``uvm_gpu_cache.py:305-398``).
+
+        ``metadata`` / ``stats`` are accepted for signature compatibility: the readers already recorded
+        what missed.  With ``stream`` the work runs there, after everything enqueued so far on the current
+        stream; the next attention call waits for it.
+        """
+        if stream is None:
+            self.wait()
+            N.cache_schedule(self.handle, self.device)
+            N.cache_commit(self.handle, self.device)
+            return
+        stream.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(stream):
+            N.cache_schedule(self.handle, self.device)
+            N.cache_commit(self.handle, self.device)
+            self._ready = torch.cuda.Event()
+            self._ready.record(stream)
+
+    def on_set_kv_buffer(self, table: Tensor, cache_k: Tensor, cache_v: Optional[Tensor]):
+        """Resident blocks receive freshly written rows (``uvm_gpu_cache.py:548-563``)."""
+        self.wait()
+        rows = table.reshape(-1).to(device=self.device, dtype=torch.int64).contiguous()
+        k_rows = cache_k.to(self.device).contiguous()
+        v_rows = cache_v.to(self.device).contiguous() if (self.kv_packed and cache_v is not None) else None
+        N.cache_write_rows(self.handle, rows, k_rows, v_rows, self.device)
+
+    def statistics(self) -> dict:
+        s = N.cache_stats(self.handle, self.device)
+        keys = ("steps", "blocks_hit", "blocks_missed", "blocks_fetched", "blocks_evicted", "last_hit", "last_missed",
+                "last_fetched")
+        return dict(zip(keys, s))
+
+
+class HiPOffloadCache:
+    """Host-resident K/V of one layer with its two device caches (``uvm_gpu_cache.py:569-700``)."""
+
+    def __init__(self, layer_id: int, max_token_size: int, max_mask_cache_token_size: int,
+                 max_sa_cache_token_size: int, head_num: int, head_dim: int, dtype: torch.dtype,
+                 device: torch.device, online_cache_update: bool = False, block_tokens: int = 16,
+                 max_fetch: Optional[int] = None):
+        self.layer_id = layer_id
+        self.device = torch.device(device)
+        self.head_kv = head_num
+        self.head_dim = head_dim
+        self.page_size = 1
+        self.k_uvm = UVMCache(layer_id, max_token_size, head_num, head_dim, dtype, device)
+        self.v_uvm = UVMCache(layer_id, max_token_size, head_num, head_dim, dtype, device)
+        self.mask_k_cache = GPUCache(self.k_uvm, None, max_mask_cache_token_size, online_cache_update,
+                                     block_tokens=block_tokens, max_fetch=max_fetch)
+        self.sa_kv_cache = GPUCache(self.k_uvm, self.v_uvm, max_sa_cache_token_size, online_cache_update,
+                                    block_tokens=block_tokens, max_fetch=max_fetch)
+        self.miss_stream: Optional[torch.cuda.Stream] = None
+
+    def get_page_count(self) -> int:
+        assert self.k_uvm.bank_cpu.shape == self.v_uvm.bank_cpu.shape
+        return self.k_uvm.bank_cpu.shape[0]
+
+    # ------------------------------------------------------------------ what the operator needs
+    def kv_struct(self, block_table: Tensor, cache_seq_lens: Tensor, max_tsrc: int, masking: bool):
+        """Paged (page size 1) description of the host pools with the cache that serves this phase."""
+        cache = self.mask_k_cache if masking else self.sa_kv_cache
+        cache.wait()
+        kb, vb = self.k_uvm.bank_cpu, self.v_uvm.bank_cpu
+        s = N.KVStruct()
+        s.k, s.v = self.k_uvm.device_ptr, self.v_uvm.device_ptr
+        s.k_stride_b, s.k_stride_t, s.k_stride_h = kb.stride(0), kb.stride(0), kb.stride(1)
+        s.v_stride_b, s.v_stride_t, s.v_stride_h = vb.stride(0), vb.stride(0), vb.stride(1)
+        s.tsrc = 0
+        s.max_tsrc = max_tsrc
+        s.block_table = block_table.data_ptr()
+        s.cache_seq_lens = cache_seq_lens.data_ptr()
+        s.bt_stride_b = block_table.stride(0)
+        s.bt_is64 = int(block_table.dtype == torch.int64)
+        s.sl_is64 = int(cache_seq_lens.dtype == torch.int64)
+        s.paged = 1
+        s.page_size = 1
+        s.HKV = self.head_kv
+        s.cache = cache.handle
+        return s
+
+    # ------------------------------------------------------------------ reference methods
+    def prefetch_prefix_kv_buffer(self, table: Tensor, device: torch.device) -> Tuple[Tensor, Tensor]:
+        """Dense device copies ``[1, n, head, dim]`` of the pool rows listed in ``table``."""
+        if table.device != torch.device("cpu"):
+            table = table.to("cpu", non_blocking=False)
+        k = self.k_uvm.gather_cpu(table, pin_memory=True).to(device, non_blocking=False).unsqueeze(0)
+        v = self.v_uvm.gather_cpu(table, pin_memory=True).to(device, non_blocking=False).unsqueeze(0)
+        return k, v
+
+    def set_kv_buffer(self, table: Tensor, table_gpu: Tensor, cache_k: Tensor, cache_v: Tensor):
+        """Store rows into the host pools and keep resident cache blocks current."""
+        assert table.device == cache_k.device and cache_v.device == cache_k.device
+        if cache_k.device.type == "cpu":
+            idx = table.reshape(-1).to(torch.int64)
+            self.k_uvm.bank_cpu.index_copy_(0, idx, cache_k.reshape(-1, self.head_kv, self.head_dim))
+            self.v_uvm.bank_cpu.index_copy_(0, idx, cache_v.reshape(-1, self.head_kv, self.head_dim))
+        else:
+            rows = table.reshape(-1).to(torch.int64).contiguous()
+            for pool, src in ((self.k_uvm, cache_k), (self.v_uvm, cache_v)):
+                src = src.reshape(-1, self.head_kv, self.head_dim).to(pool.dtype).contiguous()
+                N.pool_write_rows(pool.device_ptr, pool.bank_cpu.stride(0), pool.bank_cpu.stride(1), self.head_kv,
+                                  self.head_dim, N.dtype_code(pool.bank_cpu), rows, src, self.device)
+        self.mask_k_cache.on_set_kv_buffer(table_gpu, cache_k, None)
+        self.sa_kv_cache.on_set_kv_buffer(table_gpu, cache_k, cache_v)
+        idx_gpu = table_gpu.reshape(-1).to(torch.int64)
+        for pool in (self.k_uvm, self.v_uvm):
+            pool.metadata.index_put_((idx_gpu,), torch.index_select(pool.metadata, 0, idx_gpu) + 1)
+
+    def handle_cache_miss(self, metadata=None):
+        stats_m = getattr(metadata, "mask_cache_statistics", None)
+        stats_s = getattr(metadata, "sa_cache_statistics", None)
+        self.mask_k_cache.handle_cache_miss(metadata=metadata, stats=stats_m, stream=self.miss_stream)
+        self.sa_kv_cache.handle_cache_miss(metadata=metadata, stats=stats_s, stream=self.miss_stream)
+
+    def flush(self):
+        self.mask_k_cache.flush()
+        self.sa_kv_cache.flush()

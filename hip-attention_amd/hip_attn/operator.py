@@ -60,33 +60,51 @@ def _reject_unsupported(args: HiPAttentionArgs):
         raise NotImplementedError("low_percent / low_k_ratio pruning is dead code in the reference and not built")
 
 
-def _kv_struct(args: HiPAttentionArgs, k: Optional[Tensor], v: Optional[Tensor], max_tsrc: int):
-    """Returns (struct, keepalive) describing where K/V rows live."""
+def _kv_struct(args: HiPAttentionArgs, k: Optional[Tensor], v: Optional[Tensor], max_tsrc: int,
+               masking: bool = False, stats: Optional[HiPAttentionCacheAccessStatistics] = None):
+    """Returns (struct, keepalive) describing where K/V rows live.
+
+    ``masking`` picks the key-only cache of an offload cache; ``stats`` attaches access / miss flags.
+    """
     if k is not None:
         kk = k if k.stride(-1) == 1 else k.contiguous()
         vv = v if v.stride(-1) == 1 else v.contiguous()
-        return N.make_kv_dense(kk, vv), (kk, vv)
-    if args.offload_cache is not None:
-        return args.offload_cache.kv_struct(max_tsrc)
-    bt = args.block_table
-    sl = args.cache_seq_lens
-    assert args.k_cache is not None and args.v_cache is not None, "paged mode needs k_cache and v_cache"
-    assert bt is not None and bt.ndim == 2, "paged mode needs block_table [B, pages]"
-    assert sl is not None and sl.ndim == 1, "paged mode needs cache_seq_lens [B]"
-    assert args.k_cache.ndim == 4 and args.v_cache.ndim == 4
-    if bt.dtype not in (torch.int32, torch.int64):
-        bt = bt.to(torch.int64)
-    if bt.stride(1) != 1:
-        bt = bt.contiguous()
-    if sl.dtype not in (torch.int32, torch.int64):
-        sl = sl.to(torch.int64)
-    if sl.stride(0) != 1:
-        sl = sl.contiguous()
-    return N.make_kv_paged(args.k_cache, args.v_cache, bt, sl, max_tsrc), (bt, sl)
+        st, keep = N.make_kv_dense(kk, vv), (kk, vv)
+    else:
+        bt = args.block_table
+        sl = args.cache_seq_lens
+        assert bt is not None and bt.ndim == 2, "paged mode needs block_table [B, pages]"
+        assert sl is not None and sl.ndim == 1, "paged mode needs cache_seq_lens [B]"
+        if bt.dtype not in (torch.int32, torch.int64):
+            bt = bt.to(torch.int64)
+        if bt.stride(1) != 1:
+            bt = bt.contiguous()
+        if sl.dtype not in (torch.int32, torch.int64):
+            sl = sl.to(torch.int64)
+        if sl.stride(0) != 1:
+            sl = sl.contiguous()
+        if args.k_cache is None and args.offload_cache is not None:
+            st, keep = args.offload_cache.kv_struct(bt, sl, max_tsrc, masking), (bt, sl)
+        else:
+            assert args.k_cache is not None and args.v_cache is not None, "paged mode needs k_cache and v_cache"
+            assert args.k_cache.ndim == 4 and args.v_cache.ndim == 4
+            st, keep = N.make_kv_paged(args.k_cache, args.v_cache, bt, sl, max_tsrc), (bt, sl)
+    if stats is not None and stats.access_counter is not None:
+        st = N.set_flags(st, stats.access_counter, stats.cache_miss_counter if st.cache else None)
+    return st, keep
+
+
+def _new_statistics(args: HiPAttentionArgs, B: int, head_kv: int, pages: int, device):
+    """Zeroed ``int32 [B, HEAD_KV, pages]`` access and miss flags (attention_extend.py:1994-2006)."""
+    if not args.require_cache_statistics:
+        return HiPAttentionCacheAccessStatistics(None, None)
+    return HiPAttentionCacheAccessStatistics(
+        torch.zeros((B, head_kv, pages), dtype=torch.int32, device=device),
+        torch.zeros((B, head_kv, pages), dtype=torch.int32, device=device))
 
 
 def _mask_kv(args: HiPAttentionArgs, k_mask: Optional[Tensor], max_tsrc: int, q: Tensor, programs_rows: int,
-             chunk_count: int, device):
+             chunk_count: int, device, stats=None):
     """KV description for the scan kernels, with keys pre-scaled when that saves work."""
     stage0 = args.stages[0]
     iters = max(1, int(stage0.stage_chunk_size).bit_length())
@@ -99,13 +117,13 @@ def _mask_kv(args: HiPAttentionArgs, k_mask: Optional[Tensor], max_tsrc: int, q:
             if force == "1" or (force != "0" and sampled_rows >= 4 * rows_total):
                 khat = N.prescale_k(src, device)
                 if k_mask is not None:
-                    st, keep = _kv_struct(args, khat, khat, max_tsrc)
+                    st, keep = _kv_struct(args, khat, khat, max_tsrc, masking=True, stats=stats)
                 else:
                     a2 = args.clone()
                     a2.k_cache, a2.v_cache = khat, khat
-                    st, keep = _kv_struct(a2, None, None, max_tsrc)
+                    st, keep = _kv_struct(a2, None, None, max_tsrc, masking=True, stats=stats)
                 return st, (keep, khat), khat
-    st, keep = _kv_struct(args, k_mask, k_mask, max_tsrc)
+    st, keep = _kv_struct(args, k_mask, k_mask, max_tsrc, masking=True, stats=stats)
     return st, keep, None
 
 
@@ -194,6 +212,11 @@ def dual_stage_quadratic_hip_attention(
     if not args.require_stage_caches:
         stage_caches = None
 
+    args.update_flags()
+    MAX_PAGE = args.paged_cache_page_count if (k is None and args.using_paged_cache) else MAX_TSRC
+    mask_stats = None
+    sa_stats = _new_statistics(args, BSZ, HEAD_KV, MAX_PAGE, device)
+
     qq = q if q.stride(-1) == 1 else q.contiguous()
     hg = 1 if _head_reduce_enabled() else HEAD
     mask_kv = None  # built lazily: cached-mask steps never touch the estimation path
@@ -217,7 +240,9 @@ def dual_stage_quadratic_hip_attention(
 
         # Keys are scaled by c_k and re-rounded every time they are sampled.  When the scan will sample
         # far more rows than the key tensor holds (prefill), scale the whole tensor once instead.
-        mask_kv, keep_mask_kv, khat = _mask_kv(args, k_mask, MAX_TSRC, q, BSZ * HEAD * BDST_SCAN, chunk_count, device)
+        mask_stats = _new_statistics(args, BSZ, HEAD_KV, MAX_PAGE, device)
+        mask_kv, keep_mask_kv, khat = _mask_kv(args, k_mask, MAX_TSRC, q, BSZ * HEAD * BDST_SCAN, chunk_count, device,
+                                               stats=mask_stats)
         k_prescaled = khat is not None
 
         scores = None
@@ -363,7 +388,7 @@ def dual_stage_quadratic_hip_attention(
     seq_pos = position_ids[:, -q_bsa.shape[1]:]
     context = block_sparse_attention(
         q_bsa, k, v, seq_pos, indices, ks_start_end, args, MAX_TSRC, decode=use_decode, rows_shared=rows_shared,
-        khat=khat if (args.k_mask is None) else None,
+        khat=khat if (args.k_mask is None) else None, stats=sa_stats,
     )
 
     metadata = HiPAttentionOutputMetadata(
@@ -371,8 +396,8 @@ def dual_stage_quadratic_hip_attention(
         ks=ks,
         ks_count=ks_count,
         ks_start_end=ks_start_end,
-        mask_cache_statistics=(HiPAttentionCacheAccessStatistics(None, None) if fresh_mask else None),
-        sa_cache_statistics=HiPAttentionCacheAccessStatistics(None, None),
+        mask_cache_statistics=(mask_stats if fresh_mask else None),
+        sa_cache_statistics=sa_stats,
         stage_caches=stage_caches,
     )
     # private hint for later calls that reuse this metadata: index rows are identical across heads,
@@ -384,7 +409,8 @@ def dual_stage_quadratic_hip_attention(
 @torch.no_grad()
 def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], position_ids: Tensor, indices: Tensor,
                            ks_start_end: Tensor, args: HiPAttentionArgs, max_tsrc: int, decode: bool = False,
-                           impl: int = 0, rows_shared: bool = False, khat: Optional[Tensor] = None) -> Tensor:
+                           impl: int = 0, rows_shared: bool = False, khat: Optional[Tensor] = None,
+                           stats: Optional[HiPAttentionCacheAccessStatistics] = None) -> Tensor:
     """Sparse attention over (selected blocks, sink, sliding window) given the metadata tensors.
 
     ``position_ids`` are 0-based (the reference passes ``seq_lens = position_ids + 1``,
@@ -398,7 +424,7 @@ def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], 
     """
     device = q.device
     qq = q if q.stride(-1) == 1 else q.contiguous()
-    kvs, keep = _kv_struct(args, k, v, max_tsrc)
+    kvs, keep = _kv_struct(args, k, v, max_tsrc, masking=False, stats=stats)
     if position_ids.dtype != torch.int64:
         position_ids = position_ids.to(torch.int64)
     qs = N.make_q(qq, position_ids)
@@ -419,7 +445,8 @@ def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], 
             if "is not built" not in str(e):
                 raise
     ksrc = k if k is not None else args.k_cache
-    if khat is not None and (ksrc is None or khat.shape != ksrc.shape or khat.stride() != ksrc.stride()):
+    if khat is not None and (ksrc is None or khat.shape != ksrc.shape or khat.stride() != ksrc.stride()
+                             or kvs.cache):
         khat = None
     N.bsa_prefill(qs, kvs, indices, ks_start_end, BK, args.block_size_q, args.block_size_k,
                   args.sliding_window_size, args.sink_token_size, decode or rows_shared, impl, out, device,

@@ -60,6 +60,17 @@ typedef struct hipattn_kv {
     int32_t bt_is64, sl_is64;
     int32_t paged, page_size;
     int32_t HKV;
+    /* Offload: NULL, or a block cache in device memory in front of K/V that live in pinned host
+     * memory (see hipattn_cache_create).  Requires paged != 0. */
+    const struct hipattn_cache *cache;
+    /* Access statistics (HiPAttentionCacheAccessStatistics, src/hip_attn/v1_2/attention_metadata.py:76-81,
+     * stores at src/hip_attn/v1_2/uvm_gpu_cache.py:845-862,1365-1372): NULL, or int32 [B, HKV, pages]
+     * (pages = tsrc when dense) where every page whose key row was loaded is set to 1, and the same
+     * for loads the offload cache could not serve.  Only hipattn_mask_stage and the bsa entry points
+     * write them. */
+    int32_t *access_flags;
+    int32_t *miss_flags;
+    int64_t flags_stride_b, flags_stride_h;
 } hipattn_kv_t;
 
 const char *hipattn_version(void);
@@ -155,6 +166,79 @@ int hipattn_bsa_decode_partial(const hipattn_q_t *q, const hipattn_kv_t *kv, con
 int hipattn_bsa_decode_merge(const void *workspace, int32_t B, int32_t HEAD, int32_t HID,
                              int32_t nsplits, int32_t dtype, void *out, int64_t out_stride_b,
                              int64_t out_stride_h, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Offload cache: K (and V) of a layer live in pinned host memory as a pool [pool_rows, HKV, HID]
+ * addressed through the paged view (row = page * page_size + offset); a block cache in device
+ * memory holds `slots` blocks of `block_tokens` consecutive pool rows of ONE kv head.  Stands in for
+ * GPUCache / HiPOffloadCache, src/hip_attn/v1_2/uvm_gpu_cache.py:204-566,569-700: token -> slot
+ * table, least-recently-used replacement by last-access step, reads that miss go to host memory and
+ * are recorded, recorded misses are brought in after the step.
+ *
+ * Kernels given kv->cache look every row up in `table`; a resident block is read from `bank` and
+ * stamped with the current step, a missing one is read from the host pool over the host link and
+ * flagged in `miss`.  Results are therefore the same bytes with or without the cache.
+ * After the step:  hipattn_cache_lookup_and_schedule gathers the flagged blocks (ascending
+ * head-major block id, at most max_fetch) and picks as many victims: the slots with the smallest
+ * (last-use step, slot id), never one used in the current step;  hipattn_cache_commit copies the
+ * blocks host -> bank, relinks the table, and advances the step counter.  Both only enqueue work;
+ * the caller orders them after the kernels of the step and before those of the next one (they may
+ * run on another stream, overlapped with unrelated work).
+ * All buffers are the caller's; sizes from hipattn_cache_sizes. */
+typedef struct hipattn_cache hipattn_cache_t;
+
+typedef struct hipattn_cache_desc {
+    int32_t dtype;        /* HIPATTN_F32 / HIPATTN_BF16 */
+    int32_t HKV, HID;
+    int32_t block_tokens; /* power of two, 1..64 */
+    int32_t with_v;       /* 0: K only (mask estimation cache), 1: K and V per slot (attention cache) */
+    int64_t pool_rows;    /* rows of the host pool */
+    int64_t slots;
+    const void *host_k;   /* device-visible address of the pinned pool; strides in elements */
+    const void *host_v;   /* NULL when with_v == 0 */
+    int64_t host_stride_row, host_stride_h;
+    void *bank;           /* slots * (1 + with_v) * block_tokens * HID elements */
+    int32_t *table;       /* [HKV, n_blocks], n_blocks = ceil(pool_rows / block_tokens) */
+    int32_t *last_use;    /* [slots] */
+    int32_t *backref;     /* [slots] */
+    uint8_t *miss;        /* [HKV, n_blocks] */
+    void *workspace;      /* hipattn_cache_sizes(...).workspace bytes */
+} hipattn_cache_desc_t;
+
+typedef struct hipattn_cache_sizes {
+    int64_t n_blocks;
+    int64_t bank_bytes, table_bytes, last_use_bytes, backref_bytes, miss_bytes, workspace_bytes;
+} hipattn_cache_sizes_t;
+
+int hipattn_cache_sizes(const hipattn_cache_desc_t *desc, int64_t max_fetch, hipattn_cache_sizes_t *out);
+/* Builds the handle (host memory only) and enqueues the kernels that empty the cache. max_fetch bounds
+ * the blocks one commit can bring in. */
+int hipattn_cache_create(const hipattn_cache_desc_t *desc, int64_t max_fetch, hipattn_cache_t **out, void *stream);
+void hipattn_cache_destroy(hipattn_cache_t *cache);
+/* Empties the cache (GPUCache.flush, src/hip_attn/v1_2/uvm_gpu_cache.py:294-300). */
+int hipattn_cache_flush(hipattn_cache_t *cache, void *stream);
+int hipattn_cache_lookup_and_schedule(hipattn_cache_t *cache, void *stream);
+int hipattn_cache_commit(hipattn_cache_t *cache, void *stream);
+/* Write-through after the host pool changed (HiPOffloadCache.set_kv_buffer / on_set_kv_buffer,
+ * src/hip_attn/v1_2/uvm_gpu_cache.py:629-688,548-563): rows int64 [n] pool rows, k_rows / v_rows
+ * device [n, HKV, HID] contiguous; resident blocks receive the new rows, others are left alone. */
+int hipattn_cache_write_rows(hipattn_cache_t *cache, const int64_t *rows, int64_t n, const void *k_rows,
+                             const void *v_rows, void *stream);
+/* Scatter device rows src[n, HKV, HID] (contiguous) into a pinned host pool at int64 rows[n] -- the GPU-side
+ * store of HiPOffloadCache.set_kv_buffer (src/hip_attn/v1_2/uvm_gpu_cache.py:665-668). */
+int hipattn_pool_write_rows(void *pool, int64_t stride_row, int64_t stride_h, int32_t HKV, int32_t HID,
+                            int32_t dtype, const int64_t *rows, int64_t n, const void *src, void *stream);
+/* Pinned host memory for a pool.  coherent != 0 asks for memory the GPU never caches, so that rows the CPU
+ * writes are seen by the next kernel without any cache maintenance; pools written by the CPU need it. */
+int hipattn_host_alloc(int64_t bytes, int32_t coherent, void **host_out);
+int hipattn_host_free(void *host);
+/* Device-visible address of memory obtained from hipHostMalloc (HOST pointer in, device pointer out). */
+int hipattn_host_device_pointer(void *host, void **device_out);
+/* Copies the counters to host memory and waits for `stream`:
+ * out[0] steps committed, [1] resident blocks touched (summed over steps), [2] blocks missed,
+ * [3] blocks fetched, [4] blocks evicted, [5] touched in the last step, [6] missed in the last step,
+ * [7] fetched in the last step. */
+int hipattn_cache_stats(hipattn_cache_t *cache, int64_t out[8], void *stream);
 
 #ifdef __cplusplus
 }
