@@ -48,7 +48,7 @@ int check_q(const hipattn_q_t *q) {
     return 0;
 }
 
-int make_kv_view(const hipattn_kv_t *kv, int B, int HID, int dtype, KVView *o) {
+int make_kv_view(const hipattn_kv_t *kv, int B, int HID, int dtype, KVView *o, KVExt *x) {
     (void)B;
     HIPATTN_CHECK_ARG(kv && kv->k, HIPATTN_E_ARG, "kv: null K pointer");
     HIPATTN_CHECK_ARG(kv->HKV > 0, HIPATTN_E_ARG, "kv: HKV <= 0");
@@ -77,13 +77,12 @@ int make_kv_view(const hipattn_kv_t *kv, int B, int HID, int dtype, KVView *o) {
     o->block_table = kv->block_table; o->cache_seq_lens = kv->cache_seq_lens; o->bt_stride_b = kv->bt_stride_b;
     o->bt_is64 = kv->bt_is64; o->sl_is64 = kv->sl_is64; o->paged = kv->paged; o->page_size = kv->page_size ? kv->page_size : 1;
     o->HKV = kv->HKV;
-    o->cached = 0;
-    memset(&o->cache, 0, sizeof(o->cache));
-    o->access_flags = kv->access_flags;
-    o->miss_flags = kv->miss_flags;
-    o->flags_stride_b = kv->flags_stride_b;
-    o->flags_stride_h = kv->flags_stride_h;
-    if (kv->cache) return cache_view_for(kv->cache, kv, HID, dtype, o);
+    memset(x, 0, sizeof(*x));
+    x->access_flags = kv->access_flags;
+    x->miss_flags = kv->miss_flags;
+    x->flags_stride_b = kv->flags_stride_b;
+    x->flags_stride_h = kv->flags_stride_h;
+    if (kv->cache) return cache_view_for(kv->cache, kv, o, HID, dtype, x);
     return 0;
 }
 

@@ -1,11 +1,13 @@
 // Parameter block shared by the block-sparse attention kernels.
 #pragma once
 
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace hipattn {
 
-struct BsaParams {
+struct BsaParamsBase {
     const void *q;
     int64_t q_sb, q_st, q_sh;
     const int64_t *pos;
@@ -20,6 +22,13 @@ struct BsaParams {
     void *out;
     int64_t o_sb, o_st, o_sh;
 };
+
+// the extended kernels (statistics, offload cache) take the same block with the extras appended
+struct BsaParams : BsaParamsBase {
+    KVExt kx;
+};
+template <bool EXT>
+using BsaParamsFor = std::conditional_t<EXT, BsaParams, BsaParamsBase>;
 
 // validates arguments and fills the parameter block (host)
 int bsa_fill_params(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t *indices, const int32_t *kse,

@@ -9,16 +9,20 @@
 
 namespace hipattn {
 
-struct DecodeParams {
-    BsaParams a;
+template <bool EXT>
+struct DecodeParamsT {
+    BsaParamsFor<EXT> a;
     int nsplits;
     float *ws;  // [B, HEAD, nsplits, HID + 4]: acc / l, then m + log2(l)
 };
+using DecodeParams = DecodeParamsT<true>;
 
 template <typename T, int HID, int G, bool EXT>
-__global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParams dp) {
+__global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<EXT> dp) {
     constexpr int SEG = HID / 16;
-    const BsaParams &p = dp.a;
+    const BsaParamsFor<EXT> &p = dp.a;
+    const KVExt *kx = nullptr;
+    if constexpr (EXT) kx = &p.kx;
     __shared__ float s_m[16][G];
     __shared__ float s_l[16][G];
     __shared__ float s_acc[16][G][HID];
@@ -88,9 +92,13 @@ __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParams dp
             }
         }
         const bool att = valid && (kind == 0 ? (t + p.sw <= ppos) : (t <= ppos && ppos < t + p.sw));
-        if (!att) continue;  // uniform inside the 16-lane group; shuffles below stay inside the group
         int64_t koff, voff;
-        p.kv.rows<true, EXT>(b, t, kvh, seqlen, koff, voff);
+        if (!att) {  // uniform inside the 16-lane group; shuffles below stay inside the group
+            // staged but masked out: still an access as far as the statistics and the cache are concerned
+            if (EXT && valid && dl == 0) kv_rows<false, EXT>(p.kv, kx, b, t, kvh, seqlen, koff, voff, true);
+            continue;
+        }
+        kv_rows<true, EXT>(p.kv, kx, b, t, kvh, seqlen, koff, voff, dl == 0);
         float kh[SEG], vv[SEG];
         if (koff != NO_ROW) {
             load_elems<T, SEG>(kbase + koff + dl * SEG, kh);
@@ -184,10 +192,15 @@ static int launch_partial(const DecodeParams &dp, hipStream_t st) {
 #define DEC_CASE(GG)                                                                                   \
     if constexpr (GG * HID <= 512) {                                                                   \
         if (dp.a.G == GG) {                                                                            \
-            if (dp.a.kv.extended())                                                                    \
+            if (dp.a.kx.extended()) {                                                                  \
                 hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG, true>), grid, block, 0, st, dp);  \
-            else                                                                                       \
-                hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG, false>), grid, block, 0, st, dp); \
+            } else {                                                                                   \
+                DecodeParamsT<false> dq;                                                               \
+                dq.a = static_cast<const BsaParamsBase &>(dp.a);                                       \
+                dq.nsplits = dp.nsplits;                                                               \
+                dq.ws = dp.ws;                                                                         \
+                hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG, false>), grid, block, 0, st, dq); \
+            }                                                                                          \
             launched = true;                                                                           \
         }                                                                                              \
     }

@@ -51,7 +51,9 @@ struct MfmaSmem {
 };
 
 template <int HID, bool KSCALED, bool EXT>
-__global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParams p, int hgroups, int hpw, long long total_wg) {
+__global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p, int hgroups, int hpw, long long total_wg) {
+    const KVExt *kx = nullptr;
+    if constexpr (EXT) kx = &p.kx;
     constexpr int KS = HID / 16;   // k-steps of the first product
     constexpr int DB = HID / 32;   // 32-row blocks of O^T
     constexpr int CPT = TN * (HID / 8) / NTHREADS;  // 16-byte chunks per thread per tile
@@ -179,7 +181,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParams p, int hgr
             vreg[j] = make_uint4(0, 0, 0, 0);
             if (t >= 0) {
                 int64_t ko, vo;
-                p.kv.rows<true, EXT>(b, t, kvh, seqlen, ko, vo);
+                kv_rows<true, EXT>(p.kv, kx, b, t, kvh, seqlen, ko, vo, piece == 0);
                 if (ko != NO_ROW) kreg[j] = *reinterpret_cast<const uint4 *>(kbase + ko + piece * 8);
                 if (vo != NO_ROW) vreg[j] = *reinterpret_cast<const uint4 *>(vbase + vo + piece * 8);
             }
@@ -339,6 +341,55 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParams p, int hgr
         }
 }
 
+// Access statistics without touching the attention kernel: walks exactly the tokens the tile kernel stages
+// for a (batch, kv head, head group, query block) and records them, loading no keys.
+__global__ __launch_bounds__(256) void bsa_mark_kernel(BsaParams p, int hgroups, int hpw) {
+    long long L = blockIdx.x;
+    const int qb = (int)(L % p.NBQ);
+    L /= p.NBQ;
+    const int hgrp = (int)(L % hgroups);
+    L /= hgroups;
+    const int kvh = (int)(L % p.kv.HKV);
+    const int b = (int)(L / p.kv.HKV);
+    const int hrow = p.share_first_head ? kvh * p.G : kvh * p.G + hgrp * hpw;
+    const int64_t irow = ((int64_t)b * p.HEAD + hrow) * p.idx_rows + qb;
+    __shared__ long long s_cur;
+    if (threadIdx.x == 0) s_cur = -1;
+    __syncthreads();
+    for (int j = threadIdx.x; j < p.bq; j += blockDim.x) {
+        const long long it = (long long)qb * p.bq + j;
+        if (it < p.TDST) atomicMax(&s_cur, (long long)p.pos[(int64_t)b * p.pos_sb + it * p.pos_st]);
+    }
+    __syncthreads();
+    const int curr = (int)s_cur + 1;
+    int rs = p.kse[irow * 2 + 0], re = p.kse[irow * 2 + 1];
+    if (p.BK <= 0) { rs = 0; re = 0; }
+    const int jend = rs + p.BK < re ? rs + p.BK : re;
+    const int n_sel_tok = (jend > rs ? jend - rs : 0) * p.bk;
+    const int sink_end = curr < p.sink ? curr : p.sink;
+    int ws = curr - p.sw - p.bq;
+    if (ws < 0) ws = 0;
+    const int n_win = p.sw > 0 ? curr - ws : 0;
+    const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
+    const int total = n_sel_tok + sink_end + n_win;
+    for (int o = threadIdx.x; o < total; o += blockDim.x) {
+        long long t = -1;
+        if (o < n_sel_tok) {
+            const long long st = p.indices[irow * p.BK + rs + o / p.bk];
+            t = st + o % p.bk;
+            if (!(t >= 0 && t < p.kv.max_tsrc && t < curr && t >= p.sink)) t = -1;
+        } else if (o < n_sel_tok + sink_end) {
+            t = o - n_sel_tok;
+        } else {
+            t = ws + (o - n_sel_tok - sink_end);
+        }
+        if (t >= 0) {
+            int64_t ko, vo;
+            kv_rows<false, true, false>(p.kv, &p.kx, b, t, kvh, seqlen, ko, vo, true);
+        }
+    }
+}
+
 template <int HID, bool KSCALED, bool EXT>
 static int launch_mfma(const BsaParams &p, hipStream_t st) {
     const int hpw = p.share_first_head ? 4 : 1;  // per-head index rows: one head per workgroup
@@ -352,7 +403,8 @@ static int launch_mfma(const BsaParams &p, hipStream_t st) {
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
-    hipLaunchKernelGGL((bsa_mfma_kernel<HID, KSCALED, EXT>), dim3((unsigned)total), dim3(NTHREADS), smem, st, p, hgroups,
+    const BsaParamsFor<EXT> &pk = p;  // the plain kernel takes the block without the extras
+    hipLaunchKernelGGL((bsa_mfma_kernel<HID, KSCALED, EXT>), dim3((unsigned)total), dim3(NTHREADS), smem, st, pk, hgroups,
                        hpw, total);
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
@@ -362,7 +414,21 @@ int bsa_mfma_launch(const BsaParams &p, int dtype, int HID, hipStream_t st) {
     if (dtype != HIPATTN_BF16) return HIPATTN_E_UNSUPPORTED;
     if (p.bq > 64) return HIPATTN_E_UNSUPPORTED;
     if ((p.o_st % 4) != 0 || (p.o_sh % 4) != 0 || (p.o_sb % 4) != 0) return HIPATTN_E_UNSUPPORTED;
-    const bool ext = p.kv.extended();
+    bool ext = p.kx.extended();
+    BsaParams plain;
+    if (ext && !p.kx.cached && (HID == 64 || HID == 128)) {
+        // statistics only: a cheap marking pass, then the plain kernel
+        const int hpw = p.share_first_head ? 4 : 1;
+        const int hgroups = (p.G + hpw - 1) / hpw;
+        const long long total = (long long)p.B * p.kv.HKV * hgroups * p.NBQ;
+        if (total >= 0x7fffffffLL) return HIPATTN_E_UNSUPPORTED;
+        hipLaunchKernelGGL(bsa_mark_kernel, dim3((unsigned)total), dim3(256), 0, st, p, hgroups, hpw);
+        HIPATTN_CHECK_HIP(hipGetLastError());
+        plain = p;
+        plain.kx.access_flags = nullptr;
+        plain.kx.miss_flags = nullptr;
+        return bsa_mfma_launch(plain, dtype, HID, st);
+    }
 #define BSA_PICK(H)                                                                  \
     case H:                                                                          \
         if (p.k_prescaled) return ext ? launch_mfma<H, true, true>(p, st) : launch_mfma<H, true, false>(p, st); \

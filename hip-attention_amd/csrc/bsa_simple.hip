@@ -85,7 +85,7 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
             int64_t voff = NO_ROW;
             if (att) {
                 int64_t koff;
-                p.kv.rows<true, true>(b, t, kvh, seqlen, koff, voff);
+                kv_rows<true, true>(p.kv, &p.kx, b, t, kvh, seqlen, koff, voff);
                 float dot = 0.0f;
                 if (koff != NO_ROW) {
                     constexpr int CH = 16 / (int)sizeof(T) < HID ? 16 / (int)sizeof(T) : HID;
@@ -152,7 +152,7 @@ int bsa_fill_params(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t 
     HIPATTN_CHECK_ARG(kv && out && kse, HIPATTN_E_ARG, "bsa: null pointer");
     HIPATTN_CHECK_ARG(BK <= 0 || indices, HIPATTN_E_ARG, "bsa: indices is null with BK > 0");
     HIPATTN_CHECK_ARG(bq > 0 && bk > 0 && sw >= 0 && sink >= 0 && idx_rows > 0, HIPATTN_E_ARG, "bsa: bad sizes");
-    rc = make_kv_view(kv, q->B, q->HID, q->dtype, &p->kv);
+    rc = make_kv_view(kv, q->B, q->HID, q->dtype, &p->kv, &p->kx);
     if (rc) return rc;
     HIPATTN_CHECK_ARG(q->HEAD % p->kv.HKV == 0, HIPATTN_E_ARG, "bsa: HEAD %% HKV != 0");
     p->q = q->ptr; p->q_sb = q->stride_b; p->q_st = q->stride_t; p->q_sh = q->stride_h;

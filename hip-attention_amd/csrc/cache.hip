@@ -505,7 +505,7 @@ static int launch_fill(int32_t *p, int64_t n, int32_t value, hipStream_t st) {
     return 0;
 }
 
-int cache_view_for(const hipattn_cache *c, const hipattn_kv_t *kv, int HID, int dtype, KVView *o) {
+int cache_view_for(const hipattn_cache *c, const hipattn_kv_t *kv, const KVView *o, int HID, int dtype, KVExt *x) {
     HIPATTN_CHECK_ARG(kv->paged, HIPATTN_E_ARG, "kv: an offload cache needs the paged view");
     HIPATTN_CHECK_ARG(c->d.dtype == dtype && c->d.HID == HID && c->d.HKV == kv->HKV, HIPATTN_E_ARG,
                       "kv: cache was built for dtype %d, head dim %d, %d kv heads", c->d.dtype, c->d.HID, c->d.HKV);
@@ -515,8 +515,8 @@ int cache_view_for(const hipattn_cache *c, const hipattn_kv_t *kv, int HID, int 
     HIPATTN_CHECK_ARG(kv->k_stride_t == c->d.host_stride_row && kv->k_stride_b == c->d.host_stride_row * ps &&
                           kv->k_stride_h == c->d.host_stride_h,
                       HIPATTN_E_ARG, "kv: paged strides do not describe the pool the cache was built over");
-    o->cached = 1;
-    CacheView &v = o->cache;
+    x->cached = 1;
+    CacheView &v = x->cache;
     v.table = c->d.table;
     v.last_use = c->d.last_use;
     v.miss = c->d.miss;

@@ -145,8 +145,12 @@ struct CacheView {
     int32_t with_v;         // slots hold V rows too
 };
 
+// CHECK = true reads first and stores only a flag that is still clear (right for readers that revisit the
+// same rows many times); CHECK = false stores blindly (right for one pass over mostly distinct rows).
+// Racing lanes store the same value; a stale read only repeats the store.
+template <bool CHECK = true>
 __device__ __forceinline__ void mark_flag(int32_t *f) {
-    if (*f == 0) *f = 1;  // racing lanes store the same value; a stale read only repeats the store
+    if (!CHECK || *f == 0) *f = 1;
 }
 
 struct KVView {
@@ -160,10 +164,6 @@ struct KVView {
     const void *cache_seq_lens;
     int64_t bt_stride_b;
     int bt_is64, sl_is64, paged, page_size, HKV;
-    int cached;
-    CacheView cache;
-    int32_t *access_flags, *miss_flags;
-    int64_t flags_stride_b, flags_stride_h;
 
     __device__ __forceinline__ int64_t seq_len(int b) const {
         return sl_is64 ? reinterpret_cast<const int64_t *>(cache_seq_lens)[b]
@@ -178,59 +178,108 @@ struct KVView {
         }
         return page;
     }
-    // Element offsets (from k and v) of the rows of token t, kv head h; NO_ROW = "zero row".
-    // WANT_V = false skips the V side.  EXT = true also records the access and consults the block cache;
-    // kernels are built both ways so that the plain path does not carry the extra arguments.
-    template <bool WANT_V, bool EXT>
-    __device__ __forceinline__ void rows(int b, int64_t t, int h, int64_t seqlen, int64_t &ko, int64_t &vo) const {
-        ko = NO_ROW;
-        vo = NO_ROW;
+    __device__ __forceinline__ int64_t k_plain(int b, int64_t t, int h, int64_t seqlen) const {
         if (!paged) {
-            if (t < 0 || t >= tsrc) return;
-            if (EXT && access_flags)
-                mark_flag(access_flags + (int64_t)b * flags_stride_b + (int64_t)h * flags_stride_h + t);
-            ko = (int64_t)b * k_stride_b + t * k_stride_t + (int64_t)h * k_stride_h;
-            if (WANT_V) vo = (int64_t)b * v_stride_b + t * v_stride_t + (int64_t)h * v_stride_h;
-            return;
+            if (t < 0 || t >= tsrc) return NO_ROW;
+            return (int64_t)b * k_stride_b + t * k_stride_t + (int64_t)h * k_stride_h;
         }
-        if (t < 0) return;
         const int64_t page = page_of(b, t, seqlen);
-        const int64_t inpage = t % page_size;
-        if (EXT && access_flags)
-            mark_flag(access_flags + (int64_t)b * flags_stride_b + (int64_t)h * flags_stride_h + page);
-        if (EXT && cached) {
-            const int64_t row = page * page_size + inpage;
-            const int64_t e = (int64_t)h * cache.n_blocks + (row >> cache.shift);
-            const int32_t slot = cache.table[e];
-            if (slot >= 0) {
-                const int32_t now = *cache.step;
-                if (cache.last_use[slot] != now) cache.last_use[slot] = now;
-                const int64_t o = (int64_t)slot * cache.slot_stride +
-                                  (row & ((1LL << cache.shift) - 1)) * cache.row_elems;
-                ko = cache.k_delta + o;
-                if (WANT_V)
-                    vo = cache.with_v ? cache.v_delta + o
-                                      : page * v_stride_b + inpage * v_stride_t + (int64_t)h * v_stride_h;
-                return;
-            }
-            if (cache.miss[e] == 0) cache.miss[e] = 1;
-            if (miss_flags) mark_flag(miss_flags + (int64_t)b * flags_stride_b + (int64_t)h * flags_stride_h + page);
+        if (t < 0) return NO_ROW;
+        return page * k_stride_b + (t % page_size) * k_stride_t + (int64_t)h * k_stride_h;
+    }
+    __device__ __forceinline__ int64_t v_plain(int b, int64_t t, int h, int64_t seqlen) const {
+        if (!paged) {
+            if (t < 0 || t >= tsrc) return NO_ROW;
+            return (int64_t)b * v_stride_b + t * v_stride_t + (int64_t)h * v_stride_h;
         }
-        ko = page * k_stride_b + inpage * k_stride_t + (int64_t)h * k_stride_h;
-        if (WANT_V) vo = page * v_stride_b + inpage * v_stride_t + (int64_t)h * v_stride_h;
+        const int64_t page = page_of(b, t, seqlen);
+        if (t < 0) return NO_ROW;
+        return page * v_stride_b + (t % page_size) * v_stride_t + (int64_t)h * v_stride_h;
     }
-    template <bool EXT>
-    __device__ __forceinline__ int64_t k_row(int b, int64_t t, int h, int64_t seqlen) const {
-        int64_t ko, vo;
-        rows<false, EXT>(b, t, h, seqlen, ko, vo);
-        return ko;
-    }
+};
+
+// What only the extended builds of the kernels read: the offload cache and the statistics flags.  Kept out
+// of KVView (and at the end of the parameter blocks) so that the plain kernels' arguments stay small.
+struct KVExt {
+    int cached;
+    CacheView cache;
+    int32_t *access_flags, *miss_flags;
+    int64_t flags_stride_b, flags_stride_h;
     // host: does a launch need the EXT build of its kernel
     bool extended() const { return cached || access_flags || miss_flags; }
 };
 
-int make_kv_view(const hipattn_kv_t *kv, int B, int HID, int dtype, KVView *out);
-int cache_view_for(const hipattn_cache *c, const hipattn_kv_t *kv, int HID, int dtype, KVView *out);
+// Element offsets (from kv.k and kv.v) of the rows of token t, kv head h; NO_ROW = "zero row".
+// WANT_V = false skips the V side.  EXT = true also records the access and consults the block cache through
+// `kx` (ignored otherwise).  Several lanes usually fetch pieces of one row: `leader` is true for the one that
+// records the access.
+template <bool WANT_V, bool EXT, bool CHECK = true>
+__device__ __forceinline__ void kv_rows(const KVView &kv, const KVExt *kx, int b, int64_t t, int h, int64_t seqlen,
+                                        int64_t &ko, int64_t &vo, bool leader = true) {
+    if constexpr (!EXT) {
+        // Plain path: K and V offsets as two independent selects.  Sharing the range test and the page lookup
+        // between them reads better but made the attention tile kernel 18% slower (the compiler then keeps both
+        // row loads inside one divergent region and serialises them behind its waits).
+        ko = kv.k_plain(b, t, h, seqlen);
+        vo = WANT_V ? kv.v_plain(b, t, h, seqlen) : NO_ROW;
+        return;
+    }
+    ko = NO_ROW;
+    vo = NO_ROW;
+    if (!kv.paged) {
+        if (t < 0 || t >= kv.tsrc) return;
+        if constexpr (EXT) {
+            if (kx->access_flags && leader)
+                mark_flag<CHECK>(kx->access_flags + (int64_t)b * kx->flags_stride_b + (int64_t)h * kx->flags_stride_h + t);
+        }
+        ko = (int64_t)b * kv.k_stride_b + t * kv.k_stride_t + (int64_t)h * kv.k_stride_h;
+        if (WANT_V) vo = (int64_t)b * kv.v_stride_b + t * kv.v_stride_t + (int64_t)h * kv.v_stride_h;
+        return;
+    }
+    if (t < 0) return;
+    const int64_t page = kv.page_of(b, t, seqlen);
+    const int64_t inpage = t % kv.page_size;
+    if constexpr (EXT) {
+        if (kx->access_flags && leader)
+            mark_flag<CHECK>(kx->access_flags + (int64_t)b * kx->flags_stride_b + (int64_t)h * kx->flags_stride_h + page);
+        if (kx->cached) {
+            const CacheView &c = kx->cache;
+            const int64_t row = page * kv.page_size + inpage;
+            const int64_t e = (int64_t)h * c.n_blocks + (row >> c.shift);
+            const int32_t slot = c.table[e];
+            if (slot >= 0) {
+                if (leader) {
+                    const int32_t now = *c.step;
+                    if (c.last_use[slot] != now) c.last_use[slot] = now;
+                }
+                const int64_t o = (int64_t)slot * c.slot_stride + (row & ((1LL << c.shift) - 1)) * c.row_elems;
+                ko = c.k_delta + o;
+                if (WANT_V)
+                    vo = c.with_v ? c.v_delta + o
+                                  : page * kv.v_stride_b + inpage * kv.v_stride_t + (int64_t)h * kv.v_stride_h;
+                return;
+            }
+            if (leader) {
+                if (c.miss[e] == 0) c.miss[e] = 1;
+                if (kx->miss_flags)
+                    mark_flag(kx->miss_flags + (int64_t)b * kx->flags_stride_b + (int64_t)h * kx->flags_stride_h + page);
+            }
+        }
+    }
+    ko = page * kv.k_stride_b + inpage * kv.k_stride_t + (int64_t)h * kv.k_stride_h;
+    if (WANT_V) vo = page * kv.v_stride_b + inpage * kv.v_stride_t + (int64_t)h * kv.v_stride_h;
+}
+
+template <bool EXT>
+__device__ __forceinline__ int64_t kv_k_row(const KVView &kv, const KVExt *kx, int b, int64_t t, int h,
+                                            int64_t seqlen, bool leader = true) {
+    int64_t ko, vo;
+    kv_rows<false, EXT>(kv, kx, b, t, h, seqlen, ko, vo, leader);
+    return ko;
+}
+
+int make_kv_view(const hipattn_kv_t *kv, int B, int HID, int dtype, KVView *out, KVExt *ext);
+int cache_view_for(const hipattn_cache *c, const hipattn_kv_t *kv, const KVView *view, int HID, int dtype, KVExt *ext);
 int check_q(const hipattn_q_t *q);
 
 // ---------------------------------------------------------------- wave helpers

@@ -165,8 +165,8 @@ __global__ __launch_bounds__(64) void mask_stage_kernel(MaskParams p) {
         if (lane < BC) {
             int64_t o0 = NO_ROW, o1 = NO_ROW;
             if (active) {
-                o0 = p.kv.k_row<true>(b, (l + c) >> 1, kvh, seqlen);
-                o1 = p.kv.k_row<true>(b, (c + r) >> 1, kvh, seqlen);
+                o0 = kv_k_row<true>(p.kv, &p.kx, b, (l + c) >> 1, kvh, seqlen);
+                o1 = kv_k_row<true>(p.kv, &p.kx, b, (c + r) >> 1, kvh, seqlen);
             }
             s_koff[2 * lane] = o0;
             s_koff[2 * lane + 1] = o1;
@@ -279,7 +279,7 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
     HIPATTN_CHECK_ARG(terminate_size >= 1, HIPATTN_E_ARG, "mask stage: terminate_size < 1");
     if (n == 0) return 0;
     MaskParams p;
-    rc = make_kv_view(kv, q->B, q->HID, q->dtype, &p.kv);
+    rc = make_kv_view(kv, q->B, q->HID, q->dtype, &p.kv, &p.kx);
     if (rc) return rc;
     HIPATTN_CHECK_ARG(q->HEAD % p.kv.HKV == 0, HIPATTN_E_ARG, "mask stage: HEAD %% HKV != 0");
     p.q = q->ptr; p.q_sb = q->stride_b; p.q_st = q->stride_t; p.q_sh = q->stride_h;

@@ -44,7 +44,9 @@ __device__ __forceinline__ uint32_t scale_pack(uint32_t w, float c) {
 }
 
 template <int HID, int MB, int NB, bool PRESCALED, bool VIA_LDS, bool EXT>
-__global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(MaskParams p, int nsub, int hpw) {
+__global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
+    const KVExt *kx = nullptr;
+    if constexpr (EXT) kx = &p.kx;
     constexpr int KS = HID / 16;
     constexpr int HALF = HID / 2;
     constexpr int PPR = HID / 8;                  // 16-byte pieces per key row
@@ -192,7 +194,7 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
             int64_t off = NO_ROW;
             if (active[tb]) {
                 const int t = side ? ((ctr[tb] + cr[tb]) >> 1) : ((cl[tb] + ctr[tb]) >> 1);
-                off = p.kv.k_row<EXT>(b, t, kvh, seqlen);
+                off = kv_k_row<EXT>(p.kv, kx, b, t, kvh, seqlen, hh == 0);
             }
             if constexpr (VIA_LDS) {
                 if (hh == 0) s_off[tb * 32 + n] = off;
@@ -348,7 +350,7 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
         const char *e = getenv("HIPATTN_MASK_VIA_LDS");
         g_mask_via_lds = e ? (e[0] == '1' ? 1 : 0) : 2;
     }
-    const bool ext = p.kv.extended();  // statistics / offload cache: built for the direct path only
+    const bool ext = p.kx.extended();  // statistics / offload cache: built for the direct path only
     const bool via_lds = !ext && (g_mask_via_lds == 2 ? !wide : (g_mask_via_lds == 1));
     const int hpw = (via_lds || two) ? 1 : (p.G < 4 ? p.G : 4);
     const int hblocks = (p.G + hpw - 1) / hpw;
@@ -363,12 +365,13 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
         hipLaunchKernelGGL(qhat_kernel, dim3((unsigned)blocks), dim3(256), 0, st, p, HID, const_cast<uint16_t *>(p.qhat));
     }
     dim3 grid((unsigned)p.total), block(64 * hpw);
+    const MaskParamsBase &pb = p;  // the plain kernels take the block without the extras
 #define MS_LAUNCH(MBv, NBv, PSv, VLv)                                                                                 \
     do {                                                                                                              \
         if (ext && !VLv)                                                                                              \
             hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, NBv, PSv, false, true>), grid, block, 0, st, p, nsub, hpw); \
         else                                                                                                          \
-            hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, NBv, PSv, VLv, false>), grid, block, 0, st, p, nsub, hpw);  \
+            hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, NBv, PSv, VLv, false>), grid, block, 0, st, pb, nsub, hpw); \
     } while (0)
 #define MS_PICK(MBv, NBv)                                                \
     do {                                                                  \

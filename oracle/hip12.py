@@ -51,6 +51,8 @@ class _Tensors(ctypes.Structure):
         ("bt_cols", ctypes.c_int64),
         ("cache_seq_lens", ctypes.c_void_p),
         ("MAX_TSRC", ctypes.c_int64),
+        ("access", ctypes.c_void_p),
+        ("access_pages", ctypes.c_int64),
     ]
 
 
@@ -145,6 +147,7 @@ class OInputs:
     v_cache: Optional[np.ndarray] = None
     block_table: Optional[np.ndarray] = None  # [B,cols] int64
     cache_seq_lens: Optional[np.ndarray] = None  # [B] int64
+    access: Optional[np.ndarray] = None  # int32 [B,HKV,pages]: flags set by every key row the kernels fetch
 
     def c_struct(self, max_tsrc: int):
         np_t = np.uint16 if self.dtype == "bf16" else np.float32
@@ -181,6 +184,10 @@ class OInputs:
             S.bt_cols = self.block_table.shape[1]
             S.cache_seq_lens = arr(self.cache_seq_lens, np.int64)
         S.MAX_TSRC = max_tsrc
+        if self.access is not None:
+            assert self.access.dtype == np.int32 and self.access.flags.c_contiguous and self.access.ndim == 3
+            S.access = self.access.ctypes.data
+            S.access_pages = self.access.shape[2]
         return S, keep
 
 
@@ -251,6 +258,8 @@ class OMetadata:
     ks_count: Optional[np.ndarray]
     ks_start_end: Optional[np.ndarray]
     stage_caches: Optional[List[OStageCache]]
+    mask_access: Optional[np.ndarray] = None  # int32 [B,HKV,pages] (None when the mask was reused)
+    sa_access: Optional[np.ndarray] = None
 
 
 def hip_attention_12(X: OInputs, A: OArgs, cached: Optional[OMetadata] = None):
@@ -281,7 +290,16 @@ def hip_attention_12(X: OInputs, A: OArgs, cached: Optional[OMetadata] = None):
 
     stage_caches = [] if (cached is None or cached.stage_caches is None) else cached.stage_caches
 
+    # access flags (attention_extend.py:1988-2006): one entry per token (dense) or pool page (paged)
+    HKV = X.k.shape[2] if X.k is not None else X.k_cache.shape[2]
+    pages = MAX_TSRC if X.k is not None else X.k_cache.shape[0]
+    mask_access = None
+    sa_access = np.zeros((B, HKV, pages), dtype=np.int32)
+    user_access = X.access
+
     if cached is None or cached.indices is None:
+        mask_access = np.zeros((B, HKV, pages), dtype=np.int32)
+        X.access = mask_access
         fresh = cached is None or cached.stage_caches is None
         # A cache holding only the (empty) stage-0 entry carries no tensors: the reference would fail on
         # None.clone() (attention_extend.py:2052-2056) although its own replay test passes such a list
@@ -405,6 +423,7 @@ def hip_attention_12(X: OInputs, A: OArgs, cached: Optional[OMetadata] = None):
             ks_count = np.repeat(ks_count, rep, 1)
             ks_start_end = np.repeat(ks_start_end, rep, 1)
             block_size_q = bsbq
+        X.access = user_access
         if A.mask_only:
             return None, None
     else:
@@ -421,8 +440,12 @@ def hip_attention_12(X: OInputs, A: OArgs, cached: Optional[OMetadata] = None):
         sw_bsa = A.model_context_length - sink - A.second_stage_k - block_size_q
 
     decode = (TDST == 1) and (not A.disable_flashdecode)
-    context = bsa(X, MAX_TSRC, indices, ks_start_end, block_size_q, block_size_k, sw_bsa, sink,
-                  share_first_head=decode)
+    X.access = sa_access
+    try:
+        context = bsa(X, MAX_TSRC, indices, ks_start_end, block_size_q, block_size_k, sw_bsa, sink,
+                      share_first_head=decode)
+    finally:
+        X.access = user_access
     meta = OMetadata(indices=indices, ks=ks, ks_count=ks_count, ks_start_end=ks_start_end,
-                     stage_caches=stage_caches)
+                     stage_caches=stage_caches, mask_access=mask_access, sa_access=sa_access)
     return context, meta

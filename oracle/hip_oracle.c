@@ -61,6 +61,10 @@ typedef struct {
     int64_t bt_cols;
     const int64_t *cache_seq_lens; /* [B] */
     int64_t MAX_TSRC;        /* TSRC (dense) or extend_context_length (paged) */
+    /* optional access flags int32 [B, HKV, access_pages]: every fetched key row sets the flag of its token
+     * (dense) or page (paged) -- the ACCESS_COUNTER stores of uvm_gpu_cache.py:845-862,893-907 */
+    int32_t *access;
+    int64_t access_pages;
 } hipo_tensors_t;
 
 /* ---------------------------------------------------------------- scalar helpers */
@@ -223,6 +227,7 @@ static void fetch_row(const hipo_tensors_t *X, int want_v, int b, int64_t t, int
             for (int d = 0; d < HID; d++) out[d] = 0.0f;
             return;
         }
+        if (X->access && !want_v) X->access[((int64_t)b * X->HKV + kvh) * X->access_pages + t] = 1;
         int64_t off = (((int64_t)b * X->TSRC + t) * X->HKV + kvh) * HID;
         for (int d = 0; d < HID; d++) out[d] = load_T(base, off + d, X->dtype);
     } else {
@@ -231,6 +236,7 @@ static void fetch_row(const hipo_tensors_t *X, int want_v, int b, int64_t t, int
         int64_t page = 0;
         if (t >= 0 && t < seq_len) page = X->block_table[(int64_t)b * X->bt_cols + t / X->page_size];
         int64_t offp = t % X->page_size;
+        if (X->access && !want_v && t >= 0) X->access[((int64_t)b * X->HKV + kvh) * X->access_pages + page] = 1;
         int64_t off = ((page * X->page_size + offp) * X->HKV + kvh) * HID;
         for (int d = 0; d < HID; d++) out[d] = load_T(base, off + d, X->dtype);
     }

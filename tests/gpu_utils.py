@@ -61,6 +61,15 @@ def assert_metadata_equal(meta, ometa):
     assert np.array_equal(meta.ks.cpu().numpy(), ometa.ks), "ks differ"
     assert np.array_equal(meta.ks_count.cpu().numpy(), ometa.ks_count)
     assert np.array_equal(meta.ks_start_end.cpu().numpy(), ometa.ks_start_end)
+    # access statistics, whenever both sides recorded them
+    for got, want, name in ((meta.mask_cache_statistics, getattr(ometa, "mask_access", None), "mask"),
+                            (meta.sa_cache_statistics, getattr(ometa, "sa_access", None), "attention")):
+        if got is None or got.access_counter is None or want is None:
+            continue
+        a = got.access_counter.cpu().numpy()
+        if a.shape != want.shape:
+            continue  # oracle ran on the dense tensors, product on a paged copy: flags are indexed differently
+        assert np.array_equal(a, want), f"{name} access flags differ in {int((a != want).sum())} entries"
 
 
 def assert_context_close(ctx, octx, dtype):
