@@ -130,36 +130,78 @@ def run_decode(args, device, TK=1 << 20, steps=64, refresh_every=8):
         k[:, s:s + step] = torch.randn((1, step, HKV, D), generator=g, dtype=torch.float32).to(torch.bfloat16).to(device)
     v = k.clone()
     q = torch.randn((1, 1, H, D), generator=g, dtype=torch.float32).to(torch.bfloat16).to(device)
-    hargs = HiPAttentionArgs12(sliding_window_size=1024,
-                               position_ids=torch.full((1, 1), TK - 1, dtype=torch.int64, device=device))
+    pos = torch.full((1, 1), TK - 1, dtype=torch.int64, device=device)
+
+    def step_args(refresh):
+        # statistics only when the mask is estimated, as the serving entry point asks for them (paged_hip.py:400-406)
+        return HiPAttentionArgs12(sliding_window_size=1024, position_ids=pos, require_cache_statistics=refresh)
+
+    def step(meta_in):
+        return hip_attention_12(q, k, v, step_args(meta_in is None), cached_metadata=meta_in)
+
     meta = None
     for i in range(16):
-        _, meta = hip_attention_12(q, k, v, hargs, cached_metadata=None if i % refresh_every == 0 else meta)
+        _, meta = step(None if i % refresh_every == 0 else meta)
     torch.cuda.synchronize()
 
-    def timed(n, cached_fn):
+    def timed(n, fn):
         s_ev = torch.cuda.Event(enable_timing=True)
         e_ev = torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         s_ev.record()
-        m = meta
         for i in range(n):
-            _, m = hip_attention_12(q, k, v, hargs, cached_metadata=cached_fn(i, m))
+            fn(i)
         e_ev.record()
         torch.cuda.synchronize()
         return s_ev.elapsed_time(e_ev) * 1e3 / n
 
-    us_mixed = timed(steps, lambda i, m: None if i % refresh_every == 0 else m)
-    us_refresh = timed(16, lambda i, m: None)
-    us_cached = timed(64, lambda i, m: m)
-    # wall-clock per step including host launch overhead
+    # eager: one Python call per step
+    state = {"m": meta}
+
+    def eager(kind):
+        def run(i):
+            fresh = (i % refresh_every == 0) if kind == "mixed" else (kind == "refresh")
+            _, state["m"] = step(None if fresh else state["m"])
+        return run
+
+    eager_mixed = timed(steps, eager("mixed"))
+    eager_refresh = timed(16, eager("refresh"))
+    eager_cached = timed(64, eager("cached"))
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    m = meta
     for i in range(steps):
-        _, m = hip_attention_12(q, k, v, hargs, cached_metadata=None if i % refresh_every == 0 else m)
+        eager("mixed")(i)
+    torch.cuda.synchronize()
+    eager_wall = (time.perf_counter() - t0) * 1e6 / steps
+
+    # the serving form: the refresh step and the cached step each captured once in a HIP graph and replayed
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        _, m_warm = step(None)
+        step(m_warm)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g_refresh = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g_refresh):
+        out_r, meta_r = step(None)
+    g_cached = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g_cached, pool=g_refresh.pool()):
+        out_c, _ = step(meta_r)
+    torch.cuda.synchronize()
+    us_mixed = timed(steps, lambda i: (g_refresh if i % refresh_every == 0 else g_cached).replay())
+    us_refresh = timed(16, lambda i: g_refresh.replay())
+    us_cached = timed(64, lambda i: g_cached.replay())
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        (g_refresh if i % refresh_every == 0 else g_cached).replay()
     torch.cuda.synchronize()
     wall_us = (time.perf_counter() - t0) * 1e6 / steps
+    # the replayed cached step must agree with an eager one on the same mask
+    eager_out, _ = step(meta_r)
+    torch.cuda.synchronize()
+    graph_matches = bool(torch.equal(eager_out.view(torch.int16), out_c.view(torch.int16)))
 
     sink, sw = 256, 1024
     n0 = cdiv(TK - sink - sw, 256)
@@ -171,13 +213,18 @@ def run_decode(args, device, TK=1 << 20, steps=64, refresh_every=8):
     gbs_refresh = refresh_bytes / (us_refresh * 1e-6) / 1e9
     gbs_cached = attn_bytes / (us_cached * 1e-6) / 1e9
     N.profile_begin()
-    hip_attention_12(q, k, v, hargs)
+    step(None)
     prof = N.profile_end()
+    del g_refresh, g_cached, out_r, out_c, meta_r
     del k, v
     torch.cuda.empty_cache()
     return {
-        "kv_len": TK, "us_per_step_mixed": us_mixed, "us_per_step_refresh": us_refresh,
+        "kv_len": TK, "launch": "hip graph replay (one graph per step kind)",
+        "us_per_step_mixed": us_mixed, "us_per_step_refresh": us_refresh,
         "us_per_step_cached": us_cached, "wall_us_per_step_mixed": wall_us, "refresh_every": refresh_every,
+        "graph_replay_matches_eager": graph_matches,
+        "eager": {"us_per_step_mixed": eager_mixed, "us_per_step_refresh": eager_refresh,
+                  "us_per_step_cached": eager_cached, "wall_us_per_step_mixed": eager_wall},
         "refresh_algorithmic_bytes": refresh_bytes, "cached_algorithmic_bytes": attn_bytes,
         "hbm_frac_refresh": gbs_refresh / HBM_PEAK_GBS, "hbm_frac_cached": gbs_cached / HBM_PEAK_GBS,
         "refresh_GBps": gbs_refresh, "cached_GBps": gbs_cached,

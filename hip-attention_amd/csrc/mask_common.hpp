@@ -22,6 +22,7 @@ struct MaskParamsBase {
     long long total;
     float c_q, c_k;
     float *scores;
+    int reduce_heads;  // scores is [B, BS, 1, n], pre-filled with -inf, and receives the max over heads
     int32_t *left_out;
     const uint16_t *qhat;  // bf16 path: workspace [B, BS, HEAD, nrows, HID] filled by the entry point
 };
@@ -32,6 +33,20 @@ struct MaskParams : MaskParamsBase {
 };
 template <bool EXT>
 using MaskParamsFor = std::conditional_t<EXT, MaskParams, MaskParamsBase>;
+
+// Score of one (head, chunk): a plain store, or the running maximum over heads.  The maximum uses the usual
+// split on the sign (ordered as int for non-negative floats, reverse-ordered as unsigned for negative ones);
+// -0 is folded into +0 first, and the target starts at -inf.
+__device__ __forceinline__ void store_score(const MaskParamsBase &p, int64_t row_out, int64_t red_out, int c, float v) {
+    if (!p.reduce_heads) {
+        p.scores[row_out + c] = v;
+        return;
+    }
+    if (v == 0.0f) v = 0.0f;
+    float *a = p.scores + red_out + c;
+    if (v >= 0.0f) atomicMax(reinterpret_cast<int *>(a), __float_as_int(v));
+    else atomicMin(reinterpret_cast<unsigned int *>(a), __float_as_uint(v));
+}
 
 // bf16 path on the matrix cores (mask_stage_mfma.hip)
 int mask_stage_mfma_launch(const MaskParams &p, int HID, int rows_eff, int prescaled, hipStream_t st);

@@ -80,6 +80,7 @@ __global__ __launch_bounds__(64) void mask_stage_kernel(MaskParams p) {
     const int hgi = p.hg == 1 ? 0 : h;
     const int64_t row_in = (((int64_t)b * p.BS + s) * p.hg + hgi) * p.n;
     const int64_t row_out = (((int64_t)b * p.BS + s) * p.HEAD + h) * p.n;
+    const int64_t red_out = ((int64_t)b * p.BS + s) * p.n;
 
     int l = (int)p.kv.max_tsrc, r = (int)p.kv.max_tsrc;
     if (real) {
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(64) void mask_stage_kernel(MaskParams p) {
     }
     if (!run || !(width >= p.terminate)) {
         if (real) {
-            p.scores[row_out + ci] = score;
+            store_score(p, row_out, red_out, ci, score);
             if (p.left_out) p.left_out[row_out + ci] = l;
         }
         return;
@@ -231,7 +232,7 @@ __global__ __launch_bounds__(64) void mask_stage_kernel(MaskParams p) {
         __syncthreads();
     }
     if (real) {
-        p.scores[row_out + ci] = score;
+        store_score(p, row_out, red_out, ci, score);
         if (p.left_out) p.left_out[row_out + ci] = l;
     }
 }
@@ -266,7 +267,8 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
                                   int32_t hg, int32_t n, int32_t chunk_size, int64_t right_clamp,
                                   int32_t bs, int32_t bq, int32_t stride_q, int32_t block_chunk,
                                   int32_t scan_stride, int32_t sw_eff, int32_t terminate_size,
-                                  int32_t k_prescaled, void *workspace, float *scores, int32_t *left_out, void *stream) {
+                                  int32_t k_prescaled, int32_t reduce_heads, void *workspace, float *scores,
+                                  int32_t *left_out, void *stream) {
     int rc = check_q(q);
     if (rc) return rc;
     HIPATTN_CHECK_ARG(kv && chunk_left && scores, HIPATTN_E_ARG, "mask stage: null pointer");
@@ -298,6 +300,8 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
     HIPATTN_CHECK_ARG(p.total < 0x7fffffffLL, HIPATTN_E_UNSUPPORTED, "mask stage: grid too large");
     scale_constants(q->HID, q->dtype, &p.c_q, &p.c_k);
     p.scores = scores; p.left_out = left_out;
+    p.reduce_heads = reduce_heads ? 1 : 0;
+    HIPATTN_CHECK_ARG(!reduce_heads || hg == 1, HIPATTN_E_ARG, "mask stage: reduce_heads needs one shared chunk list (hg == 1)");
     int rows_max = (q->TDST + stride_q - 1) / stride_q;
     int rows_eff = p.nrows < rows_max ? p.nrows : rows_max;
     if (p.nrows > 64) {

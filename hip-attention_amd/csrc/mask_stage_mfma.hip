@@ -81,6 +81,7 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
     const int hgi = p.hg == 1 ? 0 : h;
     const int64_t row_in = (((int64_t)b * p.BS + s) * p.hg + hgi) * p.n;
     const int64_t row_out = (((int64_t)b * p.BS + s) * p.HEAD + h) * p.n;
+    const int64_t red_out = ((int64_t)b * p.BS + s) * p.n;
 
     // ---- program-level quantities over the whole group of BC chunks
     int gl = (int)p.kv.max_tsrc, gr = (int)p.kv.max_tsrc;
@@ -133,7 +134,7 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
 #pragma unroll
             for (int tb = 0; tb < NB; tb++)
                 if (real[tb]) {
-                    p.scores[row_out + cidx[tb]] = score[tb];
+                    store_score(p, row_out, red_out, cidx[tb], score[tb]);
                     if (p.left_out) p.left_out[row_out + cidx[tb]] = cl[tb];
                 }
         }

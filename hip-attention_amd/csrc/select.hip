@@ -64,19 +64,33 @@ __device__ void topk_threshold(const float *scores_row /* [nheads, n] with strid
             if ((key & mask) == prefix) atomicAdd(&s_hist[(key >> shift) & 255u], 1);
         }
         __syncthreads();
-        if (tid == 0) {
-            int cum = 0, digit = 0, nd = need;
-            for (int bin = 255; bin >= 0; bin--) {
-                int hcount = s_hist[bin];
-                if (cum + hcount >= need) {
-                    digit = bin;
-                    nd = need - cum;
-                    break;
-                }
-                cum += hcount;
+        if (tid < 64) {
+            // first wave: lane l owns bins 255-4l .. 252-4l; a prefix sum from the top finds the bin in which
+            // the need-th largest key falls
+            int hv[4];
+            int mine = 0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                hv[j] = s_hist[255 - 4 * tid - j];
+                mine += hv[j];
             }
-            s_misc[0] = digit;
-            s_misc[1] = nd;
+            int incl = mine;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const int up = __shfl_up(incl, o);
+                if (tid >= o) incl += up;
+            }
+            int cum = incl - mine;
+            if (cum < need && need <= incl) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    if (cum < need && need <= cum + hv[j]) {
+                        s_misc[0] = 255 - 4 * tid - j;
+                        s_misc[1] = need - cum;
+                    }
+                    cum += hv[j];
+                }
+            }
         }
         __syncthreads();
         prefix |= ((uint32_t)s_misc[0]) << shift;
@@ -161,22 +175,28 @@ __global__ __launch_bounds__(SEL_THREADS) void select_stage_kernel(const float *
 
 __global__ __launch_bounds__(SEL_THREADS) void finalize_kernel(const float *scores, const int32_t *left_out,
                                                                const int64_t *pos, int64_t pos_sb, int64_t pos_st,
-                                                               int bs, int bdst, int scan_stride, int HEAD, int hg,
-                                                               int n, int K, int chunk, int bq, int64_t *indices,
-                                                               int64_t *ks, int32_t *ks_start_end) {
+                                                               int bs, int bdst, int scan_stride, int HEAD,
+                                                               int score_heads, int hg, int hsplit, int n, int K,
+                                                               int chunk, int bq, int64_t *indices, int64_t *ks,
+                                                               int32_t *ks_start_end) {
     __shared__ uint32_t s_keys[SEL_MAX_N];
     __shared__ int s_hist[256];
     __shared__ int s_misc[2];
     __shared__ int s_tmp[SEL_THREADS / 64];
     int *s_sel = reinterpret_cast<int *>(s_keys);  // reused after selection: positions of selected chunks
 
-    const int hgi = blockIdx.x % hg;
-    const int qb = (blockIdx.x / hg) % bdst;
-    const int b = blockIdx.x / (hg * bdst);
+    // workgroup = (batch, query block, head group, slice of the group's heads): every slice repeats the
+    // selection, then lays out the rows of its own heads
+    const int hs = blockIdx.x % hsplit;
+    const int wg = blockIdx.x / hsplit;
+    const int hgi = wg % hg;
+    const int qb = (wg / hg) % bdst;
+    const int b = wg / (hg * bdst);
     const int i = (qb + scan_stride * bs - bdst) / scan_stride;
     const int nheads = HEAD / hg;
+    const int nsh = score_heads / hg;
     const int BK = K < n ? K : n;
-    const float *srow = scores + (((int64_t)b * bs + i) * HEAD + (int64_t)hgi * nheads) * n;
+    const float *srow = scores + (((int64_t)b * bs + i) * score_heads + (int64_t)hgi * nsh) * n;
 
     uint32_t thr;
     int need;
@@ -186,7 +206,7 @@ __global__ __launch_bounds__(SEL_THREADS) void finalize_kernel(const float *scor
         for (int c = threadIdx.x; c < n; c += SEL_THREADS) s_keys[c] = 1u;
         __syncthreads();
     } else {
-        topk_threshold(srow, nheads, n, BK, s_keys, s_hist, s_misc, &thr, &need);
+        topk_threshold(srow, nsh, n, BK, s_keys, s_hist, s_misc, &thr, &need);
     }
     SegScan sc = selection_scan(s_keys, n, thr, need, s_tmp);
     // each thread lists its selected positions in registers first (keys are still being read by others)
@@ -212,7 +232,9 @@ __global__ __launch_bounds__(SEL_THREADS) void finalize_kernel(const float *scor
     const int per = (BK + SEL_THREADS - 1) / SEL_THREADS;
     const int o0 = threadIdx.x * per;
     const int o1 = o0 + per < BK ? o0 + per : BK;
-    for (int hh = 0; hh < nheads; hh++) {
+    const int hper = (nheads + hsplit - 1) / hsplit;
+    const int hh_end = (hs + 1) * hper < nheads ? (hs + 1) * hper : nheads;
+    for (int hh = hs * hper; hh < hh_end; hh++) {
         const int h = hgi * nheads + hh;
         const int32_t *lrow = left_out + (((int64_t)b * bs + i) * HEAD + h) * n;
         int64_t *irow = indices + (((int64_t)b * HEAD + h) * bdst + qb) * BK;
@@ -273,20 +295,29 @@ extern "C" int hipattn_select_stage(const float *scores, const int32_t *chunk_le
 
 extern "C" int hipattn_finalize_indices(const float *scores, const int32_t *left_out, const int64_t *pos,
                                         int64_t pos_stride_b, int64_t pos_stride_t, int32_t B, int32_t bs,
-                                        int32_t bdst, int32_t scan_stride, int32_t HEAD, int32_t hg, int32_t n,
-                                        int32_t K, int32_t chunk_size, int32_t bq, int64_t *indices, int64_t *ks,
-                                        int32_t *ks_start_end, void *stream) {
+                                        int32_t bdst, int32_t scan_stride, int32_t HEAD, int32_t score_heads,
+                                        int32_t hg, int32_t n, int32_t K, int32_t chunk_size, int32_t bq,
+                                        int64_t *indices, int64_t *ks, int32_t *ks_start_end, void *stream) {
     HIPATTN_CHECK_ARG(scores && left_out && pos && indices && ks && ks_start_end, HIPATTN_E_ARG,
                       "finalize: null pointer");
     HIPATTN_CHECK_ARG(B > 0 && bs > 0 && bdst > 0 && scan_stride > 0 && HEAD > 0 && n > 0 && K > 0 && chunk_size > 0 &&
                           bq > 0,
                       HIPATTN_E_ARG, "finalize: non-positive size");
     HIPATTN_CHECK_ARG(hg == 1 || hg == HEAD, HIPATTN_E_ARG, "finalize: hg must be 1 or HEAD");
+    HIPATTN_CHECK_ARG(score_heads == HEAD || (score_heads == 1 && hg == 1), HIPATTN_E_ARG,
+                      "finalize: score_heads must be HEAD, or 1 with hg == 1");
     HIPATTN_CHECK_ARG(bdst <= scan_stride * bs, HIPATTN_E_ARG, "finalize: bdst > scan_stride*bs");
     HIPATTN_CHECK_ARG(n <= SEL_MAX_N, HIPATTN_E_UNSUPPORTED, "finalize: %d chunks exceed the limit %d", n, SEL_MAX_N);
-    dim3 grid((unsigned)(B * bdst * hg)), block(SEL_THREADS);
+    // few query blocks (decode): slice each group's heads over several workgroups so that the chip is not idle
+    const long long groups = (long long)B * bdst * hg;
+    const int nheads = HEAD / hg;
+    int hsplit = 1;
+    while (hsplit < nheads && groups * hsplit < 512) hsplit *= 2;
+    if (hsplit > nheads) hsplit = nheads;
+    dim3 grid((unsigned)(groups * hsplit)), block(SEL_THREADS);
     hipLaunchKernelGGL(finalize_kernel, grid, block, 0, (hipStream_t)stream, scores, left_out, pos, pos_stride_b,
-                       pos_stride_t, bs, bdst, scan_stride, HEAD, hg, n, K, chunk_size, bq, indices, ks, ks_start_end);
+                       pos_stride_t, bs, bdst, scan_stride, HEAD, score_heads, hg, hsplit, n, K, chunk_size, bq, indices,
+                       ks, ks_start_end);
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
 }

@@ -240,7 +240,7 @@ def prescale_k(k: torch.Tensor, device) -> torch.Tensor:
 
 
 def mask_stage(qs, kvs, chunk_left, hg, n, chunk, right_clamp, bs, bq, stride_q, block_chunk, scan_stride,
-               sw_eff, terminate, scores, left_out, device, k_prescaled=False):
+               sw_eff, terminate, scores, left_out, device, k_prescaled=False, reduce_heads=False):
     need = lib().hipattn_mask_stage_workspace_bytes(
         ctypes.c_int32(qs.dtype), ctypes.c_int32(qs.B), ctypes.c_int32(bs), ctypes.c_int32(qs.HEAD),
         ctypes.c_int32(qs.HID), ctypes.c_int32(bq), ctypes.c_int32(stride_q))
@@ -250,7 +250,8 @@ def mask_stage(qs, kvs, chunk_left, hg, n, chunk, right_clamp, bs, bq, stride_q,
         ctypes.byref(qs), ctypes.byref(kvs), _p(chunk_left), ctypes.c_int32(hg), ctypes.c_int32(n),
         ctypes.c_int32(chunk), ctypes.c_int64(right_clamp), ctypes.c_int32(bs), ctypes.c_int32(bq),
         ctypes.c_int32(stride_q), ctypes.c_int32(block_chunk), ctypes.c_int32(scan_stride),
-        ctypes.c_int32(sw_eff), ctypes.c_int32(terminate), ctypes.c_int32(int(k_prescaled)), _p(workspace),
+        ctypes.c_int32(sw_eff), ctypes.c_int32(terminate), ctypes.c_int32(int(k_prescaled)),
+        ctypes.c_int32(int(reduce_heads)), _p(workspace),
         _p(scores),
         _p(left_out), stream_ptr(device))
     check(rc, "hipattn_mask_stage")
@@ -265,13 +266,14 @@ def select_stage(scores, chunk_left, B, bs_in, bs_out, row_rep, HEAD, hg, n, k, 
     check(rc, "hipattn_select_stage")
 
 
-def finalize_indices(scores, left_out, pos, B, bs, bdst, scan_stride, HEAD, hg, n, K, chunk, bq,
+def finalize_indices(scores, left_out, pos, B, bs, bdst, scan_stride, HEAD, score_heads, hg, n, K, chunk, bq,
                      indices, ks, ks_start_end, device):
     with _timed("finalize_indices"):
       rc = lib().hipattn_finalize_indices(
         _p(scores), _p(left_out), _p(pos), ctypes.c_int64(pos.stride(0)), ctypes.c_int64(pos.stride(1)),
         ctypes.c_int32(B), ctypes.c_int32(bs), ctypes.c_int32(bdst), ctypes.c_int32(scan_stride),
-        ctypes.c_int32(HEAD), ctypes.c_int32(hg), ctypes.c_int32(n), ctypes.c_int32(K), ctypes.c_int32(chunk),
+        ctypes.c_int32(HEAD), ctypes.c_int32(score_heads), ctypes.c_int32(hg), ctypes.c_int32(n), ctypes.c_int32(K),
+        ctypes.c_int32(chunk),
         ctypes.c_int32(bq), _p(indices), _p(ks), _p(ks_start_end), stream_ptr(device))
     check(rc, "hipattn_finalize_indices")
 

@@ -284,7 +284,7 @@ def dual_stage_quadratic_hip_attention(
                 splits = chunk_size // stage.stage_chunk_size
                 next_left = torch.empty((BSZ, bs_out, hg, keep * splits), dtype=torch.int32, device=device)
                 if keep > 0:
-                    N.select_stage(scores, chunk_left, BSZ, bs_in, bs_out, row_rep, HEAD, hg, prev_n, keep,
+                    N.select_stage(scores, chunk_left, BSZ, bs_in, bs_out, row_rep, scores.shape[2], hg, prev_n, keep,
                                    chunk_size, splits, next_left, device)
                 chunk_left = next_left
                 right_clamp = _BIG
@@ -308,15 +308,22 @@ def dual_stage_quadratic_hip_attention(
             last = i_stage == len(stages) - 1
 
             if isinstance(stage, ScanStage):
-                scores = torch.empty((BSZ, bs, HEAD, chunk_count), dtype=torch.float32, device=device)
+                # one shared chunk list: the scan kernels fold the maximum over heads into their score store
+                reduce = hg == 1
+                if reduce:
+                    scores = torch.full((BSZ, bs, 1, chunk_count), float("-inf"), dtype=torch.float32, device=device)
+                else:
+                    scores = torch.empty((BSZ, bs, HEAD, chunk_count), dtype=torch.float32, device=device)
                 left_out = torch.empty((BSZ, bs, HEAD, chunk_count), dtype=torch.int32, device=device) if last else None
                 if chunk_count > 0:
                     qs = N.make_q(qq, position_ids)
                     N.mask_stage(qs, mask_kv, chunk_left, hg, chunk_count, chunk_size, right_clamp, bs,
                                  BLOCK_SIZE_Q, stage.stage_block_stride_q, BLOCK_CHUNK, STAGE_STRIDE, sw_eff,
-                                 args.stage_early_terminate, scores, left_out, device, k_prescaled=k_prescaled)
+                                 args.stage_early_terminate, scores, left_out, device, k_prescaled=k_prescaled,
+                                 reduce_heads=reduce)
             elif isinstance(stage, NopStage):
-                scores = torch.full((BSZ, bs, HEAD, chunk_count), -32000.0, dtype=torch.float32, device=device)
+                scores = torch.full((BSZ, bs, 1 if hg == 1 else HEAD, chunk_count), -32000.0, dtype=torch.float32,
+                                    device=device)
                 left_out = chunk_left.expand(BSZ, bs, HEAD, chunk_count).contiguous() if last else None
             else:
                 raise NotImplementedError(f"stage type {type(stage).__name__} raises in the reference as well")
@@ -331,8 +338,8 @@ def dual_stage_quadratic_hip_attention(
         ks = torch.empty((BSZ * HEAD, BDST), dtype=torch.int64, device=device)
         ks_start_end = torch.empty((BSZ * HEAD, BDST, 2), dtype=torch.int32, device=device)
         if BK > 0:
-            N.finalize_indices(scores, left_out, position_ids, BSZ, chunk_left.shape[1], BDST, STAGE_STRIDE, HEAD, hg,
-                               chunk_count, K, chunk_size, stages[-1].stage_block_size_q, indices, ks, ks_start_end,
+            N.finalize_indices(scores, left_out, position_ids, BSZ, chunk_left.shape[1], BDST, STAGE_STRIDE, HEAD,
+                               scores.shape[2], hg, chunk_count, K, chunk_size, stages[-1].stage_block_size_q, indices, ks, ks_start_end,
                                device)
         else:
             indices = indices[:, :, :0]

@@ -82,7 +82,9 @@ const char *hipattn_last_error(void);
  *   chunk_left  int32 [B, BS, HG, n]   start of every candidate chunk, ascending; HG = 1 when
  *                                      scores are max-reduced over heads, else HEAD
  *   right = min(left + chunk_size, right_clamp)
- *   scores      f32   [B, BS, HEAD, n] written for every chunk (-32000 where not scored)
+ *   scores      f32   [B, BS, HEAD, n] written for every chunk (-32000 where not scored); with
+ *                     reduce_heads != 0 (needs hg == 1): [B, BS, 1, n], filled with -inf by the caller,
+ *                     receives the maximum over heads (the torch.max at :2566-2570 folded into the scan)
  *   left_out    int32 [B, BS, HEAD, n] refined left edge per head, or NULL
  *   block_chunk = chunks per reference program (16/32/64): fixes the program-level gate and
  *   iteration count (:595-601,736-737).
@@ -92,8 +94,8 @@ int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, const int32
                        int32_t hg, int32_t n, int32_t chunk_size, int64_t right_clamp,
                        int32_t bs, int32_t bq, int32_t stride_q, int32_t block_chunk,
                        int32_t scan_stride, int32_t sw_eff, int32_t terminate_size,
-                       int32_t k_prescaled, void *workspace, float *scores, int32_t *left_out,
-                       void *stream);
+                       int32_t k_prescaled, int32_t reduce_heads, void *workspace, float *scores,
+                       int32_t *left_out, void *stream);
 
 /* Bytes of caller-allocated scratch hipattn_mask_stage needs (bf16: the averaged, scaled query rows
  * of every scan program, [B, BS, HEAD, bq/stride_q, HID]; f32: 0, workspace may be NULL). */
@@ -110,7 +112,7 @@ int hipattn_prescale_k(const void *k, int64_t stride0, int64_t stride1, int64_t 
 /* Between two stages: max over heads, top-k under (score desc, position asc), realign, split.
  * Replaces the ATen glue at src/hip_attn/v1_2/attention_extend.py:2566-2570 (head reduce),
  * :2710-2728 (topk + gather) and :2072-2165 (truncate, realign, sort, re-tile, split).
- *   scores      f32   [B, BS_in, HEAD, n]
+ *   scores      f32   [B, BS_in, HEAD, n]  (HEAD = 1 for scores already reduced over heads)
  *   chunk_left  int32 [B, BS_in, HG, n]
  *   next_left   int32 [B, BS_out, HG, k*splits]; chunk j of a kept parent starts at
  *               left + j*(chunk_size/splits)
@@ -124,6 +126,7 @@ int hipattn_select_stage(const float *scores, const int32_t *chunk_left, int32_t
 /* After the last stage: top-K chunks, block alignment, de-duplication, active count, in the
  * reference's metadata layout.  Replaces src/hip_attn/v1_2/attention_extend.py:2757-2776 and
  * :2906-2924.
+ *   scores      f32   [B, BS, score_heads, n], score_heads = HEAD or 1 (already reduced, needs hg == 1)
  *   left_out    int32 [B, BS, HEAD, n]  refined left edges from the last hipattn_mask_stage
  *   indices     int64 [B*HEAD, BDST, BK] ascending unique block starts then INT64_MAX
  *   ks          int64 [B*HEAD, BDST]     entries below pos[b, qb*bq] + bq
@@ -131,8 +134,8 @@ int hipattn_select_stage(const float *scores, const int32_t *chunk_left, int32_t
  *   BK = min(K, n); output row qb reads scan row (qb + scan_stride*BS - BDST) / scan_stride. */
 int hipattn_finalize_indices(const float *scores, const int32_t *left_out, const int64_t *pos,
                              int64_t pos_stride_b, int64_t pos_stride_t, int32_t B, int32_t bs,
-                             int32_t bdst, int32_t scan_stride, int32_t HEAD, int32_t hg, int32_t n,
-                             int32_t K, int32_t chunk_size, int32_t bq, int64_t *indices,
+                             int32_t bdst, int32_t scan_stride, int32_t HEAD, int32_t score_heads, int32_t hg,
+                             int32_t n, int32_t K, int32_t chunk_size, int32_t bq, int64_t *indices,
                              int64_t *ks, int32_t *ks_start_end, void *stream);
 
 /* Block-sparse flash attention over selected blocks + sink + sliding window.  Replaces
