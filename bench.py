@@ -9,6 +9,8 @@ attention) on synthetic inputs already resident in HBM.  ``value`` = queries / s
 Also reported in the same JSON line:
   * ``decode``: a 1M-token KV decode loop (configs[3] phase B: mask refreshed every 8 steps),
     microseconds per step and the HBM roofline fraction of a refresh step;
+  * ``offload``: configs[4], a 3M-token KV held in pinned host memory behind a 16 GB HBM block cache: cold,
+    warm and drifting-query decode steps beside the same steps with the KV resident;
   * ``roofline``: the dominant kernel of the prefill step, timed with HIP events inside the timed
     region, against its algorithmic bytes (mask stage: sampled key rows) or flops (attention);
   * ``cpu_baseline``: the CPU oracle (a port of the reference algorithm, OpenMP) on a bounded sample
@@ -232,6 +234,132 @@ def run_decode(args, device, TK=1 << 20, steps=64, refresh_every=8):
     }
 
 
+def run_offload(args, device, TK=3_000_000, warm_steps=4, drift_steps=12):
+    """configs[4]: one layer, 3M keys in pinned host memory, 16 GB of HBM cache, batch 1 decode.
+
+    The key-only cache for mask estimation is sized to hold every key block (6.1 GB), the key+value cache
+    for attention gets the rest of the 16 GB budget.  Reported: a resident run of the same steps, the cold
+    step (every read goes to host memory), warm steps (every read served from HBM), and a drifting-query
+    phase in which each refresh selects partly new blocks, with the measured miss fraction.
+    """
+    import torch
+    from hip_attn import HiPAttentionArgs12, HiPOffloadCache, hip_attention_12
+
+    H, HKV, D, BT = 32, 8, 128, 16
+    blocks = cdiv(TK + 1, BT)
+    mask_slots = blocks * HKV
+    budget = 16 * (1 << 30)
+    sa_slots = (budget - mask_slots * BT * D * 2) // (2 * BT * D * 2)
+    cache = HiPOffloadCache(0, TK + 1, mask_slots * BT, sa_slots * BT, HKV, D, torch.bfloat16, device,
+                            block_tokens=BT, max_fetch=1 << 20)
+    g = torch.Generator(device="cpu").manual_seed(4)
+    chunk = 1 << 17
+    for s0 in range(0, TK, chunk):
+        n = min(chunk, TK - s0)
+        rows = torch.arange(s0, s0 + n, dtype=torch.int64, device=device)
+        kc = torch.randn((n, HKV, D), generator=g, dtype=torch.float32).to(torch.bfloat16).to(device)
+        cache.set_kv_buffer(rows, rows, kc, kc)
+    torch.cuda.synchronize()
+    bt = torch.arange(0, TK, dtype=torch.int32, device=device)[None]
+    sl = torch.tensor([TK], dtype=torch.int32, device=device)
+    pos = torch.full((1, 1), TK - 1, dtype=torch.int64, device=device)
+    q0 = torch.randn((1, 1, H, D), generator=g, dtype=torch.float32)
+    noise = [torch.randn((1, 1, H, D), generator=g, dtype=torch.float32) for _ in range(drift_steps)]
+
+    def call(q, meta=None, resident=None):
+        kw = dict(sliding_window_size=1024, position_ids=pos, block_table=bt, cache_seq_lens=sl,
+                  extend_context_length=TK, require_cache_statistics=False)
+        if resident is None:
+            kw["offload_cache"] = cache
+        else:
+            kw["k_cache"], kw["v_cache"] = resident
+        return hip_attention_12(q, None, None, HiPAttentionArgs12(**kw), cached_metadata=meta)
+
+    def timed(fn, n=1):
+        s_ev = torch.cuda.Event(enable_timing=True)
+        e_ev = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        s_ev.record()
+        for _ in range(n):
+            r = fn()
+        e_ev.record()
+        torch.cuda.synchronize()
+        return s_ev.elapsed_time(e_ev) * 1e3 / n, r
+
+    q = q0.to(torch.bfloat16).to(device)
+    # --- offloaded: cold step, then repeat the step until both caches serve everything
+    us_cold, (out_cold, meta) = timed(lambda: call(q))
+    us_commit_cold, _ = timed(lambda: cache.handle_cache_miss(meta))
+    cold_stats = (cache.mask_k_cache.statistics(), cache.sa_kv_cache.statistics())
+    warmup_steps = 0
+    for _ in range(32):
+        _, meta = call(q)
+        cache.handle_cache_miss(meta)
+        warmup_steps += 1
+        if cache.mask_k_cache.statistics()["last_missed"] == 0 and cache.sa_kv_cache.statistics()["last_missed"] == 0:
+            break
+    us_warm_refresh, (out_warm, meta) = timed(lambda: call(q), 8)
+    us_warm_cached, (out_warm_c, _) = timed(lambda: call(q, meta), 32)
+    cache.handle_cache_miss(meta)
+    warm_stats = (cache.mask_k_cache.statistics(), cache.sa_kv_cache.statistics())
+    us_commit_idle, _ = timed(lambda: cache.handle_cache_miss(meta), 8)
+
+    # --- drifting query: each refresh selects partly new blocks.  The blend is picked from a short list so
+    # that about a tenth of the attention blocks miss; the measured fraction is what gets reported.
+    def drift_step(qd):
+        us_step, (_, md) = timed(lambda: call(qd))
+        us_commit, _ = timed(lambda: cache.handle_cache_miss(md))
+        st, sm = cache.sa_kv_cache.statistics(), cache.mask_k_cache.statistics()
+        return {"step_us": us_step, "commit_us": us_commit,
+                "miss_fraction": st["last_missed"] / max(1, st["last_hit"] + st["last_missed"]),
+                "fetched_blocks": st["last_fetched"] + sm["last_fetched"], "mask_cache_missed": sm["last_missed"],
+                "mask_miss_fraction": sm["last_missed"] / max(1, sm["last_hit"] + sm["last_missed"])}
+
+    def blended(a, nz):
+        return ((1 - a) * q0 + a * nz).to(torch.bfloat16).to(device)
+
+    trial = {}
+    for a in (0.02, 0.05, 0.1, 0.2):
+        trial[a] = drift_step(blended(a, noise[0]))["miss_fraction"]
+        call(q)  # back to the base query so that trials do not build on each other
+    blend = min(trial, key=lambda a: abs(trial[a] - 0.10))
+    drift = [drift_step(blended(blend, nz)) for nz in noise]
+    # --- the same data resident in HBM
+    kres = cache.k_uvm.bank_cpu.to(device).unsqueeze(1)
+    resident = (kres, kres)
+    out_res, meta_res = call(q, resident=resident)
+    us_res_refresh, _ = timed(lambda: call(q, resident=resident), 8)
+    us_res_cached, _ = timed(lambda: call(q, meta_res, resident=resident), 32)
+    same = bool(torch.equal(out_res.view(torch.int16), out_cold.view(torch.int16)) and
+                torch.equal(out_res.view(torch.int16), out_warm.view(torch.int16)) and
+                torch.equal(meta_res.indices, meta.indices))
+    tail = drift[2:]
+    block_bytes = 2 * BT * D * 2  # upper bound per fetched block (key-only blocks are half of it)
+    res = {
+        "kv_len": TK, "host_pool_GB": 2 * (TK + 1) * HKV * D * 2 / 1e9,
+        "hbm_cache_GB": (mask_slots * BT * D * 2 + sa_slots * block_bytes) / 1e9, "block_tokens": BT,
+        "resident_us": {"refresh": us_res_refresh, "cached": us_res_cached},
+        "offload_cold_us": {"refresh": us_cold, "commit": us_commit_cold,
+                            "blocks_fetched": [cold_stats[0]["last_fetched"], cold_stats[1]["last_fetched"]]},
+        "offload_warm_us": {"refresh": us_warm_refresh, "cached": us_warm_cached, "commit_nothing_to_fetch": us_commit_idle,
+                            "steps_until_warm": warmup_steps,
+                            "missed_last_step": [warm_stats[0]["last_missed"], warm_stats[1]["last_missed"]]},
+        "drifting_query": {
+            "blend": blend, "blend_trials": trial, "steps": len(tail),
+            "mask_miss_fraction": sum(d["mask_miss_fraction"] for d in tail) / len(tail),
+            "miss_fraction": sum(d["miss_fraction"] for d in tail) / len(tail),
+            "refresh_us": sum(d["step_us"] for d in tail) / len(tail),
+            "commit_us": sum(d["commit_us"] for d in tail) / len(tail),
+            "fetched_MB_per_step": sum(d["fetched_blocks"] for d in tail) / len(tail) * block_bytes / 1e6,
+            "mask_cache_missed": sum(d["mask_cache_missed"] for d in tail),
+        },
+        "offloaded_equals_resident": same,
+    }
+    del cache, kres, resident
+    torch.cuda.empty_cache()
+    return res
+
+
 def run_cpu_baseline(args):
     """The CPU oracle on a bounded sample of the prefill workload: last 128 queries, all heads, full keys."""
     import numpy as np
@@ -264,6 +392,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--skip-decode", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--skip-offload", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; every figure is one MI355X's throughput (--gpus 1).",
@@ -275,6 +404,7 @@ def main():
     torch.cuda.set_device(device)
     pre = run_prefill(args, device)
     dec = None if args.skip_decode else run_decode(args, device)
+    off = None if args.skip_offload else run_offload(args, device)
     cpu = None if args.skip_cpu else run_cpu_baseline(args)
     dom = pre["dominant"] or {}
     line = {
@@ -297,6 +427,7 @@ def main():
         "roofline_all": pre["rooflines"],
         "kernels_ms": pre["kernels_ms"],
         "decode": dec,
+        "offload": off,
         "cpu_baseline": cpu,
     }
     print(json.dumps(line))

@@ -364,38 +364,38 @@ __global__ __launch_bounds__(CT_THREADS) void cache_emit_kernel(CacheDev c) {
     }
 }
 
-// one workgroup per fetched block: unlink the victim, copy host -> bank, link
+// a workgroup per fetched block (grid-stride over the list): unlink the victim, copy host -> bank, link
 __global__ __launch_bounds__(CT_THREADS) void cache_fetch_kernel(CacheDev c) {
-    const int i = blockIdx.x;
-    if (i >= c.ctl[C_M]) return;
-    const int32_t e = c.miss_list[i];
-    const int32_t slot = c.victim_list[i];
-    const int64_t h = e / c.n_blocks, blk = e % c.n_blocks;
+    const int m = c.ctl[C_M];
     const int pieces_per_row = (int)(c.row_bytes / 16);
-    const int parts = 1 + c.with_v;
-    const int total = c.block_tokens * pieces_per_row * parts;
-    char *dst = c.bank + (int64_t)slot * c.slot_bytes;
-    for (int w = threadIdx.x; w < total; w += CT_THREADS) {
-        const int part = w / (c.block_tokens * pieces_per_row);
-        const int r = (w / pieces_per_row) % c.block_tokens;
-        const int piece = w % pieces_per_row;
-        const int64_t row = (blk << c.shift) + r;
-        uint4 val = make_uint4(0, 0, 0, 0);
-        if (row < c.pool_rows) {
-            const char *src = (part ? c.host_v : c.host_k) + row * c.host_stride_row_b + h * c.host_stride_h_b;
-            val = *reinterpret_cast<const uint4 *>(src + piece * 16);
+    const int total = c.block_tokens * pieces_per_row * (1 + c.with_v);
+    for (int i = blockIdx.x; i < m; i += gridDim.x) {
+        const int32_t e = c.miss_list[i];
+        const int32_t slot = c.victim_list[i];
+        const int64_t h = e / c.n_blocks, blk = e % c.n_blocks;
+        char *dst = c.bank + (int64_t)slot * c.slot_bytes;
+        for (int w = threadIdx.x; w < total; w += CT_THREADS) {
+            const int part = w / (c.block_tokens * pieces_per_row);
+            const int r = (w / pieces_per_row) % c.block_tokens;
+            const int piece = w % pieces_per_row;
+            const int64_t row = (blk << c.shift) + r;
+            uint4 val = make_uint4(0, 0, 0, 0);
+            if (row < c.pool_rows) {
+                const char *src = (part ? c.host_v : c.host_k) + row * c.host_stride_row_b + h * c.host_stride_h_b;
+                val = *reinterpret_cast<const uint4 *>(src + piece * 16);
+            }
+            *reinterpret_cast<uint4 *>(dst + ((int64_t)part * c.block_tokens + r) * c.row_bytes + piece * 16) = val;
         }
-        *reinterpret_cast<uint4 *>(dst + ((int64_t)part * c.block_tokens + r) * c.row_bytes + piece * 16) = val;
-    }
-    if (threadIdx.x == 0) {
-        const int32_t old = c.backref[slot];
-        if (old >= 0) {
-            c.table[old] = -1;
-            atomicAdd(c.ctl + C_EVICTED, 1);
+        if (threadIdx.x == 0) {
+            const int32_t old = c.backref[slot];
+            if (old >= 0) {
+                c.table[old] = -1;
+                atomicAdd(c.ctl + C_EVICTED, 1);
+            }
+            c.backref[slot] = e;
+            c.table[e] = slot;
+            c.last_use[slot] = *c.step;
         }
-        c.backref[slot] = e;
-        c.table[e] = slot;
-        c.last_use[slot] = *c.step;
     }
 }
 
@@ -634,7 +634,9 @@ extern "C" int hipattn_cache_commit(hipattn_cache_t *c, void *stream) {
     HIPATTN_CHECK_ARG(c, HIPATTN_E_ARG, "cache: null handle");
     hipStream_t st = (hipStream_t)stream;
     const CacheDev v = dev_of(c);
-    hipLaunchKernelGGL(cache_fetch_kernel, dim3((unsigned)c->max_fetch), dim3(CT_THREADS), 0, st, v);
+    // a bounded grid walks the fetch list: how many blocks there are is only known on the device
+    const unsigned fetch_grid = (unsigned)(c->max_fetch < 4096 ? c->max_fetch : 4096);
+    hipLaunchKernelGGL(cache_fetch_kernel, dim3(fetch_grid), dim3(CT_THREADS), 0, st, v);
     hipLaunchKernelGGL(cache_step_kernel, dim3(1), dim3(64), 0, st, v);
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
