@@ -30,6 +30,16 @@ for _p in (ROOT, os.path.join(ROOT, "hip-attention_amd"), os.path.join(ROOT, "te
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
+# HBM bytes per launch of the prefill kernels, from two rocprofv3 --pmc runs of this file (FETCH_SIZE, then
+# WRITE_SIZE, KiB per dispatch).  A 268 435 456-byte device copy reads 131 094 KiB of FETCH_SIZE and 262 144 KiB of
+# WRITE_SIZE in the same runs, so FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0.
+MEASURED_TRAFFIC_BYTES = {
+    "mask_stage[n=507,chunk=256,rows=16]": 2.0 * 772743.5 * 1024 + 53366.8 * 1024,
+    "mask_stage[n=1024,chunk=32,rows=16]": 2.0 * 2149794.1 * 1024 + 65683.6 * 1024,
+    "mask_stage[n=1024,chunk=8,rows=64]": 2.0 * 3694235.9 * 1024 + 131098.5 * 1024,
+    "bsa_prefill": 2.0 * 1831309.1 * 1024 + 262144.0 * 1024,
+}
+
 
 def cdiv(a, b):
     return -(-a // b)
@@ -98,12 +108,13 @@ def run_prefill(args, device):
         if nm in kern:
             gbs = by / (kern[nm] * 1e-3) / 1e9
             rooflines.append({"kernel": nm, "bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                              "frac": gbs / HBM_PEAK_GBS, "traffic": None, "ms": kern[nm],
+                              "frac": gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(nm), "ms": kern[nm],
                               "algorithmic_bytes": by})
     if "bsa_prefill" in kern:
         tf = bsa_flops / (kern["bsa_prefill"] * 1e-3) / 1e12
         rooflines.append({"kernel": "bsa_prefill", "bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS,
-                          "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                          "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS,
+                          "traffic": MEASURED_TRAFFIC_BYTES.get("bsa_prefill"),
                           "ms": kern["bsa_prefill"], "algorithmic_flops": bsa_flops})
     dominant = max(rooflines, key=lambda r: r["ms"]) if rooflines else None
     del q, k, v, ctx, meta
@@ -367,7 +378,7 @@ def run_cpu_baseline(args):
     from oracle import hip12 as O
 
     TQ_full, TK, H, HKV, D = 32768, 131072, 32, 8, 128
-    TQs = 128
+    TQs = 512
     g = torch.Generator(device="cpu").manual_seed(1)
     q = torch.randn((1, TQ_full, H, D), generator=g, dtype=torch.float32).to(torch.bfloat16)[:, -TQs:]
     k = torch.randn((1, TK, HKV, D), generator=g, dtype=torch.float32).to(torch.bfloat16)
@@ -381,7 +392,7 @@ def run_cpu_baseline(args):
     O.hip_attention_12(X, A)
     dt = time.perf_counter() - t0
     return {"value": TQs / dt, "unit": "tok/s", "cores": int(threads), "kind": "port",
-            "sample": f"last {TQs} of 32768 queries (2 query blocks) x 32 heads against all 131072 keys, "
+            "sample": f"last {TQs} of 32768 queries ({TQs // 64} query blocks) x 32 heads against all 131072 keys, "
                       f"{dt:.1f} s of CPU time; throughput is per query token, so it compares directly"}
 
 
@@ -393,6 +404,8 @@ def main():
     ap.add_argument("--skip-decode", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-offload", action="store_true")
+    ap.add_argument("--only", choices=["prefill", "decode", "offload", "cpu"], default=None,
+                    help="profiling aid: run one part; the other fields of the JSON line are null")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; every figure is one MI355X's throughput (--gpus 1).",
@@ -402,10 +415,12 @@ def main():
 
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
-    pre = run_prefill(args, device)
-    dec = None if args.skip_decode else run_decode(args, device)
-    off = None if args.skip_offload else run_offload(args, device)
-    cpu = None if args.skip_cpu else run_cpu_baseline(args)
+    want = (lambda part: args.only in (None, part))
+    pre = run_prefill(args, device) if want("prefill") else {
+        "tok_per_s": None, "ms_per_step": None, "rooflines": [], "kernels_ms": {}, "dominant": None}
+    dec = run_decode(args, device) if (want("decode") and not args.skip_decode) else None
+    off = run_offload(args, device) if (want("offload") and not args.skip_offload) else None
+    cpu = run_cpu_baseline(args) if (want("cpu") and not args.skip_cpu) else None
     dom = pre["dominant"] or {}
     line = {
         "metric": "prefill tok/s at 128k KV (hip_attention_12, mask estimation + block-sparse attention)",

@@ -166,23 +166,46 @@ __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<E
     }
 }
 
+// Merge of the per-split partials of one (batch, head): out = sum_s w_s x_s / sum_s w_s with w_s = 2^(lse_s - max lse),
+// summed in split order.  The partials were written by workgroups all over the chip, so every read is a long-latency
+// one: the rows are first pulled into LDS with all loads of a chunk in flight at once, then combined from there.
+constexpr int MERGE_THREADS = 256;
+constexpr int MERGE_CHUNK = 32;  // splits staged per round
+
 template <typename T, int HID>
-__global__ void bsa_decode_merge_kernel(const float *ws, int HEAD, int nsplits, T *out, int64_t o_sb, int64_t o_sh) {
-    const int h = blockIdx.x, b = blockIdx.y;
-    const float *base = ws + ((int64_t)b * HEAD + h) * nsplits * (HID + 4);
+__global__ __launch_bounds__(MERGE_THREADS) void bsa_decode_merge_kernel(const float *ws, int HEAD, int nsplits, T *out,
+                                                                        int64_t o_sb, int64_t o_sh) {
+    constexpr int ROW = HID + 4;
+    __shared__ __align__(16) float s_rows[MERGE_CHUNK * ROW];
+    __shared__ float s_red[MERGE_THREADS / 64];
+    const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    const float *base = ws + ((int64_t)b * HEAD + h) * nsplits * ROW;
+    // max of the log-sum-exps
     float mm = -INFINITY;
-    for (int s = 0; s < nsplits; s++) mm = fmaxf(mm, base[(int64_t)s * (HID + 4) + HID]);
-    for (int d = threadIdx.x; d < HID; d += blockDim.x) {
-        float num = 0.0f, den = 0.0f;
-        if (mm > -INFINITY) {
-            for (int s = 0; s < nsplits; s++) {
-                const float w = exp2f(base[(int64_t)s * (HID + 4) + HID] - mm);
-                num += w * base[(int64_t)s * (HID + 4) + d];
+    for (int s = tid; s < nsplits; s += MERGE_THREADS) mm = fmaxf(mm, base[(int64_t)s * ROW + HID]);
+    mm = wave_max(mm);
+    if ((tid & 63) == 0) s_red[tid >> 6] = mm;
+    __syncthreads();
+    mm = s_red[0];
+#pragma unroll
+    for (int w = 1; w < MERGE_THREADS / 64; w++) mm = fmaxf(mm, s_red[w]);
+    float num = 0.0f, den = 0.0f;
+    for (int s0 = 0; s0 < nsplits; s0 += MERGE_CHUNK) {
+        const int ns = nsplits - s0 < MERGE_CHUNK ? nsplits - s0 : MERGE_CHUNK;
+        __syncthreads();
+        const float4 *src = reinterpret_cast<const float4 *>(base + (int64_t)s0 * ROW);  // rows are 16-byte multiples
+        float4 *dst = reinterpret_cast<float4 *>(s_rows);
+        for (int i = tid; i < ns * ROW / 4; i += MERGE_THREADS) dst[i] = src[i];
+        __syncthreads();
+        if (tid < HID && mm > -INFINITY) {
+            for (int s = 0; s < ns; s++) {
+                const float w = exp2f(s_rows[s * ROW + HID] - mm);
+                num += w * s_rows[s * ROW + tid];
                 den += w;
             }
         }
-        out[(int64_t)b * o_sb + (int64_t)h * o_sh + d] = Elem<T>::narrow(den > 0.0f ? num / den : 0.0f);
     }
+    if (tid < HID) out[(int64_t)b * o_sb + (int64_t)h * o_sh + tid] = Elem<T>::narrow(den > 0.0f ? num / den : 0.0f);
 }
 
 template <typename T, int HID>
@@ -271,7 +294,8 @@ extern "C" int hipattn_bsa_decode_merge(const void *workspace, int32_t B, int32_
                                         void *stream) {
     HIPATTN_CHECK_ARG(workspace && out, HIPATTN_E_ARG, "decode merge: null pointer");
     HIPATTN_CHECK_ARG(B > 0 && HEAD > 0 && nsplits > 0, HIPATTN_E_ARG, "decode merge: non-positive size");
-    dim3 grid((unsigned)HEAD, (unsigned)B), block(HID < 64 ? 64 : (HID > 256 ? 256 : HID));
+    HIPATTN_CHECK_ARG(aligned16(workspace), HIPATTN_E_ALIGN, "decode merge: workspace must be 16-byte aligned");
+    dim3 grid((unsigned)HEAD, (unsigned)B), block(MERGE_THREADS);
     const float *ws = reinterpret_cast<const float *>(workspace);
     hipStream_t st = (hipStream_t)stream;
 #define MERGE_CASE(TT, HH)                                                                                         \

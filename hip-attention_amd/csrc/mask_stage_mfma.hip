@@ -351,11 +351,13 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
         const char *e = getenv("HIPATTN_MASK_VIA_LDS");
         g_mask_via_lds = e ? (e[0] == '1' ? 1 : 0) : 2;
     }
-    // statistics / offload cache: built for the direct path only.  The extended build is also used for wide
-    // single-row-block launches without extras: measured 10-15% faster there than the plain build of the same
-    // source (the compiler schedules its row loads earlier), and its extra branches are never taken.
+    // The extended build (statistics, offload cache) exists for the direct path and for the one-block LDS path.
+    // It is also used for wide single-row-block launches without extras: measured 10-15% faster there than the
+    // plain build of the same source (the compiler schedules its row loads earlier), and its extra branches are
+    // never taken.
     const bool ext = p.kx.extended() || (wide && !two);
-    const bool via_lds = !ext && (g_mask_via_lds == 2 ? !wide : (g_mask_via_lds == 1));
+    bool via_lds = g_mask_via_lds == 2 ? !wide : (g_mask_via_lds == 1);
+    if (ext && nb == 2) via_lds = false;
     const int hpw = (via_lds || two) ? 1 : (p.G < 4 ? p.G : 4);
     const int hblocks = (p.G + hpw - 1) / hpw;
     p.total = (long long)p.B * p.kv.HKV * hblocks * p.BS * p.ngroups * nsub;
@@ -372,8 +374,10 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
     const MaskParamsBase &pb = p;  // the plain kernels take the block without the extras
 #define MS_LAUNCH(MBv, NBv, PSv, VLv)                                                                                 \
     do {                                                                                                              \
-        if (ext && !VLv)                                                                                              \
-            hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, NBv, PSv, false, true>), grid, block, 0, st, p, nsub, hpw); \
+        constexpr bool EXT_BUILT = !(VLv) || (NBv) == 1;                                                              \
+        if (ext && EXT_BUILT)                                                                                         \
+            hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, NBv, PSv, VLv, EXT_BUILT>), grid, block, 0, st, p, nsub, \
+                               hpw);                                                                                  \
         else                                                                                                          \
             hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, NBv, PSv, VLv, false>), grid, block, 0, st, pb, nsub, hpw); \
     } while (0)

@@ -376,10 +376,12 @@ def dual_stage_quadratic_hip_attention(
         args.sliding_window_size += args.mask_k
         args.block_size_k = stages[-1].stage_chunk_size
         args.mask_k = args.second_stage_k
-        indices = cached_metadata.indices.clone()
-        ks = cached_metadata.ks.clone()
-        ks_count = cached_metadata.ks_count.clone()
-        ks_start_end = cached_metadata.ks_start_end.clone()
+        # The reference clones these four tensors (:3063-3066).  Nothing here writes to them, so the returned
+        # metadata shares them with the cached one: four copy kernels less on every cached decode step.
+        indices = cached_metadata.indices
+        ks = cached_metadata.ks
+        ks_count = cached_metadata.ks_count
+        ks_start_end = cached_metadata.ks_start_end
         fresh_mask = False
         rows_shared = bool(getattr(cached_metadata, "_rows_shared", False))
 
