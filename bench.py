@@ -72,7 +72,7 @@ def run_prefill(args, device):
 
     TQ, TK, H, HKV, D = 32768, 131072, 32, 8, 128
     q, k, v = prefill_workload(device, 1, TQ, TK, H, HKV, D)
-    hargs = HiPAttentionArgs12(sliding_window_size=1024)
+    hargs = HiPAttentionArgs12(sliding_window_size=1024, require_cache_statistics=not args.no_statistics)
     for _ in range(args.warmup):
         hip_attention_12(q, k, v, hargs)
     torch.cuda.synchronize()
@@ -404,6 +404,8 @@ def main():
     ap.add_argument("--skip-decode", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-offload", action="store_true")
+    ap.add_argument("--no-statistics", action="store_true",
+                    help="profiling aid: prefill without the access-statistics flags the default arguments ask for")
     ap.add_argument("--only", choices=["prefill", "decode", "offload", "cpu"], default=None,
                     help="profiling aid: run one part; the other fields of the JSON line are null")
     args = ap.parse_args()

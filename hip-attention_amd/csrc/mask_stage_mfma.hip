@@ -355,9 +355,9 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
     // It is also used for wide single-row-block launches without extras: measured 10-15% faster there than the
     // plain build of the same source (the compiler schedules its row loads earlier), and its extra branches are
     // never taken.
-    const bool ext = p.kx.extended() || (wide && !two);
     bool via_lds = g_mask_via_lds == 2 ? !wide : (g_mask_via_lds == 1);
-    if (ext && nb == 2) via_lds = false;
+    if (p.kx.extended() && nb == 2) via_lds = false;
+    const bool ext = p.kx.extended() || (wide && !two && !via_lds);
     const int hpw = (via_lds || two) ? 1 : (p.G < 4 ? p.G : 4);
     const int hblocks = (p.G + hpw - 1) / hpw;
     p.total = (long long)p.B * p.kv.HKV * hblocks * p.BS * p.ngroups * nsub;
