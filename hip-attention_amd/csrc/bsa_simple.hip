@@ -83,6 +83,12 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
             const bool att = valid && (kind == 0 ? (t + p.sw <= ppos) : (t <= ppos && ppos < t + p.sw));
             float logit = -INFINITY;
             int64_t voff = NO_ROW;
+            if (valid && !att && j == wid && (p.kx.access_flags || p.kx.cached)) {
+                // staged for this query block but masked out for this row: the tile kernel loads such rows, so
+                // they count as accessed (first row pass of each wave records them)
+                int64_t ko, vo;
+                kv_rows<false, true>(p.kv, &p.kx, b, t, kvh, seqlen, ko, vo);
+            }
             if (att) {
                 int64_t koff;
                 kv_rows<true, true>(p.kv, &p.kx, b, t, kvh, seqlen, koff, voff);
