@@ -7,8 +7,10 @@ default stages, sink 256, window 1024.  A "step" is one full call (mask estimati
 attention) on synthetic inputs already resident in HBM.  ``value`` = queries / second.
 
 Also reported in the same JSON line:
-  * ``decode``: a 1M-token KV decode loop (configs[3] phase B: mask refreshed every 8 steps),
-    microseconds per step and the HBM roofline fraction of a refresh step;
+  * ``decode``: configs[3], one sequence of 1M keys with planted needle blocks: the chunked prefill (8 calls of
+    131072 queries against the growing prefix), then the decode loop (mask refreshed every 8 steps) with
+    microseconds per step, the HBM roofline fraction of a refresh step and the needle recall;
+  * ``batched_decode``: configs[2], 16 sequences of 64k-256k keys in a paged cache (page 16), same decode loop;
   * ``offload``: configs[4], a 3M-token KV held in pinned host memory behind a 16 GB HBM block cache: cold,
     warm and drifting-query decode steps beside the same steps with the KV resident;
   * ``roofline``: the dominant kernel of the prefill step, timed with HIP events inside the timed
@@ -129,28 +131,10 @@ def run_prefill(args, device):
     }
 
 
-def run_decode(args, device, TK=1 << 20, steps=64, refresh_every=8):
-    """configs[3] phase B: single sequence, 1M keys, q_len 1, mask refreshed every 8 steps."""
+def _time_decode(step, steps, refresh_every):
+    """Times a decode loop given ``step(meta_or_None) -> (out, meta)``: eager calls, then HIP-graph replay."""
     import torch
-    from hip_attn import HiPAttentionArgs12, hip_attention_12
     from hip_attn import _native as N
-
-    H, HKV, D = 32, 8, 128
-    g = torch.Generator(device="cpu").manual_seed(3)
-    k = torch.empty((1, TK, HKV, D), dtype=torch.bfloat16, device=device)
-    step = 1 << 17
-    for s in range(0, TK, step):
-        k[:, s:s + step] = torch.randn((1, step, HKV, D), generator=g, dtype=torch.float32).to(torch.bfloat16).to(device)
-    v = k.clone()
-    q = torch.randn((1, 1, H, D), generator=g, dtype=torch.float32).to(torch.bfloat16).to(device)
-    pos = torch.full((1, 1), TK - 1, dtype=torch.int64, device=device)
-
-    def step_args(refresh):
-        # statistics only when the mask is estimated, as the serving entry point asks for them (paged_hip.py:400-406)
-        return HiPAttentionArgs12(sliding_window_size=1024, position_ids=pos, require_cache_statistics=refresh)
-
-    def step(meta_in):
-        return hip_attention_12(q, k, v, step_args(meta_in is None), cached_metadata=meta_in)
 
     meta = None
     for i in range(16):
@@ -215,34 +199,145 @@ def run_decode(args, device, TK=1 << 20, steps=64, refresh_every=8):
     eager_out, _ = step(meta_r)
     torch.cuda.synchronize()
     graph_matches = bool(torch.equal(eager_out.view(torch.int16), out_c.view(torch.int16)))
-
-    sink, sw = 256, 1024
-    n0 = cdiv(TK - sink - sw, 256)
-    n1 = min(32768 // 256, n0) * 8
-    n2 = min(8192 // 32, n1) * 4
-    mb = sum(mask_stage_bytes(1, 1, H, D, 2, [(64, n0, 256), (64, n1, 32), (64, n2, 8)]))
-    attn_bytes = HKV * (2048 + sink + sw) * 2 * D * 2
-    refresh_bytes = mb + attn_bytes
-    gbs_refresh = refresh_bytes / (us_refresh * 1e-6) / 1e9
-    gbs_cached = attn_bytes / (us_cached * 1e-6) / 1e9
     N.profile_begin()
-    step(None)
+    _, meta_last = step(None)
     prof = N.profile_end()
     del g_refresh, g_cached, out_r, out_c, meta_r
-    del k, v
-    torch.cuda.empty_cache()
     return {
-        "kv_len": TK, "launch": "hip graph replay (one graph per step kind)",
+        "launch": "hip graph replay (one graph per step kind)",
         "us_per_step_mixed": us_mixed, "us_per_step_refresh": us_refresh,
         "us_per_step_cached": us_cached, "wall_us_per_step_mixed": wall_us, "refresh_every": refresh_every,
         "graph_replay_matches_eager": graph_matches,
         "eager": {"us_per_step_mixed": eager_mixed, "us_per_step_refresh": eager_refresh,
                   "us_per_step_cached": eager_cached, "wall_us_per_step_mixed": eager_wall},
-        "refresh_algorithmic_bytes": refresh_bytes, "cached_algorithmic_bytes": attn_bytes,
-        "hbm_frac_refresh": gbs_refresh / HBM_PEAK_GBS, "hbm_frac_cached": gbs_cached / HBM_PEAK_GBS,
-        "refresh_GBps": gbs_refresh, "cached_GBps": gbs_cached,
         "refresh_kernels_us": [(n, round(ms * 1e3, 1)) for n, ms in prof],
-    }
+    }, meta_last
+
+
+def _decode_bytes(lens, H, HKV, D):
+    """Algorithmic bytes of a refresh step and of a cached step, summed over the batch (default stages)."""
+    sink, sw = 256, 1024
+    mb = 0
+    for TK in lens:
+        n0 = cdiv(TK - sink - sw, 256)
+        n1 = min(32768 // 256, n0) * 8
+        n2 = min(8192 // 32, n1) * 4
+        mb += sum(mask_stage_bytes(1, 1, H, D, 2, [(64, n0, 256), (64, n1, 32), (64, n2, 8)]))
+    attn = len(lens) * HKV * (2048 + sink + sw) * 2 * D * 2
+    return mb + attn, attn
+
+
+def _with_rooflines(res, refresh_bytes, attn_bytes):
+    gbs_refresh = refresh_bytes / (res["us_per_step_refresh"] * 1e-6) / 1e9
+    gbs_cached = attn_bytes / (res["us_per_step_cached"] * 1e-6) / 1e9
+    res.update({"refresh_algorithmic_bytes": refresh_bytes, "cached_algorithmic_bytes": attn_bytes,
+                "hbm_frac_refresh": gbs_refresh / HBM_PEAK_GBS, "hbm_frac_cached": gbs_cached / HBM_PEAK_GBS,
+                "refresh_GBps": gbs_refresh, "cached_GBps": gbs_cached})
+    return res
+
+
+def run_decode(args, device, TK=1 << 20, steps=64, refresh_every=8, needles=64):
+    """configs[3]: one sequence of 1M keys with planted needle blocks; chunked prefill, then decode steps."""
+    import torch
+    from hip_attn import HiPAttentionArgs12, hip_attention_12
+
+    H, HKV, D = 32, 8, 128
+    g = torch.Generator(device="cpu").manual_seed(3)
+    k = torch.empty((1, TK, HKV, D), dtype=torch.bfloat16, device=device)
+    chunk = 1 << 17
+    for s in range(0, TK, chunk):
+        k[:, s:s + chunk] = torch.randn((1, chunk, HKV, D), generator=g, dtype=torch.float32).to(torch.bfloat16).to(device)
+    # needles: 8-token blocks at seeded positions whose component along a unit direction u is set to +12;
+    # the decode query is noise + 12 u, so a needle token scores ~144 against ~N(0, 17^2) for ordinary keys
+    u = torch.randn((D,), generator=g, dtype=torch.float32)
+    u = u / u.norm()
+    starts = (torch.randperm((TK - 4096) // 8, generator=g)[:needles] * 8 + 2048).sort().values
+    ud = u.to(device)
+    for st in starts.tolist():
+        blk = k[0, st:st + 8].float()
+        blk = blk - (blk @ ud)[..., None] * ud + 12.0 * ud
+        k[0, st:st + 8] = blk.to(torch.bfloat16)
+    v = k.clone()
+    q = (torch.randn((1, 1, H, D), generator=g, dtype=torch.float32) + 12.0 * u).to(torch.bfloat16).to(device)
+    pos = torch.full((1, 1), TK - 1, dtype=torch.int64, device=device)
+
+    # phase A: the context is prefilled in 131072-query chunks, each against the prefix it has seen so far
+    TQA = 1 << 17
+    qa = torch.randn((1, TQA, H, D), generator=g, dtype=torch.float32).to(torch.bfloat16).to(device)
+    prefill_ms = []
+    for c in range(TK // TQA):
+        end = (c + 1) * TQA
+        a = HiPAttentionArgs12(sliding_window_size=1024)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        hip_attention_12(qa, k[:, :end], v[:, :end], a)
+        torch.cuda.synchronize()
+        prefill_ms.append((time.perf_counter() - t0) * 1e3)
+    del qa
+    torch.cuda.empty_cache()
+
+    def step(meta_in):
+        # statistics only when the mask is estimated, as the serving entry point asks for them (paged_hip.py:400-406)
+        a = HiPAttentionArgs12(sliding_window_size=1024, position_ids=pos, require_cache_statistics=meta_in is None)
+        return hip_attention_12(q, k, v, a, cached_metadata=meta_in)
+
+    res, meta = _time_decode(step, steps, refresh_every)
+    # needle recall: a needle counts as found when its 8-token block is among the selected blocks of a head
+    idx = meta.indices[:, 0, :]  # [H, BK]
+    found = (idx[:, :, None] == starts.to(device)[None, None, :]).any(dim=1).float()  # [H, needles]
+    res.update({"kv_len": TK, "needle_blocks": needles, "needle_recall_mean_over_heads": float(found.mean()),
+                "needle_recall_any_head": float(found.any(dim=0).float().mean()),
+                "prefill_chunks_ms": [round(x, 1) for x in prefill_ms],
+                "prefill_tok_per_s": TK / (sum(prefill_ms) * 1e-3)})
+    refresh_bytes, attn_bytes = _decode_bytes([TK], H, HKV, D)
+    del k, v
+    torch.cuda.empty_cache()
+    return _with_rooflines(res, refresh_bytes, attn_bytes)
+
+
+def run_batched_decode(args, device, B=16, steps=64, refresh_every=8):
+    """configs[2]: 16 sequences of 64k-256k keys in a paged cache (page 16, shuffled block table), q_len 1."""
+    import torch
+    from hip_attn import HiPAttentionArgs12, hip_attention_12
+
+    H, HKV, D, PAGE, MAXLEN = 32, 8, 128, 16, 262144
+    g = torch.Generator(device="cpu").manual_seed(2)
+    lens = torch.randint(65536, MAXLEN + 1, (B,), generator=g)
+    per = [cdiv(int(x), PAGE) for x in lens]
+    pages = sum(per) + 1
+    kc = torch.empty((pages, PAGE, HKV, D), dtype=torch.bfloat16, device=device)
+    chunk = 8192
+    for s in range(0, pages, chunk):
+        n = min(chunk, pages - s)
+        kc[s:s + n] = torch.randn((n, PAGE, HKV, D), generator=g, dtype=torch.float32).to(torch.bfloat16).to(device)
+    kc[0].zero_()  # page 0 is the dummy page
+    vc = kc.clone()
+    perm = torch.randperm(pages - 1, generator=g) + 1
+    bt = torch.zeros((B, cdiv(MAXLEN, PAGE)), dtype=torch.int32)
+    o = 0
+    for b in range(B):
+        bt[b, :per[b]] = perm[o:o + per[b]].to(torch.int32)
+        o += per[b]
+    bt = bt.to(device)
+    sl = lens.to(torch.int32).to(device)
+    pos = (lens - 1).to(torch.int64)[:, None].to(device)
+    q = torch.randn((B, 1, H, D), generator=g, dtype=torch.float32).to(torch.bfloat16).to(device)
+
+    def step(meta_in):
+        a = HiPAttentionArgs12(sliding_window_size=1024, position_ids=pos, k_cache=kc, v_cache=vc, block_table=bt,
+                               cache_seq_lens=sl, extend_context_length=MAXLEN,
+                               require_cache_statistics=meta_in is None)
+        return hip_attention_12(q, None, None, a, cached_metadata=meta_in)
+
+    res, _ = _time_decode(step, steps, refresh_every)
+    # every sequence scans the chunk grid of the full 262144-token table (the reference sizes the first stage by
+    # extend_context_length); chunks beyond a sequence's length end their search after the activity test
+    refresh_bytes, attn_bytes = _decode_bytes([int(x) for x in lens], H, HKV, D)
+    res.update({"batch": B, "kv_lens_min_max": [int(lens.min()), int(lens.max())], "page_size": PAGE,
+                "paged_cache_GB": 2 * kc.numel() * 2 / 1e9})
+    del kc, vc
+    torch.cuda.empty_cache()
+    return _with_rooflines(res, refresh_bytes, attn_bytes)
 
 
 def run_offload(args, device, TK=3_000_000, warm_steps=4, drift_steps=12):
@@ -406,7 +501,7 @@ def main():
     ap.add_argument("--skip-offload", action="store_true")
     ap.add_argument("--no-statistics", action="store_true",
                     help="profiling aid: prefill without the access-statistics flags the default arguments ask for")
-    ap.add_argument("--only", choices=["prefill", "decode", "offload", "cpu"], default=None,
+    ap.add_argument("--only", choices=["prefill", "decode", "batched_decode", "offload", "cpu"], default=None,
                     help="profiling aid: run one part; the other fields of the JSON line are null")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -421,6 +516,7 @@ def main():
     pre = run_prefill(args, device) if want("prefill") else {
         "tok_per_s": None, "ms_per_step": None, "rooflines": [], "kernels_ms": {}, "dominant": None}
     dec = run_decode(args, device) if (want("decode") and not args.skip_decode) else None
+    bdec = run_batched_decode(args, device) if (want("batched_decode") and not args.skip_decode) else None
     off = run_offload(args, device) if (want("offload") and not args.skip_offload) else None
     cpu = run_cpu_baseline(args) if (want("cpu") and not args.skip_cpu) else None
     dom = pre["dominant"] or {}
@@ -444,6 +540,7 @@ def main():
         "roofline_all": pre["rooflines"],
         "kernels_ms": pre["kernels_ms"],
         "decode": dec,
+        "batched_decode": bdec,
         "offload": off,
         "cpu_baseline": cpu,
     }
