@@ -199,6 +199,16 @@ def _time_decode(step, steps, refresh_every):
     eager_out, _ = step(meta_r)
     torch.cuda.synchronize()
     graph_matches = bool(torch.equal(eager_out.view(torch.int16), out_c.view(torch.int16)))
+    # the same refresh step without the access-statistics flags (an option of the operator, not the serving default)
+    with torch.cuda.stream(side):
+        step(None, False)
+    torch.cuda.synchronize()
+    g_plain = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g_plain, pool=g_refresh.pool()):
+        out_p, _ = step(None, False)
+    torch.cuda.synchronize()
+    us_refresh_plain = timed(16, lambda i: g_plain.replay())
+    del g_plain, out_p
     N.profile_begin()
     _, meta_last = step(None)
     prof = N.profile_end()
@@ -207,6 +217,7 @@ def _time_decode(step, steps, refresh_every):
         "launch": "hip graph replay (one graph per step kind)",
         "us_per_step_mixed": us_mixed, "us_per_step_refresh": us_refresh,
         "us_per_step_cached": us_cached, "wall_us_per_step_mixed": wall_us, "refresh_every": refresh_every,
+        "us_per_step_refresh_without_statistics": us_refresh_plain,
         "graph_replay_matches_eager": graph_matches,
         "eager": {"us_per_step_mixed": eager_mixed, "us_per_step_refresh": eager_refresh,
                   "us_per_step_cached": eager_cached, "wall_us_per_step_mixed": eager_wall},
@@ -230,6 +241,8 @@ def _decode_bytes(lens, H, HKV, D):
 def _with_rooflines(res, refresh_bytes, attn_bytes):
     gbs_refresh = refresh_bytes / (res["us_per_step_refresh"] * 1e-6) / 1e9
     gbs_cached = attn_bytes / (res["us_per_step_cached"] * 1e-6) / 1e9
+    res["hbm_frac_refresh_without_statistics"] = (
+        refresh_bytes / (res["us_per_step_refresh_without_statistics"] * 1e-6) / 1e9 / HBM_PEAK_GBS)
     res.update({"refresh_algorithmic_bytes": refresh_bytes, "cached_algorithmic_bytes": attn_bytes,
                 "hbm_frac_refresh": gbs_refresh / HBM_PEAK_GBS, "hbm_frac_cached": gbs_cached / HBM_PEAK_GBS,
                 "refresh_GBps": gbs_refresh, "cached_GBps": gbs_cached})
@@ -276,9 +289,10 @@ def run_decode(args, device, TK=1 << 20, steps=64, refresh_every=8, needles=64):
     del qa
     torch.cuda.empty_cache()
 
-    def step(meta_in):
+    def step(meta_in, stats=None):
         # statistics only when the mask is estimated, as the serving entry point asks for them (paged_hip.py:400-406)
-        a = HiPAttentionArgs12(sliding_window_size=1024, position_ids=pos, require_cache_statistics=meta_in is None)
+        a = HiPAttentionArgs12(sliding_window_size=1024, position_ids=pos,
+                               require_cache_statistics=(meta_in is None) if stats is None else stats)
         return hip_attention_12(q, k, v, a, cached_metadata=meta_in)
 
     res, meta = _time_decode(step, steps, refresh_every)
@@ -323,10 +337,10 @@ def run_batched_decode(args, device, B=16, steps=64, refresh_every=8):
     pos = (lens - 1).to(torch.int64)[:, None].to(device)
     q = torch.randn((B, 1, H, D), generator=g, dtype=torch.float32).to(torch.bfloat16).to(device)
 
-    def step(meta_in):
+    def step(meta_in, stats=None):
         a = HiPAttentionArgs12(sliding_window_size=1024, position_ids=pos, k_cache=kc, v_cache=vc, block_table=bt,
                                cache_seq_lens=sl, extend_context_length=MAXLEN,
-                               require_cache_statistics=meta_in is None)
+                               require_cache_statistics=(meta_in is None) if stats is None else stats)
         return hip_attention_12(q, None, None, a, cached_metadata=meta_in)
 
     res, _ = _time_decode(step, steps, refresh_every)

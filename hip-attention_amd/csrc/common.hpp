@@ -270,11 +270,11 @@ __device__ __forceinline__ void kv_rows(const KVView &kv, const KVExt *kx, int b
     if (WANT_V) vo = page * kv.v_stride_b + inpage * kv.v_stride_t + (int64_t)h * kv.v_stride_h;
 }
 
-template <bool EXT>
+template <bool EXT, bool CHECK = true>
 __device__ __forceinline__ int64_t kv_k_row(const KVView &kv, const KVExt *kx, int b, int64_t t, int h,
                                             int64_t seqlen, bool leader = true) {
     int64_t ko, vo;
-    kv_rows<false, EXT>(kv, kx, b, t, h, seqlen, ko, vo, leader);
+    kv_rows<false, EXT, CHECK>(kv, kx, b, t, h, seqlen, ko, vo, leader);
     return ko;
 }
 

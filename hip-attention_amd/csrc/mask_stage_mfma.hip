@@ -195,7 +195,9 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
             int64_t off = NO_ROW;
             if (active[tb]) {
                 const int t = side ? ((ctr[tb] + cr[tb]) >> 1) : ((cl[tb] + ctr[tb]) >> 1);
-                off = kv_k_row<EXT>(p.kv, kx, b, t, kvh, seqlen, hh == 0);
+                // access flags: wide launches (prefill) revisit rows constantly, so they look before they store;
+                // narrow ones (decode) touch mostly fresh rows and store blindly
+                off = kv_k_row<EXT, NB == 2>(p.kv, kx, b, t, kvh, seqlen, hh == 0);
             }
             if constexpr (VIA_LDS) {
                 if (hh == 0) s_off[tb * 32 + n] = off;
@@ -343,7 +345,12 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
     // two token blocks (32 chunks) per wave when programs are plentiful, else one block per wave
     const long long programs = (long long)p.B * p.HEAD * p.BS * p.ngroups;
     const bool wide = (BC >= 32) && (programs >= 16384);
-    const int nb = wide ? 2 : 1;
+    static int env_nb = -1;
+    if (env_nb < 0) {
+        const char *e = getenv("HIPATTN_MASK_NB");
+        env_nb = e ? atoi(e) : 0;
+    }
+    const int nb = (env_nb == 2 && BC >= 32) ? 2 : (wide ? 2 : 1);
     const int nsub = (BC / 16) / nb;
     // LDS path: one wave per workgroup (it uses workgroup barriers); direct path: up to 4 heads per workgroup
     // (measured: sharing pays with one query-row block per program, not with two)
@@ -386,8 +393,8 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
         if (prescaled) { if (via_lds) MS_LAUNCH(MBv, NBv, true, true); else MS_LAUNCH(MBv, NBv, true, false); } \
         else { if (via_lds) MS_LAUNCH(MBv, NBv, false, true); else MS_LAUNCH(MBv, NBv, false, false); }        \
     } while (0)
-    if (two) { if (wide) MS_PICK(2, 2); else MS_PICK(2, 1); }
-    else { if (wide) MS_PICK(1, 2); else MS_PICK(1, 1); }
+    if (two) { if (nb == 2) MS_PICK(2, 2); else MS_PICK(2, 1); }
+    else { if (nb == 2) MS_PICK(1, 2); else MS_PICK(1, 1); }
 #undef MS_PICK
 #undef MS_LAUNCH
     HIPATTN_CHECK_HIP(hipGetLastError());

@@ -53,7 +53,15 @@ class _Tensors(ctypes.Structure):
         ("MAX_TSRC", ctypes.c_int64),
         ("access", ctypes.c_void_p),
         ("access_pages", ctypes.c_int64),
+        ("rope_cos", ctypes.c_void_p),
+        ("rope_sin", ctypes.c_void_p),
+        ("rope_len", ctypes.c_int64),
+        ("scan_backend", ctypes.c_int),
+        ("sa_backend", ctypes.c_int),
     ]
+
+
+EXTEND_BACKENDS = {None: 0, "relative": 1, "streaming": 2, "infllm": 3}
 
 
 def build(force: bool = False) -> str:
@@ -78,6 +86,7 @@ def lib():
         L.hipo_scale_constants.restype = None
         L.hipo_mask_stage.restype = ctypes.c_int
         L.hipo_bsa.restype = ctypes.c_int
+        L.hipo_rope_row.restype = None
         L.hipo_num_threads.restype = ctypes.c_int
         _LIB = L
     return _LIB
@@ -113,6 +122,7 @@ class OStage:
     stage_chunk_size: int
     stage_k: Optional[int]
     stage_stride: int = 1
+    stage_extend_backend: Optional[str] = None
 
 
 def default_stages() -> List[OStage]:
@@ -134,6 +144,11 @@ class OArgs:
     disable_flashdecode: bool = False
     head_reduce: bool = True  # env HIP_HEAD_REDUCE, default on (attention_extend.py:2566)
     mask_only: bool = False
+    # RoPE applied on load (attention_metadata.py:191-198); only using_extend with need_apply_rope is modelled
+    using_extend: bool = False
+    need_apply_rope: bool = False
+    scan_extend_backend: str = "relative"
+    sa_extend_backend: str = "streaming"
 
 
 @dataclass
@@ -148,6 +163,10 @@ class OInputs:
     block_table: Optional[np.ndarray] = None  # [B,cols] int64
     cache_seq_lens: Optional[np.ndarray] = None  # [B] int64
     access: Optional[np.ndarray] = None  # int32 [B,HKV,pages]: flags set by every key row the kernels fetch
+    rope_cos: Optional[np.ndarray] = None  # float32 [L,HID] (values of the tables' own dtype, widened)
+    rope_sin: Optional[np.ndarray] = None
+    scan_backend: Optional[str] = None  # rotation rule of the mask stage / of sparse attention; None = no RoPE
+    sa_backend: Optional[str] = None
 
     def c_struct(self, max_tsrc: int):
         np_t = np.uint16 if self.dtype == "bf16" else np.float32
@@ -188,6 +207,14 @@ class OInputs:
             assert self.access.dtype == np.int32 and self.access.flags.c_contiguous and self.access.ndim == 3
             S.access = self.access.ctypes.data
             S.access_pages = self.access.shape[2]
+        if self.scan_backend is not None or self.sa_backend is not None:
+            assert self.rope_cos is not None and self.rope_cos.shape == self.rope_sin.shape
+            assert self.rope_cos.ndim == 2 and self.rope_cos.shape[1] == HID
+            S.rope_cos = arr(self.rope_cos, np.float32)
+            S.rope_sin = arr(self.rope_sin, np.float32)
+            S.rope_len = self.rope_cos.shape[0]
+            S.scan_backend = EXTEND_BACKENDS[self.scan_backend]
+            S.sa_backend = EXTEND_BACKENDS[self.sa_backend]
         return S, keep
 
 
@@ -222,6 +249,15 @@ def mask_stage(X: OInputs, max_tsrc, left, right, scores, BS, BQ, stride_q, bloc
     if rc != 0:
         raise RuntimeError(f"hipo_mask_stage failed: {rc}")
     del keep
+
+
+def rope_row(X: OInputs, row: np.ndarray, pos: int) -> np.ndarray:
+    """One row (float32 values of X's dtype) rotated to ``pos`` with X's tables."""
+    S, keep = X.c_struct(0)
+    out = np.ascontiguousarray(row, dtype=np.float32).copy()
+    lib().hipo_rope_row(ctypes.byref(S), ctypes.c_void_p(out.ctypes.data), ctypes.c_int64(pos))
+    del keep
+    return out
 
 
 def bsa(X: OInputs, max_tsrc, indices, ks_start_end, block_size_q, block_size_k, sw, sink,
@@ -289,6 +325,14 @@ def hip_attention_12(X: OInputs, A: OArgs, cached: Optional[OMetadata] = None):
     assert pos.shape == (B, TDST)
 
     stage_caches = [] if (cached is None or cached.stage_caches is None) else cached.stage_caches
+
+    user_backends = (X.scan_backend, X.sa_backend)
+    if A.using_extend:
+        assert A.need_apply_rope, "only keys stored without rotation are modelled"
+        assert X.rope_cos is not None and X.rope_sin is not None
+        X.scan_backend, X.sa_backend = A.scan_extend_backend, A.sa_extend_backend
+    else:
+        X.scan_backend = X.sa_backend = None
 
     # access flags (attention_extend.py:1988-2006): one entry per token (dense) or pool page (paged)
     HKV = X.k.shape[2] if X.k is not None else X.k_cache.shape[2]
@@ -377,6 +421,8 @@ def hip_attention_12(X: OInputs, A: OArgs, cached: Optional[OMetadata] = None):
             left = np.ascontiguousarray(left)
             right = np.ascontiguousarray(right)
             scores = np.ascontiguousarray(scores)
+            if A.using_extend:  # :2200-2204
+                X.scan_backend = st.stage_extend_backend or A.scan_extend_backend
             mask_stage(X, MAX_TSRC, left, right, scores, BS=left.shape[1], BQ=BQ,
                        stride_q=st.stage_block_stride_q, block_chunk=BLOCK_CHUNK,
                        scan_stride=STAGE_STRIDE, sw_eff=sw_eff, terminate=A.stage_early_terminate)
@@ -425,6 +471,7 @@ def hip_attention_12(X: OInputs, A: OArgs, cached: Optional[OMetadata] = None):
             block_size_q = bsbq
         X.access = user_access
         if A.mask_only:
+            X.scan_backend, X.sa_backend = user_backends
             return None, None
     else:
         sw_bsa = sw_eff + mask_k
@@ -446,6 +493,7 @@ def hip_attention_12(X: OInputs, A: OArgs, cached: Optional[OMetadata] = None):
                       share_first_head=decode)
     finally:
         X.access = user_access
+        X.scan_backend, X.sa_backend = user_backends
     meta = OMetadata(indices=indices, ks=ks, ks_count=ks_count, ks_start_end=ks_start_end,
                      stage_caches=stage_caches, mask_access=mask_access, sa_access=sa_access)
     return context, meta

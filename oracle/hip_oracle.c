@@ -44,6 +44,11 @@
 #define HIPO_F32 0
 #define HIPO_BF16 1
 
+#define HIPO_EXT_NONE 0
+#define HIPO_EXT_RELATIVE 1
+#define HIPO_EXT_STREAMING 2
+#define HIPO_EXT_INFLLM 3
+
 typedef struct {
     int dtype;               /* HIPO_F32 / HIPO_BF16 (q, k, v, caches all share it) */
     int B, TDST, HEAD, HKV, HID;
@@ -65,6 +70,13 @@ typedef struct {
      * (dense) or page (paged) -- the ACCESS_COUNTER stores of uvm_gpu_cache.py:845-862,893-907 */
     int32_t *access;
     int64_t access_pages;
+    /* RoPE applied on load ("extend" modes, keys and queries stored without rotation):
+     * cos/sin tables f32 [rope_len, HID] whose two halves repeat the HID/2 frequencies; values are rounded to T on
+     * use, as the reference casts the loaded table entries to the tensor's dtype.  NULL -> no rotation. */
+    const float *rope_cos, *rope_sin;
+    int64_t rope_len;
+    int scan_backend;        /* HIPO_EXT_* for the mask stage */
+    int sa_backend;          /* HIPO_EXT_* for block sparse attention */
 } hipo_tensors_t;
 
 /* ---------------------------------------------------------------- scalar helpers */
@@ -242,8 +254,32 @@ static void fetch_row(const hipo_tensors_t *X, int want_v, int b, int64_t t, int
     }
 }
 
-static void scaled_key(const hipo_tensors_t *X, int b, int64_t t, int kvh, float c_k, float *out) {
+/* Rotate one row in place to position `pos`: x*cos[pos] + rot(x)*sin[pos] with rot(x)[i] = -x[i+HID/2] for
+ * i < HID/2 and +x[i-HID/2] above, table column i % (HID/2), every product and the sum rounded to T
+ * (attention_extend.py:380-407, :640-690; attention_extend_bsa.py:303-380, :818-852). */
+static void rope_rotate(const hipo_tensors_t *X, float *x, int64_t pos) {
+    const int HID = X->HID, H2 = X->HID / 2, dt = X->dtype;
+    if (pos < 0) pos = 0;
+    if (pos >= X->rope_len) pos = X->rope_len - 1;
+    for (int d = 0; d < H2; d++) {
+        float c = round_T(X->rope_cos[pos * HID + d], dt);
+        float s = round_T(X->rope_sin[pos * HID + d], dt);
+        float lo = x[d], hi = x[d + H2];
+        float nlo = round_T(round_T(lo * c, dt) + round_T(-hi * s, dt), dt);
+        float nhi = round_T(round_T(hi * c, dt) + round_T(lo * s, dt), dt);
+        x[d] = nlo;
+        x[d + H2] = nhi;
+    }
+}
+
+/* exported so tests can check the rotation against the complex-number form of RoPE */
+void hipo_rope_row(const hipo_tensors_t *X, float *x, int64_t pos) { rope_rotate(X, x, pos); }
+
+/* key row -> (rotate to rope_pos when tables are given) -> scale */
+static void scaled_key_at(const hipo_tensors_t *X, int b, int64_t t, int kvh, float c_k, int64_t rope_pos,
+                          float *out) {
     fetch_row(X, 0, b, t, kvh, out);
+    if (X->rope_cos) rope_rotate(X, out, rope_pos);
     for (int d = 0; d < X->HID; d++) out[d] = round_T(out[d] * c_k, X->dtype);
 }
 
@@ -273,6 +309,7 @@ int hipo_mask_stage(const hipo_tensors_t *X, int64_t *left, int64_t *right, floa
     {
         float *qhat = (float *)malloc(sizeof(float) * nrows * HID);
         float *kbuf = (float *)malloc(sizeof(float) * HID);
+        float *qsum = (float *)malloc(sizeof(float) * HID);
         int *rowvalid = (int *)malloc(sizeof(int) * nrows);
         int32_t *l = (int32_t *)malloc(sizeof(int32_t) * block_chunk);
         int32_t *r = (int32_t *)malloc(sizeof(int32_t) * block_chunk);
@@ -299,20 +336,30 @@ int hipo_mask_stage(const hipo_tensors_t *X, int64_t *left, int64_t *right, floa
             if (pmin < 0) continue;
             int32_t lim = (int32_t)(pmin - sw_eff);
             if (lim < 0) lim = 0;
-            /* strided mean of query rows, then scale: :607-734, :924-931 */
+            /* strided mean of query rows, then scale: :607-734, :924-931.  With RoPE tables every strided row is
+             * rotated before it is summed, all of them to the position derived from the base row (:626-690). */
             for (int j = 0; j < nrows; j++) {
                 int64_t it = qb * BQ + (int64_t)j * stride_q;
+                int cnt = 0;
+                for (int d = 0; d < HID; d++) qsum[d] = 0.0f;
+                int64_t qpos = 0;
+                if (rowvalid[j] && X->rope_cos) {
+                    int64_t p = X->pos[(int64_t)b * TDST + it];
+                    if (X->scan_backend == HIPO_EXT_RELATIVE) qpos = 1 + (int64_t)sw_eff;
+                    else if (X->scan_backend == HIPO_EXT_INFLLM) qpos = sw_eff;
+                    else qpos = p < (int64_t)n + sw_eff ? p : (int64_t)n + sw_eff;
+                }
+                for (int o = 0; o < stride_q; o++) {
+                    int64_t iti = it + o;
+                    if (!(rowvalid[j] && iti < TDST)) continue;
+                    for (int d = 0; d < HID; d++)
+                        kbuf[d] = load_T(X->q, (((int64_t)b * TDST + iti) * HEAD + h) * HID + d, X->dtype);
+                    if (X->rope_cos) rope_rotate(X, kbuf, qpos);
+                    for (int d = 0; d < HID; d++) qsum[d] += kbuf[d];
+                    cnt++;
+                }
                 for (int d = 0; d < HID; d++) {
-                    float sum = 0.0f;
-                    int cnt = 0;
-                    for (int o = 0; o < stride_q; o++) {
-                        int64_t iti = it + o;
-                        if (rowvalid[j] && iti < TDST) {
-                            sum += load_T(X->q, (((int64_t)b * TDST + iti) * HEAD + h) * HID + d, X->dtype);
-                            cnt++;
-                        }
-                    }
-                    float mean = sum / ((float)cnt + 1e-12f);
+                    float mean = qsum[d] / ((float)cnt + 1e-12f);
                     if (!rowvalid[j]) mean = 0.0f;
                     mean = round_T(mean, X->dtype);
                     qhat[j * HID + d] = round_T(mean * c_q, X->dtype);
@@ -348,13 +395,17 @@ int hipo_mask_stage(const hipo_tensors_t *X, int64_t *left, int64_t *right, floa
                         int32_t tl_ = (l[lane] + ctr) / 2;
                         int32_t tr_ = (ctr + r[lane]) / 2;
                         float sL = -INFINITY, sR = -INFINITY;
-                        scaled_key(X, b, tl_, h / G, c_k, kbuf);
+                        /* rotated key positions: attention_extend.py:289-298 */
+                        int64_t kposL = 0, kposR = 0;
+                        if (X->scan_backend == HIPO_EXT_RELATIVE) kposR = 1;
+                        else if (X->scan_backend == HIPO_EXT_STREAMING) kposL = kposR = c;
+                        scaled_key_at(X, b, tl_, h / G, c_k, kposL, kbuf);
                         for (int j = 0; j < nrows; j++) {
                             if (!rowvalid[j]) continue;
                             float v = round_T(score_dot(qhat + j * HID, kbuf, HID, X->dtype), X->dtype);
                             if (v > sL) sL = v;
                         }
-                        scaled_key(X, b, tr_, h / G, c_k, kbuf);
+                        scaled_key_at(X, b, tr_, h / G, c_k, kposR, kbuf);
                         for (int j = 0; j < nrows; j++) {
                             if (!rowvalid[j]) continue;
                             float v = round_T(score_dot(qhat + j * HID, kbuf, HID, X->dtype), X->dtype);
@@ -375,7 +426,7 @@ int hipo_mask_stage(const hipo_tensors_t *X, int64_t *left, int64_t *right, floa
                 }
             }
         }
-        free(qhat); free(kbuf); free(rowvalid); free(l); free(r); free(sc);
+        free(qhat); free(kbuf); free(qsum); free(rowvalid); free(l); free(r); free(sc);
     }
     return 0;
 }
@@ -409,6 +460,7 @@ int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_
     {
         int64_t *tok = (int64_t *)malloc(sizeof(int64_t) * cap);
         int *kind = (int *)malloc(sizeof(int) * cap); /* 0: excluded-window rule, 1: window rule */
+        int64_t *rpos = (int64_t *)malloc(sizeof(int64_t) * cap); /* rotated position of the key (RoPE on load) */
         float *khat = (float *)malloc(sizeof(float) * (size_t)cap * HID);
         float *vrow = (float *)malloc(sizeof(float) * (size_t)cap * HID);
         float *qhat = (float *)malloc(sizeof(float) * HID);
@@ -422,16 +474,21 @@ int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_
             int kvh = h / G;
             int hrow = share_first_head ? (h / G) * G : h;
             int64_t irow = ((int64_t)b * HEAD + hrow) * NBQ_rows + qb;
-            int64_t curr = 0;
+            int64_t curr = 0, pos_min = INT64_MAX;
             for (int j = 0; j < block_size_q; j++) {
                 int64_t it = (int64_t)qb * block_size_q + j;
                 if (it < TDST) {
                     int64_t sl = X->pos[(int64_t)b * TDST + it] + 1;
                     if (sl > curr) curr = sl;
+                    if (sl - 1 < pos_min) pos_min = sl - 1;
                 }
             }
             int nt = 0;
             int rs = ks_start_end[irow * 2 + 0], re = ks_start_end[irow * 2 + 1];
+            /* Rotated positions of keys outside the window (attention_extend_bsa.py:256-299): "streaming" packs
+             * sink and selected tokens, in the order of the index row, into the positions just below the window of
+             * the block's first query; "infllm" puts all of them at the window's edge. */
+            const int64_t shift = pos_min - sw - sink - (int64_t)(re - rs) * block_size_k + 1;
             if (BK <= 0) { rs = 0; re = 0; }
             for (int j = rs; j < rs + BK && j < re; j++) {
                 int64_t st = indices[irow * BK + j];
@@ -439,18 +496,25 @@ int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_
                     int64_t t = st + e;
                     if (t < 0 || t >= MAXT) continue;
                     if (!(t < curr && t >= sink)) continue;
-                    tok[nt] = t; kind[nt] = 0; nt++;
+                    tok[nt] = t; kind[nt] = 0;
+                    rpos[nt] = (int64_t)(j + sink / block_size_k) * block_size_k + e + shift;
+                    nt++;
                 }
             }
             int64_t sink_end = curr < sink ? curr : sink;
-            for (int64_t t = 0; t < sink_end; t++) { tok[nt] = t; kind[nt] = 0; nt++; }
+            for (int64_t t = 0; t < sink_end; t++) { tok[nt] = t; kind[nt] = 0; rpos[nt] = t + shift; nt++; }
             if (sw > 0) {
                 int64_t ws = curr - sw - block_size_q;
                 if (ws < 0) ws = 0;
-                for (int64_t t = ws; t < curr; t++) { tok[nt] = t; kind[nt] = 1; nt++; }
+                for (int64_t t = ws; t < curr; t++) { tok[nt] = t; kind[nt] = 1; rpos[nt] = t; nt++; }
             }
             for (int i = 0; i < nt; i++) {
-                scaled_key(X, b, tok[i], kvh, c_k, khat + (size_t)i * HID);
+                int64_t rp = rpos[i];
+                if (kind[i] == 0) {
+                    if (X->sa_backend == HIPO_EXT_INFLLM) rp = pos_min - sw;
+                    if (rp < 0) rp = 0;
+                }
+                scaled_key_at(X, b, tok[i], kvh, c_k, rp, khat + (size_t)i * HID);
                 fetch_row(X, 1, b, tok[i], kvh, vrow + (size_t)i * HID);
             }
             for (int j = 0; j < block_size_q; j++) {
@@ -458,8 +522,9 @@ int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_
                 if (it >= TDST) continue;
                 int64_t p = X->pos[(int64_t)b * TDST + it];
                 int64_t qoff = (((int64_t)b * TDST + it) * HEAD + h) * HID;
-                for (int d = 0; d < HID; d++)
-                    qhat[d] = round_T(load_T(X->q, qoff + d, X->dtype) * c_q, X->dtype);
+                for (int d = 0; d < HID; d++) qhat[d] = load_T(X->q, qoff + d, X->dtype);
+                if (X->rope_cos) rope_rotate(X, qhat, p); /* :796-852: the query keeps its true position */
+                for (int d = 0; d < HID; d++) qhat[d] = round_T(qhat[d] * c_q, X->dtype);
                 float m = -INFINITY;
                 for (int i = 0; i < nt; i++) {
                     int64_t t = tok[i];
@@ -486,7 +551,7 @@ int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_
                 for (int d = 0; d < HID; d++) store_T(out, qoff + d, (float)(acc[d] / lsum), X->dtype);
             }
         }
-        free(tok); free(kind); free(khat); free(vrow); free(qhat); free(logit); free(acc);
+        free(tok); free(kind); free(rpos); free(khat); free(vrow); free(qhat); free(logit); free(acc);
     }
     return 0;
 }

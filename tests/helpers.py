@@ -47,3 +47,25 @@ def tiny_args(**kw):
                 stages=[O.OStage(32, 2, 64, None, 1), O.OStage(32, 2, 16, 2048, 1), O.OStage(32, 1, 2, 1024, 1)])
     base.update(kw)
     return O.OArgs(**base)
+
+
+def rope_tables(length, D, dtype="f32", theta=10000.0):
+    """cos/sin tables [length, D] in the layout serving stacks keep (both halves repeat the D/2 frequencies),
+    as float32 values representable in ``dtype``; also returns the float64 angles [length, D/2]."""
+    inv = theta ** (-np.arange(0, D, 2, dtype=np.float64) / D)
+    ang = np.arange(length, dtype=np.float64)[:, None] * inv[None, :]
+    cos = np.concatenate([np.cos(ang), np.cos(ang)], axis=1).astype(np.float32)
+    sin = np.concatenate([np.sin(ang), np.sin(ang)], axis=1).astype(np.float32)
+    if dtype == "bf16":
+        cos = O.bf16_bits_to_f32(O.f32_to_bf16_bits(cos))
+        sin = O.bf16_bits_to_f32(O.f32_to_bf16_bits(sin))
+    return cos, sin, ang
+
+
+def with_rope(X, length, dtype=None, scan_backend=None, sa_backend=None):
+    """Attach RoPE tables (and optionally the rotation rules) to an OInputs."""
+    D = X.q.shape[-1]
+    cos, sin, _ = rope_tables(length, D, dtype or X.dtype)
+    X.rope_cos, X.rope_sin = cos, sin
+    X.scan_backend, X.sa_backend = scan_backend, sa_backend
+    return X
