@@ -48,6 +48,22 @@ int check_q(const hipattn_q_t *q) {
     return 0;
 }
 
+int make_rope_view(const hipattn_q_t *q, unsigned allowed, const char *who, RopeView *o) {
+    memset(o, 0, sizeof(*o));
+    const hipattn_rope_t *r = q->rope;
+    if (!r) return 0;
+    HIPATTN_CHECK_ARG(r->cos && r->sin && r->len > 0, HIPATTN_E_ARG, "%s: rope tables are null or empty", who);
+    HIPATTN_CHECK_ARG(r->backend >= 1 && r->backend < 32 && ((allowed >> r->backend) & 1u), HIPATTN_E_UNSUPPORTED,
+                      "%s: extend backend %d is not built for this entry point", who, r->backend);
+    const int esz = q->dtype == HIPATTN_BF16 ? 2 : 4;
+    HIPATTN_CHECK_ARG(aligned16(r->cos) && aligned16(r->sin) && (r->stride_t * esz) % 16 == 0 &&
+                          r->stride_t >= q->HID / 2,
+                      HIPATTN_E_ALIGN, "%s: rope table rows must be 16-byte aligned and hold HID/2 columns", who);
+    HIPATTN_CHECK_ARG(q->HID % 32 == 0, HIPATTN_E_UNSUPPORTED, "%s: rope needs a head dim that is a multiple of 32", who);
+    o->cos = r->cos; o->sin = r->sin; o->stride_t = r->stride_t; o->len = r->len; o->backend = r->backend;
+    return 0;
+}
+
 int make_kv_view(const hipattn_kv_t *kv, int B, int HID, int dtype, KVView *o, KVExt *x) {
     (void)B;
     HIPATTN_CHECK_ARG(kv && kv->k, HIPATTN_E_ARG, "kv: null K pointer");

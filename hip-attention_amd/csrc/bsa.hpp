@@ -26,7 +26,18 @@ struct BsaParamsBase {
 // the extended kernels (statistics, offload cache) take the same block with the extras appended
 struct BsaParams : BsaParamsBase {
     KVExt kx;
+    RopeView rope;
 };
+// Rotated position of a sink or selected key (attention_extend_bsa.py:256-299): "streaming" packs them, in the
+// order of the index row, into the positions that end just below the window of the block's first query;
+// "infllm" puts all of them at that edge.  `slot` = token for sink tokens, (j + sink / bk) * bk + e for element e
+// of index entry j; `shift` = pmin - sw - sink - (ks_end - ks_start) * bk + 1.
+__device__ __forceinline__ int64_t bsa_rope_far_pos(const RopeView &r, long long slot, long long shift, long long pmin,
+                                                    int sw) {
+    const long long v = r.backend == HIPATTN_EXTEND_INFLLM ? pmin - sw : slot + shift;
+    return v < 0 ? 0 : v;
+}
+
 template <bool EXT>
 using BsaParamsFor = std::conditional_t<EXT, BsaParams, BsaParamsBase>;
 

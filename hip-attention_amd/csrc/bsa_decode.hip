@@ -17,8 +17,11 @@ struct DecodeParamsT {
 };
 using DecodeParams = DecodeParamsT<true>;
 
-template <typename T, int HID, int G, bool EXT>
+// ROPE = true (extended parameter block only): query and keys are rotated on load; lanes dl and dl ^ 8 of a
+// 16-lane group hold the two halves of a row.
+template <typename T, int HID, int G, bool EXT, bool ROPE = false>
 __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<EXT> dp) {
+    static_assert(!ROPE || EXT, "rope variant takes the extended parameter block");
     constexpr int SEG = HID / 16;
     const BsaParamsFor<EXT> &p = dp.a;
     const KVExt *kx = nullptr;
@@ -37,6 +40,7 @@ __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<E
     const long long ppos = p.pos[(int64_t)b * p.pos_sb];
     const long long curr = ppos + 1;
     int rs = p.kse[irow * 2 + 0], re = p.kse[irow * 2 + 1];
+    const long long rope_shift = ppos - p.sw - p.sink - (long long)(re - rs) * p.bk + 1;
     if (p.BK <= 0) { rs = 0; re = 0; }
     const int jend = rs + p.BK < re ? rs + p.BK : re;
     const int nsel = jend > rs ? jend - rs : 0;
@@ -60,6 +64,15 @@ __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<E
     for (int g = 0; g < G; g++) {
         const T *qrow = reinterpret_cast<const T *>(p.q) + (int64_t)b * p.q_sb + (int64_t)(h0 + g) * p.q_sh;
         load_elems<T, SEG>(qrow + dl * SEG, qh[g]);
+        if constexpr (ROPE) {  // the query keeps its own position (attention_decode_bsa.py:135-262)
+            float other[SEG], rc[SEG], rsn[SEG];
+            load_elems<T, SEG>(qrow + (dl ^ 8) * SEG, other);
+            const int64_t tr = p.rope.row(ppos) + (dl & 7) * SEG;
+            load_elems<T, SEG>(reinterpret_cast<const T *>(p.rope.cos) + tr, rc);
+            load_elems<T, SEG>(reinterpret_cast<const T *>(p.rope.sin) + tr, rsn);
+#pragma unroll
+            for (int e = 0; e < SEG; e++) qh[g][e] = rope_elem<T>(qh[g][e], dl < 8 ? -other[e] : other[e], rc[e], rsn[e]);
+        }
 #pragma unroll
         for (int e = 0; e < SEG; e++) qh[g][e] = Elem<T>::round(qh[g][e] * p.c_q);
     }
@@ -77,18 +90,24 @@ __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<E
         long long t = -1;
         int kind = 0;
         bool valid = false;
+        long long rpos = 0;  // rotated position of the key (ROPE only)
         if (o < o_end) {
             if (o < n_sel_tok) {
                 const long long st = p.indices[irow * p.BK + rs + o / p.bk];
                 t = st + o % p.bk;
                 valid = (t >= 0) && (t < p.kv.max_tsrc) && (t < curr) && (t >= p.sink);
+                if constexpr (ROPE)
+                    rpos = bsa_rope_far_pos(p.rope, (rs + o / p.bk + p.sink / p.bk) * (long long)p.bk + o % p.bk, rope_shift,
+                                            ppos, p.sw);
             } else if (o < n_sel_tok + sink_end) {
                 t = o - n_sel_tok;
                 valid = true;
+                if constexpr (ROPE) rpos = bsa_rope_far_pos(p.rope, t, rope_shift, ppos, p.sw);
             } else {
                 t = ws0 + (o - n_sel_tok - sink_end);
                 kind = 1;
                 valid = true;
+                rpos = t;
             }
         }
         const bool att = valid && (kind == 0 ? (t + p.sw <= ppos) : (t <= ppos && ppos < t + p.sw));
@@ -111,6 +130,17 @@ __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<E
         } else {
 #pragma unroll
             for (int e = 0; e < SEG; e++) vv[e] = 0.0f;
+        }
+        if constexpr (ROPE) {
+            float rc[SEG], rsn[SEG];
+            const int64_t tr = p.rope.row(rpos) + (dl & 7) * SEG;
+            load_elems<T, SEG>(reinterpret_cast<const T *>(p.rope.cos) + tr, rc);
+            load_elems<T, SEG>(reinterpret_cast<const T *>(p.rope.sin) + tr, rsn);
+#pragma unroll
+            for (int e = 0; e < SEG; e++) {
+                const float other = __shfl_xor(kh[e], 8);
+                kh[e] = rope_elem<T>(kh[e], dl < 8 ? -other : other, rc[e], rsn[e]);
+            }
         }
 #pragma unroll
         for (int e = 0; e < SEG; e++) kh[e] = Elem<T>::round(kh[e] * p.c_k);
@@ -215,7 +245,9 @@ static int launch_partial(const DecodeParams &dp, hipStream_t st) {
 #define DEC_CASE(GG)                                                                                   \
     if constexpr (GG * HID <= 512) {                                                                   \
         if (dp.a.G == GG) {                                                                            \
-            if (dp.a.kx.extended()) {                                                                  \
+            if (dp.a.rope.cos) {                                                                       \
+                hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG, true, true>), grid, block, 0, st, dp); \
+            } else if (dp.a.kx.extended()) {                                                           \
                 hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG, true>), grid, block, 0, st, dp);  \
             } else {                                                                                   \
                 DecodeParamsT<false> dq;                                                               \

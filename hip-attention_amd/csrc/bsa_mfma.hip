@@ -50,8 +50,12 @@ struct MfmaSmem {
     int idx[MAX_LDS_IDX];
 };
 
-template <int HID, bool KSCALED, bool EXT>
+// ROPE = true (extended parameter block, unscaled keys): query rows and staged key rows are rotated on load.
+// A query lane holds both halves of its row (k-steps ks and ks + KS/2); the two halves of a staged key row are
+// fetched by lanes tid and tid ^ (HID/16) of one wave.
+template <int HID, bool KSCALED, bool EXT, bool ROPE = false>
 __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p, int hgroups, int hpw, long long total_wg) {
+    static_assert(!ROPE || (EXT && !KSCALED), "rope variant: extended parameter block, keys scaled in the kernel");
     const KVExt *kx = nullptr;
     if constexpr (EXT) kx = &p.kx;
     constexpr int KS = HID / 16;   // k-steps of the first product
@@ -107,6 +111,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
 
     const int curr = pmax_blk + 1;
     int rs = p.kse[irow * 2 + 0], re = p.kse[irow * 2 + 1];
+    const long long rope_shift = (long long)pmin_blk - p.sw - p.sink - (long long)(re - rs) * p.bk + 1;
     if (p.BK <= 0) { rs = 0; re = 0; }
     const int jend = rs + p.BK < re ? rs + p.BK : re;
     const int nsel = jend > rs ? jend - rs : 0;
@@ -134,10 +139,29 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
     {
         const uint16_t *qbase = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
         const bool ok = head_ok && row_ok;
+        uint4 qraw[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
-            uint4 raw = make_uint4(0, 0, 0, 0);
-            if (ok) raw = *reinterpret_cast<const uint4 *>(qbase + myit * p.q_st + ks * 16 + hh * 8);
+            qraw[ks] = make_uint4(0, 0, 0, 0);
+            if (ok) qraw[ks] = *reinterpret_cast<const uint4 *>(qbase + myit * p.q_st + ks * 16 + hh * 8);
+        }
+        if constexpr (ROPE) {
+            if (ok) {  // the query keeps its own position (attention_extend_bsa.py:796-852)
+                const uint16_t *ct = reinterpret_cast<const uint16_t *>(p.rope.cos) + p.rope.row(pq);
+                const uint16_t *st = reinterpret_cast<const uint16_t *>(p.rope.sin) + p.rope.row(pq);
+#pragma unroll
+                for (int ks = 0; ks < KS / 2; ks++) {
+                    const uint4 c = *reinterpret_cast<const uint4 *>(ct + ks * 16 + hh * 8);
+                    const uint4 sn = *reinterpret_cast<const uint4 *>(st + ks * 16 + hh * 8);
+                    const uint4 lo = qraw[ks], hi = qraw[ks + KS / 2];
+                    qraw[ks] = rope_piece(lo, hi, c, sn, true);
+                    qraw[ks + KS / 2] = rope_piece(hi, lo, c, sn, false);
+                }
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const uint4 raw = qraw[ks];
             const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
             for (int e = 0; e < 4; e++)
@@ -152,6 +176,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
 
     // ---- staging: thread handles chunks c = tid + NTHREADS*j: token slot c / (HID/8), 16-byte piece c % (HID/8)
     uint4 kreg[CPT], vreg[CPT];
+    uint4 creg[ROPE ? CPT : 1], sreg[ROPE ? CPT : 1];  // cos / sin pieces of the staged key rows
     int treg[CPT];
     auto prefetch = [&](int tile) {
         int kind, base;  // kind 0 selected, 1 sink, 2 window
@@ -164,21 +189,32 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
             const int slot = c / (HID / 8), piece = c % (HID / 8);
             const int o = base + slot;
             long long t = -1;
+            long long rpos = 0;  // rotated position of the key (ROPE only)
             if (kind == 0) {
                 if (o < n_sel_tok) {
                     const int bi = o / p.bk;
                     const long long st = idx_in_lds ? (long long)sm.idx[bi] : p.indices[irow * p.BK + rs + bi];
                     t = st + o % p.bk;
                     if (!(t >= 0 && t < p.kv.max_tsrc && t < curr && t >= p.sink)) t = -1;
+                    if constexpr (ROPE)
+                        rpos = bsa_rope_far_pos(p.rope, (long long)(rs + bi + p.sink / p.bk) * p.bk + o % p.bk, rope_shift,
+                                                pmin_blk, p.sw);
                 }
             } else if (kind == 1) {
                 if (o < sink_end) t = o;
+                if constexpr (ROPE) rpos = bsa_rope_far_pos(p.rope, o, rope_shift, pmin_blk, p.sw);
             } else {
                 if (o < n_win) t = ws + o;
+                rpos = t;
             }
             treg[j] = (int)t;
             kreg[j] = make_uint4(0, 0, 0, 0);
             vreg[j] = make_uint4(0, 0, 0, 0);
+            if constexpr (ROPE) {
+                const int64_t tr = p.rope.row(rpos) + (piece % (HID / 16)) * 8;
+                creg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr);
+                sreg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr);
+            }
             if (t >= 0) {
                 int64_t ko, vo;
                 kv_rows<true, EXT>(p.kv, kx, b, t, kvh, seqlen, ko, vo, piece == 0);
@@ -193,6 +229,11 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
             const int c = tid + NTHREADS * j;
             const int slot = c / (HID / 8), piece = c % (HID / 8);
             uint4 kq = kreg[j];
+            if constexpr (ROPE) {
+                const uint4 oth = make_uint4(__shfl_xor(kq.x, HID / 16), __shfl_xor(kq.y, HID / 16),
+                                             __shfl_xor(kq.z, HID / 16), __shfl_xor(kq.w, HID / 16));
+                kq = rope_piece(kq, oth, creg[j], sreg[j], piece < HID / 16);
+            }
             if (!KSCALED) {
                 kq.x = cvt_pk_bf16(__uint_as_float(kq.x << 16) * p.c_k, __uint_as_float(kq.x & 0xffff0000u) * p.c_k);
                 kq.y = cvt_pk_bf16(__uint_as_float(kq.y << 16) * p.c_k, __uint_as_float(kq.y & 0xffff0000u) * p.c_k);
@@ -390,7 +431,7 @@ __global__ __launch_bounds__(256) void bsa_mark_kernel(BsaParams p, int hgroups,
     }
 }
 
-template <int HID, bool KSCALED, bool EXT>
+template <int HID, bool KSCALED, bool EXT, bool ROPE = false>
 static int launch_mfma(const BsaParams &p, hipStream_t st) {
     const int hpw = p.share_first_head ? 4 : 1;  // per-head index rows: one head per workgroup
     const int hgroups = (p.G + hpw - 1) / hpw;
@@ -399,12 +440,12 @@ static int launch_mfma(const BsaParams &p, hipStream_t st) {
     const size_t smem = sizeof(MfmaSmem<HID>);
     static bool attr_set = false;
     if (!attr_set) {
-        HIPATTN_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&bsa_mfma_kernel<HID, KSCALED, EXT>),
+        HIPATTN_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&bsa_mfma_kernel<HID, KSCALED, EXT, ROPE>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
     const BsaParamsFor<EXT> &pk = p;  // the plain kernel takes the block without the extras
-    hipLaunchKernelGGL((bsa_mfma_kernel<HID, KSCALED, EXT>), dim3((unsigned)total), dim3(NTHREADS), smem, st, pk, hgroups,
+    hipLaunchKernelGGL((bsa_mfma_kernel<HID, KSCALED, EXT, ROPE>), dim3((unsigned)total), dim3(NTHREADS), smem, st, pk, hgroups,
                        hpw, total);
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
@@ -429,8 +470,13 @@ int bsa_mfma_launch(const BsaParams &p, int dtype, int HID, hipStream_t st) {
         plain.kx.miss_flags = nullptr;
         return bsa_mfma_launch(plain, dtype, HID, st);
     }
+    if (p.rope.cos && p.k_prescaled) {
+        set_error("bsa: prescaled keys cannot be combined with rope applied on load");
+        return HIPATTN_E_ARG;
+    }
 #define BSA_PICK(H)                                                                  \
     case H:                                                                          \
+        if (p.rope.cos) return launch_mfma<H, false, true, true>(p, st);             \
         if (p.k_prescaled) return ext ? launch_mfma<H, true, true>(p, st) : launch_mfma<H, true, false>(p, st); \
         return ext ? launch_mfma<H, false, true>(p, st) : launch_mfma<H, false, false>(p, st);
     switch (HID) {

@@ -10,9 +10,10 @@
 
 namespace hipattn {
 
-template <typename T, int HID>
+template <typename T, int HID, bool ROPE>
 __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
     constexpr int DPL = (HID + 63) / 64;  // output elements per lane
+    constexpr int HALF = HID / 2;
     __shared__ float s_q[4][HID];
     const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
     const int qb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -21,20 +22,24 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
     const int64_t irow = ((int64_t)b * p.HEAD + hrow) * p.idx_rows + qb;
 
     // CURR = largest position + 1 over the block's rows
-    long long curr = 0;
+    long long curr = 0, pmin = 0x7fffffffffffffffLL;
     for (int j = lane; j < p.bq; j += 64) {
         long long it = (long long)qb * p.bq + j;
         if (it < p.TDST) {
             long long sl = p.pos[(int64_t)b * p.pos_sb + it * p.pos_st] + 1;
             curr = sl > curr ? sl : curr;
+            pmin = sl - 1 < pmin ? sl - 1 : pmin;
         }
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
         long long w = __shfl_xor(curr, o);
         curr = w > curr ? w : curr;
+        long long w2 = __shfl_xor(pmin, o);
+        pmin = w2 < pmin ? w2 : pmin;
     }
     int rs = p.kse[irow * 2 + 0], re = p.kse[irow * 2 + 1];
+    const long long rope_shift = pmin - p.sw - p.sink - (long long)(re - rs) * p.bk + 1;
     if (p.BK <= 0) { rs = 0; re = 0; }
     int jend = rs + p.BK < re ? rs + p.BK : re;
     const int nsel = jend > rs ? jend - rs : 0;
@@ -53,7 +58,16 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
         if (it >= p.TDST) break;  // uniform per wave
         const long long ppos = p.pos[(int64_t)b * p.pos_sb + it * p.pos_st];
         const T *qrow = reinterpret_cast<const T *>(p.q) + (int64_t)b * p.q_sb + it * p.q_st + (int64_t)h * p.q_sh;
-        for (int d = lane; d < HID; d += 64) s_q[wid][d] = Elem<T>::round(Elem<T>::widen(qrow[d]) * p.c_q);
+        for (int d = lane; d < HID; d += 64) {
+            float x = Elem<T>::widen(qrow[d]);
+            if constexpr (ROPE) {  // the query keeps its own position (attention_extend_bsa.py:796-852)
+                const int64_t tr = p.rope.row(ppos) + d % HALF;
+                const float other = Elem<T>::widen(qrow[(d + HALF) % HID]);
+                x = rope_elem<T>(x, d < HALF ? -other : other, Elem<T>::widen(reinterpret_cast<const T *>(p.rope.cos)[tr]),
+                                 Elem<T>::widen(reinterpret_cast<const T *>(p.rope.sin)[tr]));
+            }
+            s_q[wid][d] = Elem<T>::round(x * p.c_q);
+        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -68,17 +82,23 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
             long long t = -1;
             int kind = 0;
             bool valid = false;
+            long long rpos = 0;  // rotated position of the key (ROPE only)
             if (o < n_sel_tok) {
                 const long long st = p.indices[irow * p.BK + rs + o / p.bk];
                 t = st + o % p.bk;
                 valid = (t >= 0) && (t < p.kv.max_tsrc) && (t < curr) && (t >= p.sink);
+                if constexpr (ROPE)
+                    rpos = bsa_rope_far_pos(p.rope, (rs + o / p.bk + p.sink / p.bk) * (long long)p.bk + o % p.bk, rope_shift,
+                                            pmin, p.sw);
             } else if (o < n_sel_tok + sink_end) {
                 t = o - n_sel_tok;
                 valid = true;
+                if constexpr (ROPE) rpos = bsa_rope_far_pos(p.rope, t, rope_shift, pmin, p.sw);
             } else if (o < total) {
                 t = ws + (o - n_sel_tok - sink_end);
                 kind = 1;
                 valid = true;
+                rpos = t;
             }
             const bool att = valid && (kind == 0 ? (t + p.sw <= ppos) : (t <= ppos && ppos < t + p.sw));
             float logit = -INFINITY;
@@ -98,6 +118,16 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
                     for (int d0 = 0; d0 < HID; d0 += CH) {
                         float kk[CH];
                         load_elems<T, CH>(kbase + koff + d0, kk);
+                        if constexpr (ROPE) {
+                            float other[CH], rc[CH], rsn[CH];
+                            load_elems<T, CH>(kbase + koff + (d0 + HALF) % HID, other);
+                            const int64_t tr = p.rope.row(rpos) + d0 % HALF;
+                            load_elems<T, CH>(reinterpret_cast<const T *>(p.rope.cos) + tr, rc);
+                            load_elems<T, CH>(reinterpret_cast<const T *>(p.rope.sin) + tr, rsn);
+#pragma unroll
+                            for (int e = 0; e < CH; e++)
+                                kk[e] = rope_elem<T>(kk[e], d0 < HALF ? -other[e] : other[e], rc[e], rsn[e]);
+                        }
 #pragma unroll
                         for (int e = 0; e < CH; e++)
                             dot = __fmaf_rn(s_q[wid][d0 + e], Elem<T>::round(kk[e] * p.c_k), dot);
@@ -145,7 +175,8 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
 template <typename T, int HID>
 static int launch_simple(const BsaParams &p, hipStream_t stream) {
     dim3 grid((unsigned)p.NBQ, (unsigned)p.HEAD, (unsigned)p.B), block(256);
-    hipLaunchKernelGGL((bsa_simple_kernel<T, HID>), grid, block, 0, stream, p);
+    if (p.rope.cos) hipLaunchKernelGGL((bsa_simple_kernel<T, HID, true>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((bsa_simple_kernel<T, HID, false>), grid, block, 0, stream, p);
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
 }
@@ -159,6 +190,8 @@ int bsa_fill_params(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t 
     HIPATTN_CHECK_ARG(BK <= 0 || indices, HIPATTN_E_ARG, "bsa: indices is null with BK > 0");
     HIPATTN_CHECK_ARG(bq > 0 && bk > 0 && sw >= 0 && sink >= 0 && idx_rows > 0, HIPATTN_E_ARG, "bsa: bad sizes");
     rc = make_kv_view(kv, q->B, q->HID, q->dtype, &p->kv, &p->kx);
+    if (rc) return rc;
+    rc = make_rope_view(q, (1u << HIPATTN_EXTEND_STREAMING) | (1u << HIPATTN_EXTEND_INFLLM), "bsa", &p->rope);
     if (rc) return rc;
     HIPATTN_CHECK_ARG(q->HEAD % p->kv.HKV == 0, HIPATTN_E_ARG, "bsa: HEAD %% HKV != 0");
     p->q = q->ptr; p->q_sb = q->stride_b; p->q_st = q->stride_t; p->q_sh = q->stride_h;

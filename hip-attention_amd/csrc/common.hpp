@@ -278,6 +278,49 @@ __device__ __forceinline__ int64_t kv_k_row(const KVView &kv, const KVExt *kx, i
     return ko;
 }
 
+// ---------------------------------------------------------------- rotary embedding applied on load
+// Device copy of hipattn_rope_t.  cos == nullptr: rows are used as stored.
+struct RopeView {
+    const void *cos, *sin;
+    int64_t stride_t, len;
+    int backend;  // HIPATTN_EXTEND_*
+    __device__ __forceinline__ int64_t row(int64_t pos) const {  // element offset of the table row of a position
+        pos = pos < 0 ? 0 : (pos >= len ? len - 1 : pos);
+        return pos * stride_t;
+    }
+};
+
+// One element of a rotated row: x*c + o*s with `o` the partner element, already signed (-x[i + HID/2] in the
+// lower half, +x[i - HID/2] in the upper); both products and the sum are rounded to T, never fused.
+template <typename T>
+__device__ __forceinline__ float rope_elem(float x, float o, float c, float s) {
+    return Elem<T>::round(__fadd_rn(Elem<T>::round(__fmul_rn(x, c)), Elem<T>::round(__fmul_rn(o, s))));
+}
+
+typedef __attribute__((ext_vector_type(2))) __bf16 rope_bf16x2;
+typedef __attribute__((ext_vector_type(2))) float rope_f32x2;
+__device__ __forceinline__ uint32_t rope_pk(float a, float b) {  // two f32 -> packed bf16, round to nearest even
+    rope_f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, rope_bf16x2));
+}
+// The same on a packed pair of bf16: w own pair, o partner pair, c and s table pairs; `s` must already carry the
+// sign of the half (xor 0x80008000 for the lower half).
+__device__ __forceinline__ uint32_t rope_pair(uint32_t w, uint32_t o, uint32_t c, uint32_t s) {
+    const uint32_t a = rope_pk(__fmul_rn(__uint_as_float(w << 16), __uint_as_float(c << 16)),
+                               __fmul_rn(__uint_as_float(w & 0xffff0000u), __uint_as_float(c & 0xffff0000u)));
+    const uint32_t b = rope_pk(__fmul_rn(__uint_as_float(o << 16), __uint_as_float(s << 16)),
+                               __fmul_rn(__uint_as_float(o & 0xffff0000u), __uint_as_float(s & 0xffff0000u)));
+    return rope_pk(__fadd_rn(__uint_as_float(a << 16), __uint_as_float(b << 16)),
+                   __fadd_rn(__uint_as_float(a & 0xffff0000u), __uint_as_float(b & 0xffff0000u)));
+}
+__device__ __forceinline__ uint4 rope_piece(uint4 w, uint4 o, uint4 c, uint4 s, bool lower) {
+    const uint32_t sg = lower ? 0x80008000u : 0u;
+    return make_uint4(rope_pair(w.x, o.x, c.x, s.x ^ sg), rope_pair(w.y, o.y, c.y, s.y ^ sg),
+                      rope_pair(w.z, o.z, c.z, s.z ^ sg), rope_pair(w.w, o.w, c.w, s.w ^ sg));
+}
+
+// validates q->rope (may be NULL) and fills the view; `allowed` is a bit mask of HIPATTN_EXTEND_* values
+int make_rope_view(const hipattn_q_t *q, unsigned allowed, const char *who, RopeView *out);
 int make_kv_view(const hipattn_kv_t *kv, int B, int HID, int dtype, KVView *out, KVExt *ext);
 int cache_view_for(const hipattn_cache *c, const hipattn_kv_t *kv, const KVView *view, int HID, int dtype, KVExt *ext);
 int check_q(const hipattn_q_t *q);

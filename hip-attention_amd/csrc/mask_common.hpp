@@ -30,6 +30,7 @@ struct MaskParamsBase {
 // the extended kernels (statistics, offload cache) take the same block with the extras appended
 struct MaskParams : MaskParamsBase {
     KVExt kx;
+    RopeView rope;
 };
 template <bool EXT>
 using MaskParamsFor = std::conditional_t<EXT, MaskParams, MaskParamsBase>;

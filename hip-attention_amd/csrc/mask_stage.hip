@@ -52,9 +52,24 @@ __device__ __forceinline__ float reduce16(const float (&part)[ROWS], int dl) {
     }
 }
 
-template <typename T, int HID, int ROWS, int MAXROWS, int STEPS>
+// Position a query row is rotated to in the mask stage (attention_extend.py:632-647)
+__device__ __forceinline__ int64_t mask_rope_qpos(const RopeView &r, long long pos, int n, int sw_eff) {
+    if (r.backend == HIPATTN_EXTEND_RELATIVE) return 1 + (int64_t)sw_eff;
+    if (r.backend == HIPATTN_EXTEND_INFLLM) return sw_eff;
+    const long long cap = (long long)n + sw_eff;
+    return pos < cap ? pos : cap;
+}
+// Position the sampled key of chunk `c` is rotated to (attention_extend.py:289-298)
+__device__ __forceinline__ int64_t mask_rope_kpos(const RopeView &r, int c, int side) {
+    if (r.backend == HIPATTN_EXTEND_RELATIVE) return side;
+    if (r.backend == HIPATTN_EXTEND_STREAMING) return c;
+    return 0;
+}
+
+template <typename T, int HID, int ROWS, int MAXROWS, int STEPS, bool ROPE>
 __global__ __launch_bounds__(64) void mask_stage_kernel(MaskParams p) {
     constexpr int SEG = HID / 16;
+    constexpr int HALF = HID / 2;
     __shared__ int64_t s_koff[128];
     __shared__ float s_sc[128];
     __shared__ __align__(16) T s_q[MAXROWS * HID];
@@ -126,9 +141,21 @@ __global__ __launch_bounds__(64) void mask_stage_kernel(MaskParams p) {
             const long long it = qb * p.BQ + (long long)j * p.stride_q;
             float sum = 0.0f;
             int cnt = 0;
+            float rc = 0.0f, rsn = 0.0f;
+            if constexpr (ROPE) {
+                // every strided row is rotated to the position derived from the base row
+                const int64_t tr = p.rope.row(mask_rope_qpos(p.rope, p.pos[(int64_t)b * p.pos_sb + it * p.pos_st], p.n, p.sw_eff));
+                rc = Elem<T>::widen(reinterpret_cast<const T *>(p.rope.cos)[tr + d % HALF]);
+                rsn = Elem<T>::widen(reinterpret_cast<const T *>(p.rope.sin)[tr + d % HALF]);
+            }
             for (int o = 0; o < p.stride_q; o++) {
                 if (it + o < p.TDST) {
-                    sum += Elem<T>::widen(qbase[(it + o) * p.q_st + d]);
+                    float x = Elem<T>::widen(qbase[(it + o) * p.q_st + d]);
+                    if constexpr (ROPE) {
+                        const float other = Elem<T>::widen(qbase[(it + o) * p.q_st + (d + HALF) % HID]);
+                        x = rope_elem<T>(x, d < HALF ? -other : other, rc, rsn);
+                    }
+                    sum += x;
                     cnt++;
                 }
             }
@@ -194,6 +221,19 @@ __global__ __launch_bounds__(64) void mask_stage_kernel(MaskParams p) {
                     if ((cs + st) < nsteps) {
                         float kh[SEG];
                         raw[st].widen(kh);
+                        if constexpr (ROPE) {
+                            // lanes dl and dl ^ 8 of a row group hold the two halves of the row
+                            const int krow = (cs + st) * 4 + sub;
+                            const int64_t tr = p.rope.row(mask_rope_kpos(p.rope, g * BC + (krow >> 1), krow & 1)) + (dl & 7) * SEG;
+                            float rc[SEG], rsn[SEG];
+                            load_elems<T, SEG>(reinterpret_cast<const T *>(p.rope.cos) + tr, rc);
+                            load_elems<T, SEG>(reinterpret_cast<const T *>(p.rope.sin) + tr, rsn);
+#pragma unroll
+                            for (int e = 0; e < SEG; e++) {
+                                const float other = __shfl_xor(kh[e], 8);
+                                kh[e] = rope_elem<T>(kh[e], dl < 8 ? -other : other, rc[e], rsn[e]);
+                            }
+                        }
 #pragma unroll
                         for (int e = 0; e < SEG; e++) kh[e] = Elem<T>::round(kh[e] * p.c_k);
                         float part[ROWS];
@@ -237,20 +277,20 @@ __global__ __launch_bounds__(64) void mask_stage_kernel(MaskParams p) {
     }
 }
 
-template <typename T, int HID>
+template <typename T, int HID, bool ROPE>
 static int launch_mask(const MaskParams &p, int rows_eff, hipStream_t stream) {
     dim3 grid((unsigned)p.total), block(64);
     if (rows_eff <= 1) {
         if (p.block_chunk == 64)
-            hipLaunchKernelGGL((mask_stage_kernel<T, HID, 1, 1, 32>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((mask_stage_kernel<T, HID, 1, 1, 32, ROPE>), grid, block, 0, stream, p);
         else
-            hipLaunchKernelGGL((mask_stage_kernel<T, HID, 1, 1, 8>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((mask_stage_kernel<T, HID, 1, 1, 8, ROPE>), grid, block, 0, stream, p);
     } else if (rows_eff <= 4) {
-        hipLaunchKernelGGL((mask_stage_kernel<T, HID, 4, 4, 8>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((mask_stage_kernel<T, HID, 4, 4, 8, ROPE>), grid, block, 0, stream, p);
     } else if (rows_eff <= 16) {
-        hipLaunchKernelGGL((mask_stage_kernel<T, HID, 16, 16, 8>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((mask_stage_kernel<T, HID, 16, 16, 8, ROPE>), grid, block, 0, stream, p);
     } else if (rows_eff <= 64) {
-        hipLaunchKernelGGL((mask_stage_kernel<T, HID, 16, 64, 8>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((mask_stage_kernel<T, HID, 16, 64, 8, ROPE>), grid, block, 0, stream, p);
     } else {
         set_error("mask stage: %d query rows per program exceed the supported 64", rows_eff);
         return HIPATTN_E_UNSUPPORTED;
@@ -283,6 +323,11 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
     MaskParams p;
     rc = make_kv_view(kv, q->B, q->HID, q->dtype, &p.kv, &p.kx);
     if (rc) return rc;
+    rc = make_rope_view(q, (1u << HIPATTN_EXTEND_RELATIVE) | (1u << HIPATTN_EXTEND_STREAMING) | (1u << HIPATTN_EXTEND_INFLLM),
+                        "mask stage", &p.rope);
+    if (rc) return rc;
+    HIPATTN_CHECK_ARG(!(p.rope.cos && k_prescaled), HIPATTN_E_ARG,
+                      "mask stage: prescaled keys cannot be combined with rope applied on load");
     HIPATTN_CHECK_ARG(q->HEAD % p.kv.HKV == 0, HIPATTN_E_ARG, "mask stage: HEAD %% HKV != 0");
     p.q = q->ptr; p.q_sb = q->stride_b; p.q_st = q->stride_t; p.q_sh = q->stride_h;
     p.pos = q->pos; p.pos_sb = q->pos_stride_b; p.pos_st = q->pos_stride_t;
@@ -317,10 +362,11 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
         return mask_stage_mfma_launch(p, q->HID, rows_eff, k_prescaled, st);
     } else if (q->dtype == HIPATTN_F32) {
         HIPATTN_CHECK_ARG(!k_prescaled, HIPATTN_E_ARG, "mask stage: prescaled keys are a bf16-only option");
+        const bool rope = p.rope.cos != nullptr;
         switch (q->HID) {
-            case 32: return launch_mask<float, 32>(p, rows_eff, st);
-            case 64: return launch_mask<float, 64>(p, rows_eff, st);
-            case 128: return launch_mask<float, 128>(p, rows_eff, st);
+            case 32: return rope ? launch_mask<float, 32, true>(p, rows_eff, st) : launch_mask<float, 32, false>(p, rows_eff, st);
+            case 64: return rope ? launch_mask<float, 64, true>(p, rows_eff, st) : launch_mask<float, 64, false>(p, rows_eff, st);
+            case 128: return rope ? launch_mask<float, 128, true>(p, rows_eff, st) : launch_mask<float, 128, false>(p, rows_eff, st);
         }
     }
     set_error("mask stage: head dim %d with dtype %d is not built", q->HID, q->dtype);

@@ -43,8 +43,26 @@ __device__ __forceinline__ uint32_t scale_pack(uint32_t w, float c) {
     return cvt_pk_bf16(__uint_as_float(w << 16) * c, __uint_as_float(w & 0xffff0000u) * c);
 }
 
-template <int HID, int MB, int NB, bool PRESCALED, bool VIA_LDS, bool EXT>
+// rotated position of a query row / of the sampled key of chunk c (attention_extend.py:632-647, :289-298)
+__device__ __forceinline__ int64_t rope_qpos(const RopeView &r, long long pos, int n, int sw_eff) {
+    if (r.backend == HIPATTN_EXTEND_RELATIVE) return 1 + (int64_t)sw_eff;
+    if (r.backend == HIPATTN_EXTEND_INFLLM) return sw_eff;
+    const long long cap = (long long)n + sw_eff;
+    return pos < cap ? pos : cap;
+}
+__device__ __forceinline__ int64_t rope_kpos(const RopeView &r, int c, int side) {
+    if (r.backend == HIPATTN_EXTEND_RELATIVE) return side;
+    if (r.backend == HIPATTN_EXTEND_STREAMING) return c;
+    return 0;
+}
+
+// ROPE = true (direct path, one token block per wave, extended parameter block): every sampled key row is rotated
+// before it is scaled.  The two halves of a row sit in the two half-waves (lane and lane ^ 32) at the same k-step,
+// and the rotated position of a lane's key never changes over the iterations, so its cos/sin entries are loaded
+// once and stay in registers.
+template <int HID, int MB, int NB, bool PRESCALED, bool VIA_LDS, bool EXT, bool ROPE = false>
 __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
+    static_assert(!ROPE || (EXT && !VIA_LDS && !PRESCALED), "rope variant: direct path of the extended build");
     const KVExt *kx = nullptr;
     if constexpr (EXT) kx = &p.kx;
     constexpr int KS = HID / 16;
@@ -182,6 +200,19 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
     const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
     const uint16_t *kbase = reinterpret_cast<const uint16_t *>(p.kv.k);
 
+    uint4 rcos[ROPE ? NB : 1][ROPE ? KS : 1], rsin[ROPE ? NB : 1][ROPE ? KS : 1];
+    if constexpr (ROPE) {
+#pragma unroll
+        for (int tb = 0; tb < NB; tb++) {
+            const int64_t tr = p.rope.row(rope_kpos(p.rope, cidx[tb], side));
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                rcos[tb][ks] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr + ks * 8);
+                rsin[tb][ks] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr + ks * 8);
+            }
+        }
+    }
+
     const int lrow = lane / PPR, lpos = lane % PPR;  // loader role: row within an instruction, piece slot
     while (width >= p.terminate) {
         width *= 0.5f;
@@ -245,6 +276,15 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
                     kf.q = s_rows[r * PPR + ((hh * (PPR / 2) + ks) ^ sw)];
                 } else if constexpr (PRESCALED) {
                     kf.q = raw[tb][ks];
+                } else if constexpr (ROPE) {
+                    const uint4 own = raw[tb][ks];
+                    const uint4 oth = make_uint4(__shfl_xor(own.x, 32), __shfl_xor(own.y, 32), __shfl_xor(own.z, 32),
+                                                 __shfl_xor(own.w, 32));
+                    const uint4 rot = rope_piece(own, oth, rcos[tb][ks], rsin[tb][ks], hh == 0);
+                    kf.u[0] = scale_pack(rot.x, p.c_k);
+                    kf.u[1] = scale_pack(rot.y, p.c_k);
+                    kf.u[2] = scale_pack(rot.z, p.c_k);
+                    kf.u[3] = scale_pack(rot.w, p.c_k);
                 } else {
                     kf.u[0] = scale_pack(raw[tb][ks].x, p.c_k);
                     kf.u[1] = scale_pack(raw[tb][ks].y, p.c_k);
@@ -310,9 +350,23 @@ __global__ void qhat_kernel(MaskParams p, int hid, uint16_t *out) {
         const uint16_t *qbase = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
         float sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         int cnt = 0;
+        const bool rope = p.rope.cos != nullptr;
+        const int ppiece = (piece + per_row / 2) % per_row;  // the piece holding the partner elements
+        uint4 rc = make_uint4(0, 0, 0, 0), rs = rc;
+        if (rope) {
+            // every strided row is rotated to the position derived from the base row (attention_extend.py:626-690)
+            const int64_t tr = p.rope.row(rope_qpos(p.rope, p.pos[(int64_t)b * p.pos_sb + it * p.pos_st], p.n, p.sw_eff)) +
+                               (piece % (per_row / 2)) * 8;
+            rc = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr);
+            rs = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr);
+        }
         for (int oo = 0; oo < p.stride_q; oo++) {
             if (it + oo < p.TDST) {
-                const uint4 raw = *reinterpret_cast<const uint4 *>(qbase + (it + oo) * p.q_st + piece * 8);
+                uint4 raw = *reinterpret_cast<const uint4 *>(qbase + (it + oo) * p.q_st + piece * 8);
+                if (rope) {
+                    const uint4 oth = *reinterpret_cast<const uint4 *>(qbase + (it + oo) * p.q_st + ppiece * 8);
+                    raw = rope_piece(raw, oth, rc, rs, piece < per_row / 2);
+                }
                 const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
@@ -350,8 +404,7 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
         const char *e = getenv("HIPATTN_MASK_NB");
         env_nb = e ? atoi(e) : 0;
     }
-    const int nb = (env_nb == 2 && BC >= 32) ? 2 : (wide ? 2 : 1);
-    const int nsub = (BC / 16) / nb;
+    const int nb0 = (env_nb == 2 && BC >= 32) ? 2 : (wide ? 2 : 1);
     // LDS path: one wave per workgroup (it uses workgroup barriers); direct path: up to 4 heads per workgroup
     // (measured: sharing pays with one query-row block per program, not with two)
     if (g_mask_via_lds < 0) {
@@ -362,9 +415,16 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
     // It is also used for wide single-row-block launches without extras: measured 10-15% faster there than the
     // plain build of the same source (the compiler schedules its row loads earlier), and its extra branches are
     // never taken.
+    const bool rope = p.rope.cos != nullptr;
+    if (rope && prescaled) {
+        set_error("mask stage: prescaled keys cannot be combined with rope applied on load");
+        return HIPATTN_E_ARG;
+    }
+    const int nb = rope ? 1 : nb0;
+    const int nsub = (BC / 16) / nb;
     bool via_lds = g_mask_via_lds == 2 ? !wide : (g_mask_via_lds == 1);
-    if (p.kx.extended() && nb == 2) via_lds = false;
-    const bool ext = p.kx.extended() || (wide && !two && !via_lds);
+    if ((p.kx.extended() && nb == 2) || rope) via_lds = false;
+    const bool ext = rope || p.kx.extended() || (wide && !two && !via_lds);
     const int hpw = (via_lds || two) ? 1 : (p.G < 4 ? p.G : 4);
     const int hblocks = (p.G + hpw - 1) / hpw;
     p.total = (long long)p.B * p.kv.HKV * hblocks * p.BS * p.ngroups * nsub;
@@ -393,7 +453,10 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
         if (prescaled) { if (via_lds) MS_LAUNCH(MBv, NBv, true, true); else MS_LAUNCH(MBv, NBv, true, false); } \
         else { if (via_lds) MS_LAUNCH(MBv, NBv, false, true); else MS_LAUNCH(MBv, NBv, false, false); }        \
     } while (0)
-    if (two) { if (nb == 2) MS_PICK(2, 2); else MS_PICK(2, 1); }
+    if (rope) {
+        if (two) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 2, 1, false, false, true, true>), grid, block, 0, st, p, nsub, hpw);
+        else hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, false, false, true, true>), grid, block, 0, st, p, nsub, hpw);
+    } else if (two) { if (nb == 2) MS_PICK(2, 2); else MS_PICK(2, 1); }
     else { if (nb == 2) MS_PICK(1, 2); else MS_PICK(1, 1); }
 #undef MS_PICK
 #undef MS_LAUNCH

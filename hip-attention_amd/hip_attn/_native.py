@@ -31,7 +31,19 @@ class QStruct(ctypes.Structure):
         ("pos_stride_b", ctypes.c_int64), ("pos_stride_t", ctypes.c_int64),
         ("B", ctypes.c_int32), ("TDST", ctypes.c_int32), ("HEAD", ctypes.c_int32), ("HID", ctypes.c_int32),
         ("dtype", ctypes.c_int32),
+        ("rope", ctypes.c_void_p),
     ]
+
+
+class RopeStruct(ctypes.Structure):
+    _fields_ = [
+        ("cos", ctypes.c_void_p), ("sin", ctypes.c_void_p),
+        ("stride_t", ctypes.c_int64), ("len", ctypes.c_int64),
+        ("backend", ctypes.c_int32),
+    ]
+
+
+EXTEND_BACKENDS = {"relative": 1, "streaming": 2, "infllm": 3}
 
 
 class KVStruct(ctypes.Structure):
@@ -125,10 +137,26 @@ def _p(t: Optional[torch.Tensor]):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
 
 
-def make_q(q: torch.Tensor, pos: torch.Tensor) -> QStruct:
+def make_rope(cos: torch.Tensor, sin: torch.Tensor, backend: str) -> RopeStruct:
+    """Describe RoPE tables ``[len, >= HID/2]`` (q's dtype, unit inner stride) and the rotation rule of one call."""
+    if backend not in EXTEND_BACKENDS:
+        raise NotImplementedError(f"extend backend {backend!r} is not built (built: {sorted(EXTEND_BACKENDS)})")
+    assert cos.ndim == 2 and sin.shape == cos.shape and cos.stride(1) == 1 and sin.stride(1) == 1
+    assert cos.stride(0) == sin.stride(0) and cos.dtype == sin.dtype
+    r = RopeStruct()
+    r.cos, r.sin = cos.data_ptr(), sin.data_ptr()
+    r.stride_t, r.len = cos.stride(0), cos.shape[0]
+    r.backend = EXTEND_BACKENDS[backend]
+    return r
+
+
+def make_q(q: torch.Tensor, pos: torch.Tensor, rope: Optional[RopeStruct] = None) -> QStruct:
     assert q.ndim == 4 and q.stride(3) == 1
     assert pos.dtype == torch.int64 and pos.ndim == 2
     s = QStruct()
+    if rope is not None:
+        s._rope_keep = rope  # the struct holds a bare pointer to it
+        s.rope = ctypes.addressof(rope)
     s.ptr = q.data_ptr()
     s.stride_b, s.stride_t, s.stride_h = q.stride(0), q.stride(1), q.stride(2)
     s.pos = pos.data_ptr()

@@ -46,8 +46,9 @@ def _head_reduce_enabled() -> bool:
 
 
 def _reject_unsupported(args: HiPAttentionArgs):
-    if args.using_extend or args.need_apply_rope:
-        raise NotImplementedError("RoPE 'extend' modes (using_extend / need_apply_rope) are not built yet")
+    if args.using_extend and not args.need_apply_rope:
+        raise NotImplementedError("using_extend with keys stored WITH rotation (need_apply_rope=False) is not built; "
+                                  "store q and k without RoPE and pass need_apply_rope=True")
     if args.logit_softcap is not None:
         raise NotImplementedError("logit_softcap is not built yet")
     if not args.is_causal:
@@ -58,6 +59,35 @@ def _reject_unsupported(args: HiPAttentionArgs):
         raise NotImplementedError("online_update_cache (in-kernel cache fill) is not built")
     if (args.low_percent > 0) and (args.low_k_ratio < 1):
         raise NotImplementedError("low_percent / low_k_ratio pruning is dead code in the reference and not built")
+
+
+_ROPE_TABLES = {}  # (cos ptr, sin ptr, versions, dtype) -> (cos, sin) in the compute dtype; tiny, most recent last
+
+
+def _rope_tables(args: HiPAttentionArgs, dtype: torch.dtype):
+    """RoPE tables as 2-D tensors of the query dtype (the reference casts every loaded entry to it,
+    attention_extend.py:395-405).  Converted tables are remembered so a serving loop converts once."""
+    cos, sin = args.rope_cos, args.rope_sin
+    if cos is None or sin is None:
+        raise ValueError("using_extend with need_apply_rope needs rope_cos and rope_sin")
+    if cos.ndim == 3:
+        cos, sin = cos.view(-1, cos.shape[-1]), sin.view(-1, sin.shape[-1])
+    assert cos.ndim == 2 and cos.shape == sin.shape, "rope tables are [positions, head_dim]"
+    esz = torch.empty((), dtype=dtype).element_size()
+
+    def usable(t):
+        return (t.dtype == dtype and t.stride(1) == 1 and (t.stride(0) * esz) % 16 == 0 and t.data_ptr() % 16 == 0)
+
+    if usable(cos) and usable(sin) and cos.stride(0) == sin.stride(0):
+        return cos, sin
+    key = (cos.data_ptr(), sin.data_ptr(), cos._version, sin._version, tuple(cos.shape), dtype)
+    hit = _ROPE_TABLES.get(key)
+    if hit is None:
+        hit = (cos.to(dtype).contiguous(), sin.to(dtype).contiguous())
+        if len(_ROPE_TABLES) >= 8:
+            _ROPE_TABLES.pop(next(iter(_ROPE_TABLES)))
+        _ROPE_TABLES[key] = hit
+    return hit
 
 
 def _kv_struct(args: HiPAttentionArgs, k: Optional[Tensor], v: Optional[Tensor], max_tsrc: int,
@@ -109,7 +139,8 @@ def _mask_kv(args: HiPAttentionArgs, k_mask: Optional[Tensor], max_tsrc: int, q:
     stage0 = args.stages[0]
     iters = max(1, int(stage0.stage_chunk_size).bit_length())
     sampled_rows = 2 * iters * programs_rows * chunk_count  # stage 0 alone
-    if q.dtype == torch.bfloat16 and args.offload_cache is None:
+    rope = args.using_extend and args.need_apply_rope  # keys are rotated per sample: nothing to scale ahead
+    if q.dtype == torch.bfloat16 and args.offload_cache is None and not rope:
         src = k_mask if k_mask is not None else args.k_cache
         if src is not None and src.dtype == torch.bfloat16 and src.ndim == 4 and src.stride(-1) == 1:
             rows_total = src.shape[0] * src.shape[1] * src.shape[2]
@@ -218,6 +249,7 @@ def dual_stage_quadratic_hip_attention(
     sa_stats = _new_statistics(args, BSZ, HEAD_KV, MAX_PAGE, device)
 
     qq = q if q.stride(-1) == 1 else q.contiguous()
+    rope_tabs = _rope_tables(args, q.dtype) if (args.using_extend and args.need_apply_rope) else None
     hg = 1 if _head_reduce_enabled() else HEAD
     mask_kv = None  # built lazily: cached-mask steps never touch the estimation path
     k_prescaled = False
@@ -316,7 +348,10 @@ def dual_stage_quadratic_hip_attention(
                     scores = torch.empty((BSZ, bs, HEAD, chunk_count), dtype=torch.float32, device=device)
                 left_out = torch.empty((BSZ, bs, HEAD, chunk_count), dtype=torch.int32, device=device) if last else None
                 if chunk_count > 0:
-                    qs = N.make_q(qq, position_ids)
+                    rope = None
+                    if rope_tabs is not None:  # :2200-2204
+                        rope = N.make_rope(*rope_tabs, stage.stage_extend_backend or args.scan_extend_backend)
+                    qs = N.make_q(qq, position_ids, rope)
                     N.mask_stage(qs, mask_kv, chunk_left, hg, chunk_count, chunk_size, right_clamp, bs,
                                  BLOCK_SIZE_Q, stage.stage_block_stride_q, BLOCK_CHUNK, STAGE_STRIDE, sw_eff,
                                  args.stage_early_terminate, scores, left_out, device, k_prescaled=k_prescaled,
@@ -397,7 +432,7 @@ def dual_stage_quadratic_hip_attention(
     seq_pos = position_ids[:, -q_bsa.shape[1]:]
     context = block_sparse_attention(
         q_bsa, k, v, seq_pos, indices, ks_start_end, args, MAX_TSRC, decode=use_decode, rows_shared=rows_shared,
-        khat=khat if (args.k_mask is None) else None, stats=sa_stats,
+        khat=khat if (args.k_mask is None) else None, stats=sa_stats, rope_tables=rope_tabs,
     )
 
     metadata = HiPAttentionOutputMetadata(
@@ -419,7 +454,8 @@ def dual_stage_quadratic_hip_attention(
 def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], position_ids: Tensor, indices: Tensor,
                            ks_start_end: Tensor, args: HiPAttentionArgs, max_tsrc: int, decode: bool = False,
                            impl: int = 0, rows_shared: bool = False, khat: Optional[Tensor] = None,
-                           stats: Optional[HiPAttentionCacheAccessStatistics] = None) -> Tensor:
+                           stats: Optional[HiPAttentionCacheAccessStatistics] = None,
+                           rope_tables=None) -> Tensor:
     """Sparse attention over (selected blocks, sink, sliding window) given the metadata tensors.
 
     ``position_ids`` are 0-based (the reference passes ``seq_lens = position_ids + 1``,
@@ -429,14 +465,18 @@ def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], 
     index row of the group's first head.  ``rows_shared`` promises that all heads of a GQA group hold
     identical index rows (true for masks estimated with head reduction), which lets one gathered
     K/V tile serve the whole group.  ``khat`` is an optional ``bf16(k * c_k)`` tensor with the shape and
-    strides of the key storage (dense ``k`` or ``args.k_cache``).
+    strides of the key storage (dense ``k`` or ``args.k_cache``).  ``rope_tables`` = ``(cos, sin)`` in q's dtype
+    turns on rotation on load under ``args.sa_extend_backend``.
     """
     device = q.device
     qq = q if q.stride(-1) == 1 else q.contiguous()
     kvs, keep = _kv_struct(args, k, v, max_tsrc, masking=False, stats=stats)
     if position_ids.dtype != torch.int64:
         position_ids = position_ids.to(torch.int64)
-    qs = N.make_q(qq, position_ids)
+    rope = N.make_rope(*rope_tables, args.sa_extend_backend) if rope_tables is not None else None
+    qs = N.make_q(qq, position_ids, rope)
+    if rope is not None:
+        khat = None
     if not indices.is_contiguous():
         indices = indices.contiguous()
     if not ks_start_end.is_contiguous():

@@ -27,6 +27,34 @@ extern "C" {
 #define HIPATTN_E_UNSUPPORTED (-2) /* valid request the kernels do not cover (head dim, limits) */
 #define HIPATTN_E_ALIGN (-3)     /* pointer or stride not aligned for 16-byte row loads */
 
+/* Rotary embedding applied while rows are loaded -- HiPAttentionArgs.using_extend with need_apply_rope,
+ * rope_cos / rope_sin, scan_extend_backend / sa_extend_backend (src/hip_attn/v1_2/attention_metadata.py:191-198):
+ * q and K are stored WITHOUT rotation and every loaded row x becomes x*cos[p] + rot(x)*sin[p], rot(x)[i] =
+ * -x[i + HID/2] below HID/2 and x[i - HID/2] above, each product and the sum rounded to the element type
+ * (load_keys_with_rope, src/hip_attn/v1_2/attention_extend.py:289-407; queries :626-690;
+ * src/hip_attn/v1_2/attention_extend_bsa.py:248-380, :796-852).  The position p depends on `backend`:
+ *   mask stage   RELATIVE  left sample 0, right sample 1, query 1 + sw_eff
+ *                STREAMING key: number of its chunk in the stage's list, query: min(pos, n + sw_eff)
+ *                INFLLM    key 0, query sw_eff
+ *   attention    query: its own position; window keys: their own position; sink and selected keys:
+ *                STREAMING max(0, slot + pmin - sliding_window - sink - (ks_end - ks_start)*block_size_k + 1),
+ *                          slot = token for sink tokens, (j + sink / block_size_k) * block_size_k + e for
+ *                          element e of index entry j; pmin = smallest position in the query block
+ *                INFLLM    max(0, pmin - sliding_window)
+ * Positions are clamped into [0, len).  The reference's "dynamic_extend" and "self_extend" rules and the mode
+ * that re-rotates keys stored WITH rotation (need_apply_rope = False) are not built. */
+#define HIPATTN_EXTEND_RELATIVE 1
+#define HIPATTN_EXTEND_STREAMING 2
+#define HIPATTN_EXTEND_INFLLM 3
+
+typedef struct hipattn_rope {
+    const void *cos; /* [len, >= HID/2], q's dtype, 16-byte aligned rows; column i = frequency i */
+    const void *sin;
+    int64_t stride_t; /* elements between rows */
+    int64_t len;
+    int32_t backend;  /* HIPATTN_EXTEND_* for this call */
+} hipattn_rope_t;
+
 /* Query tensor q[B, TDST, HEAD, HID] and its token positions (0-based, int64)
  * -- the (q, position_ids) pair of dual_stage_quadratic_hip_attention,
  * src/hip_attn/v1_2/attention_extend.py:1918-1987. */
@@ -37,6 +65,7 @@ typedef struct hipattn_q {
     int64_t pos_stride_b, pos_stride_t;
     int32_t B, TDST, HEAD, HID;
     int32_t dtype; /* HIPATTN_F32 / HIPATTN_BF16; K and V share it */
+    const hipattn_rope_t *rope; /* host pointer; NULL: rows are used as stored */
 } hipattn_q_t;
 
 /* Key/value storage: dense k,v[B, TSRC, HKV, HID] or a paged cache [pages, page_size, HKV, HID]

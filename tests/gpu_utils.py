@@ -27,7 +27,8 @@ def product_args(A: O.OArgs, X: O.OInputs, device="cuda", **extra):
         sink_token_size=A.sink_token_size, sliding_window_size=A.sliding_window_size,
         block_size_k=A.block_size_k, second_stage_k=A.second_stage_k,
         stages=[ScanStage12(stage_block_size_q=s.stage_block_size_q, stage_block_stride_q=s.stage_block_stride_q,
-                            stage_chunk_size=s.stage_chunk_size, stage_k=s.stage_k, stage_stride=s.stage_stride)
+                            stage_chunk_size=s.stage_chunk_size, stage_k=s.stage_k, stage_stride=s.stage_stride,
+                            stage_extend_backend=getattr(s, "stage_extend_backend", None))
                 for s in A.stages],
         model_context_length=A.model_context_length, extend_context_length=A.extend_context_length,
         block_sparse_block_size_q=A.block_sparse_block_size_q, stage_early_terminate=A.stage_early_terminate,
@@ -38,6 +39,11 @@ def product_args(A: O.OArgs, X: O.OInputs, device="cuda", **extra):
         kw.update(k_cache=to_torch(X.k_cache, X.dtype, device), v_cache=to_torch(X.v_cache, X.dtype, device),
                   block_table=torch.from_numpy(X.block_table).to(device),
                   cache_seq_lens=torch.from_numpy(X.cache_seq_lens).to(device))
+    if A.using_extend:
+        kw.update(using_extend=True, need_apply_rope=A.need_apply_rope, scan_extend_backend=A.scan_extend_backend,
+                  sa_extend_backend=A.sa_extend_backend,
+                  rope_cos=to_torch(O.f32_to_bf16_bits(X.rope_cos) if X.dtype == "bf16" else X.rope_cos, X.dtype, device),
+                  rope_sin=to_torch(O.f32_to_bf16_bits(X.rope_sin) if X.dtype == "bf16" else X.rope_sin, X.dtype, device))
     kw.update(extra)
     return HiPAttentionArgs12(**kw)
 

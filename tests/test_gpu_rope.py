@@ -1,0 +1,122 @@
+"""GPU parity of RoPE applied on load (the "extend" modes): mask stage rules relative / streaming / infllm, sparse
+attention rules streaming / infllm, through every kernel that loads query or key rows (scan on the matrix cores and
+portable scan, tile kernel, portable attention kernel, decode kernel).
+
+Indices must match the oracle bit for bit; outputs within 2e-2 abs / 1e-2 rel (bf16) or 1e-4 (f32).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import hip12 as O
+from helpers import make_inputs, tiny_args, to_paged, with_rope
+from gpu_utils import assert_context_close, assert_metadata_equal, run_product, to_torch
+from test_oracle_bsa import random_indices
+
+pytestmark = pytest.mark.gpu
+
+
+def _ext(**kw):
+    return tiny_args(using_extend=True, need_apply_rope=True, **kw)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("scan", ["relative", "streaming", "infllm"])
+def test_prefill_with_rope_matches_oracle(dtype, scan):
+    print(f"[case] rope prefill {dtype} scan={scan}", flush=True)
+    # ragged last query block, GQA, strided query mean in the first two stages
+    X = with_rope(make_inputs(31, B=2, TQ=200, TK=2048, H=4, HKV=2, D=64, dtype=dtype, scale=0.5), 4096)
+    A = _ext(scan_extend_backend=scan, sa_extend_backend="streaming")
+    octx, ometa = O.hip_attention_12(X, A)
+    ctx, meta = run_product(X, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, dtype)
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_prefill_with_rope_paged_bf16_default_like_stages(D):
+    print(f"[case] rope prefill paged D={D}", flush=True)
+    X = with_rope(make_inputs(32, B=1, TQ=256, TK=4096, H=8, HKV=2, D=D, dtype="bf16", scale=0.5), 8192)
+    XP = with_rope(to_paged(X, 16, seed=4), 8192)
+    A = _ext(scan_extend_backend="relative", sa_extend_backend="streaming", extend_context_length=4096,
+             sliding_window_size=512, second_stage_k=1024, block_sparse_block_size_q=64,
+             stages=[O.OStage(64, 4, 256, None, 1), O.OStage(64, 4, 32, 2048, 1, "streaming"), O.OStage(64, 1, 8, 1024, 1)])
+    octx, ometa = O.hip_attention_12(XP, A)
+    ctx, meta = run_product(XP, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, "bf16")
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("sa", ["streaming", "infllm"])
+def test_batched_paged_decode_with_rope(dtype, sa):
+    print(f"[case] rope decode {dtype} sa={sa}", flush=True)
+    B, TK, H, HKV, D = 3, 3000, 8, 2, 128 if dtype == "bf16" else 64
+    lens = np.array([3000, 1777, 900])
+    X = make_inputs(33, B=B, TQ=1, TK=TK, H=H, HKV=HKV, D=D, dtype=dtype, pos=(lens - 1)[:, None], scale=0.5)
+    XP = with_rope(to_paged(X, 16, seed=5, seq_lens=lens), 4096)
+    A = _ext(scan_extend_backend="relative", sa_extend_backend=sa, extend_context_length=3072)
+    octx, ometa = O.hip_attention_12(XP, A)
+    ctx, meta = run_product(XP, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, dtype)
+    # cached mask: attention only
+    octx2, _ = O.hip_attention_12(XP, A, cached=O.OMetadata(ometa.indices, ometa.ks, ometa.ks_count, ometa.ks_start_end, None))
+    ctx2, _ = run_product(XP, A, cached=meta)
+    assert_context_close(ctx2, octx2, dtype)
+
+
+def _run_bsa(X, max_tsrc, idx, kse, bq, bk, sw, sink, impl, backend, share=True, decode=False):
+    from hip_attn import HiPAttentionArgs12
+    from hip_attn.operator import block_sparse_attention
+
+    dev = "cuda"
+    bits = (lambda a: O.f32_to_bf16_bits(a)) if X.dtype == "bf16" else (lambda a: a)
+    args = HiPAttentionArgs12(sink_token_size=sink, sliding_window_size=sw, sa_extend_backend=backend)
+    args.block_size_q, args.block_size_k = bq, bk
+    tabs = (to_torch(bits(X.rope_cos), X.dtype, dev), to_torch(bits(X.rope_sin), X.dtype, dev))
+    out = block_sparse_attention(to_torch(X.q, X.dtype, dev), to_torch(X.k, X.dtype, dev), to_torch(X.v, X.dtype, dev),
+                                 torch.from_numpy(X.pos.copy()).to(dev), torch.from_numpy(idx).to(dev),
+                                 torch.from_numpy(kse).to(dev), args, max_tsrc, decode=decode, impl=impl,
+                                 rows_shared=share, rope_tables=tabs)
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("backend", ["streaming", "infllm"])
+@pytest.mark.parametrize("D,bq,TQ,bk", [(64, 64, 200, 8), (128, 32, 96, 2), (128, 16, 40, 16)])
+def test_attention_kernels_with_rope_given_indices(backend, D, bq, TQ, bk):
+    print(f"[case] rope bsa {backend} D={D} bq={bq} TQ={TQ} bk={bk}", flush=True)
+    rng = np.random.default_rng(D + bq + bk)
+    TK, H, HKV, BK, sw, sink = 1536, 8, 2, 24, 100, 32
+    X = with_rope(make_inputs(34, B=2, TQ=TQ, TK=TK, H=H, HKV=HKV, D=D, dtype="bf16", scale=0.5), 2048,
+                  sa_backend=backend)
+    idx, ks, kse = random_indices(rng, 2, H, O.cdiv(TQ, bq), BK, bk, TK, same_heads=True)
+    ref = O.bsa(X, TK, idx, kse, bq, bk, sw, sink)
+    assert_context_close(_run_bsa(X, TK, idx, kse, bq, bk, sw, sink, 2, backend), ref, "bf16")
+    assert_context_close(_run_bsa(X, TK, idx, kse, bq, bk, sw, sink, 1, backend), ref, "bf16")
+
+
+def test_float32_tables_with_bf16_queries_are_cast_like_the_reference():
+    print("[case] rope f32 tables, bf16 q", flush=True)
+    # tables handed over in float32 (and as [1, L, D]): entries are cast to the query dtype on use
+    X = with_rope(make_inputs(35, B=1, TQ=64, TK=1024, H=2, HKV=1, D=64, dtype="bf16", scale=0.5), 2048, dtype="f32")
+    A = _ext(scan_extend_backend="relative", sa_extend_backend="streaming")
+    cos32 = torch.from_numpy(X.rope_cos.copy()).cuda()[None]
+    sin32 = torch.from_numpy(X.rope_sin.copy()).cuda()[None]
+    octx, ometa = O.hip_attention_12(X, A)
+    ctx, meta = run_product(X, A, rope_cos=cos32, rope_sin=sin32)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, "bf16")
+
+
+def test_unbuilt_rules_fail_loudly():
+    from hip_attn import _native as N
+    print("[case] rope unbuilt rules", flush=True)
+    X = with_rope(make_inputs(36, B=1, TQ=32, TK=512, H=2, HKV=1, D=32, dtype="f32"), 1024)
+    with pytest.raises(NotImplementedError):
+        run_product(X, _ext(scan_extend_backend="dynamic_extend"))
+    with pytest.raises((N.HipAttnError, NotImplementedError)):
+        run_product(X, _ext(sa_extend_backend="relative"))
+    with pytest.raises(NotImplementedError):
+        run_product(X, tiny_args(using_extend=True, need_apply_rope=False))
