@@ -61,6 +61,7 @@ int make_rope_view(const hipattn_q_t *q, unsigned allowed, const char *who, Rope
                       HIPATTN_E_ALIGN, "%s: rope table rows must be 16-byte aligned and hold HID/2 columns", who);
     HIPATTN_CHECK_ARG(q->HID % 32 == 0, HIPATTN_E_UNSUPPORTED, "%s: rope needs a head dim that is a multiple of 32", who);
     o->cos = r->cos; o->sin = r->sin; o->stride_t = r->stride_t; o->len = r->len; o->backend = r->backend;
+    o->k_side_delta = r->k_side_delta;
     return 0;
 }
 

@@ -284,6 +284,7 @@ struct RopeView {
     const void *cos, *sin;
     int64_t stride_t, len;
     int backend;  // HIPATTN_EXTEND_*
+    int64_t k_side_delta;  // prescaled RELATIVE scan: offset of the position-1 copy of the keys
     __device__ __forceinline__ int64_t row(int64_t pos) const {  // element offset of the table row of a position
         pos = pos < 0 ? 0 : (pos >= len ? len - 1 : pos);
         return pos * stride_t;

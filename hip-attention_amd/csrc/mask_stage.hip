@@ -326,8 +326,11 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
     rc = make_rope_view(q, (1u << HIPATTN_EXTEND_RELATIVE) | (1u << HIPATTN_EXTEND_STREAMING) | (1u << HIPATTN_EXTEND_INFLLM),
                         "mask stage", &p.rope);
     if (rc) return rc;
-    HIPATTN_CHECK_ARG(!(p.rope.cos && k_prescaled), HIPATTN_E_ARG,
-                      "mask stage: prescaled keys cannot be combined with rope applied on load");
+    HIPATTN_CHECK_ARG(!(p.rope.cos && k_prescaled) || p.rope.backend == HIPATTN_EXTEND_RELATIVE ||
+                          p.rope.backend == HIPATTN_EXTEND_INFLLM,
+                      HIPATTN_E_ARG, "mask stage: prescaled keys need a rule with fixed key positions (relative, infllm)");
+    if (p.rope.backend != HIPATTN_EXTEND_RELATIVE || !k_prescaled) p.rope.k_side_delta = 0;
+    HIPATTN_CHECK_ARG(p.rope.k_side_delta % 8 == 0, HIPATTN_E_ALIGN, "mask stage: k_side_delta must keep 16-byte alignment");
     HIPATTN_CHECK_ARG(q->HEAD % p.kv.HKV == 0, HIPATTN_E_ARG, "mask stage: HEAD %% HKV != 0");
     p.q = q->ptr; p.q_sb = q->stride_b; p.q_st = q->stride_t; p.q_sh = q->stride_h;
     p.pos = q->pos; p.pos_sb = q->pos_stride_b; p.pos_st = q->pos_stride_t;

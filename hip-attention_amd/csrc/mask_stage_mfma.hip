@@ -56,13 +56,17 @@ __device__ __forceinline__ int64_t rope_kpos(const RopeView &r, int c, int side)
     return 0;
 }
 
-// ROPE = true (direct path, one token block per wave, extended parameter block): every sampled key row is rotated
+// RMODE = 1 (direct path, one token block per wave, extended parameter block): every sampled key row is rotated
 // before it is scaled.  The two halves of a row sit in the two half-waves (lane and lane ^ 32) at the same k-step,
 // and the rotated position of a lane's key never changes over the iterations, so its cos/sin entries are loaded
 // once and stay in registers.
-template <int HID, int MB, int NB, bool PRESCALED, bool VIA_LDS, bool EXT, bool ROPE = false>
+// RMODE = 2 (prescaled keys, extended parameter block): the keys were rotated and scaled ahead of the scan, one
+// copy per sample side; right-hand samples read the copy k_side_delta elements further on.
+template <int HID, int MB, int NB, bool PRESCALED, bool VIA_LDS, bool EXT, int RMODE = 0>
 __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
+    constexpr bool ROPE = RMODE == 1;
     static_assert(!ROPE || (EXT && !VIA_LDS && !PRESCALED), "rope variant: direct path of the extended build");
+    static_assert(RMODE != 2 || (EXT && PRESCALED), "two-sided prescaled keys: extended build of the prescaled path");
     const KVExt *kx = nullptr;
     if constexpr (EXT) kx = &p.kx;
     constexpr int KS = HID / 16;
@@ -229,6 +233,9 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
                 // access flags: wide launches (prefill) revisit rows constantly, so they look before they store;
                 // narrow ones (decode) touch mostly fresh rows and store blindly
                 off = kv_k_row<EXT, NB == 2>(p.kv, kx, b, t, kvh, seqlen, hh == 0);
+                if constexpr (RMODE == 2) {
+                    if (side && off != NO_ROW) off += p.rope.k_side_delta;
+                }
             }
             if constexpr (VIA_LDS) {
                 if (hh == 0) s_off[tb * 32 + n] = off;
@@ -415,16 +422,13 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
     // It is also used for wide single-row-block launches without extras: measured 10-15% faster there than the
     // plain build of the same source (the compiler schedules its row loads earlier), and its extra branches are
     // never taken.
-    const bool rope = p.rope.cos != nullptr;
-    if (rope && prescaled) {
-        set_error("mask stage: prescaled keys cannot be combined with rope applied on load");
-        return HIPATTN_E_ARG;
-    }
+    const bool rope = p.rope.cos != nullptr && !prescaled;  // rotate every sample in the kernel
+    const bool two_sided = p.rope.cos != nullptr && prescaled;
     const int nb = rope ? 1 : nb0;
     const int nsub = (BC / 16) / nb;
     bool via_lds = g_mask_via_lds == 2 ? !wide : (g_mask_via_lds == 1);
-    if ((p.kx.extended() && nb == 2) || rope) via_lds = false;
-    const bool ext = rope || p.kx.extended() || (wide && !two && !via_lds);
+    if (((p.kx.extended() || two_sided) && nb == 2) || rope) via_lds = false;
+    const bool ext = rope || two_sided || p.kx.extended() || (wide && !two && !via_lds);
     const int hpw = (via_lds || two) ? 1 : (p.G < 4 ? p.G : 4);
     const int hblocks = (p.G + hpw - 1) / hpw;
     p.total = (long long)p.B * p.kv.HKV * hblocks * p.BS * p.ngroups * nsub;
@@ -442,6 +446,13 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
 #define MS_LAUNCH(MBv, NBv, PSv, VLv)                                                                                 \
     do {                                                                                                              \
         constexpr bool EXT_BUILT = !(VLv) || (NBv) == 1;                                                              \
+        if constexpr ((PSv) && EXT_BUILT) {                                                                           \
+            if (two_sided) {                                                                                          \
+                hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, NBv, true, VLv, true, 2>), grid, block, 0, st, p, \
+                                   nsub, hpw);                                                                        \
+                break;                                                                                                \
+            }                                                                                                         \
+        }                                                                                                             \
         if (ext && EXT_BUILT)                                                                                         \
             hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, NBv, PSv, VLv, EXT_BUILT>), grid, block, 0, st, p, nsub, \
                                hpw);                                                                                  \
@@ -454,8 +465,8 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
         else { if (via_lds) MS_LAUNCH(MBv, NBv, false, true); else MS_LAUNCH(MBv, NBv, false, false); }        \
     } while (0)
     if (rope) {
-        if (two) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 2, 1, false, false, true, true>), grid, block, 0, st, p, nsub, hpw);
-        else hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, false, false, true, true>), grid, block, 0, st, p, nsub, hpw);
+        if (two) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 2, 1, false, false, true, 1>), grid, block, 0, st, p, nsub, hpw);
+        else hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, false, false, true, 1>), grid, block, 0, st, p, nsub, hpw);
     } else if (two) { if (nb == 2) MS_PICK(2, 2); else MS_PICK(2, 1); }
     else { if (nb == 2) MS_PICK(1, 2); else MS_PICK(1, 1); }
 #undef MS_PICK
@@ -494,9 +505,57 @@ __global__ void prescale_k_kernel(const uint16_t *in, uint16_t *out, long long r
     *reinterpret_cast<uint4 *>(out + r * hid + piece * 8) = o;
 }
 
+// the same after rotating every row to one fixed position (table rows cos_row / sin_row)
+__global__ void prescale_k_rope_kernel(const uint16_t *in, uint16_t *out, long long rows, int hid, int64_t s0, int64_t s1,
+                                       int64_t s2, int d1, int d2, float c_k, const uint16_t *cos_row,
+                                       const uint16_t *sin_row) {
+    const int per_row = hid / 8;
+    const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= rows * per_row) return;
+    const long long r = gid / per_row;
+    const int piece = (int)(gid % per_row);
+    const int ppiece = (piece + per_row / 2) % per_row;
+    const long long i2 = r % d2, i1 = (r / d2) % d1, i0 = r / ((long long)d1 * d2);
+    const uint16_t *row = in + i0 * s0 + i1 * s1 + i2 * s2;
+    const uint4 raw = *reinterpret_cast<const uint4 *>(row + piece * 8);
+    const uint4 oth = *reinterpret_cast<const uint4 *>(row + ppiece * 8);
+    const uint4 c = *reinterpret_cast<const uint4 *>(cos_row + (piece % (per_row / 2)) * 8);
+    const uint4 sn = *reinterpret_cast<const uint4 *>(sin_row + (piece % (per_row / 2)) * 8);
+    const uint4 rot = rope_piece(raw, oth, c, sn, piece < per_row / 2);
+    uint4 o;
+    o.x = scale_pack(rot.x, c_k);
+    o.y = scale_pack(rot.y, c_k);
+    o.z = scale_pack(rot.z, c_k);
+    o.w = scale_pack(rot.w, c_k);
+    *reinterpret_cast<uint4 *>(out + r * hid + piece * 8) = o;
+}
+
 }  // namespace hipattn
 
 using namespace hipattn;
+
+extern "C" int hipattn_prescale_k_rope(const void *k, int64_t stride0, int64_t stride1, int64_t stride2, int64_t n0,
+                                       int32_t n1, int32_t n2, int32_t HID, const void *cos_row, const void *sin_row,
+                                       void *out, void *stream) {
+    HIPATTN_CHECK_ARG(k && out && cos_row && sin_row, HIPATTN_E_ARG, "prescale: null pointer");
+    HIPATTN_CHECK_ARG(n0 > 0 && n1 > 0 && n2 > 0 && HID > 0 && HID % 32 == 0, HIPATTN_E_ARG, "prescale: bad sizes");
+    HIPATTN_CHECK_ARG(aligned16(k) && aligned16(out) && aligned16(cos_row) && aligned16(sin_row) && stride0 % 8 == 0 &&
+                          stride1 % 8 == 0 && stride2 % 8 == 0,
+                      HIPATTN_E_ALIGN, "prescale: pointers and strides must be 16-byte aligned");
+    float c_q, c_k;
+    scale_constants(HID, HIPATTN_BF16, &c_q, &c_k);
+    const long long rows = (long long)n0 * n1 * n2;
+    const long long work = rows * (HID / 8);
+    const int threads = 256;
+    const long long blocks = (work + threads - 1) / threads;
+    HIPATTN_CHECK_ARG(blocks < 0x7fffffffLL, HIPATTN_E_UNSUPPORTED, "prescale: tensor too large");
+    hipLaunchKernelGGL(prescale_k_rope_kernel, dim3((unsigned)blocks), dim3(threads), 0, (hipStream_t)stream,
+                       reinterpret_cast<const uint16_t *>(k), reinterpret_cast<uint16_t *>(out), rows, HID, stride0,
+                       stride1, stride2, n1, n2, c_k, reinterpret_cast<const uint16_t *>(cos_row),
+                       reinterpret_cast<const uint16_t *>(sin_row));
+    HIPATTN_CHECK_HIP(hipGetLastError());
+    return 0;
+}
 
 extern "C" int hipattn_prescale_k(const void *k, int64_t stride0, int64_t stride1, int64_t stride2, int64_t n0,
                                   int32_t n1, int32_t n2, int32_t HID, void *out, void *stream) {

@@ -40,6 +40,7 @@ class RopeStruct(ctypes.Structure):
         ("cos", ctypes.c_void_p), ("sin", ctypes.c_void_p),
         ("stride_t", ctypes.c_int64), ("len", ctypes.c_int64),
         ("backend", ctypes.c_int32),
+        ("k_side_delta", ctypes.c_int64),
     ]
 
 
@@ -137,7 +138,7 @@ def _p(t: Optional[torch.Tensor]):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
 
 
-def make_rope(cos: torch.Tensor, sin: torch.Tensor, backend: str) -> RopeStruct:
+def make_rope(cos: torch.Tensor, sin: torch.Tensor, backend: str, k_side_delta: int = 0) -> RopeStruct:
     """Describe RoPE tables ``[len, >= HID/2]`` (q's dtype, unit inner stride) and the rotation rule of one call."""
     if backend not in EXTEND_BACKENDS:
         raise NotImplementedError(f"extend backend {backend!r} is not built (built: {sorted(EXTEND_BACKENDS)})")
@@ -147,6 +148,7 @@ def make_rope(cos: torch.Tensor, sin: torch.Tensor, backend: str) -> RopeStruct:
     r.cos, r.sin = cos.data_ptr(), sin.data_ptr()
     r.stride_t, r.len = cos.stride(0), cos.shape[0]
     r.backend = EXTEND_BACKENDS[backend]
+    r.k_side_delta = k_side_delta
     return r
 
 
@@ -264,6 +266,23 @@ def prescale_k(k: torch.Tensor, device) -> torch.Tensor:
         ctypes.c_int64(k.shape[0]), ctypes.c_int32(k.shape[1]), ctypes.c_int32(k.shape[2]),
         ctypes.c_int32(k.shape[3]), _p(out), stream_ptr(device))
     check(rc, "hipattn_prescale_k")
+    return out
+
+
+def prescale_k_rope(k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions, device) -> torch.Tensor:
+    """``[len(positions), *k.shape]``: for each position p the copy ``bf16(rot(k, p) * c_k)`` of a 4-D bf16 key tensor."""
+    assert k.ndim == 4 and k.dtype == torch.bfloat16 and k.stride(3) == 1
+    assert cos.dtype == torch.bfloat16 and sin.dtype == torch.bfloat16 and cos.stride(1) == 1 and sin.stride(1) == 1
+    out = torch.empty((len(positions),) + tuple(k.shape), dtype=k.dtype, device=k.device)
+    esz = 2
+    for i, p in enumerate(positions):
+        with _timed("prescale_k"):
+          rc = lib().hipattn_prescale_k_rope(
+            _p(k), ctypes.c_int64(k.stride(0)), ctypes.c_int64(k.stride(1)), ctypes.c_int64(k.stride(2)),
+            ctypes.c_int64(k.shape[0]), ctypes.c_int32(k.shape[1]), ctypes.c_int32(k.shape[2]),
+            ctypes.c_int32(k.shape[3]), ctypes.c_void_p(cos.data_ptr() + p * cos.stride(0) * esz),
+            ctypes.c_void_p(sin.data_ptr() + p * sin.stride(0) * esz), _p(out[i]), stream_ptr(device))
+        check(rc, "hipattn_prescale_k_rope")
     return out
 
 

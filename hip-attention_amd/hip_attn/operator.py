@@ -134,28 +134,37 @@ def _new_statistics(args: HiPAttentionArgs, B: int, head_kv: int, pages: int, de
 
 
 def _mask_kv(args: HiPAttentionArgs, k_mask: Optional[Tensor], max_tsrc: int, q: Tensor, programs_rows: int,
-             chunk_count: int, device, stats=None):
-    """KV description for the scan kernels, with keys pre-scaled when that saves work."""
+             chunk_count: int, device, stats=None, rope_tabs=None):
+    """KV descriptions for the scan kernels: ``(plain, prescaled or None, keepalive, khat, k_side_delta)``.
+
+    ``prescaled`` describes keys scaled (and, with RoPE on load under the relative / infllm rules, rotated) once for
+    the whole tensor; it is built when the scan will sample far more rows than the key tensor holds.
+    """
     stage0 = args.stages[0]
     iters = max(1, int(stage0.stage_chunk_size).bit_length())
     sampled_rows = 2 * iters * programs_rows * chunk_count  # stage 0 alone
-    rope = args.using_extend and args.need_apply_rope  # keys are rotated per sample: nothing to scale ahead
-    if q.dtype == torch.bfloat16 and args.offload_cache is None and not rope:
+    plain, keep = _kv_struct(args, k_mask, k_mask, max_tsrc, masking=True, stats=stats)
+    if q.dtype == torch.bfloat16 and args.offload_cache is None:
         src = k_mask if k_mask is not None else args.k_cache
         if src is not None and src.dtype == torch.bfloat16 and src.ndim == 4 and src.stride(-1) == 1:
             rows_total = src.shape[0] * src.shape[1] * src.shape[2]
             force = os.getenv("HIP_ATTN_PRESCALE_K", "")  # "0" / "1" override the heuristic (testing)
             if force == "1" or (force != "0" and sampled_rows >= 4 * rows_total):
-                khat = N.prescale_k(src, device)
+                delta = 0
+                if rope_tabs is None:
+                    khat = khat0 = N.prescale_k(src, device)
+                else:
+                    # rotated to position 0 (left samples, and everything under infllm) and 1 (right samples, relative)
+                    khat = N.prescale_k_rope(src, rope_tabs[0], rope_tabs[1], (0, 1), device)
+                    khat0, delta = khat[0], khat.stride(0)
                 if k_mask is not None:
-                    st, keep = _kv_struct(args, khat, khat, max_tsrc, masking=True, stats=stats)
+                    st, keep2 = _kv_struct(args, khat0, khat0, max_tsrc, masking=True, stats=stats)
                 else:
                     a2 = args.clone()
-                    a2.k_cache, a2.v_cache = khat, khat
-                    st, keep = _kv_struct(a2, None, None, max_tsrc, masking=True, stats=stats)
-                return st, (keep, khat), khat
-    st, keep = _kv_struct(args, k_mask, k_mask, max_tsrc, masking=True, stats=stats)
-    return st, keep, None
+                    a2.k_cache, a2.v_cache = khat0, khat0
+                    st, keep2 = _kv_struct(a2, None, None, max_tsrc, masking=True, stats=stats)
+                return plain, st, (keep, keep2, khat), (khat if rope_tabs is None else None), delta
+    return plain, None, keep, None, 0
 
 
 def _stage_cache_views(chunk_left: Tensor, HEAD: int, chunk: int) -> HiPAttentionStageInputCache:
@@ -251,8 +260,6 @@ def dual_stage_quadratic_hip_attention(
     qq = q if q.stride(-1) == 1 else q.contiguous()
     rope_tabs = _rope_tables(args, q.dtype) if (args.using_extend and args.need_apply_rope) else None
     hg = 1 if _head_reduce_enabled() else HEAD
-    mask_kv = None  # built lazily: cached-mask steps never touch the estimation path
-    k_prescaled = False
     khat = None
 
     if (cached_metadata is None) or (cached_metadata.indices is None):
@@ -273,9 +280,8 @@ def dual_stage_quadratic_hip_attention(
         # Keys are scaled by c_k and re-rounded every time they are sampled.  When the scan will sample
         # far more rows than the key tensor holds (prefill), scale the whole tensor once instead.
         mask_stats = _new_statistics(args, BSZ, HEAD_KV, MAX_PAGE, device)
-        mask_kv, keep_mask_kv, khat = _mask_kv(args, k_mask, MAX_TSRC, q, BSZ * HEAD * BDST_SCAN, chunk_count, device,
-                                               stats=mask_stats)
-        k_prescaled = khat is not None
+        mask_kv, mask_kv_pre, keep_mask_kv, khat, k_side_delta = _mask_kv(
+            args, k_mask, MAX_TSRC, q, BSZ * HEAD * BDST_SCAN, chunk_count, device, stats=mask_stats, rope_tabs=rope_tabs)
 
         scores = None
         left_out = None
@@ -349,12 +355,15 @@ def dual_stage_quadratic_hip_attention(
                 left_out = torch.empty((BSZ, bs, HEAD, chunk_count), dtype=torch.int32, device=device) if last else None
                 if chunk_count > 0:
                     rope = None
+                    use_pre = mask_kv_pre is not None
                     if rope_tabs is not None:  # :2200-2204
-                        rope = N.make_rope(*rope_tabs, stage.stage_extend_backend or args.scan_extend_backend)
+                        backend = stage.stage_extend_backend or args.scan_extend_backend
+                        use_pre = use_pre and backend in ("relative", "infllm")  # key positions fixed per sample side
+                        rope = N.make_rope(*rope_tabs, backend, k_side_delta if use_pre else 0)
                     qs = N.make_q(qq, position_ids, rope)
-                    N.mask_stage(qs, mask_kv, chunk_left, hg, chunk_count, chunk_size, right_clamp, bs,
-                                 BLOCK_SIZE_Q, stage.stage_block_stride_q, BLOCK_CHUNK, STAGE_STRIDE, sw_eff,
-                                 args.stage_early_terminate, scores, left_out, device, k_prescaled=k_prescaled,
+                    N.mask_stage(qs, mask_kv_pre if use_pre else mask_kv, chunk_left, hg, chunk_count, chunk_size,
+                                 right_clamp, bs, BLOCK_SIZE_Q, stage.stage_block_stride_q, BLOCK_CHUNK, STAGE_STRIDE,
+                                 sw_eff, args.stage_early_terminate, scores, left_out, device, k_prescaled=use_pre,
                                  reduce_heads=reduce)
             elif isinstance(stage, NopStage):
                 scores = torch.full((BSZ, bs, 1 if hg == 1 else HEAD, chunk_count), -32000.0, dtype=torch.float32,

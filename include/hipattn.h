@@ -53,6 +53,10 @@ typedef struct hipattn_rope {
     int64_t stride_t; /* elements between rows */
     int64_t len;
     int32_t backend;  /* HIPATTN_EXTEND_* for this call */
+    /* hipattn_mask_stage with k_prescaled != 0 and the RELATIVE rule: kv->k holds the keys rotated to position 0
+     * and scaled (hipattn_prescale_k_rope), and the copy rotated to position 1, which the right-hand samples
+     * read, starts this many elements behind it.  INFLLM needs the position-0 copy only.  Unused otherwise. */
+    int64_t k_side_delta;
 } hipattn_rope_t;
 
 /* Query tensor q[B, TDST, HEAD, HID] and its token positions (0-based, int64)
@@ -137,6 +141,14 @@ int64_t hipattn_mask_stage_workspace_bytes(int32_t dtype, int32_t B, int32_t bs,
  * every loaded key (src/hip_attn/v1_2/attention_extend.py:932-937); results are identical. */
 int hipattn_prescale_k(const void *k, int64_t stride0, int64_t stride1, int64_t stride2, int64_t n0,
                        int32_t n1, int32_t n2, int32_t HID, void *out, void *stream);
+
+/* The same with a rotation first: out = bf16(rot(K, p) * c_k) for ONE position p whose table rows (HID/2 bf16
+ * entries each, 16-byte aligned) are cos_row / sin_row.  The RELATIVE and INFLLM scan rules rotate every sampled
+ * key to position 0 or 1 whatever the token, so two such copies replace the per-sample rotation
+ * (see hipattn_rope_t.k_side_delta). */
+int hipattn_prescale_k_rope(const void *k, int64_t stride0, int64_t stride1, int64_t stride2, int64_t n0,
+                            int32_t n1, int32_t n2, int32_t HID, const void *cos_row, const void *sin_row,
+                            void *out, void *stream);
 
 /* Between two stages: max over heads, top-k under (score desc, position asc), realign, split.
  * Replaces the ATen glue at src/hip_attn/v1_2/attention_extend.py:2566-2570 (head reduce),

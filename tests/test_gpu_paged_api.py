@@ -103,3 +103,39 @@ def test_forward_paged_hip_long_prefill_splits_off_last_64_queries():
     got = out.view(B, TQ, H, D)
     assert_context_close(got[:, :-64], octx1, "bf16")
     assert_context_close(got[:, -64:], octx2, "bf16")
+
+
+def test_forward_paged_hip_decode_with_rope_applied_on_load():
+    """using_extend on (the configuration default): the KV pool holds keys without rotation and the serving stack
+    hands over its cos/sin tables; dense layers scan with the streaming rule, the others with the relative one."""
+    from hip_attn import HiPAttentionConfig, forward_paged_hip
+    from helpers import rope_tables
+
+    print("[case] forward_paged_hip decode, rope on load", flush=True)
+    B, TK, H, HKV, D, sw = 2, 3072, 8, 2, 128, 512
+    lens = np.array([3072, 2000])
+    X = make_inputs(23, B=B, TQ=1, TK=TK, H=H, HKV=HKV, D=D, dtype="bf16", pos=(lens - 1)[:, None])
+    kc, vc, r2t, pool_idx = _pool(X, 3)
+    spec = ('{"dense_layers": [0], "layers": [{"second_stage_k": 256, "sliding_window_size": %d},'
+            '{"second_stage_k": 128, "sliding_window_size": %d}]}') % (sw, sw)
+    cfg = HiPAttentionConfig(json_or_path=spec)
+    assert cfg.using_extend
+    cos, sin, _ = rope_tables(4096, D, "bf16")
+    sm = D ** -0.5
+    dev = "cuda"
+    common = dict(sm_scale=sm, batch_size=B, k_cache=to_torch(kc, "bf16", dev), v_cache=to_torch(vc, "bf16", dev),
+                  offload_cache=None, seq_lens=torch.from_numpy(lens).to(dev), req_to_tokens=torch.from_numpy(r2t).to(dev),
+                  req_pool_indices=torch.from_numpy(pool_idx).to(dev),
+                  rope_cos=to_torch(O.f32_to_bf16_bits(cos), "bf16", dev), rope_sin=to_torch(O.f32_to_bf16_bits(sin), "bf16", dev),
+                  logit_cap=0.0, orig_context_len=131072, max_context_len=TK, hip_config=cfg)
+    q = to_torch(X.q, "bf16", dev).view(B, H, D)
+    for layer_id, second_k, scan in ((0, 256, "streaming"), (5, 128, "relative")):
+        out, meta = forward_paged_hip(q, positions=torch.from_numpy(X.pos.reshape(-1).copy()).to(dev), layer_id=layer_id,
+                                      is_prefill=False, is_decode=True, **common)
+        XP, A = _oracle(X, kc, vc, r2t, pool_idx, lens, sm, second_k, sw, TK, False)
+        XP.rope_cos, XP.rope_sin = cos, sin
+        A.using_extend = A.need_apply_rope = True
+        A.scan_extend_backend, A.sa_extend_backend = scan, "streaming"
+        octx, ometa = O.hip_attention_12(XP, A)
+        assert_metadata_equal(meta, ometa)
+        assert_context_close(out.view(B, 1, H, D), octx, "bf16")

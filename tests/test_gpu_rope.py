@@ -120,3 +120,22 @@ def test_unbuilt_rules_fail_loudly():
         run_product(X, _ext(sa_extend_backend="relative"))
     with pytest.raises(NotImplementedError):
         run_product(X, tiny_args(using_extend=True, need_apply_rope=False))
+
+
+@pytest.mark.parametrize("scan", ["relative", "infllm"])
+@pytest.mark.parametrize("force", ["0", "1"])
+def test_keys_rotated_and_scaled_ahead_give_identical_masks(scan, force, monkeypatch):
+    """relative / infllm rotate sampled keys to position 0 or 1 whatever the token: rotating and scaling the whole
+    key tensor once per position must give the same mask as rotating every sample (one stage keeps the streaming
+    rule, which cannot be prepared ahead, to cover the mix)."""
+    print(f"[case] rope prescaled scan={scan} force={force}", flush=True)
+    monkeypatch.setenv("HIP_ATTN_PRESCALE_K", force)
+    X = with_rope(make_inputs(37, B=2, TQ=200, TK=2048, H=4, HKV=2, D=64, dtype="bf16", scale=0.5), 4096)
+    A = _ext(scan_extend_backend=scan, sa_extend_backend="streaming",
+             stages=[O.OStage(32, 2, 64, None, 1), O.OStage(32, 2, 16, 2048, 1, "streaming"), O.OStage(32, 1, 2, 1024, 1)])
+    octx, ometa = O.hip_attention_12(X, A)
+    for XX in (X, with_rope(to_paged(X, 16, seed=6), 4096)):
+        AA = A if XX is X else O.OArgs(**{**A.__dict__, "extend_context_length": 2048})
+        ctx, meta = run_product(XX, AA)
+        assert np.array_equal(meta.indices.cpu().numpy(), ometa.indices)
+        assert_context_close(ctx, octx, "bf16")
