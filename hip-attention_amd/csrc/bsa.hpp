@@ -27,7 +27,14 @@ struct BsaParamsBase {
 struct BsaParams : BsaParamsBase {
     KVExt kx;
     RopeView rope;
+    float softcap;  // 0 = off; logits become tanh(qk / softcap) * softcap (attention_extend_bsa.py:507-508)
 };
+
+// tanh(x / cap) * cap through one exp2 and one reciprocal: tanh(y) = 1 - 2 / (exp(2y) + 1)
+__device__ __forceinline__ float softcap_logit(float x, float cap, float two_log2e_over_cap) {
+    const float e = __builtin_amdgcn_exp2f(x * two_log2e_over_cap);
+    return cap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f));
+}
 // Rotated position of a sink or selected key (attention_extend_bsa.py:256-299): "streaming" packs them, in the
 // order of the index row, into the positions that end just below the window of the block's first query;
 // "infllm" puts all of them at that edge.  `slot` = token for sink tokens, (j + sink / bk) * bk + e for element e

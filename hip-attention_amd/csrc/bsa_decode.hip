@@ -19,9 +19,10 @@ using DecodeParams = DecodeParamsT<true>;
 
 // ROPE = true (extended parameter block only): query and keys are rotated on load; lanes dl and dl ^ 8 of a
 // 16-lane group hold the two halves of a row.
-template <typename T, int HID, int G, bool EXT, bool ROPE = false>
+// CAP = true (extended parameter block only): logits are soft-capped.
+template <typename T, int HID, int G, bool EXT, bool ROPE = false, bool CAP = false>
 __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<EXT> dp) {
-    static_assert(!ROPE || EXT, "rope variant takes the extended parameter block");
+    static_assert((!ROPE && !CAP) || EXT, "rope / softcap variants take the extended parameter block");
     constexpr int SEG = HID / 16;
     const BsaParamsFor<EXT> &p = dp.a;
     const KVExt *kx = nullptr;
@@ -153,6 +154,7 @@ __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<E
             d += __shfl_xor(d, 2);
             d += __shfl_xor(d, 4);
             d += __shfl_xor(d, 8);
+            if constexpr (CAP) d = tanhf(d / p.softcap) * p.softcap;
             const float x = d * 1.44269504f;
             const float m_new = fmaxf(m[g], x);
             const float alpha = exp2f(m[g] - m_new);
@@ -245,7 +247,12 @@ static int launch_partial(const DecodeParams &dp, hipStream_t st) {
 #define DEC_CASE(GG)                                                                                   \
     if constexpr (GG * HID <= 512) {                                                                   \
         if (dp.a.G == GG) {                                                                            \
-            if (dp.a.rope.cos) {                                                                       \
+            if (dp.a.softcap != 0.0f) {                                                                \
+                if (dp.a.rope.cos)                                                                     \
+                    hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG, true, true, true>), grid, block, 0, st, dp); \
+                else                                                                                   \
+                    hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG, true, false, true>), grid, block, 0, st, dp); \
+            } else if (dp.a.rope.cos) {                                                                \
                 hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG, true, true>), grid, block, 0, st, dp); \
             } else if (dp.a.kx.extended()) {                                                           \
                 hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG, true>), grid, block, 0, st, dp);  \

@@ -53,9 +53,11 @@ struct MfmaSmem {
 // ROPE = true (extended parameter block, unscaled keys): query rows and staged key rows are rotated on load.
 // A query lane holds both halves of its row (k-steps ks and ks + KS/2); the two halves of a staged key row are
 // fetched by lanes tid and tid ^ (HID/16) of one wave.
-template <int HID, bool KSCALED, bool EXT, bool ROPE = false>
+// CAP = true (extended parameter block): logits are soft-capped before the softmax.
+template <int HID, bool KSCALED, bool EXT, bool ROPE = false, bool CAP = false>
 __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p, int hgroups, int hpw, long long total_wg) {
     static_assert(!ROPE || (EXT && !KSCALED), "rope variant: extended parameter block, keys scaled in the kernel");
+    static_assert(!CAP || EXT, "softcap variant: extended parameter block");
     const KVExt *kx = nullptr;
     if constexpr (EXT) kx = &p.kx;
     constexpr int KS = HID / 16;   // k-steps of the first product
@@ -294,6 +296,14 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
             sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1.v, qf[ks].v, sacc[1], 0, 0, 0);
         }
 
+        if constexpr (CAP) {
+            const float k2 = 2.0f * LOG2E / p.softcap;
+#pragma unroll
+            for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) sacc[nb][i] = softcap_logit(sacc[nb][i], p.softcap, k2);
+        }
+
         // ---- mask + online softmax; element (nb, i) of a lane is token slot nb*32 + (i/4)*8 + hh*4 + i%4
         float mx = -INFINITY;
         if (full) {
@@ -431,7 +441,7 @@ __global__ __launch_bounds__(256) void bsa_mark_kernel(BsaParams p, int hgroups,
     }
 }
 
-template <int HID, bool KSCALED, bool EXT, bool ROPE = false>
+template <int HID, bool KSCALED, bool EXT, bool ROPE = false, bool CAP = false>
 static int launch_mfma(const BsaParams &p, hipStream_t st) {
     const int hpw = p.share_first_head ? 4 : 1;  // per-head index rows: one head per workgroup
     const int hgroups = (p.G + hpw - 1) / hpw;
@@ -440,12 +450,12 @@ static int launch_mfma(const BsaParams &p, hipStream_t st) {
     const size_t smem = sizeof(MfmaSmem<HID>);
     static bool attr_set = false;
     if (!attr_set) {
-        HIPATTN_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&bsa_mfma_kernel<HID, KSCALED, EXT, ROPE>),
+        HIPATTN_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&bsa_mfma_kernel<HID, KSCALED, EXT, ROPE, CAP>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
     const BsaParamsFor<EXT> &pk = p;  // the plain kernel takes the block without the extras
-    hipLaunchKernelGGL((bsa_mfma_kernel<HID, KSCALED, EXT, ROPE>), dim3((unsigned)total), dim3(NTHREADS), smem, st, pk, hgroups,
+    hipLaunchKernelGGL((bsa_mfma_kernel<HID, KSCALED, EXT, ROPE, CAP>), dim3((unsigned)total), dim3(NTHREADS), smem, st, pk, hgroups,
                        hpw, total);
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
@@ -476,6 +486,11 @@ int bsa_mfma_launch(const BsaParams &p, int dtype, int HID, hipStream_t st) {
     }
 #define BSA_PICK(H)                                                                  \
     case H:                                                                          \
+        if (p.softcap != 0.0f) {                                                     \
+            if (p.k_prescaled) return HIPATTN_E_UNSUPPORTED;                         \
+            return p.rope.cos ? launch_mfma<H, false, true, true, true>(p, st)       \
+                              : launch_mfma<H, false, true, false, true>(p, st);     \
+        }                                                                            \
         if (p.rope.cos) return launch_mfma<H, false, true, true>(p, st);             \
         if (p.k_prescaled) return ext ? launch_mfma<H, true, true>(p, st) : launch_mfma<H, true, false>(p, st); \
         return ext ? launch_mfma<H, false, true>(p, st) : launch_mfma<H, false, false>(p, st);

@@ -133,6 +133,7 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
                             dot = __fmaf_rn(s_q[wid][d0 + e], Elem<T>::round(kk[e] * p.c_k), dot);
                     }
                 }
+                if (p.softcap != 0.0f) dot = tanhf(dot / p.softcap) * p.softcap;
                 logit = dot * 1.44269504f;
             }
             const float tile_max = wave_max(logit);
@@ -193,6 +194,8 @@ int bsa_fill_params(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t 
     if (rc) return rc;
     rc = make_rope_view(q, (1u << HIPATTN_EXTEND_STREAMING) | (1u << HIPATTN_EXTEND_INFLLM), "bsa", &p->rope);
     if (rc) return rc;
+    HIPATTN_CHECK_ARG(q->logit_softcap >= 0.0f, HIPATTN_E_ARG, "bsa: negative logit_softcap");
+    p->softcap = q->logit_softcap;
     HIPATTN_CHECK_ARG(q->HEAD % p->kv.HKV == 0, HIPATTN_E_ARG, "bsa: HEAD %% HKV != 0");
     p->q = q->ptr; p->q_sb = q->stride_b; p->q_st = q->stride_t; p->q_sh = q->stride_h;
     p->pos = q->pos; p->pos_sb = q->pos_stride_b; p->pos_st = q->pos_stride_t;

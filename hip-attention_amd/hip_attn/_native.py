@@ -32,6 +32,7 @@ class QStruct(ctypes.Structure):
         ("B", ctypes.c_int32), ("TDST", ctypes.c_int32), ("HEAD", ctypes.c_int32), ("HID", ctypes.c_int32),
         ("dtype", ctypes.c_int32),
         ("rope", ctypes.c_void_p),
+        ("logit_softcap", ctypes.c_float),
     ]
 
 
@@ -152,10 +153,12 @@ def make_rope(cos: torch.Tensor, sin: torch.Tensor, backend: str, k_side_delta: 
     return r
 
 
-def make_q(q: torch.Tensor, pos: torch.Tensor, rope: Optional[RopeStruct] = None) -> QStruct:
+def make_q(q: torch.Tensor, pos: torch.Tensor, rope: Optional[RopeStruct] = None,
+           logit_softcap: Optional[float] = None) -> QStruct:
     assert q.ndim == 4 and q.stride(3) == 1
     assert pos.dtype == torch.int64 and pos.ndim == 2
     s = QStruct()
+    s.logit_softcap = float(logit_softcap or 0.0)
     if rope is not None:
         s._rope_keep = rope  # the struct holds a bare pointer to it
         s.rope = ctypes.addressof(rope)

@@ -49,8 +49,8 @@ def _reject_unsupported(args: HiPAttentionArgs):
     if args.using_extend and not args.need_apply_rope:
         raise NotImplementedError("using_extend with keys stored WITH rotation (need_apply_rope=False) is not built; "
                                   "store q and k without RoPE and pass need_apply_rope=True")
-    if args.logit_softcap is not None:
-        raise NotImplementedError("logit_softcap is not built yet")
+    if args.logit_softcap is not None and not (args.logit_softcap > 0):
+        raise ValueError("logit_softcap must be positive (or None)")
     if not args.is_causal:
         raise NotImplementedError("is_causal=False is not built")
     if args.sliding_window_indices is not None:
@@ -483,8 +483,8 @@ def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], 
     if position_ids.dtype != torch.int64:
         position_ids = position_ids.to(torch.int64)
     rope = N.make_rope(*rope_tables, args.sa_extend_backend) if rope_tables is not None else None
-    qs = N.make_q(qq, position_ids, rope)
-    if rope is not None:
+    qs = N.make_q(qq, position_ids, rope, args.logit_softcap)
+    if rope is not None or args.logit_softcap is not None:
         khat = None
     if not indices.is_contiguous():
         indices = indices.contiguous()

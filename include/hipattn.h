@@ -70,6 +70,10 @@ typedef struct hipattn_q {
     int32_t B, TDST, HEAD, HID;
     int32_t dtype; /* HIPATTN_F32 / HIPATTN_BF16; K and V share it */
     const hipattn_rope_t *rope; /* host pointer; NULL: rows are used as stored */
+    /* HiPAttentionArgs.logit_softcap: 0 = off, else attention logits become tanh(qk / cap) * cap before the
+     * softmax (src/hip_attn/v1_2/attention_extend_bsa.py:507-508).  Read by the bsa entry points only; the mask
+     * stage scores are never capped (the reference's scan kernel has no such option). */
+    float logit_softcap;
 } hipattn_q_t;
 
 /* Key/value storage: dense k,v[B, TSRC, HKV, HID] or a paged cache [pages, page_size, HKV, HID]

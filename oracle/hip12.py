@@ -58,6 +58,7 @@ class _Tensors(ctypes.Structure):
         ("rope_len", ctypes.c_int64),
         ("scan_backend", ctypes.c_int),
         ("sa_backend", ctypes.c_int),
+        ("logit_softcap", ctypes.c_float),
     ]
 
 
@@ -149,6 +150,7 @@ class OArgs:
     need_apply_rope: bool = False
     scan_extend_backend: str = "relative"
     sa_extend_backend: str = "streaming"
+    logit_softcap: Optional[float] = None  # attention logits only (attention_extend_bsa.py:507-508)
 
 
 @dataclass
@@ -167,6 +169,7 @@ class OInputs:
     rope_sin: Optional[np.ndarray] = None
     scan_backend: Optional[str] = None  # rotation rule of the mask stage / of sparse attention; None = no RoPE
     sa_backend: Optional[str] = None
+    logit_softcap: float = 0.0
 
     def c_struct(self, max_tsrc: int):
         np_t = np.uint16 if self.dtype == "bf16" else np.float32
@@ -203,6 +206,7 @@ class OInputs:
             S.bt_cols = self.block_table.shape[1]
             S.cache_seq_lens = arr(self.cache_seq_lens, np.int64)
         S.MAX_TSRC = max_tsrc
+        S.logit_softcap = float(self.logit_softcap or 0.0)
         if self.access is not None:
             assert self.access.dtype == np.int32 and self.access.flags.c_contiguous and self.access.ndim == 3
             S.access = self.access.ctypes.data
@@ -488,11 +492,14 @@ def hip_attention_12(X: OInputs, A: OArgs, cached: Optional[OMetadata] = None):
 
     decode = (TDST == 1) and (not A.disable_flashdecode)
     X.access = sa_access
+    user_cap = X.logit_softcap
+    X.logit_softcap = float(A.logit_softcap or 0.0)
     try:
         context = bsa(X, MAX_TSRC, indices, ks_start_end, block_size_q, block_size_k, sw_bsa, sink,
                       share_first_head=decode)
     finally:
         X.access = user_access
+        X.logit_softcap = user_cap
         X.scan_backend, X.sa_backend = user_backends
     meta = OMetadata(indices=indices, ks=ks, ks_count=ks_count, ks_start_end=ks_start_end,
                      stage_caches=stage_caches, mask_access=mask_access, sa_access=sa_access)

@@ -77,6 +77,7 @@ typedef struct {
     int64_t rope_len;
     int scan_backend;        /* HIPO_EXT_* for the mask stage */
     int sa_backend;          /* HIPO_EXT_* for block sparse attention */
+    float logit_softcap;     /* 0 = off; attention logits become tanh(qk / cap) * cap (attention_extend_bsa.py:507-508) */
 } hipo_tensors_t;
 
 /* ---------------------------------------------------------------- scalar helpers */
@@ -530,7 +531,9 @@ int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_
                     int64_t t = tok[i];
                     int att = kind[i] == 0 ? (t + sw <= p) : (t <= p && p < t + sw);
                     if (!att) { logit[i] = -INFINITY; continue; }
-                    logit[i] = hipo_dot(qhat, khat + (size_t)i * HID, HID) * 1.44269504f;
+                    float qk = hipo_dot(qhat, khat + (size_t)i * HID, HID);
+                    if (X->logit_softcap != 0.0f) qk = tanhf(qk / X->logit_softcap) * X->logit_softcap;
+                    logit[i] = qk * 1.44269504f;
                     if (logit[i] > m) m = logit[i];
                 }
                 double lsum = 0.0;

@@ -39,6 +39,8 @@ def product_args(A: O.OArgs, X: O.OInputs, device="cuda", **extra):
         kw.update(k_cache=to_torch(X.k_cache, X.dtype, device), v_cache=to_torch(X.v_cache, X.dtype, device),
                   block_table=torch.from_numpy(X.block_table).to(device),
                   cache_seq_lens=torch.from_numpy(X.cache_seq_lens).to(device))
+    if getattr(A, "logit_softcap", None) is not None:
+        kw.update(logit_softcap=A.logit_softcap)
     if A.using_extend:
         kw.update(using_extend=True, need_apply_rope=A.need_apply_rope, scan_extend_backend=A.scan_extend_backend,
                   sa_extend_backend=A.sa_extend_backend,

@@ -11,7 +11,7 @@ from test_oracle_bsa import random_indices
 pytestmark = pytest.mark.gpu
 
 
-def _run(X, max_tsrc, idx, kse, bq, bk, sw, sink, impl, share=False, decode=False):
+def _run(X, max_tsrc, idx, kse, bq, bk, sw, sink, impl, share=False, decode=False, softcap=None):
     from hip_attn import HiPAttentionArgs12
     from hip_attn.operator import block_sparse_attention
 
@@ -22,7 +22,7 @@ def _run(X, max_tsrc, idx, kse, bq, bk, sw, sink, impl, share=False, decode=Fals
         kw = dict(k_cache=to_torch(X.k_cache, X.dtype, dev), v_cache=to_torch(X.v_cache, X.dtype, dev),
                   block_table=torch.from_numpy(X.block_table).to(dev),
                   cache_seq_lens=torch.from_numpy(X.cache_seq_lens).to(dev))
-    args = HiPAttentionArgs12(sink_token_size=sink, sliding_window_size=sw, **kw)
+    args = HiPAttentionArgs12(sink_token_size=sink, sliding_window_size=sw, logit_softcap=softcap, **kw)
     args.block_size_q, args.block_size_k = bq, bk
     out = block_sparse_attention(q, to_torch(X.k, X.dtype, dev), to_torch(X.v, X.dtype, dev),
                                  torch.from_numpy(X.pos.copy()).to(dev), torch.from_numpy(idx).to(dev),
@@ -90,3 +90,26 @@ def test_decode_kernel_matches_oracle(dtype, D, G):
     ref = O.bsa(X, TK, idx, kse, 1, bk, sw, sink, share_first_head=True)
     out = _run(X, TK, idx, kse, 1, bk, sw, sink, impl=0, decode=True)
     assert_context_close(out, ref, dtype)
+
+
+@pytest.mark.parametrize("dtype,D", [("bf16", 128), ("bf16", 64), ("f32", 64)])
+def test_logit_softcap_in_every_attention_kernel(dtype, D):
+    print(f"[case] bsa softcap {dtype} D={D}", flush=True)
+    rng = np.random.default_rng(D)
+    TK, TQ, H, HKV, bq, bk, BK, sw, sink = 1024, 96, 8, 2, 32, 8, 16, 64, 16
+    X = make_inputs(42, B=2, TQ=TQ, TK=TK, H=H, HKV=HKV, D=D, dtype=dtype, scale=1.5)
+    X.logit_softcap = 3.0
+    idx, ks, kse = random_indices(rng, 2, H, O.cdiv(TQ, bq), BK, bk, TK, same_heads=True)
+    ref = O.bsa(X, TK, idx, kse, bq, bk, sw, sink)
+    uncapped = O.OInputs(X.dtype, X.q, X.pos, k=X.k, v=X.v)
+    assert np.abs(O.bf16_bits_to_f32(ref) - O.bf16_bits_to_f32(O.bsa(uncapped, TK, idx, kse, bq, bk, sw, sink))).max() > 0.05 \
+        if dtype == "bf16" else True
+    assert_context_close(_run(X, TK, idx, kse, bq, bk, sw, sink, impl=1, share=True, softcap=3.0), ref, dtype)
+    if dtype == "bf16":
+        assert_context_close(_run(X, TK, idx, kse, bq, bk, sw, sink, impl=2, share=True, softcap=3.0), ref, dtype)
+    # decode: one query at the end of each sequence
+    Xd = make_inputs(43, B=2, TQ=1, TK=TK, H=H, HKV=HKV, D=D, dtype=dtype, scale=1.5)
+    Xd.logit_softcap = 3.0
+    idx, ks, kse = random_indices(rng, 2, H, 1, BK, bk, TK, same_heads=True)
+    ref = O.bsa(Xd, TK, idx, kse, 1, bk, sw, sink, share_first_head=True)
+    assert_context_close(_run(Xd, TK, idx, kse, 1, bk, sw, sink, impl=0, decode=True, softcap=3.0), ref, dtype)

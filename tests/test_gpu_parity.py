@@ -150,3 +150,15 @@ def test_short_context_and_mask_only():
     assert_context_close(ctx, octx, "f32")
     A.mask_only = True
     assert run_product(X, A) == (None, None)
+
+
+def test_operator_with_logit_softcap():
+    _case("operator softcap")
+    X = make_inputs(44, B=1, TQ=128, TK=2048, H=4, HKV=2, D=64, dtype="bf16", scale=1.5)
+    A = tiny_args(logit_softcap=4.0)
+    octx, ometa = O.hip_attention_12(X, A)
+    ctx, meta = run_product(X, A)
+    assert_metadata_equal(meta, ometa)  # the cap never touches mask estimation
+    assert_context_close(ctx, octx, "bf16")
+    plain, _ = O.hip_attention_12(X, tiny_args())
+    assert np.abs(O.bf16_bits_to_f32(plain) - O.bf16_bits_to_f32(octx)).max() > 0.05

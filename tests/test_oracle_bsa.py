@@ -7,7 +7,7 @@ from oracle import hip12 as O
 from helpers import make_inputs, to_paged, widen
 
 
-def dense_reference(X, indices, ks, bq, bk, sw, sink, max_tsrc, share_first_head=False):
+def dense_reference(X, indices, ks, bq, bk, sw, sink, max_tsrc, share_first_head=False, softcap=None):
     """softmax over the attended set written as an explicit boolean mask, float64 arithmetic.
 
     Built from the set definition only (no tiling): sink tokens and selected-block tokens at
@@ -43,6 +43,8 @@ def dense_reference(X, indices, ks, bq, bk, sw, sink, max_tsrc, share_first_head
                        (t[None, :] >= max(0, curr - sw - bq)) & (sw > 0)
                 mask = (far & (sel | (t < sink))[None, :]) | near
                 logits = qh[b, rows, h] @ kh[b, :, h // G].T
+                if softcap is not None:
+                    logits = np.tanh(logits / softcap) * softcap
                 logits = np.where(mask, logits, -np.inf)
                 m = logits.max(axis=1, keepdims=True)
                 m = np.where(np.isfinite(m), m, 0.0)
@@ -137,3 +139,17 @@ def test_paged_equals_dense_bit_exact(page_size):
     XP = to_paged(X, page_size, seed=page_size)
     paged = O.bsa(XP, 4096, idx, kse, 16, bk, 16, 4)
     assert np.array_equal(dense, paged)
+
+
+@pytest.mark.parametrize("dtype,tol", [("f32", 2e-5), ("bf16", 1.5e-2)])
+def test_logit_softcap_is_tanh_capping_of_the_logits(dtype, tol):
+    rng = np.random.default_rng(9)
+    B, TQ, TK, H, HKV, D, bq, bk, sw, sink = 1, 40, 256, 4, 2, 32, 16, 8, 24, 8
+    X = make_inputs(41, B=B, TQ=TQ, TK=TK, H=H, HKV=HKV, D=D, dtype=dtype, scale=1.5)
+    idx, ks, kse = random_indices(rng, B, H, O.cdiv(TQ, bq), 6, bk, TK)
+    plain = widen(O.bsa(X, TK, idx, kse, bq, bk, sw, sink), dtype)
+    X.logit_softcap = 2.0
+    got = widen(O.bsa(X, TK, idx, kse, bq, bk, sw, sink), dtype)
+    want = dense_reference(X, idx, ks, bq, bk, sw, sink, TK, softcap=2.0)
+    assert np.abs(got - want).max() <= tol
+    assert np.abs(got - plain).max() > 10 * tol  # the cap matters at this scale
