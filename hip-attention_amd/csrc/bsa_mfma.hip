@@ -7,8 +7,9 @@
 // Per 64-token tile:   S^T[token, query] = K^ . Q^^T      (v_mfma_f32_32x32x16_bf16, K^ from LDS,
 //                                                           Q^ resident in registers)
 //                      online softmax down the token axis  (a lane owns one query column)
-//                      O^T[d, query]    += V^T . P^T        (V staged transposed in LDS; P^T is
-//                                                           taken straight from the S^T registers)
+//                      O^T[d, query]    += V^T . P^T        (V staged row-major in LDS and read through
+//                                                           the transposing LDS load; P^T is taken
+//                                                           straight from the S^T registers)
 // Working on the transposed problem keeps the softmax statistics lane-local and lets P feed the
 // second MFMA without a trip through LDS.  Global loads of tile i+1 are issued before the math of
 // tile i; LDS is double-buffered so one barrier per tile suffices.  The running maximum is only
@@ -24,7 +25,7 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 constexpr int TN = 64;        // tokens per tile
 constexpr int KPAD = 8;       // bf16 elements of row padding for the K^ tile
-constexpr int VPAD = 4;       // bf16 elements of row padding for the V^T tile
+constexpr int VPAD = 32;      // bf16 elements of row padding for the V tile: four consecutive rows tile all banks
 constexpr int NTHREADS = 512;
 constexpr int MAX_LDS_IDX = 1024;  // selected-block starts kept in LDS
 constexpr float LOG2E = 1.44269504f;
@@ -35,6 +36,12 @@ __device__ __forceinline__ uint32_t cvt_pk_bf16(float a, float b) {  // one v_cv
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
 
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+__device__ __forceinline__ uint2 lds_read_tr16(const uint16_t *p) {  // ds_read_b64_tr_b16
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p);
+    return __builtin_bit_cast(uint2, v);
+}
+
 union Frag {
     bf16x8 v;
     uint32_t u[4];
@@ -42,11 +49,18 @@ union Frag {
     uint4 q;
 };
 
+// what wave 0 posts about the 64 token slots of a tile
+struct MfmaMeta {
+    long long ko[TN], vo[TN];  // K / V row offsets (NO_ROW: zero row)
+    int tok[TN];               // token, -1 for an empty slot
+    int rp[TN];                // row of the RoPE tables the key is rotated with
+};
+
 template <int HID>
 struct MfmaSmem {
     uint16_t k[2][TN][HID + KPAD];
-    uint16_t vt[2][HID][TN + VPAD];
-    int tok[2][TN];
+    uint16_t v[2][TN][HID + VPAD];
+    MfmaMeta meta[4];
     int idx[MAX_LDS_IDX];
 };
 
@@ -176,53 +190,70 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
     const uint16_t *kbase = reinterpret_cast<const uint16_t *>(p.kv.k);
     const uint16_t *vbase = reinterpret_cast<const uint16_t *>(p.kv.v);
 
-    // ---- staging: thread handles chunks c = tid + NTHREADS*j: token slot c / (HID/8), 16-byte piece c % (HID/8)
-    uint4 kreg[CPT], vreg[CPT];
-    uint4 creg[ROPE ? CPT : 1], sreg[ROPE ? CPT : 1];  // cos / sin pieces of the staged key rows
-    int treg[CPT];
-    auto prefetch = [&](int tile) {
+    // ---- staging.  Wave 0 walks the token list: lane = token slot of a tile; it resolves the token, its K / V row
+    // offsets (page lookup, statistics, offload cache) and, with RoPE, its rotated position, one tile ahead of the
+    // loads, and posts them in LDS (four slots, so that a slot is rewritten only after every wave is done with it).
+    // All threads then fetch rows by posted offset: chunk c = tid + NTHREADS*j is 16-byte piece c % (HID/8) of token
+    // slot c / (HID/8).
+    long long m_ko = NO_ROW, m_vo = NO_ROW;
+    int m_t = -1, m_rp = 0;
+    auto resolve = [&](int tile) {  // wave 0 only
         int kind, base;  // kind 0 selected, 1 sink, 2 window
         if (tile < tiles_sel) { kind = 0; base = tile * TN; }
         else if (tile < tiles_sel + tiles_sink) { kind = 1; base = (tile - tiles_sel) * TN; }
         else { kind = 2; base = (tile - tiles_sel - tiles_sink) * TN; }
+        const int o = base + lane;
+        long long t = -1;
+        long long rpos = 0;  // rotated position of the key (ROPE only)
+        if (kind == 0) {
+            if (o < n_sel_tok) {
+                const int bi = o / p.bk;
+                const long long st = idx_in_lds ? (long long)sm.idx[bi] : p.indices[irow * p.BK + rs + bi];
+                t = st + o % p.bk;
+                if (!(t >= 0 && t < p.kv.max_tsrc && t < curr && t >= p.sink)) t = -1;
+                if constexpr (ROPE)
+                    rpos = bsa_rope_far_pos(p.rope, (long long)(rs + bi + p.sink / p.bk) * p.bk + o % p.bk, rope_shift,
+                                            pmin_blk, p.sw);
+            }
+        } else if (kind == 1) {
+            if (o < sink_end) t = o;
+            if constexpr (ROPE) rpos = bsa_rope_far_pos(p.rope, o, rope_shift, pmin_blk, p.sw);
+        } else {
+            if (o < n_win) t = ws + o;
+            rpos = t;
+        }
+        int64_t ko = NO_ROW, vo = NO_ROW;
+        if (t >= 0) kv_rows<true, EXT>(p.kv, kx, b, t, kvh, seqlen, ko, vo, true);
+        m_ko = ko;
+        m_vo = vo;
+        m_t = (int)t;
+        if constexpr (ROPE) m_rp = (int)(p.rope.row(rpos) / p.rope.stride_t);
+    };
+    auto post = [&](int tile) {  // wave 0 only
+        MfmaMeta &mt = sm.meta[tile & 3];
+        mt.ko[lane] = m_ko;
+        mt.vo[lane] = m_vo;
+        mt.tok[lane] = m_t;
+        if constexpr (ROPE) mt.rp[lane] = m_rp;
+    };
+    uint4 kreg[CPT], vreg[CPT];
+    uint4 creg[ROPE ? CPT : 1], sreg[ROPE ? CPT : 1];  // cos / sin pieces of the staged key rows
+    auto prefetch = [&](int tile) {
+        const MfmaMeta &mt = sm.meta[tile & 3];
 #pragma unroll
         for (int j = 0; j < CPT; j++) {
             const int c = tid + NTHREADS * j;
             const int slot = c / (HID / 8), piece = c % (HID / 8);
-            const int o = base + slot;
-            long long t = -1;
-            long long rpos = 0;  // rotated position of the key (ROPE only)
-            if (kind == 0) {
-                if (o < n_sel_tok) {
-                    const int bi = o / p.bk;
-                    const long long st = idx_in_lds ? (long long)sm.idx[bi] : p.indices[irow * p.BK + rs + bi];
-                    t = st + o % p.bk;
-                    if (!(t >= 0 && t < p.kv.max_tsrc && t < curr && t >= p.sink)) t = -1;
-                    if constexpr (ROPE)
-                        rpos = bsa_rope_far_pos(p.rope, (long long)(rs + bi + p.sink / p.bk) * p.bk + o % p.bk, rope_shift,
-                                                pmin_blk, p.sw);
-                }
-            } else if (kind == 1) {
-                if (o < sink_end) t = o;
-                if constexpr (ROPE) rpos = bsa_rope_far_pos(p.rope, o, rope_shift, pmin_blk, p.sw);
-            } else {
-                if (o < n_win) t = ws + o;
-                rpos = t;
-            }
-            treg[j] = (int)t;
+            const long long ko = mt.ko[slot], vo = mt.vo[slot];
             kreg[j] = make_uint4(0, 0, 0, 0);
             vreg[j] = make_uint4(0, 0, 0, 0);
             if constexpr (ROPE) {
-                const int64_t tr = p.rope.row(rpos) + (piece % (HID / 16)) * 8;
+                const int64_t tr = (int64_t)mt.rp[slot] * p.rope.stride_t + (piece % (HID / 16)) * 8;
                 creg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr);
                 sreg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr);
             }
-            if (t >= 0) {
-                int64_t ko, vo;
-                kv_rows<true, EXT>(p.kv, kx, b, t, kvh, seqlen, ko, vo, piece == 0);
-                if (ko != NO_ROW) kreg[j] = *reinterpret_cast<const uint4 *>(kbase + ko + piece * 8);
-                if (vo != NO_ROW) vreg[j] = *reinterpret_cast<const uint4 *>(vbase + vo + piece * 8);
-            }
+            if (ko != NO_ROW) kreg[j] = *reinterpret_cast<const uint4 *>(kbase + ko + piece * 8);
+            if (vo != NO_ROW) vreg[j] = *reinterpret_cast<const uint4 *>(vbase + vo + piece * 8);
         }
     };
     auto commit = [&](int buf) {
@@ -243,13 +274,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
                 kq.w = cvt_pk_bf16(__uint_as_float(kq.w << 16) * p.c_k, __uint_as_float(kq.w & 0xffff0000u) * p.c_k);
             }
             *reinterpret_cast<uint4 *>(&sm.k[buf][slot][piece * 8]) = kq;
-            const uint32_t vw[4] = {vreg[j].x, vreg[j].y, vreg[j].z, vreg[j].w};
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                sm.vt[buf][piece * 8 + 2 * e][slot] = (uint16_t)(vw[e] & 0xffffu);
-                sm.vt[buf][piece * 8 + 2 * e + 1][slot] = (uint16_t)(vw[e] >> 16);
-            }
-            if (piece == 0) sm.tok[buf][slot] = treg[j];
+            *reinterpret_cast<uint4 *>(&sm.v[buf][slot][piece * 8]) = vreg[j];
         }
     };
 
@@ -262,16 +287,27 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
     float m_run = -INFINITY;   // in log2 units, already multiplied by log2(e)
     float l_run = 0.0f;
 
-    if (ntiles > 0) prefetch(0);
+    if (ntiles > 0) {
+        if (wid == 0) {
+            resolve(0);
+            post(0);
+            if (ntiles > 1) resolve(1);
+        }
+        __syncthreads();
+        prefetch(0);
+    }
     for (int tile = 0; tile < ntiles; tile++) {
         const int buf = tile & 1;
         commit(buf);
+        if (wid == 0 && tile + 1 < ntiles) post(tile + 1);
         __syncthreads();
         if (tile + 1 < ntiles) prefetch(tile + 1);
+        if (wid == 0 && tile + 2 < ntiles) resolve(tile + 2);
+        const MfmaMeta &mt = sm.meta[tile & 3];
         const bool window = tile >= tiles_sel + tiles_sink;
 
         // tile summary (token range, all valid?) computed redundantly per wave
-        const int tk = sm.tok[buf][lane];
+        const int tk = mt.tok[lane];
         int tmin = tk < 0 ? 0x7fffffff : tk, tmax = tk;
         tmin = wave_min_i(tmin);
         tmax = wave_max_i(tmax);
@@ -316,7 +352,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
             for (int nb = 0; nb < 2; nb++)
 #pragma unroll
                 for (int i4 = 0; i4 < 4; i4++) {
-                    const int4 tt = *reinterpret_cast<const int4 *>(&sm.tok[buf][nb * 32 + i4 * 8 + hh * 4]);
+                    const int4 tt = *reinterpret_cast<const int4 *>(&mt.tok[nb * 32 + i4 * 8 + hh * 4]);
                     const int ts[4] = {tt.x, tt.y, tt.z, tt.w};
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
@@ -366,9 +402,15 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
         for (int db = 0; db < DB; db++) {
 #pragma unroll
             for (int j = 0; j < 4; j++) {
+                // V^T fragments straight from the row-major tile: a transposing LDS read hands lane l of a 16-lane
+                // group column l % 4 of the four rows addressed by lanes l / 4, l / 4 + 4, + 8, + 12 of the group, so
+                // with source lane s pointing at (token T0 + s / 4, d = D0 + 4 * (s % 4)) lane l receives tokens
+                // T0 .. T0 + 3 at d = D0 + l.
                 Frag a;
-                a.d[0] = *reinterpret_cast<const uint2 *>(&sm.vt[buf][db * 32 + col][j * 16 + hh * 4]);
-                a.d[1] = *reinterpret_cast<const uint2 *>(&sm.vt[buf][db * 32 + col][j * 16 + 8 + hh * 4]);
+                const int trow = j * 16 + hh * 4 + ((lane & 15) >> 2);
+                const int tcol = db * 32 + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+                a.d[0] = lds_read_tr16(&sm.v[buf][trow][tcol]);
+                a.d[1] = lds_read_tr16(&sm.v[buf][trow + 8][tcol]);
                 oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pf[j].v, oacc[db], 0, 0, 0);
             }
         }
