@@ -93,6 +93,8 @@ int make_kv_view(const hipattn_kv_t *kv, int B, int HID, int dtype, KVView *o, K
     o->tsrc = kv->tsrc; o->max_tsrc = kv->max_tsrc;
     o->block_table = kv->block_table; o->cache_seq_lens = kv->cache_seq_lens; o->bt_stride_b = kv->bt_stride_b;
     o->bt_is64 = kv->bt_is64; o->sl_is64 = kv->sl_is64; o->paged = kv->paged; o->page_size = kv->page_size ? kv->page_size : 1;
+    o->page_shift = 0;
+    while ((1 << o->page_shift) < o->page_size) o->page_shift++;
     o->HKV = kv->HKV;
     memset(x, 0, sizeof(*x));
     x->access_flags = kv->access_flags;

@@ -54,6 +54,8 @@ struct MfmaMeta {
     long long ko[TN], vo[TN];  // K / V row offsets (NO_ROW: zero row)
     int tok[TN];               // token, -1 for an empty slot
     int rp[TN];                // row of the RoPE tables the key is rotated with
+    int tmin, tmax, all_valid; // smallest / largest token of the tile (tmax < 0: empty tile), no empty slot
+    int pad_;
 };
 
 template <int HID>
@@ -196,24 +198,33 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
     // All threads then fetch rows by posted offset: chunk c = tid + NTHREADS*j is 16-byte piece c % (HID/8) of token
     // slot c / (HID/8).
     long long m_ko = NO_ROW, m_vo = NO_ROW;
-    int m_t = -1, m_rp = 0;
+    int m_t = -1, m_rp = 0, m_tmin = 0, m_tmax = -1, m_allv = 0;
+    const int bk_shift = (p.bk & (p.bk - 1)) == 0 ? __builtin_ctz(p.bk) : -1;  // block sizes are usually powers of two
+    const int tlimit = (int)(p.kv.max_tsrc < (long long)curr ? p.kv.max_tsrc : (long long)curr);
     auto resolve = [&](int tile) {  // wave 0 only
         int kind, base;  // kind 0 selected, 1 sink, 2 window
         if (tile < tiles_sel) { kind = 0; base = tile * TN; }
         else if (tile < tiles_sel + tiles_sink) { kind = 1; base = (tile - tiles_sel) * TN; }
         else { kind = 2; base = (tile - tiles_sel - tiles_sink) * TN; }
         const int o = base + lane;
-        long long t = -1;
+        int t = -1;
         long long rpos = 0;  // rotated position of the key (ROPE only)
         if (kind == 0) {
             if (o < n_sel_tok) {
-                const int bi = o / p.bk;
-                const long long st = idx_in_lds ? (long long)sm.idx[bi] : p.indices[irow * p.BK + rs + bi];
-                t = st + o % p.bk;
-                if (!(t >= 0 && t < p.kv.max_tsrc && t < curr && t >= p.sink)) t = -1;
+                const int bi = bk_shift >= 0 ? (o >> bk_shift) : o / p.bk;
+                const int e = o - bi * p.bk;
+                int st;
+                if (idx_in_lds) {
+                    st = sm.idx[bi];
+                } else {
+                    const long long s64 = p.indices[irow * p.BK + rs + bi];
+                    st = (s64 >= 0 && s64 < 0x7fffffffLL) ? (int)s64 : -0x40000000;
+                }
+                t = st + e;  // st is below 2^31 - 1 or the large negative marker: no overflow
+                if (!(t >= p.sink && t < tlimit)) t = -1;
                 if constexpr (ROPE)
-                    rpos = bsa_rope_far_pos(p.rope, (long long)(rs + bi + p.sink / p.bk) * p.bk + o % p.bk, rope_shift,
-                                            pmin_blk, p.sw);
+                    rpos = bsa_rope_far_pos(p.rope, (long long)(rs + bi + p.sink / p.bk) * p.bk + e, rope_shift, pmin_blk,
+                                            p.sw);
             }
         } else if (kind == 1) {
             if (o < sink_end) t = o;
@@ -226,8 +237,12 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
         if (t >= 0) kv_rows<true, EXT>(p.kv, kx, b, t, kvh, seqlen, ko, vo, true);
         m_ko = ko;
         m_vo = vo;
-        m_t = (int)t;
-        if constexpr (ROPE) m_rp = (int)(p.rope.row(rpos) / p.rope.stride_t);
+        m_t = t;
+        if constexpr (ROPE) m_rp = (int)p.rope.clamp(rpos);
+        // tile summary for the mask shortcut, once for the whole workgroup
+        m_tmin = wave_min_i(t < 0 ? 0x7fffffff : t);
+        m_tmax = wave_max_i(t);
+        m_allv = __all(t >= 0) ? 1 : 0;
     };
     auto post = [&](int tile) {  // wave 0 only
         MfmaMeta &mt = sm.meta[tile & 3];
@@ -235,6 +250,11 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
         mt.vo[lane] = m_vo;
         mt.tok[lane] = m_t;
         if constexpr (ROPE) mt.rp[lane] = m_rp;
+        if (lane == 0) {
+            mt.tmin = m_tmin;
+            mt.tmax = m_tmax;
+            mt.all_valid = m_allv;
+        }
     };
     uint4 kreg[CPT], vreg[CPT];
     uint4 creg[ROPE ? CPT : 1], sreg[ROPE ? CPT : 1];  // cos / sin pieces of the staged key rows
@@ -306,12 +326,9 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
         const MfmaMeta &mt = sm.meta[tile & 3];
         const bool window = tile >= tiles_sel + tiles_sink;
 
-        // tile summary (token range, all valid?) computed redundantly per wave
-        const int tk = mt.tok[lane];
-        int tmin = tk < 0 ? 0x7fffffff : tk, tmax = tk;
-        tmin = wave_min_i(tmin);
-        tmax = wave_max_i(tmax);
-        const bool all_valid = __all(tk >= 0);
+        // tile summary (token range, all valid?) posted by wave 0
+        const int tmin = mt.tmin, tmax = mt.tmax;
+        const bool all_valid = mt.all_valid != 0;
         bool full;  // every (valid row, token) pair of the tile is attended
         if (!window) full = all_valid && ((long long)tmax + p.sw <= pmin_blk);
         else full = all_valid && (tmax <= pmin_blk) && ((long long)pmax_blk < (long long)tmin + p.sw);
@@ -357,9 +374,9 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         const int t = ts[e];
-                        bool att;
-                        if (!window) att = (t >= 0) && ((long long)t + p.sw <= pq);
-                        else att = (t >= 0) && (t <= pq) && ((long long)pq < (long long)t + p.sw);
+                        // branch-free: far keys need t + sw <= pq, window keys t <= pq < t + sw
+                        const long long tsw = (long long)t + p.sw;
+                        const bool att = (t >= 0) & (window ? ((t <= pq) & ((long long)pq < tsw)) : (tsw <= (long long)pq));
                         const float s = att ? sacc[nb][i4 * 4 + e] : -INFINITY;
                         sacc[nb][i4 * 4 + e] = s;
                         mx = fmaxf(mx, s);

@@ -164,6 +164,7 @@ struct KVView {
     const void *cache_seq_lens;
     int64_t bt_stride_b;
     int bt_is64, sl_is64, paged, page_size, HKV;
+    int page_shift;  // log2(page_size): page sizes are powers of two
 
     __device__ __forceinline__ int64_t seq_len(int b) const {
         return sl_is64 ? reinterpret_cast<const int64_t *>(cache_seq_lens)[b]
@@ -172,7 +173,7 @@ struct KVView {
     __device__ __forceinline__ int64_t page_of(int b, int64_t t, int64_t seqlen) const {
         int64_t page = 0;
         if (t >= 0 && t < seqlen) {
-            int64_t i = (int64_t)b * bt_stride_b + t / page_size;
+            int64_t i = (int64_t)b * bt_stride_b + (t >> page_shift);
             page = bt_is64 ? reinterpret_cast<const int64_t *>(block_table)[i]
                            : (int64_t) reinterpret_cast<const int32_t *>(block_table)[i];
         }
@@ -185,7 +186,7 @@ struct KVView {
         }
         const int64_t page = page_of(b, t, seqlen);
         if (t < 0) return NO_ROW;
-        return page * k_stride_b + (t % page_size) * k_stride_t + (int64_t)h * k_stride_h;
+        return page * k_stride_b + (t & (page_size - 1)) * k_stride_t + (int64_t)h * k_stride_h;
     }
     __device__ __forceinline__ int64_t v_plain(int b, int64_t t, int h, int64_t seqlen) const {
         if (!paged) {
@@ -194,7 +195,7 @@ struct KVView {
         }
         const int64_t page = page_of(b, t, seqlen);
         if (t < 0) return NO_ROW;
-        return page * v_stride_b + (t % page_size) * v_stride_t + (int64_t)h * v_stride_h;
+        return page * v_stride_b + (t & (page_size - 1)) * v_stride_t + (int64_t)h * v_stride_h;
     }
 };
 
@@ -238,13 +239,13 @@ __device__ __forceinline__ void kv_rows(const KVView &kv, const KVExt *kx, int b
     }
     if (t < 0) return;
     const int64_t page = kv.page_of(b, t, seqlen);
-    const int64_t inpage = t % kv.page_size;
+    const int64_t inpage = t & (kv.page_size - 1);
     if constexpr (EXT) {
         if (kx->access_flags && leader)
             mark_flag<CHECK>(kx->access_flags + (int64_t)b * kx->flags_stride_b + (int64_t)h * kx->flags_stride_h + page);
         if (kx->cached) {
             const CacheView &c = kx->cache;
-            const int64_t row = page * kv.page_size + inpage;
+            const int64_t row = (page << kv.page_shift) + inpage;
             const int64_t e = (int64_t)h * c.n_blocks + (row >> c.shift);
             const int32_t slot = c.table[e];
             if (slot >= 0) {
@@ -285,9 +286,9 @@ struct RopeView {
     int64_t stride_t, len;
     int backend;  // HIPATTN_EXTEND_*
     int64_t k_side_delta;  // prescaled RELATIVE scan: offset of the position-1 copy of the keys
+    __device__ __forceinline__ int64_t clamp(int64_t pos) const { return pos < 0 ? 0 : (pos >= len ? len - 1 : pos); }
     __device__ __forceinline__ int64_t row(int64_t pos) const {  // element offset of the table row of a position
-        pos = pos < 0 ? 0 : (pos >= len ? len - 1 : pos);
-        return pos * stride_t;
+        return clamp(pos) * stride_t;
     }
 };
 
