@@ -383,7 +383,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
                     }
                 }
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32)) * LOG2E;
+        mx = fmaxf(mx, swap_halves(mx)) * LOG2E;
         // raise the reference point only when the maximum grew noticeably
         float m_use = m_run;
         float alpha = 1.0f;
@@ -435,7 +435,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
 
     // ---- epilogue: O^T[d, m] / l -> out[b, m, h, d]
     if (!head_ok) return;
-    const float l = l_run + __shfl_xor(l_run, 32);
+    const float l = l_run + swap_halves(l_run);
     if (!row_ok) return;
     const float inv = 1.0f / (l == 0.0f ? 1.0f : l);
     uint16_t *obase = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + myit * p.o_st;

@@ -357,6 +357,16 @@ __device__ __forceinline__ long long wave_min_ll(long long v) {
     return v;
 }
 
+// Value held by the lane 32 positions away (lane ^ 32): one v_permlane32_swap instead of a trip through LDS.
+// The instruction swaps the upper half of its first operand with the lower half of its second; fed the same
+// value twice it leaves (lower half everywhere, upper half everywhere), and each lane picks the half that is
+// not its own.
+__device__ __forceinline__ uint32_t swap_halves(uint32_t x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+    return (threadIdx.x & 32) ? r[0] : r[1];
+}
+__device__ __forceinline__ float swap_halves(float x) { return __uint_as_float(swap_halves(__float_as_uint(x))); }
+
 // XCD-aware remap: consecutive workgroup ids are dealt round-robin to the 8 XCDs (each with its
 // own L2), so give every XCD one contiguous range of logical work ids.
 __device__ __forceinline__ long long xcd_remap(long long bid, long long total) {
