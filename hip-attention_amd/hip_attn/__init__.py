@@ -13,6 +13,7 @@ from .config import HiPAttentionConfig, HiPAttentionPerLayerConfig
 from .refresh import HiPMaskRefreshState
 from .paged import forward_paged_hip
 from .offload import HiPOffloadCache
+from .memory_pool import HiPMetadataCachePool, cuda_graph_capture_configs
 
 hip_attention = hip_attention_12
 HiPAttentionArgs = HiPAttentionArgs12
@@ -34,4 +35,6 @@ __all__ = [
     "HiPMaskRefreshState",
     "forward_paged_hip",
     "HiPOffloadCache",
+    "HiPMetadataCachePool",
+    "cuda_graph_capture_configs",
 ]

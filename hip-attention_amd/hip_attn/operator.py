@@ -488,6 +488,10 @@ def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], 
         khat = None
     if not indices.is_contiguous():
         indices = indices.contiguous()
+    if ks_start_end.dtype != torch.int32:  # metadata kept in a HiPMetadataCachePool comes back as int64
+        ks_start_end = ks_start_end.to(torch.int32)
+    if indices.dtype != torch.int64:
+        indices = indices.to(torch.int64)
     if not ks_start_end.is_contiguous():
         ks_start_end = ks_start_end.contiguous()
     BK = indices.shape[-1]

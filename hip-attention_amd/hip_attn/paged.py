@@ -17,6 +17,8 @@ from .config import HiPAttentionConfig
 from .metadata import HiPAttentionArgs, HiPAttentionOutputMetadata
 from .operator import dual_stage_quadratic_hip_attention
 
+from .memory_pool import cuda_graph_capture_configs  # noqa: F401  (paged_hip.py:27-32 keeps it here)
+
 _LAST_DENSE = 64  # trailing prefill queries served with an (effectively) dense window, paged_hip.py:462
 
 

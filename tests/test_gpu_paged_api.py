@@ -139,3 +139,43 @@ def test_forward_paged_hip_decode_with_rope_applied_on_load():
         octx, ometa = O.hip_attention_12(XP, A)
         assert_metadata_equal(meta, ometa)
         assert_context_close(out.view(B, 1, H, D), octx, "bf16")
+
+
+def test_metadata_cache_pool_hands_masks_between_decode_steps():
+    """A mask stored in HiPMetadataCachePool after a refresh step drives the next steps (finished mask, or the
+    inputs of a later stage) exactly like the metadata object itself."""
+    from hip_attn import HiPAttentionArgs12, HiPAttentionConfig, HiPMetadataCachePool, hip_attention_12
+    from helpers import to_paged
+
+    print("[case] metadata cache pool", flush=True)
+    B, TK, H, HKV, D = 2, 16384, 8, 2, 128
+    lens = np.array([16384, 9000])
+    X = make_inputs(24, B=B, TQ=1, TK=TK, H=H, HKV=HKV, D=D, dtype="bf16", pos=(lens - 1)[:, None])
+    XP = to_paged(X, 16, seed=9, seq_lens=lens)
+    dev = "cuda"
+    cfg = HiPAttentionConfig()
+    pool = HiPMetadataCachePool(max_total_num_tokens=B * TK, query_head_num=H, layer_num=2, context_length=TK,
+                                device=dev, hip_config=cfg)
+    layer = pool.layer_configs[1]
+
+    def args():
+        return HiPAttentionArgs12(
+            k_cache=to_torch(XP.k_cache, "bf16", dev), v_cache=to_torch(XP.v_cache, "bf16", dev),
+            block_table=torch.from_numpy(XP.block_table).to(dev), cache_seq_lens=torch.from_numpy(XP.cache_seq_lens).to(dev),
+            position_ids=torch.from_numpy(XP.pos.copy()).to(dev), sliding_window_size=layer.sliding_window_size,
+            sink_token_size=layer.sink_token_size, second_stage_k=layer.second_stage_k, stages=layer.stages,
+            extend_context_length=TK)
+
+    q = to_torch(X.q, "bf16", dev)
+    out, meta = hip_attention_12(q, None, None, args())
+    pool.set_hip_metadata_cache(1, B, B, meta)
+    # finished mask out of the pool
+    cached = pool.get_hip_metadata_cache(1, B, B, None)
+    assert torch.equal(cached.ks, meta.ks)
+    out_c, _ = hip_attention_12(q, None, None, args(), cached_metadata=cached)
+    assert torch.equal(out_c, out)
+    # inputs of the last stage out of the pool: estimation resumes there and ends in the same mask
+    resumed = pool.get_hip_metadata_cache(1, B, B, len(layer.stages) - 1)
+    out_r, meta_r = hip_attention_12(q, None, None, args(), cached_metadata=resumed)
+    assert torch.equal(meta_r.indices, meta.indices) and torch.equal(meta_r.ks, meta.ks)
+    assert torch.equal(out_r, out)

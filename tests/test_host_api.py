@@ -91,3 +91,53 @@ def test_unsupported_options_fail_loudly():
                dict(online_update_cache=True), dict(sliding_window_indices=torch.zeros(1))):
         with pytest.raises(NotImplementedError):
             _reject_unsupported(HiPAttentionArgs12(**kw))
+
+
+def test_metadata_cache_pool_round_trip_on_cpu():
+    """HiPMetadataCachePool: storage formats, batch slicing and stage-level getters (hip_memory_pool.py:55-409)."""
+    import torch
+    from hip_attn import HiPAttentionConfig, HiPMetadataCachePool, cuda_graph_capture_configs
+    from hip_attn.metadata import HiPAttentionOutputMetadata, HiPAttentionStageInputCache
+
+    cfg = HiPAttentionConfig()
+    assert cuda_graph_capture_configs(cfg) == [(None,), (0,), (1,), (2,)]
+    H, B = 4, 3
+    pool = HiPMetadataCachePool(max_total_num_tokens=1 << 16, query_head_num=H, layer_num=2, context_length=1 << 17,
+                                device="cpu", hip_config=cfg)
+    lc = pool.layer_configs[1]
+    nblk = lc.second_stage_k // lc.stages[-1].stage_chunk_size
+    assert pool.cache[1]["indices"].buffer.dtype == torch.uint32
+    assert pool.cache[1]["indices"].buffer.shape == (cfg.metadata_cache_max_batch_size * H, 1, nblk)
+    assert pool.cache[1]["stage_1_out_scores"].buffer.dtype == torch.bfloat16
+    assert pool.compute_allocated_bytes() == pool.allocated_gpu_bytes > 0
+    g = torch.Generator().manual_seed(0)
+    idx = torch.randint(0, 1 << 20, (B * H, 1, nblk), generator=g, dtype=torch.int64).sort(-1).values
+    idx[:, :, -5:] = torch.iinfo(torch.int64).max  # padding entries wrap to 2^32 - 1 in storage
+    ks = torch.full((B * H, 1), nblk - 5, dtype=torch.int64)
+    kse = torch.zeros((B * H, 1, 2), dtype=torch.int32); kse[..., 1] = nblk - 5
+    stage = lambda n: HiPAttentionStageInputCache(
+        torch.randint(0, 1 << 20, (B, 1, H, n), generator=g), torch.randint(0, 1 << 20, (B, 1, H, n), generator=g),
+        torch.randn((B, 1, H, n), generator=g))
+    n1 = pool.cache[1]["stage_1_indices_left"].buffer.shape[-1]
+    n2 = pool.cache[1]["stage_2_indices_left"].buffer.shape[-1]
+    meta = HiPAttentionOutputMetadata(indices=idx, ks=ks, ks_count=ks.unsqueeze(-1), ks_start_end=kse,
+                                      mask_cache_statistics=None, sa_cache_statistics=None,
+                                      stage_caches=[HiPAttentionStageInputCache(None, None, None), stage(n1), stage(n2)])
+    pool.set_hip_metadata_cache(1, B, B, meta)
+    back = pool.get_hip_metadata_cache(1, B, B, None)
+    assert back.indices.dtype == torch.int64 and back.indices.shape == idx.shape
+    assert torch.equal(back.indices[:, :, :-5], idx[:, :, :-5]) and (back.indices[:, :, -5:] == 2 ** 32 - 1).all()
+    assert torch.equal(back.ks, ks) and torch.equal(back.ks_start_end, kse.to(torch.int64))
+    assert back.stage_caches is None
+    assert pool.get_hip_metadata_cache(1, B, B, 0) is None
+    part = pool.get_hip_metadata_cache(1, B, B, 2)
+    assert part.indices is None and len(part.stage_caches) == 3 and part.stage_caches[0].indices_left is None
+    assert torch.equal(part.stage_caches[2].indices_left, meta.stage_caches[2].indices_left)
+    assert torch.equal(part.stage_caches[1].out_scores, meta.stage_caches[1].out_scores.to(torch.bfloat16).float())
+    # a smaller batch reads a prefix; a larger one than the pool holds is refused
+    small = pool.get_hip_metadata_cache(1, 2, 2, None)
+    assert torch.equal(small.indices, back.indices[: 2 * H])
+    with pytest.raises(ValueError):
+        pool.get_buffer(1, "stage_1_indices_left", cfg.metadata_cache_max_batch_size + 1)
+    with pytest.raises(KeyError):
+        pool.get_buffer(1, "nope", 1)
