@@ -69,8 +69,13 @@ int make_kv_view(const hipattn_kv_t *kv, int B, int HID, int dtype, KVView *o, K
     (void)B;
     HIPATTN_CHECK_ARG(kv && kv->k, HIPATTN_E_ARG, "kv: null K pointer");
     HIPATTN_CHECK_ARG(kv->HKV > 0, HIPATTN_E_ARG, "kv: HKV <= 0");
-    const int esz = dtype == HIPATTN_BF16 ? 2 : 4;
-    const int64_t al = 16 / esz;
+    if (kv->fp8) {
+        HIPATTN_CHECK_ARG(dtype == HIPATTN_BF16 && kv->paged && !kv->cache, HIPATTN_E_UNSUPPORTED,
+                          "kv: fp8 storage needs a bf16 query, a paged cache and no offload cache");
+        HIPATTN_CHECK_ARG(HID % 32 == 0, HIPATTN_E_UNSUPPORTED, "kv: fp8 storage needs a head dim that is a multiple of 32");
+    }
+    const int esz = kv->fp8 ? 1 : (dtype == HIPATTN_BF16 ? 2 : 4);
+    const int64_t al = kv->fp8 ? 8 : 16 / esz;  // fp8 rows are fetched in 8-byte pieces
     const void *v = kv->v ? kv->v : kv->k;
     HIPATTN_CHECK_ARG(aligned16(kv->k) && aligned16(v) && kv->k_stride_b % al == 0 && kv->k_stride_t % al == 0 &&
                           kv->k_stride_h % al == 0 && kv->v_stride_b % al == 0 && kv->v_stride_t % al == 0 &&
@@ -101,6 +106,7 @@ int make_kv_view(const hipattn_kv_t *kv, int B, int HID, int dtype, KVView *o, K
     x->miss_flags = kv->miss_flags;
     x->flags_stride_b = kv->flags_stride_b;
     x->flags_stride_h = kv->flags_stride_h;
+    x->kv8 = kv->fp8 ? 1 : 0;
     if (kv->cache) return cache_view_for(kv->cache, kv, o, HID, dtype, x);
     return 0;
 }

@@ -20,9 +20,10 @@ using DecodeParams = DecodeParamsT<true>;
 // ROPE = true (extended parameter block only): query and keys are rotated on load; lanes dl and dl ^ 8 of a
 // 16-lane group hold the two halves of a row.
 // CAP = true (extended parameter block only): logits are soft-capped.
-template <typename T, int HID, int G, bool EXT, bool ROPE = false, bool CAP = false>
+// KV8 = true (extended parameter block only): K / V rows are fp8 (e5m2) bytes, widened on load.
+template <typename T, int HID, int G, bool EXT, bool ROPE = false, bool CAP = false, bool KV8 = false>
 __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<EXT> dp) {
-    static_assert((!ROPE && !CAP) || EXT, "rope / softcap variants take the extended parameter block");
+    static_assert((!ROPE && !CAP && !KV8) || EXT, "rope / softcap / fp8 variants take the extended parameter block");
     constexpr int SEG = HID / 16;
     const BsaParamsFor<EXT> &p = dp.a;
     const KVExt *kx = nullptr;
@@ -57,8 +58,8 @@ __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<E
     const long long o_end = o_begin + per < total ? o_begin + per : total;
 
     const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
-    const T *kbase = reinterpret_cast<const T *>(p.kv.k);
-    const T *vbase = reinterpret_cast<const T *>(p.kv.v);
+    const void *kbase = p.kv.k;
+    const void *vbase = p.kv.v;
 
     float qh[G][SEG];
 #pragma unroll
@@ -121,13 +122,13 @@ __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<E
         kv_rows<true, EXT>(p.kv, kx, b, t, kvh, seqlen, koff, voff, dl == 0);
         float kh[SEG], vv[SEG];
         if (koff != NO_ROW) {
-            load_elems<T, SEG>(kbase + koff + dl * SEG, kh);
+            load_kv_elems<T, SEG, KV8>(kbase, koff + dl * SEG, kh);
         } else {
 #pragma unroll
             for (int e = 0; e < SEG; e++) kh[e] = 0.0f;
         }
         if (voff != NO_ROW) {
-            load_elems<T, SEG>(vbase + voff + dl * SEG, vv);
+            load_kv_elems<T, SEG, KV8>(vbase, voff + dl * SEG, vv);
         } else {
 #pragma unroll
             for (int e = 0; e < SEG; e++) vv[e] = 0.0f;
@@ -247,7 +248,15 @@ static int launch_partial(const DecodeParams &dp, hipStream_t st) {
 #define DEC_CASE(GG)                                                                                   \
     if constexpr (GG * HID <= 512) {                                                                   \
         if (dp.a.G == GG) {                                                                            \
-            if (dp.a.softcap != 0.0f) {                                                                \
+            if (sizeof(T) == 2 && dp.a.kx.kv8) {                                                       \
+                if constexpr (sizeof(T) == 2) {                                                        \
+                    const bool r_ = dp.a.rope.cos != nullptr, c_ = dp.a.softcap != 0.0f;               \
+                    if (r_ && c_) hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG, true, true, true, true>), grid, block, 0, st, dp); \
+                    else if (r_) hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG, true, true, false, true>), grid, block, 0, st, dp); \
+                    else if (c_) hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG, true, false, true, true>), grid, block, 0, st, dp); \
+                    else hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG, true, false, false, true>), grid, block, 0, st, dp); \
+                }                                                                                      \
+            } else if (dp.a.softcap != 0.0f) {                                                         \
                 if (dp.a.rope.cos)                                                                     \
                     hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG, true, true, true>), grid, block, 0, st, dp); \
                 else                                                                                   \

@@ -70,10 +70,12 @@ struct MfmaSmem {
 // A query lane holds both halves of its row (k-steps ks and ks + KS/2); the two halves of a staged key row are
 // fetched by lanes tid and tid ^ (HID/16) of one wave.
 // CAP = true (extended parameter block): logits are soft-capped before the softmax.
-template <int HID, bool KSCALED, bool EXT, bool ROPE = false, bool CAP = false>
+// KV8 = true (extended parameter block): K / V rows are fp8 (e5m2) bytes, widened on load.
+template <int HID, bool KSCALED, bool EXT, bool ROPE = false, bool CAP = false, bool KV8 = false>
 __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p, int hgroups, int hpw, long long total_wg) {
     static_assert(!ROPE || (EXT && !KSCALED), "rope variant: extended parameter block, keys scaled in the kernel");
     static_assert(!CAP || EXT, "softcap variant: extended parameter block");
+    static_assert(!KV8 || (EXT && !KSCALED), "fp8 storage: extended parameter block, keys scaled in the kernel");
     const KVExt *kx = nullptr;
     if constexpr (EXT) kx = &p.kx;
     constexpr int KS = HID / 16;   // k-steps of the first product
@@ -189,8 +191,6 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
     __syncthreads();  // sm.idx visible
 
     const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
-    const uint16_t *kbase = reinterpret_cast<const uint16_t *>(p.kv.k);
-    const uint16_t *vbase = reinterpret_cast<const uint16_t *>(p.kv.v);
 
     // ---- staging.  Wave 0 walks the token list: lane = token slot of a tile; it resolves the token, its K / V row
     // offsets (page lookup, statistics, offload cache) and, with RoPE, its rotated position, one tile ahead of the
@@ -272,8 +272,8 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
                 creg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr);
                 sreg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr);
             }
-            if (ko != NO_ROW) kreg[j] = *reinterpret_cast<const uint4 *>(kbase + ko + piece * 8);
-            if (vo != NO_ROW) vreg[j] = *reinterpret_cast<const uint4 *>(vbase + vo + piece * 8);
+            if (ko != NO_ROW) kreg[j] = load_kv_piece<KV8>(p.kv.k, ko + piece * 8);
+            if (vo != NO_ROW) vreg[j] = load_kv_piece<KV8>(p.kv.v, vo + piece * 8);
         }
     };
     auto commit = [&](int buf) {
@@ -500,7 +500,7 @@ __global__ __launch_bounds__(256) void bsa_mark_kernel(BsaParams p, int hgroups,
     }
 }
 
-template <int HID, bool KSCALED, bool EXT, bool ROPE = false, bool CAP = false>
+template <int HID, bool KSCALED, bool EXT, bool ROPE = false, bool CAP = false, bool KV8 = false>
 static int launch_mfma(const BsaParams &p, hipStream_t st) {
     const int hpw = p.share_first_head ? 4 : 1;  // per-head index rows: one head per workgroup
     const int hgroups = (p.G + hpw - 1) / hpw;
@@ -509,12 +509,12 @@ static int launch_mfma(const BsaParams &p, hipStream_t st) {
     const size_t smem = sizeof(MfmaSmem<HID>);
     static bool attr_set = false;
     if (!attr_set) {
-        HIPATTN_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&bsa_mfma_kernel<HID, KSCALED, EXT, ROPE, CAP>),
+        HIPATTN_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&bsa_mfma_kernel<HID, KSCALED, EXT, ROPE, CAP, KV8>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
     const BsaParamsFor<EXT> &pk = p;  // the plain kernel takes the block without the extras
-    hipLaunchKernelGGL((bsa_mfma_kernel<HID, KSCALED, EXT, ROPE, CAP>), dim3((unsigned)total), dim3(NTHREADS), smem, st, pk, hgroups,
+    hipLaunchKernelGGL((bsa_mfma_kernel<HID, KSCALED, EXT, ROPE, CAP, KV8>), dim3((unsigned)total), dim3(NTHREADS), smem, st, pk, hgroups,
                        hpw, total);
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
@@ -526,7 +526,7 @@ int bsa_mfma_launch(const BsaParams &p, int dtype, int HID, hipStream_t st) {
     if ((p.o_st % 4) != 0 || (p.o_sh % 4) != 0 || (p.o_sb % 4) != 0) return HIPATTN_E_UNSUPPORTED;
     bool ext = p.kx.extended();
     BsaParams plain;
-    if (ext && !p.kx.cached && (HID == 64 || HID == 128)) {
+    if ((p.kx.access_flags || p.kx.miss_flags) && !p.kx.cached && (HID == 64 || HID == 128)) {
         // statistics only: a cheap marking pass, then the plain kernel
         const int hpw = p.share_first_head ? 4 : 1;
         const int hgroups = (p.G + hpw - 1) / hpw;
@@ -545,6 +545,14 @@ int bsa_mfma_launch(const BsaParams &p, int dtype, int HID, hipStream_t st) {
     }
 #define BSA_PICK(H)                                                                  \
     case H:                                                                          \
+        if (p.kx.kv8) {                                                              \
+            if (p.k_prescaled) return HIPATTN_E_UNSUPPORTED;                         \
+            if (p.softcap != 0.0f)                                                   \
+                return p.rope.cos ? launch_mfma<H, false, true, true, true, true>(p, st)   \
+                                  : launch_mfma<H, false, true, false, true, true>(p, st); \
+            return p.rope.cos ? launch_mfma<H, false, true, true, false, true>(p, st)      \
+                              : launch_mfma<H, false, true, false, false, true>(p, st);    \
+        }                                                                            \
         if (p.softcap != 0.0f) {                                                     \
             if (p.k_prescaled) return HIPATTN_E_UNSUPPORTED;                         \
             return p.rope.cos ? launch_mfma<H, false, true, true, true>(p, st)       \

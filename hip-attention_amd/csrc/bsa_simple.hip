@@ -10,7 +10,7 @@
 
 namespace hipattn {
 
-template <typename T, int HID, bool ROPE>
+template <typename T, int HID, bool ROPE, bool KV8 = false>
 __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
     constexpr int DPL = (HID + 63) / 64;  // output elements per lane
     constexpr int HALF = HID / 2;
@@ -50,8 +50,8 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
     const long long n_win = p.sw > 0 ? curr - ws : 0;
     const long long total = n_sel_tok + sink_end + n_win;
     const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
-    const T *kbase = reinterpret_cast<const T *>(p.kv.k);
-    const T *vbase = reinterpret_cast<const T *>(p.kv.v);
+    const void *kbase = p.kv.k;
+    const void *vbase = p.kv.v;
 
     for (int j = wid; j < p.bq; j += 4) {
         const long long it = (long long)qb * p.bq + j;
@@ -117,10 +117,10 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
                     constexpr int CH = 16 / (int)sizeof(T) < HID ? 16 / (int)sizeof(T) : HID;
                     for (int d0 = 0; d0 < HID; d0 += CH) {
                         float kk[CH];
-                        load_elems<T, CH>(kbase + koff + d0, kk);
+                        load_kv_elems<T, CH, KV8>(kbase, koff + d0, kk);
                         if constexpr (ROPE) {
                             float other[CH], rc[CH], rsn[CH];
-                            load_elems<T, CH>(kbase + koff + (d0 + HALF) % HID, other);
+                            load_kv_elems<T, CH, KV8>(kbase, koff + (d0 + HALF) % HID, other);
                             const int64_t tr = p.rope.row(rpos) + d0 % HALF;
                             load_elems<T, CH>(reinterpret_cast<const T *>(p.rope.cos) + tr, rc);
                             load_elems<T, CH>(reinterpret_cast<const T *>(p.rope.sin) + tr, rsn);
@@ -155,7 +155,7 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
 #pragma unroll
                         for (int e = 0; e < DPL; e++) {
                             const int d = lane + e * 64;
-                            if (d < HID) acc[e] = __fmaf_rn(pj, Elem<T>::widen(vbase[vo + d]), acc[e]);
+                            if (d < HID) acc[e] = __fmaf_rn(pj, load_kv_elem<T, KV8>(vbase, vo + d), acc[e]);
                         }
                     }
                 }
@@ -176,6 +176,14 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
 template <typename T, int HID>
 static int launch_simple(const BsaParams &p, hipStream_t stream) {
     dim3 grid((unsigned)p.NBQ, (unsigned)p.HEAD, (unsigned)p.B), block(256);
+    if constexpr (sizeof(T) == 2) {
+        if (p.kx.kv8) {
+            if (p.rope.cos) hipLaunchKernelGGL((bsa_simple_kernel<T, HID, true, true>), grid, block, 0, stream, p);
+            else hipLaunchKernelGGL((bsa_simple_kernel<T, HID, false, true>), grid, block, 0, stream, p);
+            HIPATTN_CHECK_HIP(hipGetLastError());
+            return 0;
+        }
+    }
     if (p.rope.cos) hipLaunchKernelGGL((bsa_simple_kernel<T, HID, true>), grid, block, 0, stream, p);
     else hipLaunchKernelGGL((bsa_simple_kernel<T, HID, false>), grid, block, 0, stream, p);
     HIPATTN_CHECK_HIP(hipGetLastError());

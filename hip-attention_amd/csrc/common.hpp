@@ -199,6 +199,67 @@ struct KVView {
     }
 };
 
+// ---------------------------------------------------------------- fp8 (e5m2) key/value storage
+// KV8 = true: K / V rows hold one byte per element (the uint8 view of a float8_e5m2 paged cache,
+// uvm_gpu_cache.py:1043-1046); every value is widened to bf16 on load, which is exact.  Offsets stay in elements.
+typedef __attribute__((ext_vector_type(2))) float kv_f32x2;
+
+// 8 consecutive elements as four packed bf16 pairs
+template <bool KV8>
+__device__ __forceinline__ uint4 load_kv_piece(const void *base, int64_t off) {
+    if constexpr (!KV8) {
+        return *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(base) + off);
+    } else {
+        const uint2 r = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint8_t *>(base) + off);
+        const kv_f32x2 a = __builtin_amdgcn_cvt_pk_f32_bf8((int)r.x, false), b = __builtin_amdgcn_cvt_pk_f32_bf8((int)r.x, true);
+        const kv_f32x2 c = __builtin_amdgcn_cvt_pk_f32_bf8((int)r.y, false), d = __builtin_amdgcn_cvt_pk_f32_bf8((int)r.y, true);
+        // widening is exact, so plain truncation packs the pairs
+        return make_uint4((__float_as_uint(a[0]) >> 16) | (__float_as_uint(a[1]) & 0xffff0000u),
+                          (__float_as_uint(b[0]) >> 16) | (__float_as_uint(b[1]) & 0xffff0000u),
+                          (__float_as_uint(c[0]) >> 16) | (__float_as_uint(c[1]) & 0xffff0000u),
+                          (__float_as_uint(d[0]) >> 16) | (__float_as_uint(d[1]) & 0xffff0000u));
+    }
+}
+
+// N consecutive elements widened to f32 (N in {2, 4, 8, 16} for fp8 storage)
+template <typename T, int N, bool KV8>
+__device__ __forceinline__ void load_kv_elems(const void *base, int64_t off, float (&out)[N]) {
+    if constexpr (!KV8) {
+        load_elems<T, N>(reinterpret_cast<const T *>(base) + off, out);
+    } else {
+        const uint8_t *p = reinterpret_cast<const uint8_t *>(base) + off;
+        if constexpr (N == 2) {
+            const kv_f32x2 a = __builtin_amdgcn_cvt_pk_f32_bf8((int)*reinterpret_cast<const uint16_t *>(p), false);
+            out[0] = a[0]; out[1] = a[1];
+        } else {
+            static_assert(N % 4 == 0, "fp8 row slices are whole dwords");
+            uint32_t w[N / 4];
+            if constexpr (N == 4) {
+                w[0] = *reinterpret_cast<const uint32_t *>(p);
+            } else if constexpr (N == 8) {
+                const uint2 r = *reinterpret_cast<const uint2 *>(p);
+                w[0] = r.x; w[1] = r.y;
+            } else {
+                static_assert(N == 16, "fp8 row slices hold 2, 4, 8 or 16 elements");
+                const uint4 r = *reinterpret_cast<const uint4 *>(p);
+                w[0] = r.x; w[1] = r.y; w[2] = r.z; w[3] = r.w;
+            }
+#pragma unroll
+            for (int i = 0; i < N / 4; i++) {
+                const kv_f32x2 a = __builtin_amdgcn_cvt_pk_f32_bf8((int)w[i], false), b = __builtin_amdgcn_cvt_pk_f32_bf8((int)w[i], true);
+                out[4 * i] = a[0]; out[4 * i + 1] = a[1]; out[4 * i + 2] = b[0]; out[4 * i + 3] = b[1];
+            }
+        }
+    }
+}
+
+// one element
+template <typename T, bool KV8>
+__device__ __forceinline__ float load_kv_elem(const void *base, int64_t off) {
+    if constexpr (!KV8) return Elem<T>::widen(reinterpret_cast<const T *>(base)[off]);
+    else return __builtin_amdgcn_cvt_f32_bf8((int)reinterpret_cast<const uint8_t *>(base)[off], 0);
+}
+
 // What only the extended builds of the kernels read: the offload cache and the statistics flags.  Kept out
 // of KVView (and at the end of the parameter blocks) so that the plain kernels' arguments stay small.
 struct KVExt {
@@ -206,8 +267,9 @@ struct KVExt {
     CacheView cache;
     int32_t *access_flags, *miss_flags;
     int64_t flags_stride_b, flags_stride_h;
+    int kv8;  // host: K / V are stored as fp8 (e5m2) bytes, kernels are launched in their KV8 builds
     // host: does a launch need the EXT build of its kernel
-    bool extended() const { return cached || access_flags || miss_flags; }
+    bool extended() const { return cached || access_flags || miss_flags || kv8; }
 };
 
 // Element offsets (from kv.k and kv.v) of the rows of token t, kv head h; NO_ROW = "zero row".

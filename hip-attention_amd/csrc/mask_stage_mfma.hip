@@ -62,9 +62,11 @@ __device__ __forceinline__ int64_t rope_kpos(const RopeView &r, int c, int side)
 // once and stay in registers.
 // RMODE = 2 (prescaled keys, extended parameter block): the keys were rotated and scaled ahead of the scan, one
 // copy per sample side; right-hand samples read the copy k_side_delta elements further on.
-template <int HID, int MB, int NB, bool PRESCALED, bool VIA_LDS, bool EXT, int RMODE = 0>
+// KV8 = true (extended parameter block, unscaled keys): key rows are fp8 (e5m2) bytes, widened on load.
+template <int HID, int MB, int NB, bool PRESCALED, bool VIA_LDS, bool EXT, int RMODE = 0, bool KV8 = false>
 __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     constexpr bool ROPE = RMODE == 1;
+    static_assert(!KV8 || (EXT && !PRESCALED), "fp8 keys: extended build, scaled in the kernel");
     static_assert(!ROPE || (EXT && !VIA_LDS && !PRESCALED), "rope variant: direct path of the extended build");
     static_assert(RMODE != 2 || (EXT && PRESCALED), "two-sided prescaled keys: extended build of the prescaled path");
     const KVExt *kx = nullptr;
@@ -202,7 +204,6 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
     (void)all_rows;
 
     const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
-    const uint16_t *kbase = reinterpret_cast<const uint16_t *>(p.kv.k);
 
     uint4 rcos[ROPE ? NB : 1][ROPE ? KS : 1], rsin[ROPE ? NB : 1][ROPE ? KS : 1];
     if constexpr (ROPE) {
@@ -243,7 +244,7 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
 #pragma unroll
                 for (int ks = 0; ks < KS; ks++) {
                     raw[tb][ks] = make_uint4(0, 0, 0, 0);
-                    if (off != NO_ROW) raw[tb][ks] = *reinterpret_cast<const uint4 *>(kbase + off + hh * HALF + ks * 8);
+                    if (off != NO_ROW) raw[tb][ks] = load_kv_piece<KV8>(p.kv.k, off + hh * HALF + ks * 8);
                 }
             }
         }
@@ -256,7 +257,7 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
                 const int64_t off = s_off[r];
                 const int q = lpos ^ ((r / SWZ_DIV) & SWZ);
                 uint4 v = make_uint4(0, 0, 0, 0);
-                if (off != NO_ROW) v = *reinterpret_cast<const uint4 *>(kbase + off + q * 8);
+                if (off != NO_ROW) v = load_kv_piece<KV8>(p.kv.k, off + q * 8);
                 if (!PRESCALED) {
                     v.x = scale_pack(v.x, p.c_k);
                     v.y = scale_pack(v.y, p.c_k);
@@ -446,6 +447,13 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
 #define MS_LAUNCH(MBv, NBv, PSv, VLv)                                                                                 \
     do {                                                                                                              \
         constexpr bool EXT_BUILT = !(VLv) || (NBv) == 1;                                                              \
+        if constexpr (!(PSv) && EXT_BUILT) {                                                                          \
+            if (p.kx.kv8) {                                                                                           \
+                hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, NBv, false, VLv, true, 0, true>), grid, block, 0, st, \
+                                   p, nsub, hpw);                                                                     \
+                break;                                                                                                \
+            }                                                                                                         \
+        }                                                                                                             \
         if constexpr ((PSv) && EXT_BUILT) {                                                                           \
             if (two_sided) {                                                                                          \
                 hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, NBv, true, VLv, true, 2>), grid, block, 0, st, p, \
@@ -464,7 +472,14 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
         if (prescaled) { if (via_lds) MS_LAUNCH(MBv, NBv, true, true); else MS_LAUNCH(MBv, NBv, true, false); } \
         else { if (via_lds) MS_LAUNCH(MBv, NBv, false, true); else MS_LAUNCH(MBv, NBv, false, false); }        \
     } while (0)
-    if (rope) {
+    if (p.kx.kv8 && prescaled) {
+        set_error("mask stage: prescaled keys cannot be combined with fp8 key storage");
+        return HIPATTN_E_ARG;
+    }
+    if (rope && p.kx.kv8) {
+        if (two) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 2, 1, false, false, true, 1, true>), grid, block, 0, st, p, nsub, hpw);
+        else hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, false, false, true, 1, true>), grid, block, 0, st, p, nsub, hpw);
+    } else if (rope) {
         if (two) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 2, 1, false, false, true, 1>), grid, block, 0, st, p, nsub, hpw);
         else hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, false, false, true, 1>), grid, block, 0, st, p, nsub, hpw);
     } else if (two) { if (nb == 2) MS_PICK(2, 2); else MS_PICK(2, 1); }

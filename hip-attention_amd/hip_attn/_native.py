@@ -62,7 +62,11 @@ class KVStruct(ctypes.Structure):
         ("cache", ctypes.c_void_p),
         ("access_flags", ctypes.c_void_p), ("miss_flags", ctypes.c_void_p),
         ("flags_stride_b", ctypes.c_int64), ("flags_stride_h", ctypes.c_int64),
+        ("fp8", ctypes.c_int32),
     ]
+
+
+_FP8_DTYPES = (torch.uint8, torch.float8_e5m2)  # a float8_e5m2 cache, or its uint8 view (paged_hip.py:409-418)
 
 
 class CacheDesc(ctypes.Structure):
@@ -218,6 +222,12 @@ def make_kv_paged(k_cache, v_cache, block_table, cache_seq_lens, max_tsrc: int) 
     s.paged = 1
     s.page_size = k_cache.shape[1]
     s.HKV = k_cache.shape[2]
+    if k_cache.dtype in _FP8_DTYPES:
+        if v_cache.dtype not in _FP8_DTYPES:
+            raise HipAttnError("k_cache is fp8 but v_cache is not")
+        s.fp8 = 1
+    elif k_cache.dtype == torch.float8_e4m3fn:
+        raise NotImplementedError("fp8 KV caches are read as e5m2 (as the reference does); e4m3 is not built")
     return s
 
 

@@ -108,6 +108,11 @@ typedef struct hipattn_kv {
     int32_t *access_flags;
     int32_t *miss_flags;
     int64_t flags_stride_b, flags_stride_h;
+    /* fp8 != 0: k and v hold one byte per element, the uint8 view of a float8_e5m2 paged cache
+     * (src/hip_attn/v1_2/paged_hip.py:409-418, src/hip_attn/v1_2/uvm_gpu_cache.py:1043-1046); every loaded value is
+     * widened to bf16 (exact).  Needs paged != 0, a bf16 q, no offload cache; strides stay in elements (= bytes) and
+     * must be multiples of 8. */
+    int32_t fp8;
 } hipattn_kv_t;
 
 const char *hipattn_version(void);
