@@ -526,7 +526,7 @@ int bsa_mfma_launch(const BsaParams &p, int dtype, int HID, hipStream_t st) {
     if ((p.o_st % 4) != 0 || (p.o_sh % 4) != 0 || (p.o_sb % 4) != 0) return HIPATTN_E_UNSUPPORTED;
     bool ext = p.kx.extended();
     BsaParams plain;
-    if ((p.kx.access_flags || p.kx.miss_flags) && !p.kx.cached && (HID == 64 || HID == 128)) {
+    if ((p.kx.access_flags || p.kx.miss_flags) && !p.kx.cached && (HID == 64 || HID == 128 || HID == 256)) {
         // statistics only: a cheap marking pass, then the plain kernel
         const int hpw = p.share_first_head ? 4 : 1;
         const int hgroups = (p.G + hpw - 1) / hpw;
@@ -564,6 +564,7 @@ int bsa_mfma_launch(const BsaParams &p, int dtype, int HID, hipStream_t st) {
     switch (HID) {
         BSA_PICK(64)
         BSA_PICK(128)
+        BSA_PICK(256)
     }
 #undef BSA_PICK
     return HIPATTN_E_UNSUPPORTED;

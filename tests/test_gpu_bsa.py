@@ -32,7 +32,7 @@ def _run(X, max_tsrc, idx, kse, bq, bk, sw, sink, impl, share=False, decode=Fals
     return out
 
 
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [64, 128, 256])
 @pytest.mark.parametrize("bq,TQ,bk", [(64, 200, 8), (32, 96, 2), (16, 40, 16)])
 @pytest.mark.parametrize("paged", [False, True])
 def test_tile_kernel_matches_oracle_and_portable_kernel(D, bq, TQ, bk, paged):

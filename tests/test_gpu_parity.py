@@ -162,3 +162,13 @@ def test_operator_with_logit_softcap():
     assert_context_close(ctx, octx, "bf16")
     plain, _ = O.hip_attention_12(X, tiny_args())
     assert np.abs(O.bf16_bits_to_f32(plain) - O.bf16_bits_to_f32(octx)).max() > 0.05
+
+
+def test_head_dim_256_with_softcap_like_gemma2():
+    _case("operator D=256 softcap")
+    X = make_inputs(45, B=1, TQ=160, TK=2048, H=4, HKV=2, D=256, dtype="bf16", scale=0.7)
+    A = tiny_args(logit_softcap=50.0, block_size_k=32)
+    octx, ometa = O.hip_attention_12(X, A)
+    ctx, meta = run_product(X, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, "bf16")

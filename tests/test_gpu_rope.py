@@ -84,7 +84,7 @@ def _run_bsa(X, max_tsrc, idx, kse, bq, bk, sw, sink, impl, backend, share=True,
 
 
 @pytest.mark.parametrize("backend", ["streaming", "infllm"])
-@pytest.mark.parametrize("D,bq,TQ,bk", [(64, 64, 200, 8), (128, 32, 96, 2), (128, 16, 40, 16)])
+@pytest.mark.parametrize("D,bq,TQ,bk", [(64, 64, 200, 8), (128, 32, 96, 2), (128, 16, 40, 16), (256, 64, 100, 8)])
 def test_attention_kernels_with_rope_given_indices(backend, D, bq, TQ, bk):
     print(f"[case] rope bsa {backend} D={D} bq={bq} TQ={TQ} bk={bk}", flush=True)
     rng = np.random.default_rng(D + bq + bk)
