@@ -455,6 +455,21 @@ __global__ void pool_write_rows_kernel(char *pool, int64_t stride_row_b, int64_t
         *reinterpret_cast<const uint4 *>(src + (i * HKV + h) * (int64_t)row_bytes + piece * 16);
 }
 
+// gather: dst[i, h, :] = pool[rows[i], h, :]; rows below zero give zero rows
+__global__ void pool_read_rows_kernel(const char *pool, int64_t stride_row_b, int64_t stride_h_b, int HKV, int row_bytes,
+                                      const int64_t *rows, int64_t n, char *dst, int64_t dst_row_b) {
+    const int pieces = row_bytes / 16;
+    const int64_t w = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (w >= n * HKV * pieces) return;
+    const int piece = (int)(w % pieces);
+    const int h = (int)((w / pieces) % HKV);
+    const int64_t i = w / ((int64_t)pieces * HKV);
+    const int64_t row = rows[i];
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (row >= 0) v = *reinterpret_cast<const uint4 *>(pool + row * stride_row_b + h * stride_h_b + piece * 16);
+    *reinterpret_cast<uint4 *>(dst + i * dst_row_b + (int64_t)h * row_bytes + piece * 16) = v;
+}
+
 static int tiles_of(int64_t n) { return (int)((n + CT_TILE - 1) / CT_TILE); }
 
 static int check_desc(const hipattn_cache_desc_t *d, int64_t max_fetch, int *shift_out) {
@@ -679,6 +694,27 @@ extern "C" int hipattn_pool_write_rows(void *pool, int64_t stride_row, int64_t s
     HIPATTN_CHECK_ARG(blocks < 0x7fffffffLL, HIPATTN_E_UNSUPPORTED, "pool write: too many rows");
     hipLaunchKernelGGL(pool_write_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (char *)pool,
                        stride_row * esz, stride_h * esz, HKV, HID * esz, rows, n, (const char *)src);
+    HIPATTN_CHECK_HIP(hipGetLastError());
+    return 0;
+}
+
+extern "C" int hipattn_pool_read_rows(const void *pool, int64_t stride_row, int64_t stride_h, int32_t HKV, int32_t HID,
+                                      int32_t dtype, const int64_t *rows, int64_t n, void *dst, int64_t dst_stride_row,
+                                      void *stream) {
+    if (n == 0) return 0;
+    HIPATTN_CHECK_ARG(pool && rows && dst && n > 0 && HKV > 0 && HID > 0, HIPATTN_E_ARG, "pool read: bad argument");
+    HIPATTN_CHECK_ARG(dtype == HIPATTN_F32 || dtype == HIPATTN_BF16, HIPATTN_E_UNSUPPORTED, "pool read: dtype %d", dtype);
+    const int esz = dtype == HIPATTN_BF16 ? 2 : 4;
+    HIPATTN_CHECK_ARG(aligned16(pool) && aligned16(dst) && (stride_row * esz) % 16 == 0 && (stride_h * esz) % 16 == 0 &&
+                          (dst_stride_row * esz) % 16 == 0 && ((int64_t)HID * esz) % 16 == 0 &&
+                          dst_stride_row >= (int64_t)HKV * HID,
+                      HIPATTN_E_ALIGN, "pool read: rows must be whole, aligned 16-byte packs");
+    const int64_t total = n * HKV * ((int64_t)HID * esz / 16);
+    const int64_t blocks = (total + 255) / 256;
+    HIPATTN_CHECK_ARG(blocks < 0x7fffffffLL, HIPATTN_E_UNSUPPORTED, "pool read: too many rows");
+    hipLaunchKernelGGL(pool_read_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const char *)pool, stride_row * esz, stride_h * esz, HKV, HID * esz, rows, n, (char *)dst,
+                       dst_stride_row * esz);
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
 }

@@ -14,6 +14,7 @@ from .refresh import HiPMaskRefreshState
 from .paged import forward_paged_hip
 from .offload import HiPOffloadCache
 from .memory_pool import HiPMetadataCachePool, cuda_graph_capture_configs
+from .model_offload import HiPModelOffloadCache
 
 hip_attention = hip_attention_12
 HiPAttentionArgs = HiPAttentionArgs12
@@ -36,5 +37,6 @@ __all__ = [
     "forward_paged_hip",
     "HiPOffloadCache",
     "HiPMetadataCachePool",
+    "HiPModelOffloadCache",
     "cuda_graph_capture_configs",
 ]

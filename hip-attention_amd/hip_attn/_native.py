@@ -462,6 +462,18 @@ def cache_stats(handle: int, device) -> list:
     return list(out)
 
 
+def pool_read_rows(pool_ptr: int, stride_row: int, stride_h: int, HKV: int, HID: int, dtype: int,
+                   rows: torch.Tensor, dst: torch.Tensor, device):
+    """Gather rows of the pinned host pool into device ``dst [>= n, HKV, HID]`` (first ``n = rows.numel()`` rows)."""
+    assert rows.dtype == torch.int64 and rows.is_cuda and rows.is_contiguous() and dst.is_cuda
+    assert dst.ndim == 3 and dst.stride(2) == 1 and dst.stride(1) == HID and dst.shape[0] >= rows.numel()
+    check(lib().hipattn_pool_read_rows(ctypes.c_void_p(pool_ptr), ctypes.c_int64(stride_row), ctypes.c_int64(stride_h),
+                                       ctypes.c_int32(HKV), ctypes.c_int32(HID), ctypes.c_int32(dtype), _p(rows),
+                                       ctypes.c_int64(rows.numel()), _p(dst), ctypes.c_int64(dst.stride(0)),
+                                       stream_ptr(device)),
+          "hipattn_pool_read_rows")
+
+
 def pool_write_rows(pool_ptr: int, stride_row: int, stride_h: int, HKV: int, HID: int, dtype: int,
                     rows: torch.Tensor, src: torch.Tensor, device):
     """Scatter device rows ``src [n, HKV, HID]`` into the pinned host pool at ``rows``."""

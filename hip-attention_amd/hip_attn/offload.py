@@ -41,6 +41,8 @@ class UVMCache:
         self.device_ptr = N.host_device_pointer(self.bank_cpu)
         # per-token generation, bumped on every overwrite (uvm_gpu_cache.py:109-114,681-688)
         self.metadata = torch.zeros((max_token_size, 1), dtype=torch.int32, device=self.device)
+        self.allocated_cpu_bytes = self.bank_cpu.numel() * self.bank_cpu.element_size()
+        self.allocated_gpu_bytes = self.metadata.numel() * self.metadata.element_size()
 
     def gather_cpu(self, table: Tensor, pin_memory: bool = False) -> Tensor:
         out = torch.empty((table.numel(), self.head_num, self.head_dim), dtype=self.dtype, pin_memory=pin_memory)
@@ -91,6 +93,8 @@ class GPUCache:
         self._desc = d
         self.handle = N.cache_create(d, self.max_fetch, dev)
         self._ready: Optional[torch.cuda.Event] = None
+        self.allocated_gpu_bytes = sum(t.numel() * t.element_size() for t in (
+            self.bank, self.table, self.last_use, self.backref, self.miss, self.workspace))
 
     def __del__(self):
         h, self.handle = getattr(self, "handle", 0), 0
@@ -163,6 +167,8 @@ class HiPOffloadCache:
         self.sa_kv_cache = GPUCache(self.k_uvm, self.v_uvm, max_sa_cache_token_size, online_cache_update,
                                     block_tokens=block_tokens, max_fetch=max_fetch)
         self.miss_stream: Optional[torch.cuda.Stream] = None
+        # event of a store into the pools that was issued on another stream; readers wait for it
+        self.pending_write: Optional[torch.cuda.Event] = None
 
     def get_page_count(self) -> int:
         assert self.k_uvm.bank_cpu.shape == self.v_uvm.bank_cpu.shape
@@ -173,6 +179,8 @@ class HiPOffloadCache:
         """Paged (page size 1) description of the host pools with the cache that serves this phase."""
         cache = self.mask_k_cache if masking else self.sa_kv_cache
         cache.wait()
+        if self.pending_write is not None:
+            torch.cuda.current_stream(self.device).wait_event(self.pending_write)
         kb, vb = self.k_uvm.bank_cpu, self.v_uvm.bank_cpu
         s = N.KVStruct()
         s.k, s.v = self.k_uvm.device_ptr, self.v_uvm.device_ptr
@@ -194,11 +202,21 @@ class HiPOffloadCache:
     # ------------------------------------------------------------------ reference methods
     def prefetch_prefix_kv_buffer(self, table: Tensor, device: torch.device) -> Tuple[Tensor, Tensor]:
         """Dense device copies ``[1, n, head, dim]`` of the pool rows listed in ``table``."""
-        if table.device != torch.device("cpu"):
-            table = table.to("cpu", non_blocking=False)
-        k = self.k_uvm.gather_cpu(table, pin_memory=True).to(device, non_blocking=False).unsqueeze(0)
-        v = self.v_uvm.gather_cpu(table, pin_memory=True).to(device, non_blocking=False).unsqueeze(0)
-        return k, v
+        k, v = self.gather_rows(table, extra_rows=0)
+        return k.unsqueeze(0), v.unsqueeze(0)
+
+    def gather_rows(self, table: Tensor, extra_rows: int = 0) -> Tuple[Tensor, Tensor]:
+        """Device tensors ``[n + extra_rows, head, dim]`` whose first ``n`` rows are the pool rows listed in ``table``;
+        the device reads the pinned pools in place on the current stream (nothing blocks the host)."""
+        rows = table.reshape(-1).to(self.device, dtype=torch.int64).contiguous()
+        n = rows.numel()
+        out = []
+        for pool in (self.k_uvm, self.v_uvm):
+            dst = torch.empty((n + extra_rows, self.head_kv, self.head_dim), dtype=pool.bank_cpu.dtype, device=self.device)
+            N.pool_read_rows(pool.device_ptr, pool.bank_cpu.stride(0), pool.bank_cpu.stride(1), self.head_kv,
+                             self.head_dim, N.dtype_code(pool.bank_cpu), rows, dst, self.device)
+            out.append(dst)
+        return out[0], out[1]
 
     def set_kv_buffer(self, table: Tensor, table_gpu: Tensor, cache_k: Tensor, cache_v: Tensor):
         """Store rows into the host pools and keep resident cache blocks current."""

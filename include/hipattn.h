@@ -281,6 +281,13 @@ int hipattn_cache_write_rows(hipattn_cache_t *cache, const int64_t *rows, int64_
  * store of HiPOffloadCache.set_kv_buffer (src/hip_attn/v1_2/uvm_gpu_cache.py:665-668). */
 int hipattn_pool_write_rows(void *pool, int64_t stride_row, int64_t stride_h, int32_t HKV, int32_t HID,
                             int32_t dtype, const int64_t *rows, int64_t n, const void *src, void *stream);
+/* The gather in the other direction: dst[i, h, :] = pool[rows[i], h, :] for int64 rows[n] (negative: zero row); dst is
+ * device memory [n, HKV, HID] with dst_stride_row elements between rows.  The device reads the pinned pool in place, on
+ * `stream` -- the copy half of HiPOffloadCache.prefetch_prefix_kv_buffer (src/hip_attn/v1_2/uvm_gpu_cache.py:690-700),
+ * which the reference does with a host gather and a blocking upload. */
+int hipattn_pool_read_rows(const void *pool, int64_t stride_row, int64_t stride_h, int32_t HKV, int32_t HID,
+                           int32_t dtype, const int64_t *rows, int64_t n, void *dst, int64_t dst_stride_row,
+                           void *stream);
 /* Pinned host memory for a pool.  coherent != 0 asks for memory the GPU never caches, so that rows the CPU
  * writes are seen by the next kernel without any cache maintenance; pools written by the CPU need it. */
 int hipattn_host_alloc(int64_t bytes, int32_t coherent, void **host_out);

@@ -223,3 +223,56 @@ def test_offload_write_through_and_side_stream():
     ctx2, meta2 = hip_attention_12(q, None, None, _args(XP, A, offload_cache=cache))
     assert torch.equal(_bits(ctx2), _bits(ctx_res))
     assert torch.equal(meta2.sa_cache_statistics.cache_miss_counter, meta2.sa_cache_statistics.access_counter)
+
+
+def test_model_level_manager_prefetches_prefixes_and_orders_async_stores():
+    """HiPModelOffloadCache: per-layer pools, stores on a side stream, the next layer's prefix gathered by the device
+    from the pinned pool while the current layer runs (model_offload_cache.py:229-452)."""
+    from hip_attn import HiPAttentionArgs12, HiPAttentionConfig, HiPModelOffloadCache, hip_attention_12
+
+    print("[case] model-level offload manager", flush=True)
+    dev = torch.device("cuda", 0)
+    L, HKV, H, D, T = 3, 2, 4, 64, 4096
+    cfg = HiPAttentionConfig()
+    mgr = HiPModelOffloadCache(max_token_size=T + 64, max_mask_cache_token_size=2048, max_sa_cache_token_size=2048,
+                               dtype=torch.bfloat16, head_num=HKV, head_dim=D, layer_num=L, device=dev, hip_config=cfg)
+    host, gpu = mgr._calc_allocated_bytes()
+    assert host == L * 2 * (T + 65) * HKV * D * 2 and gpu > 0
+    g = torch.Generator().manual_seed(5)
+    perm = (torch.randperm(T + 60, generator=g)[:T] + 1).to(dev)  # pool rows of the sequence, row 0 left alone
+    ks = [torch.randn((T, HKV, D), generator=g).to(torch.bfloat16).to(dev) for _ in range(L)]
+    vs = [torch.randn((T, HKV, D), generator=g).to(torch.bfloat16).to(dev) for _ in range(L)]
+    prefix, fresh = 3072, 1024
+    for layer in range(L):  # the prefix was stored by earlier chunks; one layer asynchronously
+        mgr.set_kv_buffer(layer, perm[:prefix], ks[layer][:prefix], vs[layer][:prefix], async_copy=(layer == 1))
+    req_to_token = torch.zeros((2, T), dtype=torch.int64, device=dev)
+    req_to_token[1] = perm
+    pool_idx = torch.tensor([1], device=dev)
+    hooks = dict(batch_size=1, req_to_token=req_to_token, req_pool_indices=pool_idx,
+                 extend_prefix_lens_cpu=np.array([prefix]), extend_seq_lens_cpu=np.array([fresh]))
+    mgr.on_model_start(True, **hooks)
+    for layer in range(L):
+        mgr.on_layer_start(layer, True, **hooks)
+        new_k, new_v = ks[layer][None, prefix:], vs[layer][None, prefix:]
+        k, v, extra = mgr.get_fetched_prefix_kv_buffer(layer, 0, new_k, new_v)
+        assert extra is None and k.shape == (1, T, HKV, D)
+        assert torch.equal(k[0], ks[layer]) and torch.equal(v[0], vs[layer])
+        mgr.set_kv_buffer(layer, perm[prefix:], new_k[0], new_v[0], async_copy=True)
+        mgr.on_layer_end(layer, True)
+    mgr.on_model_end(True)
+    # decode against the offloaded layer 1 equals decode against the same rows held densely
+    cache, _ = mgr.get_kv_buffer(1)
+    q = torch.randn((1, 1, H, D), generator=g).to(torch.bfloat16).to(dev)
+    common = dict(sliding_window_size=256, sink_token_size=16, second_stage_k=512,
+                  position_ids=torch.tensor([[T - 1]], device=dev))
+    from hip_attn import ScanStage12
+    stages = [ScanStage12(stage_block_size_q=32, stage_block_stride_q=2, stage_chunk_size=64, stage_k=None, stage_stride=1),
+              ScanStage12(stage_block_size_q=32, stage_block_stride_q=2, stage_chunk_size=16, stage_k=2048, stage_stride=1),
+              ScanStage12(stage_block_size_q=32, stage_block_stride_q=1, stage_chunk_size=2, stage_k=1024, stage_stride=1)]
+    off_args = HiPAttentionArgs12(offload_cache=cache, block_table=perm[None].contiguous(),
+                                  cache_seq_lens=torch.tensor([T], device=dev), extend_context_length=T, stages=stages,
+                                  **common)
+    out_off, meta_off = hip_attention_12(q, None, None, off_args)
+    out_res, meta_res = hip_attention_12(q, ks[1][None], vs[1][None], HiPAttentionArgs12(stages=stages, **common))
+    assert torch.equal(meta_off.indices, meta_res.indices)
+    assert torch.equal(out_off, out_res)
