@@ -45,6 +45,37 @@ __device__ __forceinline__ int64_t bsa_rope_far_pos(const RopeView &r, long long
     return v < 0 ? 0 : v;
 }
 
+// ---------------------------------------------------------------- pieces shared by the matrix-core attention kernels
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+constexpr int KPAD = 8;       // bf16 elements of row padding for a K^ tile in LDS
+constexpr int VPAD = 32;      // bf16 elements of row padding for a V tile: four consecutive rows tile all banks
+constexpr float LOG2E = 1.44269504f;
+constexpr float RESCALE_STEP = 8.0f;  // raise the running max only when it grows by more than this (log2 units)
+
+__device__ __forceinline__ uint32_t cvt_pk_bf16(float a, float b) {  // one v_cvt_pk_bf16_f32
+    f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+
+// Transposing LDS read (ds_read_b64_tr_b16): lane l of a 16-lane group receives column l % 4 of the four 8-byte rows
+// addressed by lanes l / 4, l / 4 + 4, l / 4 + 8, l / 4 + 12 of its group.
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+__device__ __forceinline__ uint2 lds_read_tr16(const uint16_t *p) {
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p);
+    return __builtin_bit_cast(uint2, v);
+}
+
+union Frag {
+    bf16x8 v;
+    uint32_t u[4];
+    uint2 d[2];
+    uint4 q;
+};
+
 template <bool EXT>
 using BsaParamsFor = std::conditional_t<EXT, BsaParams, BsaParamsBase>;
 
@@ -55,5 +86,7 @@ int bsa_fill_params(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t 
 int bsa_simple_launch(const BsaParams &p, int dtype, int HID, hipStream_t st);
 // returns HIPATTN_E_UNSUPPORTED (without setting an error) when the tile kernel does not cover the case
 int bsa_mfma_launch(const BsaParams &p, int dtype, int HID, hipStream_t st);
+// decode partials on the matrix cores; HIPATTN_E_UNSUPPORTED (no error text) when the case is not covered
+int bsa_decode_mfma_launch(const BsaParams &p, int dtype, int HID, int nsplits, float *ws, hipStream_t st);
 
 }  // namespace hipattn

@@ -5,6 +5,8 @@
 // contiguous elements each: one coalesced 16-lane load per row, four rows per load instruction per
 // wave); each 16-lane group keeps its own online-softmax state and output slice, and the sixteen
 // states of a workgroup are merged through LDS before the partial is written.
+#include <stdlib.h>
+
 #include "bsa.hpp"
 
 namespace hipattn {
@@ -319,6 +321,19 @@ extern "C" int hipattn_bsa_decode_partial(const hipattn_q_t *q, const hipattn_kv
     dp.nsplits = nsplits;
     dp.ws = reinterpret_cast<float *>(workspace);
     hipStream_t st = (hipStream_t)stream;
+    {
+        // matrix-core kernel where it applies (bf16, head dim 64 / 128, groups of up to 8 heads);
+        // HIPATTN_DECODE_IMPL=1 keeps the vector-unit kernel (tuning and cross-checking aid)
+        static int impl = -1;
+        if (impl < 0) {
+            const char *e = getenv("HIPATTN_DECODE_IMPL");
+            impl = e ? atoi(e) : 0;
+        }
+        if (impl != 1) {
+            rc = bsa_decode_mfma_launch(dp.a, q->dtype, q->HID, nsplits, dp.ws, st);
+            if (rc != HIPATTN_E_UNSUPPORTED) return rc;
+        }
+    }
     if (q->dtype == HIPATTN_BF16) {
         switch (q->HID) {
             case 32: return launch_partial<bf16_t, 32>(dp, st);

@@ -18,36 +18,9 @@
 
 namespace hipattn {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-typedef __attribute__((ext_vector_type(2))) float f32x2;
-typedef __attribute__((ext_vector_type(16))) float f32x16;
-
 constexpr int TN = 64;        // tokens per tile
-constexpr int KPAD = 8;       // bf16 elements of row padding for the K^ tile
-constexpr int VPAD = 32;      // bf16 elements of row padding for the V tile: four consecutive rows tile all banks
 constexpr int NTHREADS = 512;
 constexpr int MAX_LDS_IDX = 1024;  // selected-block starts kept in LDS
-constexpr float LOG2E = 1.44269504f;
-constexpr float RESCALE_STEP = 8.0f;  // raise the running max only when it grows by more than this (log2 units)
-
-__device__ __forceinline__ uint32_t cvt_pk_bf16(float a, float b) {  // one v_cvt_pk_bf16_f32
-    f32x2 v = {a, b};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
-}
-
-typedef __attribute__((ext_vector_type(4))) short s16x4;
-__device__ __forceinline__ uint2 lds_read_tr16(const uint16_t *p) {  // ds_read_b64_tr_b16
-    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p);
-    return __builtin_bit_cast(uint2, v);
-}
-
-union Frag {
-    bf16x8 v;
-    uint32_t u[4];
-    uint2 d[2];
-    uint4 q;
-};
 
 // what wave 0 posts about the 64 token slots of a tile
 struct MfmaMeta {
