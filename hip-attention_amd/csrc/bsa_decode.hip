@@ -299,7 +299,7 @@ extern "C" int64_t hipattn_bsa_decode_workspace_bytes(int32_t B, int32_t HEAD, i
 extern "C" int32_t hipattn_bsa_decode_default_splits(int32_t B, int32_t HKV, int32_t tokens) {
     if (B <= 0 || HKV <= 0) return 1;
     int64_t groups = (int64_t)B * HKV;
-    int64_t s = (1024 + groups - 1) / groups;  // aim at ~4 workgroups per compute unit
+    int64_t s = (512 + groups - 1) / groups;  // two workgroups per compute unit: all of them resident at once
     int64_t by_tokens = (tokens + 63) / 64;
     if (s > by_tokens) s = by_tokens;
     if (s > 64) s = 64;
