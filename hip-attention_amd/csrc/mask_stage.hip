@@ -277,6 +277,11 @@ __global__ __launch_bounds__(64) void mask_stage_kernel(MaskParams p) {
     }
 }
 
+__global__ void fill_scores_kernel(float *scores, long long n, float v) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
+        scores[i] = v;
+}
+
 template <typename T, int HID, bool ROPE>
 static int launch_mask(const MaskParams &p, int rows_eff, hipStream_t stream) {
     dim3 grid((unsigned)p.total), block(64);
@@ -365,6 +370,11 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
         return mask_stage_mfma_launch(p, q->HID, rows_eff, k_prescaled, st);
     } else if (q->dtype == HIPATTN_F32) {
         HIPATTN_CHECK_ARG(!k_prescaled, HIPATTN_E_ARG, "mask stage: prescaled keys are a bf16-only option");
+        if (p.reduce_heads) {
+            const long long nscores = (long long)p.B * p.BS * p.n;
+            hipLaunchKernelGGL(fill_scores_kernel, dim3((unsigned)((nscores + 255) / 256 < 4096 ? (nscores + 255) / 256 : 4096)),
+                               dim3(256), 0, st, scores, nscores, -INFINITY);
+        }
         const bool rope = p.rope.cos != nullptr;
         switch (q->HID) {
             case 32: return rope ? launch_mask<float, 32, true>(p, rows_eff, st) : launch_mask<float, 32, false>(p, rows_eff, st);

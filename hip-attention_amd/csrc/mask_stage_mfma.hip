@@ -342,6 +342,12 @@ __global__ void qhat_kernel(MaskParams p, int hid, uint16_t *out) {
     const int per_row = hid / 8;
     const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     const long long total = (long long)p.B * p.BS * p.HEAD * p.nrows * per_row;
+    if (p.reduce_heads) {
+        // the scan folds the maximum over heads into scores [B, BS, 1, n]: start it at -inf here, in the launch that
+        // precedes the scan on the stream anyway
+        const long long nscores = (long long)p.B * p.BS * p.n;
+        for (long long i = gid; i < nscores; i += (long long)gridDim.x * blockDim.x) p.scores[i] = -INFINITY;
+    }
     if (gid >= total) return;
     const int piece = (int)(gid % per_row);
     long long r = gid / per_row;

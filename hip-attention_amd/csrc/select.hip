@@ -59,9 +59,24 @@ __device__ void topk_threshold(const float *scores_row /* [nheads, n] with strid
     for (int shift = 24; shift >= 0; shift -= 8) {
         for (int i = tid; i < 256; i += SEL_THREADS) s_hist[i] = 0;
         __syncthreads();
-        for (int c = tid; c < n; c += SEL_THREADS) {
-            uint32_t key = s_keys[c];
-            if ((key & mask) == prefix) atomicAdd(&s_hist[(key >> shift) & 255u], 1);
+        {
+            // scores cluster: most keys of a pass fall into a handful of bins, so a thread adds up the run of
+            // equal bins it meets before it touches the shared counter
+            int cur = -1, cnt = 0;
+            for (int c = tid; c < n; c += SEL_THREADS) {
+                const uint32_t key = s_keys[c];
+                if ((key & mask) == prefix) {
+                    const int bin = (int)((key >> shift) & 255u);
+                    if (bin == cur) {
+                        cnt++;
+                    } else {
+                        if (cnt) atomicAdd(&s_hist[cur], cnt);
+                        cur = bin;
+                        cnt = 1;
+                    }
+                }
+            }
+            if (cnt) atomicAdd(&s_hist[cur], cnt);
         }
         __syncthreads();
         if (tid < 64) {

@@ -167,6 +167,28 @@ def _mask_kv(args: HiPAttentionArgs, k_mask: Optional[Tensor], max_tsrc: int, q:
     return plain, None, keep, None, 0
 
 
+_INITIAL_CHUNKS = {}  # read-only stage-0 chunk lists, keyed by their shape parameters
+
+
+def _initial_chunks(chunk_count: int, chunk_size: int, sink: int, B: int, bs: int, hg: int, device) -> Tensor:
+    """``int32 [B, bs, hg, chunk_count]``: chunk c starts at ``sink + c * chunk_size`` (attention_extend.py:2020-2035).
+    Nothing writes to a chunk list, so the tensor is built once per shape and shared by later calls (a decode loop
+    would otherwise pay four small launches per mask refresh for it)."""
+    key = (chunk_count, chunk_size, sink, B, bs, hg, str(device))
+    hit = _INITIAL_CHUNKS.get(key)
+    if hit is None:
+        if torch.cuda.is_current_stream_capturing():
+            # a tensor created inside a capture lives in the graph's pool; build it the plain way and do not keep it
+            row = torch.arange(0, chunk_count, device=device, dtype=torch.int32) * chunk_size + sink
+            return row[None, None, None, :].expand(B, bs, hg, chunk_count).contiguous()
+        row = torch.arange(0, chunk_count, device=device, dtype=torch.int32) * chunk_size + sink
+        hit = row[None, None, None, :].expand(B, bs, hg, chunk_count).contiguous()
+        if len(_INITIAL_CHUNKS) >= 16:
+            _INITIAL_CHUNKS.pop(next(iter(_INITIAL_CHUNKS)))
+        _INITIAL_CHUNKS[key] = hit
+    return hit
+
+
 def _stage_cache_views(chunk_left: Tensor, HEAD: int, chunk: int) -> HiPAttentionStageInputCache:
     """Reference-layout view of a stage's inputs: int64 left/right and the reset scores."""
     B, BS, hg, n = chunk_left.shape
@@ -269,8 +291,7 @@ def dual_stage_quadratic_hip_attention(
             assert len(stage_caches) == 1
             fresh = True
         if fresh:
-            chunk_left = (torch.arange(0, chunk_count, device=device, dtype=torch.int32) * chunk_size + sink)
-            chunk_left = chunk_left[None, None, None, :].expand(BSZ, BDST_SCAN, hg, chunk_count).contiguous()
+            chunk_left = _initial_chunks(chunk_count, chunk_size, sink, BSZ, BDST_SCAN, hg, device)
             right_clamp = MAX_TSRC - sw_eff
         else:
             assert len(stage_caches) <= len(stages)
@@ -349,7 +370,7 @@ def dual_stage_quadratic_hip_attention(
                 # one shared chunk list: the scan kernels fold the maximum over heads into their score store
                 reduce = hg == 1
                 if reduce:
-                    scores = torch.full((BSZ, bs, 1, chunk_count), float("-inf"), dtype=torch.float32, device=device)
+                    scores = torch.empty((BSZ, bs, 1, chunk_count), dtype=torch.float32, device=device)  # mask_stage fills it
                 else:
                     scores = torch.empty((BSZ, bs, HEAD, chunk_count), dtype=torch.float32, device=device)
                 left_out = torch.empty((BSZ, bs, HEAD, chunk_count), dtype=torch.int32, device=device) if last else None

@@ -125,8 +125,8 @@ const char *hipattn_last_error(void);
  *                                      scores are max-reduced over heads, else HEAD
  *   right = min(left + chunk_size, right_clamp)
  *   scores      f32   [B, BS, HEAD, n] written for every chunk (-32000 where not scored); with
- *                     reduce_heads != 0 (needs hg == 1): [B, BS, 1, n], filled with -inf by the caller,
- *                     receives the maximum over heads (the torch.max at :2566-2570 folded into the scan)
+ *                     reduce_heads != 0 (needs hg == 1): [B, BS, 1, n], set to -inf by the entry point and then
+ *                     raised to the maximum over heads (the torch.max at :2566-2570 folded into the scan)
  *   left_out    int32 [B, BS, HEAD, n] refined left edge per head, or NULL
  *   block_chunk = chunks per reference program (16/32/64): fixes the program-level gate and
  *   iteration count (:595-601,736-737).
