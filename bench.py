@@ -444,6 +444,21 @@ def run_offload(args, device, TK=3_000_000, warm_steps=4, drift_steps=12):
         call(q)  # back to the base query so that trials do not build on each other
     blend = min(trial, key=lambda a: abs(trial[a] - 0.10))
     drift = [drift_step(blended(blend, nz)) for nz in noise]
+    # --- eviction: the same drifting queries against an attention cache capped at 1.25x what one step attends to
+    # (the 16 GB cache above never fills, so nothing is ever evicted there)
+    from hip_attn.offload import GPUCache
+    step_blocks = HKV * cdiv(2048 + 256 + 1024 + 1, BT)
+    capped_slots = int(step_blocks * 1.25)
+    big_sa = cache.sa_kv_cache
+    cache.sa_kv_cache = GPUCache(cache.k_uvm, cache.v_uvm, capped_slots * BT, block_tokens=BT, max_fetch=1 << 16)
+    _, md = call(q)
+    cache.handle_cache_miss(md)
+    capped = [drift_step(blended(blend, nz)) for nz in noise]
+    capped_stats = cache.sa_kv_cache.statistics()
+    out_capped, _ = call(q)
+    capped_same = bool(torch.equal(out_capped.view(torch.int16), out_warm.view(torch.int16)))
+    small_sa, cache.sa_kv_cache = cache.sa_kv_cache, big_sa
+    del small_sa
     # --- the same data resident in HBM
     kres = cache.k_uvm.bank_cpu.to(device).unsqueeze(1)
     resident = (kres, kres)
@@ -472,6 +487,14 @@ def run_offload(args, device, TK=3_000_000, warm_steps=4, drift_steps=12):
             "commit_us": sum(d["commit_us"] for d in tail) / len(tail),
             "fetched_MB_per_step": sum(d["fetched_blocks"] for d in tail) / len(tail) * block_bytes / 1e6,
             "mask_cache_missed": sum(d["mask_cache_missed"] for d in tail),
+        },
+        "capped_attention_cache": {
+            "slots": capped_slots, "blocks_attended_per_step": step_blocks, "steps": len(capped[2:]),
+            "miss_fraction": sum(d["miss_fraction"] for d in capped[2:]) / len(capped[2:]),
+            "refresh_us": sum(d["step_us"] for d in capped[2:]) / len(capped[2:]),
+            "commit_us": sum(d["commit_us"] for d in capped[2:]) / len(capped[2:]),
+            "blocks_evicted_total": capped_stats["blocks_evicted"], "blocks_fetched_total": capped_stats["blocks_fetched"],
+            "output_equals_uncapped": capped_same,
         },
         "offloaded_equals_resident": same,
     }
