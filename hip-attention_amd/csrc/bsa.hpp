@@ -17,6 +17,10 @@ struct BsaParamsBase {
     const int32_t *kse;
     int idx_rows, BK, bq, bk, sw, sink, share_first_head;
     int k_prescaled;  // kv.k already holds bf16(K * c_k) (tile kernel only)
+    // Decode only: the reference's decode kernel gives each of its programs `seam_blocks` entries of the index row but
+    // masks a program's last tile against the end of the row only, so the first `seam_extra` entries of the next
+    // program's share are attended once more (attention_decode_bsa.py:239-247); 0 / 0 = every entry once.
+    int seam_blocks, seam_extra;
     int B, TDST, HEAD, G, NBQ;
     float c_q, c_k;
     void *out;
@@ -34,6 +38,13 @@ struct BsaParams : BsaParamsBase {
 __device__ __forceinline__ float softcap_logit(float x, float cap, float two_log2e_over_cap) {
     const float e = __builtin_amdgcn_exp2f(x * two_log2e_over_cap);
     return cap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f));
+}
+// How often the reference's decode programs visit entry j of an index row: once by the program that owns it, and
+// once by each earlier program whose tile-rounded walk reaches it.
+__host__ __device__ __forceinline__ int bsa_seam_multiplicity(int j, int seam_blocks, int seam_extra) {
+    const int s = j / seam_blocks, r = j - s * seam_blocks;
+    const int earlier = (seam_blocks + seam_extra - r - 1) / seam_blocks;
+    return 1 + (earlier < s ? earlier : s);
 }
 // Rotated position of a sink or selected key (attention_extend_bsa.py:256-299): "streaming" packs them, in the
 // order of the index row, into the positions that end just below the window of the block's first query;

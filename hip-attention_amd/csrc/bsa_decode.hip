@@ -15,6 +15,7 @@ template <bool EXT>
 struct DecodeParamsT {
     BsaParamsFor<EXT> a;
     int nsplits;
+    int parts;  // workgroups that share one GQA group, G heads each (group size = parts * G)
     float *ws;  // [B, HEAD, nsplits, HID + 4]: acc / l, then m + log2(l)
 };
 using DecodeParams = DecodeParamsT<true>;
@@ -37,9 +38,9 @@ __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<E
     const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
     const int sub = lane >> 4, dl = lane & 15;
     const int grp = wid * 4 + sub;  // 16-lane group id inside the workgroup
-    const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
-    const int h0 = kvh * G;
-    const int64_t irow = ((int64_t)b * p.HEAD + h0) * p.idx_rows;  // query block 0, first head of the group
+    const int split = blockIdx.x, kvh = blockIdx.y / dp.parts, b = blockIdx.z;
+    const int h0 = kvh * p.G + (blockIdx.y % dp.parts) * G;
+    const int64_t irow = ((int64_t)b * p.HEAD + kvh * p.G) * p.idx_rows;  // query block 0, first head of the group
 
     const long long ppos = p.pos[(int64_t)b * p.pos_sb];
     const long long curr = ppos + 1;
@@ -95,9 +96,11 @@ __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<E
         int kind = 0;
         bool valid = false;
         long long rpos = 0;  // rotated position of the key (ROPE only)
+        float visits = 1.0f;  // how often the reference's programs attend this token
         if (o < o_end) {
             if (o < n_sel_tok) {
                 const long long st = p.indices[irow * p.BK + rs + o / p.bk];
+                if (p.seam_extra > 0) visits = (float)bsa_seam_multiplicity(rs + (int)(o / p.bk), p.seam_blocks, p.seam_extra);
                 t = st + o % p.bk;
                 valid = (t >= 0) && (t < p.kv.max_tsrc) && (t < curr) && (t >= p.sink);
                 if constexpr (ROPE)
@@ -162,8 +165,8 @@ __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<E
             const float m_new = fmaxf(m[g], x);
             const float alpha = exp2f(m[g] - m_new);
             const float pr = exp2f(x - m_new);
-            l[g] = l[g] * alpha + pr;
-            const float prT = Elem<T>::round(pr);
+            l[g] = l[g] * alpha + pr * visits;
+            const float prT = Elem<T>::round(pr) * visits;
 #pragma unroll
             for (int e = 0; e < SEG; e++) acc[g][e] = __fmaf_rn(prT, vv[e], acc[g][e] * alpha);
             m[g] = m_new;
@@ -244,12 +247,17 @@ __global__ __launch_bounds__(MERGE_THREADS) void bsa_decode_merge_kernel(const f
 }
 
 template <typename T, int HID>
-static int launch_partial(const DecodeParams &dp, hipStream_t st) {
-    dim3 grid((unsigned)dp.nsplits, (unsigned)dp.a.kv.HKV, (unsigned)dp.a.B), block(256);
+static int launch_partial(const DecodeParams &dp_in, hipStream_t st) {
+    // a workgroup keeps GG heads of a group in registers (GG * HID <= 512); larger groups are shared by several
+    // workgroups, each of which reads the rows again
+    dim3 grid, block(256);
     bool launched = false;
+    DecodeParams dp = dp_in;
 #define DEC_CASE(GG)                                                                                   \
     if constexpr (GG * HID <= 512) {                                                                   \
-        if (dp.a.G == GG) {                                                                            \
+        if (!launched && dp.a.G % GG == 0) {                                                           \
+            dp.parts = dp.a.G / GG;                                                                    \
+            grid = dim3((unsigned)dp.nsplits, (unsigned)(dp.a.kv.HKV * dp.parts), (unsigned)dp.a.B);   \
             if (sizeof(T) == 2 && dp.a.kx.kv8) {                                                       \
                 if constexpr (sizeof(T) == 2) {                                                        \
                     const bool r_ = dp.a.rope.cos != nullptr, c_ = dp.a.softcap != 0.0f;               \
@@ -271,18 +279,15 @@ static int launch_partial(const DecodeParams &dp, hipStream_t st) {
                 DecodeParamsT<false> dq;                                                               \
                 dq.a = static_cast<const BsaParamsBase &>(dp.a);                                       \
                 dq.nsplits = dp.nsplits;                                                               \
+                dq.parts = dp.parts;                                                                   \
                 dq.ws = dp.ws;                                                                         \
                 hipLaunchKernelGGL((bsa_decode_partial_kernel<T, HID, GG, false>), grid, block, 0, st, dq); \
             }                                                                                          \
             launched = true;                                                                           \
         }                                                                                              \
     }
-    DEC_CASE(1) DEC_CASE(2) DEC_CASE(4) DEC_CASE(8)
+    DEC_CASE(8) DEC_CASE(4) DEC_CASE(2) DEC_CASE(1)
 #undef DEC_CASE
-    if (!launched) {
-        set_error("decode: GQA group size %d with head dim %d is not built", dp.a.G, HID);
-        return HIPATTN_E_UNSUPPORTED;
-    }
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
 }
@@ -309,8 +314,8 @@ extern "C" int32_t hipattn_bsa_decode_default_splits(int32_t B, int32_t HKV, int
 
 extern "C" int hipattn_bsa_decode_partial(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t *indices,
                                           const int32_t *ks_start_end, int32_t idx_rows, int32_t BK,
-                                          int32_t block_size_k, int32_t sliding_window, int32_t sink, int32_t nsplits,
-                                          void *workspace, void *stream) {
+                                          int32_t block_size_k, int32_t sliding_window, int32_t sink,
+                                          int32_t second_stage_k, int32_t nsplits, void *workspace, void *stream) {
     DecodeParams dp;
     HIPATTN_CHECK_ARG(workspace, HIPATTN_E_ARG, "decode: null workspace");
     HIPATTN_CHECK_ARG(nsplits >= 1 && nsplits <= 1024, HIPATTN_E_ARG, "decode: nsplits %d out of range", nsplits);
@@ -318,6 +323,19 @@ extern "C" int hipattn_bsa_decode_partial(const hipattn_q_t *q, const hipattn_kv
                              workspace, 0, 0, 0, &dp.a);
     if (rc) return rc;
     HIPATTN_CHECK_ARG(q->TDST == 1, HIPATTN_E_ARG, "decode: TDST must be 1, got %d", q->TDST);
+    HIPATTN_CHECK_ARG(second_stage_k >= 0, HIPATTN_E_ARG, "decode: negative second_stage_k");
+    if (second_stage_k > 0 && BK > 0) {
+        // the reference launcher's own division of the index row (attention_decode_bsa.py:1070-1076, 1391-1393)
+        const int64_t total = (int64_t)second_stage_k + sink + sliding_window;
+        const int64_t chunk = (total + 7) / 8;
+        int64_t programs = (second_stage_k + chunk - 1) / chunk;
+        if (programs > 12) programs = 12;
+        int tile = 16 / block_size_k;
+        tile = tile < 1 ? 1 : tile;
+        const int share = (int)((BK + programs - 1) / programs);
+        dp.a.seam_blocks = share;
+        dp.a.seam_extra = (share + tile - 1) / tile * tile - share;
+    }
     dp.nsplits = nsplits;
     dp.ws = reinterpret_cast<float *>(workspace);
     hipStream_t st = (hipStream_t)stream;

@@ -20,7 +20,7 @@ struct DecWaveSmem {
     uint16_t v[DT][HID + VPAD];
     // what lanes 0..31 post about the token slots of a tile, double-buffered
     long long ko[2][DT], vo[2][DT];  // row offsets (NO_ROW: zero row)
-    int tok[2][DT];                  // token, -1: empty or masked slot
+    float bias[2][DT];               // added to the slot's logit: 0, log of the visit count, -inf: empty or masked
     int rp[2][DT];                   // row of the RoPE tables
 };
 
@@ -117,16 +117,22 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
     // page-table loads in flight), posted one tile ahead, and the K / V rows of the next tile are in flight while the
     // current tile is multiplied
     long long m_ko = NO_ROW, m_vo = NO_ROW;
-    int m_t = -1, m_rp = 0;
+    int m_rp = 0;
+    float m_bias = -INFINITY;
     auto resolve = [&](int tile) {  // lanes 0..31
         if (lane >= DT) return;
         const int o = o_begin + tile * DT + lane;
         int t = -1, win = 0;
         long long rpos = 0;
+        float bias = 0.0f;
         if (o < o_end) {
             if (o < n_sel_tok) {
                 const int bi = bk_shift >= 0 ? (o >> bk_shift) : o / p.bk;
                 const int e = o - bi * p.bk;
+                if (p.seam_extra > 0) {  // weight of a token attended v times: v * exp(logit) = exp(logit + log v)
+                    const int visits = bsa_seam_multiplicity(rs + bi, p.seam_blocks, p.seam_extra);
+                    if (visits > 1) bias = __logf((float)visits);
+                }
                 const long long s64 = p.indices[irow * p.BK + rs + bi];
                 const int st = (s64 >= 0 && s64 < 0x7fffffffLL) ? (int)s64 : -0x40000000;
                 t = st + e;
@@ -156,14 +162,14 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
         }
         m_ko = ko;
         m_vo = vo;
-        m_t = t;
+        m_bias = t >= 0 ? bias : -INFINITY;
         if constexpr (ROPE) m_rp = (int)p.rope.clamp(rpos);
     };
     auto post = [&](int slot2) {  // lanes 0..31 -> meta buffer slot2 (0 / 1)
         if (lane >= DT) return;
         sm.ko[slot2][lane] = m_ko;
         sm.vo[slot2][lane] = m_vo;
-        sm.tok[slot2][lane] = m_t;
+        sm.bias[slot2][lane] = m_bias;
         if constexpr (ROPE) sm.rp[slot2][lane] = m_rp;
     };
     auto wave_sync = [&]() {
@@ -243,11 +249,11 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
         float mx = -INFINITY;
 #pragma unroll
         for (int i4 = 0; i4 < 4; i4++) {
-            const int4 tt = *reinterpret_cast<const int4 *>(&sm.tok[cur][i4 * 8 + hh * 4]);
-            const int ts[4] = {tt.x, tt.y, tt.z, tt.w};
+            const float4 tt = *reinterpret_cast<const float4 *>(&sm.bias[cur][i4 * 8 + hh * 4]);
+            const float ts[4] = {tt.x, tt.y, tt.z, tt.w};
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                const float s = ts[e] >= 0 ? sacc[i4 * 4 + e] : -INFINITY;
+                const float s = sacc[i4 * 4 + e] + ts[e];
                 sacc[i4 * 4 + e] = s;
                 mx = fmaxf(mx, s);
             }

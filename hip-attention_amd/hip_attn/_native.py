@@ -352,7 +352,8 @@ def bsa_prefill(qs, kvs, indices, ks_start_end, BK, bq, bk, sw, sink, share_firs
     check(rc, "hipattn_bsa_prefill")
 
 
-def bsa_decode(qs, kvs, indices, ks_start_end, BK, bk, sw, sink, out, device, nsplits=0, workspace=None):
+def bsa_decode(qs, kvs, indices, ks_start_end, BK, bk, sw, sink, out, device, nsplits=0, workspace=None,
+               second_stage_k=0):
     assert indices.dtype == torch.int64 and indices.is_contiguous()
     assert ks_start_end.dtype == torch.int32 and ks_start_end.is_contiguous()
     L = lib()
@@ -367,8 +368,8 @@ def bsa_decode(qs, kvs, indices, ks_start_end, BK, bk, sw, sink, out, device, ns
     with _timed("bsa_decode"):
       rc = L.hipattn_bsa_decode_partial(
         ctypes.byref(qs), ctypes.byref(kvs), _p(indices), _p(ks_start_end), ctypes.c_int32(indices.shape[1]),
-        ctypes.c_int32(BK), ctypes.c_int32(bk), ctypes.c_int32(sw), ctypes.c_int32(sink), ctypes.c_int32(nsplits),
-        _p(workspace), stream_ptr(device))
+        ctypes.c_int32(BK), ctypes.c_int32(bk), ctypes.c_int32(sw), ctypes.c_int32(sink),
+        ctypes.c_int32(second_stage_k), ctypes.c_int32(nsplits), _p(workspace), stream_ptr(device))
     check(rc, "hipattn_bsa_decode_partial")
     rc = L.hipattn_bsa_decode_merge(
         _p(workspace), ctypes.c_int32(B), ctypes.c_int32(HEAD), ctypes.c_int32(HID), ctypes.c_int32(nsplits),

@@ -329,15 +329,19 @@ def dual_stage_quadratic_hip_attention(
                     BLOCK_SIZE_Q = stage.stage_block_size_q
                     BDST = _cdiv(TDST, BLOCK_SIZE_Q)
                     BDST_SCAN = _cdiv(BDST, STAGE_STRIDE)
-                if row_rep != 1 and STAGE_STRIDE != 1:
-                    raise NotImplementedError("a stage may shrink its query block only when stage_stride is 1")
+                shrunk = row_rep != 1
                 if STAGE_STRIDE != stage.stage_stride:
                     assert stage.stage_stride < STAGE_STRIDE and STAGE_STRIDE > 0
                     if stage.stage_stride != 1:
                         raise NotImplementedError("stage_stride may only drop to 1 between stages")
+                    # rows repeated for the smaller block and again for the smaller stride, each time keeping the
+                    # last BDST rows (:2096-2124): counted from the last row, output row e reads input row
+                    # e // (both factors), whether or not the first cut removed anything
                     row_rep *= STAGE_STRIDE // stage.stage_stride
                     STAGE_STRIDE = stage.stage_stride
                     BDST_SCAN = _cdiv(BDST, STAGE_STRIDE)
+                if shrunk and STAGE_STRIDE != 1:
+                    raise NotImplementedError("a stage may shrink its query block only when its stage_stride is 1")
                 bs_out = BDST_SCAN if row_rep == 1 else min(BDST, row_rep * bs_in)
                 assert (chunk_size % stage.stage_chunk_size) == 0
                 splits = chunk_size // stage.stage_chunk_size
@@ -481,6 +485,17 @@ def dual_stage_quadratic_hip_attention(
 
 
 @torch.no_grad()
+def _decode_seams_overlap(args: HiPAttentionArgs, BK: int) -> bool:
+    """Whether the reference's decode programs visit some selected block twice (attention_decode_bsa.py:1070-1076,
+    1391-1393, 239-247): their share of the index row is not a whole number of their tiles."""
+    if args.second_stage_k <= 0 or BK <= 0:
+        return False
+    chunk = -(-(args.second_stage_k + args.sink_token_size + args.sliding_window_size) // 8)
+    programs = min(12, -(-args.second_stage_k // chunk))
+    tile = max(1, 16 // args.block_size_k)
+    return -(-BK // programs) % tile != 0
+
+
 def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], position_ids: Tensor, indices: Tensor,
                            ks_start_end: Tensor, args: HiPAttentionArgs, max_tsrc: int, decode: bool = False,
                            impl: int = 0, rows_shared: bool = False, khat: Optional[Tensor] = None,
@@ -492,7 +507,10 @@ def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], 
     attention_extend.py:3092).  ``args.block_size_q / block_size_k / sliding_window_size`` must
     already hold the values the operator derives for this step.  ``decode`` selects the split-KV
     path, which, like the reference's decode kernel, lets every head of a GQA group read the
-    index row of the group's first head.  ``rows_shared`` promises that all heads of a GQA group hold
+    index row of the group's first head, and which weights the selected blocks as the reference's decode
+    programs do (a block at the seam of two programs' shares of the index row counts twice when
+    ``ceil(BK / programs)`` is not a multiple of ``16 // block_size_k``, attention_decode_bsa.py:239-247,1070-1076).
+    ``rows_shared`` promises that all heads of a GQA group hold
     identical index rows (true for masks estimated with head reduction), which lets one gathered
     K/V tile serve the whole group.  ``khat`` is an optional ``bf16(k * c_k)`` tensor with the shape and
     strides of the key storage (dense ``k`` or ``args.k_cache``).  ``rope_tables`` = ``(cos, sin)`` in q's dtype
@@ -522,10 +540,12 @@ def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], 
     if decode:
         try:
             N.bsa_decode(qs, kvs, indices, ks_start_end, BK, args.block_size_k, args.sliding_window_size,
-                         args.sink_token_size, out, device)
+                         args.sink_token_size, out, device, second_stage_k=args.second_stage_k)
             return out
         except N.HipAttnError as e:
-            if "is not built" not in str(e):
+            # the query-block kernel below attends every selected block once: it can stand in only where the
+            # reference's decode programs do so too
+            if "is not built" not in str(e) or _decode_seams_overlap(args, BK):
                 raise
     ksrc = k if k is not None else args.k_cache
     if khat is not None and (ksrc is None or khat.shape != ksrc.shape or khat.stride() != ksrc.stride()

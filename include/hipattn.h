@@ -209,13 +209,19 @@ int hipattn_bsa_prefill(const hipattn_q_t *q, const hipattn_kv_t *kv, const int6
  * src/hip_attn/v1_2/attention_decode_bsa.py:1331-1435: _fwd_kernel_stage1 (:22-1045) writes
  * per-split partials, _fwd_kernel_stage2 (:1148-1226) merges them by log-sum-exp.
  *   workspace: f32, hipattn_bsa_decode_workspace_bytes(...) bytes, caller-allocated.
- *   nsplits: 0 = choose from the device size. */
+ *   nsplits: how many workgroups share one (sequence, kv head); hipattn_bsa_decode_default_splits picks one.
+ *   second_stage_k: args.second_stage_k of the call being replaced, or 0.  The reference's launcher divides the
+ *   index row among min(12, ceil(second_stage_k / ceil((second_stage_k + sink + window) / 8))) programs (:1070-1076)
+ *   that walk their share in tiles of 16 / block_size_k entries (:1391-1393) and mask a tile against the end of the
+ *   row only (:239-247): when the share is not a whole number of tiles, the entries at the start of the next share
+ *   are attended twice.  With second_stage_k > 0 those entries get the same weight here, so the output equals the
+ *   reference's; with 0 every selected block counts once. */
 int64_t hipattn_bsa_decode_workspace_bytes(int32_t B, int32_t HEAD, int32_t HID, int32_t nsplits);
 int32_t hipattn_bsa_decode_default_splits(int32_t B, int32_t HKV, int32_t tokens);
 int hipattn_bsa_decode_partial(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t *indices,
                                const int32_t *ks_start_end, int32_t idx_rows, int32_t BK,
                                int32_t block_size_k, int32_t sliding_window, int32_t sink,
-                               int32_t nsplits, void *workspace, void *stream);
+                               int32_t second_stage_k, int32_t nsplits, void *workspace, void *stream);
 int hipattn_bsa_decode_merge(const void *workspace, int32_t B, int32_t HEAD, int32_t HID,
                              int32_t nsplits, int32_t dtype, void *out, int64_t out_stride_b,
                              int64_t out_stride_h, void *stream);

@@ -264,9 +264,28 @@ def rope_row(X: OInputs, row: np.ndarray, pos: int) -> np.ndarray:
     return out
 
 
+def decode_seams(second_stage_k: int, sink: int, sw: int, block_size_k: int, BK: int):
+    """``(share, overhang)`` of the decode kernel's programs over an index row of ``BK`` entries: the launcher gives
+    the selected blocks ``min(12, ceil(second_stage_k / ceil((second_stage_k + sink + sw) / 8)))`` programs
+    (attention_decode_bsa.py:1070-1076) that walk their ``share`` of the row in tiles of ``16 // block_size_k`` entries
+    (:1391-1393); ``overhang`` is how far a program's last tile reaches into the next share (:239-247)."""
+    chunk = cdiv(second_stage_k + sink + sw, 8)
+    programs = min(12, cdiv(second_stage_k, chunk)) if chunk > 0 else 0
+    if programs <= 0 or BK <= 0:
+        return 0, 0
+    share = cdiv(BK, programs)
+    tile = max(1, min(16, 16 // block_size_k))
+    return share, cdiv(share, tile) * tile - share
+
+
+def seam_multiplicity(j: int, share: int, overhang: int) -> int:
+    return int(lib().hipo_seam_multiplicity(ctypes.c_int(j), ctypes.c_int(share), ctypes.c_int(overhang)))
+
+
 def bsa(X: OInputs, max_tsrc, indices, ks_start_end, block_size_q, block_size_k, sw, sink,
-        share_first_head=False):
-    """Block-sparse attention given indices; returns context with q's shape and dtype."""
+        share_first_head=False, seams=(0, 0)):
+    """Block-sparse attention given indices; returns context with q's shape and dtype.  ``seams``: see
+    ``decode_seams`` (decode only; ``(0, 0)`` attends every selected block once)."""
     S, keep = X.c_struct(max_tsrc)
     indices = np.ascontiguousarray(indices, dtype=np.int64)
     kse = np.ascontiguousarray(ks_start_end, dtype=np.int32)
@@ -275,7 +294,7 @@ def bsa(X: OInputs, max_tsrc, indices, ks_start_end, block_size_q, block_size_k,
                         ctypes.c_int(indices.shape[1]), ctypes.c_int(indices.shape[2]),
                         ctypes.c_int(block_size_q), ctypes.c_int(block_size_k), ctypes.c_int(sw),
                         ctypes.c_int(sink), ctypes.c_int(1 if share_first_head else 0),
-                        ctypes.c_void_p(out.ctypes.data))
+                        ctypes.c_int(seams[0]), ctypes.c_int(seams[1]), ctypes.c_void_p(out.ctypes.data))
     if rc != 0:
         raise RuntimeError(f"hipo_bsa failed: {rc}")
     del keep
@@ -495,8 +514,9 @@ def hip_attention_12(X: OInputs, A: OArgs, cached: Optional[OMetadata] = None):
     user_cap = X.logit_softcap
     X.logit_softcap = float(A.logit_softcap or 0.0)
     try:
+        seams = decode_seams(A.second_stage_k, sink, sw_bsa, block_size_k, indices.shape[-1]) if decode else (0, 0)
         context = bsa(X, MAX_TSRC, indices, ks_start_end, block_size_q, block_size_k, sw_bsa, sink,
-                      share_first_head=decode)
+                      share_first_head=decode, seams=seams)
     finally:
         X.access = user_access
         X.logit_softcap = user_cap

@@ -28,9 +28,12 @@
  * Dense key reads at t >= TSRC return a zero row (the reference reads out of bounds there).
  *
  * Parity status: the reference ships no golden vectors for this path.  The functions here
- * are pinned by closed forms and brute-force checks in tests/ (see each function's comment);
- * hipo_mask_stage on multi-level hierarchies is pinned to this restatement of the source,
- * not to an execution of the Triton build: parity unpinned against the running reference.
+ * are pinned by closed forms and brute-force checks in tests/ (see each function's comment)
+ * and, for float32 inputs, by executions of the reference's own kernels under Triton's CPU
+ * interpreter (tests/golden/reference_*.npz, tests/test_golden_reference.py): multi-level scans,
+ * selection, both attention kernels, decode, RoPE on load.  Parity unpinned against the running
+ * reference: bfloat16 arithmetic (the interpreter has no bfloat16; the order of accumulation here is
+ * MI355X's, not NVIDIA's) and logit_softcap (the interpreter cannot call libdevice.tanh).
  */
 #include <math.h>
 #include <stdint.h>
@@ -442,12 +445,28 @@ int hipo_mask_stage(const hipo_tensors_t *X, int64_t *left, int64_t *right, floa
  * (:531-558).  Rows with an empty set give 0 (l stays at its initial 1.0, :764,1625).
  * share_first_head != 0 uses, for every head of a GQA group, the index row of the group's
  * first head, as the decode kernel does (attention_decode_bsa.py:150).
+ * seam_blocks > 0 restates how the decode kernel divides the index row among its programs
+ * (attention_decode_bsa.py:239-247): program s owns entries [s*seam_blocks, (s+1)*seam_blocks) but
+ * walks them in steps of its tile and masks a tile only against the end of the row, not against the
+ * end of its own share, so the first seam_extra entries of the next share (seam_extra = tile-rounded
+ * share - share) enter the softmax once per program that reaches them.  hipo_seam_multiplicity counts
+ * those visits; a token visited m times has weight m * exp2(logit - max).
  * Pinned by: dense masked softmax in f64 built from the set definition above
- * (tests/test_oracle_bsa.py), StreamingLLM and plain-causal special cases.
+ * (tests/test_oracle_bsa.py), StreamingLLM and plain-causal special cases; the seam rule by an execution
+ * of the reference (tests/golden/reference_f32_decode_paged.npz) and by a literal walk of the programs'
+ * loops (tests/test_oracle_bsa.py).
  */
+int hipo_seam_multiplicity(int j, int seam_blocks, int seam_extra) {
+    if (seam_blocks <= 0 || seam_extra <= 0) return 1;
+    int s = j / seam_blocks, r = j - s * seam_blocks;
+    int earlier = (seam_blocks + seam_extra - r - 1) / seam_blocks; /* programs before s whose last tile reaches j */
+    return 1 + (earlier < s ? earlier : s);
+}
+
 int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_start_end,
              int NBQ_rows /* rows of indices per (b,h) */, int BK, int block_size_q,
-             int block_size_k, int sw, int sink, int share_first_head, void *out) {
+             int block_size_k, int sw, int sink, int share_first_head, int seam_blocks, int seam_extra,
+             void *out) {
     const int B = X->B, TDST = X->TDST, HEAD = X->HEAD, HID = X->HID;
     const int G = HEAD / X->HKV;
     const int NBQ = (TDST + block_size_q - 1) / block_size_q;
@@ -461,6 +480,7 @@ int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_
     {
         int64_t *tok = (int64_t *)malloc(sizeof(int64_t) * cap);
         int *kind = (int *)malloc(sizeof(int) * cap); /* 0: excluded-window rule, 1: window rule */
+        int *mult = (int *)malloc(sizeof(int) * cap); /* visits of the token by the decode programs */
         int64_t *rpos = (int64_t *)malloc(sizeof(int64_t) * cap); /* rotated position of the key (RoPE on load) */
         float *khat = (float *)malloc(sizeof(float) * (size_t)cap * HID);
         float *vrow = (float *)malloc(sizeof(float) * (size_t)cap * HID);
@@ -497,17 +517,17 @@ int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_
                     int64_t t = st + e;
                     if (t < 0 || t >= MAXT) continue;
                     if (!(t < curr && t >= sink)) continue;
-                    tok[nt] = t; kind[nt] = 0;
+                    tok[nt] = t; kind[nt] = 0; mult[nt] = hipo_seam_multiplicity(j, seam_blocks, seam_extra);
                     rpos[nt] = (int64_t)(j + sink / block_size_k) * block_size_k + e + shift;
                     nt++;
                 }
             }
             int64_t sink_end = curr < sink ? curr : sink;
-            for (int64_t t = 0; t < sink_end; t++) { tok[nt] = t; kind[nt] = 0; rpos[nt] = t + shift; nt++; }
+            for (int64_t t = 0; t < sink_end; t++) { tok[nt] = t; kind[nt] = 0; mult[nt] = 1; rpos[nt] = t + shift; nt++; }
             if (sw > 0) {
                 int64_t ws = curr - sw - block_size_q;
                 if (ws < 0) ws = 0;
-                for (int64_t t = ws; t < curr; t++) { tok[nt] = t; kind[nt] = 1; rpos[nt] = t; nt++; }
+                for (int64_t t = ws; t < curr; t++) { tok[nt] = t; kind[nt] = 1; mult[nt] = 1; rpos[nt] = t; nt++; }
             }
             for (int i = 0; i < nt; i++) {
                 int64_t rp = rpos[i];
@@ -542,10 +562,10 @@ int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_
                     for (int i = 0; i < nt; i++) {
                         if (logit[i] == -INFINITY) continue;
                         float pr = exp2f(logit[i] - m);
-                        lsum += (double)pr;
-                        float prT = round_T(pr, X->dtype);
+                        lsum += (double)pr * mult[i];
+                        double prT = (double)round_T(pr, X->dtype) * mult[i];
                         const float *vr = vrow + (size_t)i * HID;
-                        for (int d = 0; d < HID; d++) acc[d] += (double)prT * (double)vr[d];
+                        for (int d = 0; d < HID; d++) acc[d] += prT * (double)vr[d];
                     }
                 } else {
                     lsum = 1.0;
@@ -554,7 +574,7 @@ int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_
                 for (int d = 0; d < HID; d++) store_T(out, qoff + d, (float)(acc[d] / lsum), X->dtype);
             }
         }
-        free(tok); free(kind); free(rpos); free(khat); free(vrow); free(qhat); free(logit); free(acc);
+        free(tok); free(kind); free(mult); free(rpos); free(khat); free(vrow); free(qhat); free(logit); free(acc);
     }
     return 0;
 }

@@ -1,0 +1,186 @@
+"""Golden vectors from an execution of the reference's own v1.2 code (mask estimation + sparse attention).
+
+Run in a container that holds the reference checkout (never on the GPU box):
+
+    python tests/golden/make_reference_fixtures.py /root/reference
+
+The reference cannot be imported as a package here: ``hip_attn/__init__.py`` pulls model code and the v1.0 / v1.1
+generations, and the v1.2 modules import ``cv2``, ``numba``, ``cuda`` (cuda-python) and a JIT-compiled cupy helper,
+none of which are installed.  This script therefore
+  * registers empty parent packages (``hip_attn``, ``hip_attn.v1_2``, ``hip_attn.utils``, ``hip_attn.v1_1...``) whose
+    ``__path__`` points into the checkout, so that the five v1.2 modules and ``utils/rope.py`` load by their own
+    names without any ``__init__`` running,
+  * registers placeholder modules for the absent third-party imports (they are only used by debug plotting and by
+    the UVM cache, which these fixtures do not touch),
+  * runs the Triton kernels under ``TRITON_INTERPRET=1`` (Triton's CPU interpreter) on CPU tensors, with the three
+    ``torch.cuda`` calls of the driver answered for a machine without a GPU.
+Only data leaves this script: inputs and the reference's outputs, saved as ``reference_*.npz`` next to it.
+"""
+import os
+import sys
+import types
+
+os.environ["TRITON_INTERPRET"] = "1"
+os.environ.setdefault("HIP_DISABLE_AUTOTUNE", "1")
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def _package(name, path):
+    m = types.ModuleType(name)
+    m.__path__ = [path]
+    sys.modules[name] = m
+    return m
+
+
+def _placeholder(name, **attrs):
+    m = types.ModuleType(name)
+    for k, v in attrs.items():
+        setattr(m, k, v)
+    sys.modules[name] = m
+    return m
+
+
+def load_reference(root):
+    src = os.path.join(root, "src", "hip_attn")
+    _package("hip_attn", src)
+    _package("hip_attn.v1_2", os.path.join(src, "v1_2"))
+    _package("hip_attn.utils", os.path.join(src, "utils"))
+    _package("hip_attn.v1_1", os.path.join(src, "v1_1"))
+    _package("hip_attn.v1_1.offload_runner", os.path.join(src, "v1_1", "offload_runner"))
+
+    def _decorator(*a, **k):  # numba.njit / numba.jit used with and without arguments
+        if len(a) == 1 and callable(a[0]) and not k:
+            return a[0]
+        return lambda f: f
+
+    _placeholder("cv2")
+    nb = _placeholder("numba", njit=_decorator, jit=_decorator, prange=range)
+    nb.cuda = _placeholder("numba.cuda", jit=_decorator)
+    cu = _placeholder("cuda")
+    cu.cudart = _placeholder("cuda.cudart")
+    _placeholder("hip_attn.v1_1.offload_runner.tensor_from_pointer", alloc_managed_tensor=None, sizeof=None)
+
+    # the driver asks the CUDA runtime about devices and graph capture (attention_extend.py:1980, 2196-2197, 2636)
+    torch.cuda.current_device = lambda: 0
+    torch.cuda.set_device = lambda *_a, **_k: None
+    torch.cuda.is_current_stream_capturing = lambda: False
+    torch.cuda.get_device_name = lambda *_a, **_k: "none"  # only picks autotune candidates (attention_extend_bsa.py:571)
+
+    import hip_attn.v1_2.attention_extend as ext
+    import hip_attn.v1_2.attention_metadata as meta
+    return ext, meta
+
+
+def rope_tables(length, D, theta=10000.0):
+    inv = theta ** (-np.arange(0, D, 2, dtype=np.float64) / D)
+    ang = np.arange(length, dtype=np.float64)[:, None] * inv[None, :]
+    cos = np.concatenate([np.cos(ang), np.cos(ang)], axis=1).astype(np.float32)
+    sin = np.concatenate([np.sin(ang), np.sin(ang)], axis=1).astype(np.float32)
+    return torch.from_numpy(cos), torch.from_numpy(sin)
+
+
+def bits16(t):
+    """Upper halves of the float32 patterns (exact: the values were rounded to 8 significant bits)."""
+    w = t.float().contiguous().view(torch.int32)
+    assert bool(((w & 0xFFFF) == 0).all())
+    return ((w >> 16) & 0xFFFF).to(torch.int32).numpy().astype(np.uint16)
+
+
+def make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, dtype=torch.float32,
+              lens=None, page_size=0, extend=None, softcap=None, block_size_k=64):
+    """One call of the reference operator; ``lens`` (decode: TQ == 1) places each sequence's query at lens[b] - 1;
+    ``page_size`` > 0 moves K/V into a paged cache behind a shuffled block table; ``extend`` = (scan rule, sa rule)
+    turns on RoPE applied on load."""
+    g = torch.Generator().manual_seed(seed)
+    # values with 8 significant bits, so that the files can hold q, k, v as 16-bit patterns
+    short = lambda t: t.to(torch.bfloat16).to(dtype)  # noqa: E731
+    q = short(torch.randn((B, TQ, H, D), generator=g, dtype=torch.float32) * 0.5)
+    k = short(torch.randn((B, TK, HKV, D), generator=g, dtype=torch.float32))
+    v = short(torch.randn((B, TK, HKV, D), generator=g, dtype=torch.float32))
+    if lens is None:
+        pos = (torch.arange(TQ) + TK - TQ)[None].expand(B, TQ).contiguous()
+    else:
+        pos = (torch.tensor(lens, dtype=torch.int64) - 1)[:, None]
+    kw = dict(sink_token_size=sink, sliding_window_size=sw, second_stage_k=second_k, block_sparse_block_size_q=bsbq,
+              stages=[meta.ScanStage(stage_block_size_q=a, stage_block_stride_q=b, stage_chunk_size=c, stage_k=d,
+                                     stage_stride=e) for (a, b, c, d, e) in stages],
+              require_cache_statistics=False, position_ids=pos, block_size_k=block_size_k)
+    extra = {}
+    if extend is not None:
+        cos, sin = rope_tables(2 * TK, D)
+        kw.update(using_extend=True, need_apply_rope=True, rope_cos=cos.to(dtype), rope_sin=sin.to(dtype),
+                  scan_extend_backend=extend[0], sa_extend_backend=extend[1])
+        extra.update(rope_cos=cos.to(dtype).float().numpy(), rope_sin=sin.to(dtype).float().numpy(),
+                     scan_backend=extend[0], sa_backend=extend[1])
+    if softcap is not None:
+        kw.update(logit_softcap=softcap)
+        extra.update(softcap=softcap)
+    if page_size > 0:
+        per = -(-TK // page_size)
+        npages = B * per + 4
+        perm = (torch.randperm(npages - 1, generator=g)[: B * per] + 1).reshape(B, per)
+        kc = torch.zeros((npages, page_size, HKV, D), dtype=dtype)
+        vc = torch.zeros_like(kc)
+        for b in range(B):
+            for pg in range(per):
+                t0, t1 = pg * page_size, min(TK, (pg + 1) * page_size)
+                kc[perm[b, pg], : t1 - t0] = k[b, t0:t1]
+                vc[perm[b, pg], : t1 - t0] = v[b, t0:t1]
+        seq = pos.max(dim=1).values + 1
+        kw.update(k_cache=kc, v_cache=vc, block_table=perm.to(torch.int64), cache_seq_lens=seq.to(torch.int64),
+                  extend_context_length=TK)
+        extra.update(k_cache=bits16(kc), v_cache=bits16(vc), block_table=perm.numpy(),
+                     cache_seq_lens=seq.numpy(), page_size=page_size)
+        args = meta.HiPAttentionArgs(**kw)
+        ctx, md = ext.dual_stage_quadratic_hip_attention(q, None, None, args=args)
+    else:
+        args = meta.HiPAttentionArgs(**kw)
+        ctx, md = ext.dual_stage_quadratic_hip_attention(q, k, v, args=args)
+    path = os.path.join(HERE, f"reference_{name}.npz")
+    if page_size > 0:  # the cache and the block table hold the same rows
+        extra.update(max_tsrc=TK)
+    else:
+        extra.update(k=bits16(k), v=bits16(v))
+    np.savez_compressed(
+        path, q=bits16(q), pos=pos.numpy(),
+        context=ctx.float().numpy(), indices=md.indices.numpy(), ks=md.ks.numpy(), ks_start_end=md.ks_start_end.numpy(),
+        stages=np.array([[-1 if x is None else x for x in s] for s in stages], dtype=np.int64),
+        sink=sink, sw=sw, second_k=second_k, bsbq=bsbq, bf16=int(dtype == torch.bfloat16), block_size_k=block_size_k,
+        **extra)
+    print("wrote", path, "context", tuple(ctx.shape), "indices", tuple(md.indices.shape), flush=True)
+
+
+def main():
+    root = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+    only = sys.argv[2:] or None
+    ext, meta = load_reference(root)
+    tiny = [(32, 2, 64, None, 1), (32, 2, 16, 2048, 1), (32, 1, 2, 1024, 1)]
+    strided = [(64, 4, 64, None, 2), (32, 2, 16, 1024, 1), (32, 1, 4, 512, 1)]
+    default = [(64, 4, 256, None, 1), (64, 4, 32, 32768, 1), (64, 1, 8, 8192, 1)]
+    cases = {
+        # name: (seed, B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, extras)
+        "f32_prefill_tiny": (0, 1, 64, 1024, 2, 1, 32, tiny, 16, 256, 512, 32, {}),
+        "f32_prefill_gqa_ragged": (1, 2, 80, 1536, 4, 2, 32, tiny, 16, 256, 512, 32, {}),
+        "f32_decode_paged": (2, 2, 1, 2048, 4, 2, 32, tiny, 16, 256, 512, 32, dict(lens=[2048, 1500], page_size=8)),
+        "f32_prefill_rope_relative": (3, 1, 64, 1024, 2, 1, 32, tiny, 16, 256, 512, 32, dict(extend=("relative", "streaming"))),
+        "f32_prefill_rope_streaming": (4, 1, 64, 1024, 2, 1, 32, tiny, 16, 256, 512, 32, dict(extend=("streaming", "streaming"))),
+        "f32_decode_rope_infllm": (5, 2, 1, 1536, 4, 2, 32, tiny, 16, 256, 512, 32,
+                                   dict(lens=[1536, 1100], extend=("infllm", "infllm"))),
+        "f32_prefill_stride_d64": (8, 1, 128, 2048, 4, 2, 64, strided, 32, 128, 256, 32, {}),
+        "f32_decode_default_stages": (9, 1, 1, 8192, 2, 1, 32, default, 256, 512, 2048, 64, {}),
+        # Not generated: Triton's interpreter has no bfloat16 constants (``get_bf16``) and cannot call
+        # ``libdevice.tanh`` (logit_softcap) outside a compiled kernel, so bfloat16 inputs and soft-capped logits
+        # have no vectors from the reference.
+    }
+    for name, (seed, B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, extra) in cases.items():
+        if only and name not in only:
+            continue
+        make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, **extra)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,7 +1,8 @@
 """Committed fixtures (tests/golden/*.npz): the oracle still reproduces them; the GPU path matches them.
 
-The vectors were written by ``tests/golden/make_fixtures.py`` from the CPU oracle (the reference repository ships no
-golden vectors for this path).
+These vectors were written by ``tests/golden/make_fixtures.py`` from the CPU oracle (the reference repository ships
+no golden vectors for this path); ``tests/golden/reference_*.npz``, written by an execution of the reference itself,
+are covered by ``tests/test_golden_reference.py``.
 """
 import glob
 import json
@@ -13,7 +14,7 @@ import pytest
 from oracle import hip12 as O
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
-FILES = sorted(glob.glob(os.path.join(GOLDEN, "*.npz")))
+FILES = sorted(f for f in glob.glob(os.path.join(GOLDEN, "*.npz")) if not os.path.basename(f).startswith("reference_"))
 
 
 def load(path):

@@ -11,7 +11,7 @@ from test_oracle_bsa import random_indices
 pytestmark = pytest.mark.gpu
 
 
-def _run(X, max_tsrc, idx, kse, bq, bk, sw, sink, impl, share=False, decode=False, softcap=None):
+def _run(X, max_tsrc, idx, kse, bq, bk, sw, sink, impl, share=False, decode=False, softcap=None, second_k=0):
     from hip_attn import HiPAttentionArgs12
     from hip_attn.operator import block_sparse_attention
 
@@ -24,6 +24,7 @@ def _run(X, max_tsrc, idx, kse, bq, bk, sw, sink, impl, share=False, decode=Fals
                   cache_seq_lens=torch.from_numpy(X.cache_seq_lens).to(dev))
     args = HiPAttentionArgs12(sink_token_size=sink, sliding_window_size=sw, logit_softcap=softcap, **kw)
     args.block_size_q, args.block_size_k = bq, bk
+    args.second_stage_k = second_k  # decode only: sizes the reference's own split of the index row
     out = block_sparse_attention(q, to_torch(X.k, X.dtype, dev), to_torch(X.v, X.dtype, dev),
                                  torch.from_numpy(X.pos.copy()).to(dev), torch.from_numpy(idx).to(dev),
                                  torch.from_numpy(kse).to(dev), args, max_tsrc, decode=decode, impl=impl,
@@ -78,18 +79,27 @@ def test_tile_kernel_empty_rows_and_early_positions():
     assert_context_close(out, ref, "bf16")
 
 
+@pytest.mark.parametrize("second_k", [0, 320, 2048])
 @pytest.mark.parametrize("dtype,D,G", [("bf16", 128, 4), ("bf16", 64, 2), ("f32", 64, 4), ("bf16", 128, 1)])
-def test_decode_kernel_matches_oracle(dtype, D, G):
-    print(f"[case] decode {dtype} D={D} G={G}", flush=True)
+def test_decode_kernel_matches_oracle(dtype, D, G, second_k):
+    """``second_k`` 0: every selected block once; 320: the reference's programs take 8 index entries each in tiles
+    of 2, no seams; 2048: 5 entries each, so the first entry of every later share is attended twice."""
+    print(f"[case] decode {dtype} D={D} G={G} second_k={second_k}", flush=True)
     rng = np.random.default_rng(D + G)
     B, HKV, TK, bk, BK, sw, sink = 3, 2, 3000, 8, 40, 200, 32
     H = HKV * G
     lens = np.array([3000, 1500, 257])
     X = make_inputs(15, B=B, TQ=1, TK=TK, H=H, HKV=HKV, D=D, dtype=dtype, scale=0.5, pos=(lens - 1)[:, None])
     idx, ks, kse = random_indices(rng, B, H, 1, BK, bk, 1400, same_heads=True)
-    ref = O.bsa(X, TK, idx, kse, 1, bk, sw, sink, share_first_head=True)
-    out = _run(X, TK, idx, kse, 1, bk, sw, sink, impl=0, decode=True)
+    seams = O.decode_seams(second_k, sink, sw, bk, BK) if second_k else (0, 0)
+    assert seams == {0: (0, 0), 320: (8, 0), 2048: (5, 1)}[second_k]
+    ref = O.bsa(X, TK, idx, kse, 1, bk, sw, sink, share_first_head=True, seams=seams)
+    out = _run(X, TK, idx, kse, 1, bk, sw, sink, impl=0, decode=True, second_k=second_k)
     assert_context_close(out, ref, dtype)
+    if seams[1]:
+        once = O.bsa(X, TK, idx, kse, 1, bk, sw, sink, share_first_head=True)
+        w = (lambda a: O.bf16_bits_to_f32(a)) if dtype == "bf16" else (lambda a: a)
+        assert np.abs(w(ref) - w(once)).max() > 0.025  # the seams matter on this input
 
 
 @pytest.mark.parametrize("dtype,D", [("bf16", 128), ("bf16", 64), ("f32", 64)])

@@ -77,12 +77,14 @@ def test_batched_paged_decode(page_size):
     ctx2, meta2 = run_product(X, A, cached=meta)
     assert torch.equal(meta2.indices, meta.indices)
     assert_context_close(ctx2, octx, "bf16")
-    # prefill kernel on the same decode problem agrees with the split-KV path
+    # the query-block kernel on the same decode problem (it attends every selected block once, while the decode
+    # path repeats the reference's double visit of the blocks at the seams of its programs: 6 programs of 43 index
+    # entries walked in tiles of 2 here)
+    assert O.decode_seams(A.second_stage_k, A.sink_token_size, 512, 8, 256) == (43, 1)
     A2 = copy.deepcopy(A); A2.disable_flashdecode = True
     ctx3, _ = run_product(X, A2)
     octx3, _ = O.hip_attention_12(X, A2)
     assert_context_close(ctx3, octx3, "bf16")
-    assert_context_close(ctx3, octx, "bf16")
 
 
 @pytest.mark.parametrize("force", ["0", "1"])

@@ -7,12 +7,12 @@ from oracle import hip12 as O
 from helpers import make_inputs, to_paged, widen
 
 
-def dense_reference(X, indices, ks, bq, bk, sw, sink, max_tsrc, share_first_head=False, softcap=None):
+def dense_reference(X, indices, ks, bq, bk, sw, sink, max_tsrc, share_first_head=False, softcap=None, visits=None):
     """softmax over the attended set written as an explicit boolean mask, float64 arithmetic.
 
     Built from the set definition only (no tiling): sink tokens and selected-block tokens at
     distance >= sw from the query, window tokens at distance < sw, everything clipped by the
-    query block's largest position.
+    query block's largest position.  ``visits[j]``: weight of the tokens of index entry j (default 1).
     """
     B, TQ, H, D = X.q.shape
     k = widen(X.k, X.dtype).astype(np.float64)
@@ -34,9 +34,12 @@ def dense_reference(X, indices, ks, bq, bk, sw, sink, max_tsrc, share_first_head
                 p = X.pos[b, rows]
                 curr = p.max() + 1
                 sel = np.zeros(TK, dtype=bool)
+                weight = np.ones(TK)
                 for j in range(int(ks[b * H + hrow, qb])):
                     st = int(indices[b * H + hrow, qb, j])
                     sel[max(st, 0): max(min(st + bk, TK, max_tsrc), 0)] = True
+                    if visits is not None:
+                        weight[max(st, 0): max(min(st + bk, TK, max_tsrc), 0)] = visits[j]
                 sel &= (t >= sink)
                 far = (t[None, :] + sw <= p[:, None]) & (t[None, :] < curr)
                 near = (t[None, :] <= p[:, None]) & (t[None, :] + sw > p[:, None]) & \
@@ -48,7 +51,7 @@ def dense_reference(X, indices, ks, bq, bk, sw, sink, max_tsrc, share_first_head
                 logits = np.where(mask, logits, -np.inf)
                 m = logits.max(axis=1, keepdims=True)
                 m = np.where(np.isfinite(m), m, 0.0)
-                pr = np.exp(logits - m)
+                pr = np.exp(logits - m) * np.where(near, 1.0, weight[None, :])
                 den = pr.sum(axis=1, keepdims=True)
                 den = np.where(den == 0, 1.0, den)
                 out[b, rows, h] = (pr / den) @ v[b, :, h // G]
@@ -153,3 +156,62 @@ def test_logit_softcap_is_tanh_capping_of_the_logits(dtype, tol):
     want = dense_reference(X, idx, ks, bq, bk, sw, sink, TK, softcap=2.0)
     assert np.abs(got - want).max() <= tol
     assert np.abs(got - plain).max() > 10 * tol  # the cap matters at this scale
+
+
+def programs_walk(BK, second_k, sink, sw, bk, rs, re):
+    """How often each entry of an index row is visited when the decode kernel's programs run their loops as written
+    (attention_decode_bsa.py:239-247) with the launcher's constants (:1070-1076, :1391-1393)."""
+    counts = np.zeros(BK, dtype=np.int64)
+    chunk = O.cdiv(second_k + sink + sw, 8)
+    programs = min(12, O.cdiv(second_k, chunk))
+    tile = max(1, min(16, 16 // bk))
+    share = O.cdiv(BK, programs)
+    for s in range(programs):
+        start, end = share * s, min(share * s + share, BK)
+        if end > start:
+            for i in range(start, end, tile):
+                for j in range(i, i + tile):
+                    if rs <= j < min(rs + BK, re):
+                        counts[j] += 1
+    return counts
+
+
+def test_seam_multiplicity_equals_a_walk_of_the_programs():
+    rng = np.random.default_rng(0)
+    seen = set()
+    for _ in range(400):
+        bk = int(rng.choice([1, 2, 4, 8, 16, 32, 64]))
+        BK = int(rng.integers(1, 300))
+        second_k = int(rng.choice([BK * bk, 2048, 512, 128, 4096]))
+        sink, sw = int(rng.choice([0, 4, 128, 256])), int(rng.choice([0, 64, 1024, 4096]))
+        re = int(rng.integers(0, BK + 1))
+        want = programs_walk(BK, second_k, sink, sw, bk, 0, re)
+        share, over = O.decode_seams(second_k, sink, sw, bk, BK)
+        got = np.array([O.seam_multiplicity(j, share, over) if j < re else 0 for j in range(BK)])
+        assert np.array_equal(got, want), (BK, second_k, sink, sw, bk, re)
+        seen.add(int(want.max(initial=0)))
+    assert {1, 2, 3} <= seen  # plain, doubled and (tiny rows) tripled entries all occurred
+    # the reference's default preset: 2048 tokens in blocks of 8 among 5 programs of 52 entries, tiles of 2 -> no seams
+    assert O.decode_seams(2048, 256, 1024, 8, 256) == (52, 0)
+
+
+@pytest.mark.parametrize("dtype,tol", [("f32", 2e-5), ("bf16", 1.5e-2)])
+def test_decode_seams_weigh_the_blocks_at_the_seams_twice(dtype, tol):
+    rng = np.random.default_rng(8)
+    TK, H, HKV, D, bk, BK, sw, sink, second_k = 512, 4, 2, 32, 2, 40, 24, 8, 80
+    lens = np.array([512, 300])
+    X = make_inputs(9, B=2, TQ=1, TK=TK, H=H, HKV=HKV, D=D, dtype=dtype, scale=0.3, pos=(lens - 1)[:, None])
+    idx, ks, kse = random_indices(rng, 2, H, 1, BK, bk, 280, same_heads=True)
+    ks[:] = BK - 3
+    kse[..., 1] = BK - 3
+    for r in range(idx.shape[0]):
+        idx[r, 0] = np.sort(rng.choice(280 // bk, size=BK, replace=False)) * bk
+    seams = O.decode_seams(second_k, sink, sw, bk, BK)
+    assert seams == (7, 1)  # 6 programs of 7 entries walking tiles of 8: 1 entry of overhang
+    visits = programs_walk(BK, second_k, sink, sw, bk, 0, BK - 3)
+    assert visits.max() == 2 and visits[:BK - 3].min() == 1
+    got = widen(O.bsa(X, TK, idx, kse, 1, bk, sw, sink, share_first_head=True, seams=seams), dtype)
+    ref = dense_reference(X, idx, ks, 1, bk, sw, sink, TK, share_first_head=True, visits=visits)
+    once = dense_reference(X, idx, ks, 1, bk, sw, sink, TK, share_first_head=True)
+    assert np.abs(got - ref).max() < tol
+    assert np.abs(ref - once).max() > 5 * tol

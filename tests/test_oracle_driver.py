@@ -115,9 +115,20 @@ def test_stage_cache_replay_and_cached_indices_reuse():
 def test_decode_shape_and_flashdecode_head_sharing_is_neutral_under_head_reduce():
     X = make_inputs(3, B=3, TQ=1, TK=1500, H=4, HKV=2, D=32, dtype="bf16",
                     pos=np.array([[1499], [700], [1200]]))
-    A = tiny_args(sliding_window_size=128, second_stage_k=64)
+    # window 256: the decode kernel's 2 programs take 16 index entries each, a whole number of their tiles of 8
+    A = tiny_args(sliding_window_size=256, second_stage_k=64)
+    assert O.decode_seams(64, A.sink_token_size, 256, 2, 32) == (16, 0)
     ctx, meta = O.hip_attention_12(X, A)
     assert meta.indices.shape == (12, 1, 32) and ctx.shape == (3, 1, 4, 32)
     A.disable_flashdecode = True
     ctx2, meta2 = O.hip_attention_12(X, A)
     assert np.array_equal(meta.indices, meta2.indices) and np.array_equal(ctx, ctx2)
+    # window 128: 3 programs of 11 entries, each walking 16: five entries per seam are attended twice, and the
+    # decode kernel's output departs from the query-block kernel's
+    A = tiny_args(sliding_window_size=128, second_stage_k=64)
+    assert O.decode_seams(64, A.sink_token_size, 128, 2, 32) == (11, 5)
+    ctx, meta = O.hip_attention_12(X, A)
+    A.disable_flashdecode = True
+    ctx2, meta2 = O.hip_attention_12(X, A)
+    assert np.array_equal(meta.indices, meta2.indices)
+    assert np.abs(O.bf16_bits_to_f32(ctx) - O.bf16_bits_to_f32(ctx2)).max() > 0.02
