@@ -21,6 +21,10 @@ struct BsaParamsBase {
     // masks a program's last tile against the end of the row only, so the first `seam_extra` entries of the next
     // program's share are attended once more (attention_decode_bsa.py:239-247); 0 / 0 = every entry once.
     int seam_blocks, seam_extra;
+    // Decode with the "streaming" rotation rule only: the reference's decode programs take `sink_share` sink tokens
+    // each and number them from their first token rounded down to a multiple of the block size
+    // (attention_decode_bsa.py:514-518, 740), so a token is rotated (share start % bk) positions lower; 0 = off.
+    int sink_share;
     int B, TDST, HEAD, G, NBQ;
     float c_q, c_k;
     void *out;
@@ -45,6 +49,10 @@ __host__ __device__ __forceinline__ int bsa_seam_multiplicity(int j, int seam_bl
     const int s = j / seam_blocks, r = j - s * seam_blocks;
     const int earlier = (seam_blocks + seam_extra - r - 1) / seam_blocks;
     return 1 + (earlier < s ? earlier : s);
+}
+// The number under which the reference's decode kernel rotates sink token t.
+__host__ __device__ __forceinline__ long long bsa_decode_sink_slot(long long t, int sink_share, int bk) {
+    return sink_share > 0 ? t - ((t / sink_share) * sink_share) % bk : t;
 }
 // Rotated position of a sink or selected key (attention_extend_bsa.py:256-299): "streaming" packs them, in the
 // order of the index row, into the positions that end just below the window of the block's first query;

@@ -109,7 +109,8 @@ __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<E
             } else if (o < n_sel_tok + sink_end) {
                 t = o - n_sel_tok;
                 valid = true;
-                if constexpr (ROPE) rpos = bsa_rope_far_pos(p.rope, t, rope_shift, ppos, p.sw);
+                if constexpr (ROPE)
+                    rpos = bsa_rope_far_pos(p.rope, bsa_decode_sink_slot(t, p.sink_share, p.bk), rope_shift, ppos, p.sw);
             } else {
                 t = ws0 + (o - n_sel_tok - sink_end);
                 kind = 1;
@@ -324,17 +325,24 @@ extern "C" int hipattn_bsa_decode_partial(const hipattn_q_t *q, const hipattn_kv
     if (rc) return rc;
     HIPATTN_CHECK_ARG(q->TDST == 1, HIPATTN_E_ARG, "decode: TDST must be 1, got %d", q->TDST);
     HIPATTN_CHECK_ARG(second_stage_k >= 0, HIPATTN_E_ARG, "decode: negative second_stage_k");
-    if (second_stage_k > 0 && BK > 0) {
-        // the reference launcher's own division of the index row (attention_decode_bsa.py:1070-1076, 1391-1393)
+    if (second_stage_k > 0) {
+        // the reference launcher's own division of the work among its programs (attention_decode_bsa.py:1070-1077)
         const int64_t total = (int64_t)second_stage_k + sink + sliding_window;
         const int64_t chunk = (total + 7) / 8;
-        int64_t programs = (second_stage_k + chunk - 1) / chunk;
-        if (programs > 12) programs = 12;
-        int tile = 16 / block_size_k;
-        tile = tile < 1 ? 1 : tile;
-        const int share = (int)((BK + programs - 1) / programs);
-        dp.a.seam_blocks = share;
-        dp.a.seam_extra = (share + tile - 1) / tile * tile - share;
+        if (BK > 0) {  // programs over the index row, walking tiles of 16 / block_size_k entries (:1391-1393, :239-247)
+            int64_t programs = (second_stage_k + chunk - 1) / chunk;
+            if (programs > 12) programs = 12;
+            int tile = 16 / block_size_k;
+            tile = tile < 1 ? 1 : tile;
+            const int share = (int)((BK + programs - 1) / programs);
+            dp.a.seam_blocks = share;
+            dp.a.seam_extra = (share + tile - 1) / tile * tile - share;
+        }
+        if (sink > 0) {  // programs over the sink (:514-518)
+            int64_t sink_programs = (sink + chunk - 1) / chunk;
+            if (sink_programs > 12) sink_programs = 12;
+            dp.a.sink_share = (int)((sink + sink_programs - 1) / sink_programs);
+        }
     }
     dp.nsplits = nsplits;
     dp.ws = reinterpret_cast<float *>(workspace);

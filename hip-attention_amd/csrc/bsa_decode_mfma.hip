@@ -141,7 +141,8 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
                     rpos = bsa_rope_far_pos(p.rope, (long long)(rs + bi + p.sink / p.bk) * p.bk + e, rope_shift, ppos, p.sw);
             } else if (o < n_sel_tok + sink_end) {
                 t = o - n_sel_tok;
-                if constexpr (ROPE) rpos = bsa_rope_far_pos(p.rope, t, rope_shift, ppos, p.sw);
+                if constexpr (ROPE)
+                    rpos = bsa_rope_far_pos(p.rope, bsa_decode_sink_slot(t, p.sink_share, p.bk), rope_shift, ppos, p.sw);
             } else {
                 t = (int)ws0 + (o - n_sel_tok - sink_end);
                 win = 1;

@@ -210,7 +210,7 @@ int bsa_fill_params(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t 
     p->indices = indices; p->kse = kse; p->idx_rows = idx_rows; p->BK = BK; p->bq = bq; p->bk = bk;
     p->sw = sw; p->sink = sink; p->share_first_head = share_first_head;
     p->k_prescaled = 0;
-    p->seam_blocks = 0; p->seam_extra = 0;
+    p->seam_blocks = 0; p->seam_extra = 0; p->sink_share = 0;
     p->B = q->B; p->TDST = q->TDST; p->HEAD = q->HEAD; p->G = q->HEAD / p->kv.HKV;
     p->NBQ = (q->TDST + bq - 1) / bq;
     HIPATTN_CHECK_ARG(p->NBQ <= idx_rows, HIPATTN_E_ARG, "bsa: %d query blocks but only %d index rows", p->NBQ, idx_rows);

@@ -215,7 +215,11 @@ int hipattn_bsa_prefill(const hipattn_q_t *q, const hipattn_kv_t *kv, const int6
  *   that walk their share in tiles of 16 / block_size_k entries (:1391-1393) and mask a tile against the end of the
  *   row only (:239-247): when the share is not a whole number of tiles, the entries at the start of the next share
  *   are attended twice.  With second_stage_k > 0 those entries get the same weight here, so the output equals the
- *   reference's; with 0 every selected block counts once. */
+ *   reference's; with 0 every selected block counts once.  The sink is likewise divided among
+ *   min(12, ceil(sink / ceil((second_stage_k + sink + window) / 8))) programs (:1077, :514-518), each numbering its
+ *   tokens from its first token rounded down to a multiple of block_size_k (:740); under the "streaming" rotation
+ *   rule a sink token is therefore rotated (share start % block_size_k) positions lower than its own number, which
+ *   second_stage_k > 0 reproduces as well. */
 int64_t hipattn_bsa_decode_workspace_bytes(int32_t B, int32_t HEAD, int32_t HID, int32_t nsplits);
 int32_t hipattn_bsa_decode_default_splits(int32_t B, int32_t HKV, int32_t tokens);
 int hipattn_bsa_decode_partial(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t *indices,

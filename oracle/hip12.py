@@ -278,14 +278,24 @@ def decode_seams(second_stage_k: int, sink: int, sw: int, block_size_k: int, BK:
     return share, cdiv(share, tile) * tile - share
 
 
+def decode_sink_share(second_stage_k: int, sink: int, sw: int) -> int:
+    """Sink tokens per program of the decode kernel: ``min(12, ceil(sink / ceil((second_stage_k + sink + sw) / 8)))``
+    programs (attention_decode_bsa.py:1077) share the sink evenly (:514)."""
+    chunk = cdiv(second_stage_k + sink + sw, 8)
+    if sink <= 0 or chunk <= 0:
+        return 0
+    return cdiv(sink, min(12, cdiv(sink, chunk)))
+
+
 def seam_multiplicity(j: int, share: int, overhang: int) -> int:
     return int(lib().hipo_seam_multiplicity(ctypes.c_int(j), ctypes.c_int(share), ctypes.c_int(overhang)))
 
 
 def bsa(X: OInputs, max_tsrc, indices, ks_start_end, block_size_q, block_size_k, sw, sink,
-        share_first_head=False, seams=(0, 0)):
+        share_first_head=False, seams=(0, 0), sink_share=0):
     """Block-sparse attention given indices; returns context with q's shape and dtype.  ``seams``: see
-    ``decode_seams`` (decode only; ``(0, 0)`` attends every selected block once)."""
+    ``decode_seams`` (decode only; ``(0, 0)`` attends every selected block once); ``sink_share``: see
+    ``decode_sink_share`` (decode with the streaming rotation rule only; 0 numbers sink tokens by themselves)."""
     S, keep = X.c_struct(max_tsrc)
     indices = np.ascontiguousarray(indices, dtype=np.int64)
     kse = np.ascontiguousarray(ks_start_end, dtype=np.int32)
@@ -294,7 +304,8 @@ def bsa(X: OInputs, max_tsrc, indices, ks_start_end, block_size_q, block_size_k,
                         ctypes.c_int(indices.shape[1]), ctypes.c_int(indices.shape[2]),
                         ctypes.c_int(block_size_q), ctypes.c_int(block_size_k), ctypes.c_int(sw),
                         ctypes.c_int(sink), ctypes.c_int(1 if share_first_head else 0),
-                        ctypes.c_int(seams[0]), ctypes.c_int(seams[1]), ctypes.c_void_p(out.ctypes.data))
+                        ctypes.c_int(seams[0]), ctypes.c_int(seams[1]), ctypes.c_int(sink_share),
+                        ctypes.c_void_p(out.ctypes.data))
     if rc != 0:
         raise RuntimeError(f"hipo_bsa failed: {rc}")
     del keep
@@ -515,8 +526,9 @@ def hip_attention_12(X: OInputs, A: OArgs, cached: Optional[OMetadata] = None):
     X.logit_softcap = float(A.logit_softcap or 0.0)
     try:
         seams = decode_seams(A.second_stage_k, sink, sw_bsa, block_size_k, indices.shape[-1]) if decode else (0, 0)
+        sink_share = decode_sink_share(A.second_stage_k, sink, sw_bsa) if decode else 0
         context = bsa(X, MAX_TSRC, indices, ks_start_end, block_size_q, block_size_k, sw_bsa, sink,
-                      share_first_head=decode, seams=seams)
+                      share_first_head=decode, seams=seams, sink_share=sink_share)
     finally:
         X.access = user_access
         X.logit_softcap = user_cap

@@ -451,6 +451,11 @@ int hipo_mask_stage(const hipo_tensors_t *X, int64_t *left, int64_t *right, floa
  * end of its own share, so the first seam_extra entries of the next share (seam_extra = tile-rounded
  * share - share) enter the softmax once per program that reaches them.  hipo_seam_multiplicity counts
  * those visits; a token visited m times has weight m * exp2(logit - max).
+ * sink_share > 0 restates the decode kernel's numbering of sink tokens for the "streaming" rotation rule: the sink
+ * is divided among programs of sink_share tokens (attention_decode_bsa.py:514-518) and a program numbers its
+ * tokens from its first token rounded down to a multiple of block_size_k (:740, i_tsrc // BLOCK_SIZE_K), so every
+ * token of a program whose share does not start on such a multiple is rotated (start % block_size_k) positions
+ * lower than its own number.
  * Pinned by: dense masked softmax in f64 built from the set definition above
  * (tests/test_oracle_bsa.py), StreamingLLM and plain-causal special cases; the seam rule by an execution
  * of the reference (tests/golden/reference_f32_decode_paged.npz) and by a literal walk of the programs'
@@ -466,7 +471,7 @@ int hipo_seam_multiplicity(int j, int seam_blocks, int seam_extra) {
 int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_start_end,
              int NBQ_rows /* rows of indices per (b,h) */, int BK, int block_size_q,
              int block_size_k, int sw, int sink, int share_first_head, int seam_blocks, int seam_extra,
-             void *out) {
+             int sink_share, void *out) {
     const int B = X->B, TDST = X->TDST, HEAD = X->HEAD, HID = X->HID;
     const int G = HEAD / X->HKV;
     const int NBQ = (TDST + block_size_q - 1) / block_size_q;
@@ -523,7 +528,10 @@ int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_
                 }
             }
             int64_t sink_end = curr < sink ? curr : sink;
-            for (int64_t t = 0; t < sink_end; t++) { tok[nt] = t; kind[nt] = 0; mult[nt] = 1; rpos[nt] = t + shift; nt++; }
+            for (int64_t t = 0; t < sink_end; t++) {
+                int64_t slip = sink_share > 0 ? ((t / sink_share) * sink_share) % block_size_k : 0;
+                tok[nt] = t; kind[nt] = 0; mult[nt] = 1; rpos[nt] = t - slip + shift; nt++;
+            }
             if (sw > 0) {
                 int64_t ws = curr - sw - block_size_q;
                 if (ws < 0) ws = 0;

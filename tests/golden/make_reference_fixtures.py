@@ -154,6 +154,56 @@ def make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, sec
     print("wrote", path, "context", tuple(ctx.shape), "indices", tuple(md.indices.shape), flush=True)
 
 
+def make_paged_api_case(name, seed, B, TQ, TK, H, HKV, D, lens, spec, layer_ids, orig_context_len, rope):
+    """``forward_paged_hip`` (the serving entry point, paged_hip.py:35-320) on a token-granular pool: one call per
+    layer id, and for decode a second call that hands the first call's metadata back."""
+    import hip_attn.v1_2.paged_hip as paged
+    from hip_attn.v1_2.hip_config import HiPAttentionConfig
+
+    g = torch.Generator().manual_seed(seed)
+    short = lambda t: t.to(torch.bfloat16).float()  # noqa: E731
+    q = short(torch.randn((B, TQ, H, D), generator=g) * 0.5)
+    k = short(torch.randn((B, TK, HKV, D), generator=g))
+    v = short(torch.randn((B, TK, HKV, D), generator=g))
+    lens_t = torch.tensor(lens, dtype=torch.int64)
+    pos = (lens_t[:, None] - TQ + torch.arange(TQ)[None, :]).contiguous()
+    slots = (torch.randperm(B * TK + 7, generator=g)[: B * TK] + 1).reshape(B, TK)
+    kc = torch.zeros((B * TK + 8, HKV, D))
+    vc = torch.zeros_like(kc)
+    for b in range(B):
+        kc[slots[b]] = k[b]
+        vc[slots[b]] = v[b]
+    req_to_tokens = torch.zeros((B + 3, TK), dtype=torch.int32)
+    pool_idx = torch.tensor([2, 0, 4][:B])
+    req_to_tokens[pool_idx] = slots.to(torch.int32)
+    cfg = HiPAttentionConfig(json_or_path=spec)
+    cos = sin = None
+    out = {}
+    if rope:
+        cos, sin = rope_tables(2 * TK, D)
+        cos, sin = short(cos), short(sin)
+        out.update(rope_cos=bits16(cos), rope_sin=bits16(sin))
+    decode = TQ == 1
+    for layer_id in layer_ids:
+        kw = dict(sm_scale=D ** -0.5, batch_size=B, k_cache=kc, v_cache=vc, offload_cache=None,
+                  positions=pos.reshape(-1), seq_lens=lens_t, req_to_tokens=req_to_tokens, req_pool_indices=pool_idx,
+                  rope_cos=cos, rope_sin=sin, layer_id=layer_id, logit_cap=0.0, orig_context_len=orig_context_len,
+                  max_context_len=TK, is_prefill=not decode, hip_config=cfg, is_decode=decode)
+        o, md = paged.forward_paged_hip(q.reshape(B * TQ, H, D), **kw)
+        out[f"o_{layer_id}"] = o.float().numpy()
+        out[f"indices_{layer_id}"] = md.indices.numpy()
+        out[f"ks_{layer_id}"] = md.ks.numpy()
+        if decode:
+            o2, _ = paged.forward_paged_hip(q.reshape(B * TQ, H, D), cached_metadata=md, **kw)
+            out[f"o_cached_{layer_id}"] = o2.float().numpy()
+    path = os.path.join(HERE, f"reference_{name}.npz")
+    np.savez_compressed(path, q=bits16(q), k_cache=bits16(kc), v_cache=bits16(vc), positions=pos.numpy(),
+                        seq_lens=lens_t.numpy(), req_to_tokens=req_to_tokens.numpy(), req_pool_indices=pool_idx.numpy(),
+                        spec=np.frombuffer(spec.encode(), dtype=np.uint8), layer_ids=np.array(layer_ids),
+                        orig_context_len=orig_context_len, max_context_len=TK, TQ=TQ, **out)
+    print("wrote", path, flush=True)
+
+
 def main():
     root = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
     only = sys.argv[2:] or None
@@ -180,6 +230,18 @@ def main():
         if only and name not in only:
             continue
         make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, **extra)
+    layers = ('"dense_layers": [0], "layers": [{"second_stage_k": 256, "sliding_window_size": 256}, '
+              '{"second_stage_k": 128, "sliding_window_size": 256}], "prefill_layers": [{"second_stage_k": 256, '
+              '"sliding_window_size": 256}, {"second_stage_k": 128, "sliding_window_size": 256}]')
+    api_cases = {
+        # name: (seed, B, TQ, TK, H, HKV, D, lens, config, layer ids, orig_context_len, rope tables)
+        "f32_paged_api_prefill": (20, 1, 192, 2048, 4, 2, 32, [2048], '{"using_extend": false, %s}' % layers, [7], 4096, False),
+        "f32_paged_api_decode_rope": (21, 2, 1, 3072, 4, 2, 32, [3072, 2000], "{%s}" % layers, [0, 5], 131072, True),
+    }
+    for name, spec in api_cases.items():
+        if only and name not in only:
+            continue
+        make_paged_api_case(name, *spec)
 
 
 if __name__ == "__main__":

@@ -14,7 +14,9 @@ import pytest
 from oracle import hip12 as O
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-FIXTURES = sorted(glob.glob(os.path.join(HERE, "golden", "reference_*.npz")))
+_ALL = sorted(glob.glob(os.path.join(HERE, "golden", "reference_*.npz")))
+FIXTURES = [f for f in _ALL if "_paged_api_" not in f]      # calls of dual_stage_quadratic_hip_attention
+API_FIXTURES = [f for f in _ALL if "_paged_api_" in f]      # calls of forward_paged_hip
 
 
 def load_case(path):
@@ -43,11 +45,12 @@ def load_case(path):
 
 
 def test_fixtures_are_present():
-    names = {os.path.basename(f) for f in FIXTURES}
+    names = {os.path.basename(f) for f in _ALL}
     assert {"reference_f32_prefill_tiny.npz", "reference_f32_prefill_gqa_ragged.npz", "reference_f32_decode_paged.npz",
             "reference_f32_prefill_rope_relative.npz", "reference_f32_prefill_rope_streaming.npz",
             "reference_f32_decode_rope_infllm.npz", "reference_f32_prefill_stride_d64.npz",
-            "reference_f32_decode_default_stages.npz"} <= names
+            "reference_f32_decode_default_stages.npz", "reference_f32_paged_api_prefill.npz",
+            "reference_f32_paged_api_decode_rope.npz"} <= names
 
 
 @pytest.mark.parametrize("path", FIXTURES, ids=[os.path.basename(f)[10:-4] for f in FIXTURES])
@@ -76,3 +79,97 @@ def test_gpu_reproduces_the_reference_run(path):
     assert np.array_equal(meta.ks_start_end.cpu().numpy(), d["ks_start_end"])
     want = O.f32_to_bf16_bits(d["context"]) if dtype == "bf16" else d["context"]
     assert_context_close(ctx, want, dtype)
+
+
+# ---------------------------------------------------------------- forward_paged_hip (paged_hip.py:35-320)
+
+def _widen16(a):
+    return (a.astype(np.uint32) << 16).view(np.float32)
+
+
+def _api_oracle_inputs(d, layer_id):
+    """The arguments ``_forward_paged_hip`` builds for this layer (paged_hip.py:356-452), as oracle inputs."""
+    import json
+
+    spec = json.loads(bytes(d["spec"]).decode())
+    TQ = int(d["TQ"])
+    kc, vc = _widen16(d["k_cache"]), _widen16(d["v_cache"])
+    q = _widen16(d["q"])
+    B, _, H, D = q.shape
+    dense = layer_id in spec["dense_layers"]
+    layer = spec["layers" if TQ == 1 else "prefill_layers"][0 if dense else 1]
+    q = (q * np.float32(D ** -0.5)).astype(np.float32)
+    X = O.OInputs("f32", q, d["positions"].astype(np.int64), k_cache=np.ascontiguousarray(kc[:, None]),
+                  v_cache=np.ascontiguousarray(vc[:, None]),
+                  block_table=d["req_to_tokens"][d["req_pool_indices"]].astype(np.int64),
+                  cache_seq_lens=d["seq_lens"].astype(np.int64))
+    kw = dict(sliding_window_size=layer["sliding_window_size"], second_stage_k=layer["second_stage_k"],
+              extend_context_length=int(d["max_context_len"]), model_context_length=int(d["orig_context_len"]),
+              disable_flashdecode=TQ != 1)
+    if spec.get("using_extend", True):
+        X.rope_cos, X.rope_sin = _widen16(d["rope_cos"]), _widen16(d["rope_sin"])
+        kw.update(using_extend=True, need_apply_rope=True, scan_extend_backend="streaming" if dense else "relative",
+                  sa_extend_backend="streaming")
+    return X, O.OArgs(**kw)
+
+
+def _sub(X, sl):
+    Y = O.OInputs(X.dtype, np.ascontiguousarray(X.q[:, sl]), np.ascontiguousarray(X.pos[:, sl]), k_cache=X.k_cache,
+                  v_cache=X.v_cache, block_table=X.block_table, cache_seq_lens=X.cache_seq_lens)
+    Y.rope_cos, Y.rope_sin = X.rope_cos, X.rope_sin
+    return Y
+
+
+@pytest.mark.parametrize("path", API_FIXTURES, ids=[os.path.basename(f)[10:-4] for f in API_FIXTURES])
+def test_oracle_reproduces_the_serving_entry_point(path):
+    d = np.load(path)
+    TQ = int(d["TQ"])
+    for layer_id in d["layer_ids"]:
+        X, A = _api_oracle_inputs(d, int(layer_id))
+        B, _, H, D = X.q.shape
+        want = d[f"o_{layer_id}"].reshape(B, TQ, H, D)
+        if TQ == 1 or TQ < 128:
+            ctx, meta = O.hip_attention_12(X, A)
+        else:  # the last 64 queries are served by a second call whose window takes what the context length leaves
+            ctx1, _ = O.hip_attention_12(_sub(X, slice(None, -64)), A)
+            ctx2, meta = O.hip_attention_12(_sub(X, slice(-64, None)), O.OArgs(**{**A.__dict__, "sliding_window_size": 777}))
+            ctx = np.concatenate([ctx1, ctx2], axis=1)
+        assert np.array_equal(meta.indices, d[f"indices_{layer_id}"])
+        assert np.array_equal(meta.ks, d[f"ks_{layer_id}"])
+        assert np.abs(ctx - want).max() <= 5e-5, np.abs(ctx - want).max()
+        if TQ == 1:
+            ctx2, _ = O.hip_attention_12(X, A, cached=meta)
+            assert np.abs(ctx2 - d[f"o_cached_{layer_id}"].reshape(B, 1, H, D)).max() <= 5e-5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("path", API_FIXTURES, ids=[os.path.basename(f)[10:-4] for f in API_FIXTURES])
+def test_gpu_reproduces_the_serving_entry_point(path):
+    import torch
+
+    from gpu_utils import assert_context_close
+    from hip_attn import HiPAttentionConfig, forward_paged_hip
+
+    print(f"[case] reference serving call {os.path.basename(path)}", flush=True)
+    d = np.load(path)
+    TQ = int(d["TQ"])
+    dev = "cuda"
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)  # noqa: E731
+    q = t(_widen16(d["q"]))
+    B, _, H, D = q.shape
+    cfg = HiPAttentionConfig(json_or_path=bytes(d["spec"]).decode())
+    rope = "rope_cos" in d.files
+    kw = dict(sm_scale=D ** -0.5, batch_size=B, k_cache=t(_widen16(d["k_cache"])), v_cache=t(_widen16(d["v_cache"])),
+              offload_cache=None, positions=t(d["positions"].reshape(-1)), seq_lens=t(d["seq_lens"]),
+              req_to_tokens=t(d["req_to_tokens"]), req_pool_indices=t(d["req_pool_indices"]),
+              rope_cos=t(_widen16(d["rope_cos"])) if rope else None, rope_sin=t(_widen16(d["rope_sin"])) if rope else None,
+              logit_cap=0.0, orig_context_len=int(d["orig_context_len"]), max_context_len=int(d["max_context_len"]),
+              is_prefill=TQ != 1, hip_config=cfg, is_decode=TQ == 1)
+    for layer_id in d["layer_ids"]:
+        o, meta = forward_paged_hip(q.reshape(B * TQ, H, D), layer_id=int(layer_id), **kw)
+        assert np.array_equal(meta.indices.cpu().numpy(), d[f"indices_{layer_id}"])
+        assert np.array_equal(meta.ks.cpu().numpy(), d[f"ks_{layer_id}"])
+        assert_context_close(o.reshape(B, TQ, H, D), d[f"o_{layer_id}"].reshape(B, TQ, H, D), "f32")
+        if TQ == 1:
+            o2, _ = forward_paged_hip(q.reshape(B * TQ, H, D), layer_id=int(layer_id), cached_metadata=meta, **kw)
+            assert_context_close(o2.reshape(B, TQ, H, D), d[f"o_cached_{layer_id}"].reshape(B, TQ, H, D), "f32")

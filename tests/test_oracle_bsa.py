@@ -215,3 +215,30 @@ def test_decode_seams_weigh_the_blocks_at_the_seams_twice(dtype, tol):
     once = dense_reference(X, idx, ks, 1, bk, sw, sink, TK, share_first_head=True)
     assert np.abs(got - ref).max() < tol
     assert np.abs(ref - once).max() > 5 * tol
+
+
+def test_sink_numbering_of_the_decode_programs_equals_a_walk_of_their_loops():
+    """attention_decode_bsa.py:514-520 and :740: a program over the sink starts at ``share * s``, steps by its tile of
+    ``BLOCK_BK * bk`` tokens and numbers the tile's entries ``arange(BLOCK_BK) + i_tsrc // bk``."""
+    rng = np.random.default_rng(1)
+    slipped = 0
+    for _ in range(200):
+        bk = int(rng.choice([1, 2, 4, 8, 16, 32, 64]))
+        sink = int(rng.choice([4, 16, 100, 256, 1024]))
+        second_k, sw = int(rng.choice([128, 256, 2048])), int(rng.choice([0, 256, 1024]))
+        chunk = O.cdiv(second_k + sink + sw, 8)
+        programs = min(12, O.cdiv(sink, chunk))
+        share = O.cdiv(sink, programs)
+        assert share == O.decode_sink_share(second_k, sink, sw)
+        block_bk = max(1, min(16, 16 // bk))
+        slot = np.full(sink, -1, dtype=np.int64)
+        for s in range(programs):
+            start, end = share * s, min(share * s + share, sink)
+            for i in range(start, end, block_bk * bk):
+                for x in range(block_bk * bk):
+                    if i + x < end:
+                        slot[i + x] = (x // bk + i // bk) * bk + x % bk
+        t = np.arange(sink)
+        assert np.array_equal(slot, t - ((t // share) * share) % bk), (bk, sink, second_k, sw)
+        slipped += int((slot != t).any())
+    assert slipped > 20
