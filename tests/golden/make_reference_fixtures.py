@@ -90,8 +90,19 @@ def bits16(t):
     return ((w >> 16) & 0xFFFF).to(torch.int32).numpy().astype(np.uint16)
 
 
+def access_flags(md, suffix):
+    """Which key rows the mask estimation and the attention touched (counters > 0), bit-packed."""
+    out = {}
+    for name, st in (("mask_access", md.mask_cache_statistics), ("sa_access", md.sa_cache_statistics)):
+        if st is not None and st.access_counter is not None:
+            flags = (st.access_counter > 0).numpy()
+            out[f"{name}_shape{suffix}"] = np.array(flags.shape)
+            out[f"{name}{suffix}"] = np.packbits(flags.reshape(-1))
+    return out
+
+
 def make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, dtype=torch.float32,
-              lens=None, page_size=0, extend=None, softcap=None, block_size_k=64):
+              lens=None, page_size=0, extend=None, softcap=None, block_size_k=64, replay=False):
     """One call of the reference operator; ``lens`` (decode: TQ == 1) places each sequence's query at lens[b] - 1;
     ``page_size`` > 0 moves K/V into a paged cache behind a shuffled block table; ``extend`` = (scan rule, sa rule)
     turns on RoPE applied on load."""
@@ -108,7 +119,7 @@ def make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, sec
     kw = dict(sink_token_size=sink, sliding_window_size=sw, second_stage_k=second_k, block_sparse_block_size_q=bsbq,
               stages=[meta.ScanStage(stage_block_size_q=a, stage_block_stride_q=b, stage_chunk_size=c, stage_k=d,
                                      stage_stride=e) for (a, b, c, d, e) in stages],
-              require_cache_statistics=False, position_ids=pos, block_size_k=block_size_k)
+              require_cache_statistics=True, position_ids=pos, block_size_k=block_size_k)
     extra = {}
     if extend is not None:
         cos, sin = rope_tables(2 * TK, D)
@@ -140,6 +151,16 @@ def make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, sec
     else:
         args = meta.HiPAttentionArgs(**kw)
         ctx, md = ext.dual_stage_quadratic_hip_attention(q, k, v, args=args)
+    extra.update(access_flags(md, ""))
+    if replay:
+        # restart from the inputs of stage 1 (the chunk list stage 0 produced), as a serving step with a cached
+        # first stage does
+        part = meta.HiPAttentionOutputMetadata(indices=None, ks=None, ks_count=None, ks_start_end=None,
+                                               mask_cache_statistics=None, sa_cache_statistics=None,
+                                               stage_caches=list(md.stage_caches[:2]))
+        kd = (None, None) if page_size > 0 else (k, v)
+        ctx_r, md_r = ext.dual_stage_quadratic_hip_attention(q, *kd, args=meta.HiPAttentionArgs(**kw), cached_metadata=part)
+        extra.update(context_replay=ctx_r.float().numpy(), indices_replay=md_r.indices.numpy())
     path = os.path.join(HERE, f"reference_{name}.npz")
     if page_size > 0:  # the cache and the block table hold the same rows
         extra.update(max_tsrc=TK)
@@ -193,6 +214,7 @@ def make_paged_api_case(name, seed, B, TQ, TK, H, HKV, D, lens, spec, layer_ids,
         out[f"o_{layer_id}"] = o.float().numpy()
         out[f"indices_{layer_id}"] = md.indices.numpy()
         out[f"ks_{layer_id}"] = md.ks.numpy()
+        out.update(access_flags(md, f"_{layer_id}"))
         if decode:
             o2, _ = paged.forward_paged_hip(q.reshape(B * TQ, H, D), cached_metadata=md, **kw)
             out[f"o_cached_{layer_id}"] = o2.float().numpy()
@@ -201,6 +223,25 @@ def make_paged_api_case(name, seed, B, TQ, TK, H, HKV, D, lens, spec, layer_ids,
                         seq_lens=lens_t.numpy(), req_to_tokens=req_to_tokens.numpy(), req_pool_indices=pool_idx.numpy(),
                         spec=np.frombuffer(spec.encode(), dtype=np.uint8), layer_ids=np.array(layer_ids),
                         orig_context_len=orig_context_len, max_context_len=TK, TQ=TQ, **out)
+    print("wrote", path, flush=True)
+
+
+def make_pool_layout_case(name, spec, heads, layers, context_length):
+    """Buffer names, shapes, formats and dtypes of ``HiPMetadataCachePool`` (hip_memory_pool.py:55-222)."""
+    import json
+
+    from hip_attn.v1_2.hip_config import HiPAttentionConfig
+    from hip_attn.v1_2.hip_memory_pool import HiPMetadataCachePool
+
+    cfg = HiPAttentionConfig(json_or_path=spec)
+    pool = HiPMetadataCachePool(max_total_num_tokens=1 << 20, query_head_num=heads, layer_num=layers,
+                                context_length=context_length, device="cpu", hip_config=cfg)
+    layout = [{n: dict(shape=list(b.buffer.shape), store=str(b.buffer.dtype), dtype=str(b.dtype), format=b.batch_format)
+               for n, b in layer.items()} for layer in pool.cache]
+    path = os.path.join(HERE, f"reference_{name}.json")
+    with open(path, "w") as f:
+        json.dump(dict(spec=spec, heads=heads, layers=layers, context_length=context_length, layout=layout,
+                       allocated_bytes=int(pool.allocated_gpu_bytes)), f, indent=1)
     print("wrote", path, flush=True)
 
 
@@ -213,9 +254,9 @@ def main():
     default = [(64, 4, 256, None, 1), (64, 4, 32, 32768, 1), (64, 1, 8, 8192, 1)]
     cases = {
         # name: (seed, B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, extras)
-        "f32_prefill_tiny": (0, 1, 64, 1024, 2, 1, 32, tiny, 16, 256, 512, 32, {}),
+        "f32_prefill_tiny": (0, 1, 64, 1024, 2, 1, 32, tiny, 16, 256, 512, 32, dict(replay=True)),
         "f32_prefill_gqa_ragged": (1, 2, 80, 1536, 4, 2, 32, tiny, 16, 256, 512, 32, {}),
-        "f32_decode_paged": (2, 2, 1, 2048, 4, 2, 32, tiny, 16, 256, 512, 32, dict(lens=[2048, 1500], page_size=8)),
+        "f32_decode_paged": (2, 2, 1, 2048, 4, 2, 32, tiny, 16, 256, 512, 32, dict(lens=[2048, 1500], page_size=8, replay=True)),
         "f32_prefill_rope_relative": (3, 1, 64, 1024, 2, 1, 32, tiny, 16, 256, 512, 32, dict(extend=("relative", "streaming"))),
         "f32_prefill_rope_streaming": (4, 1, 64, 1024, 2, 1, 32, tiny, 16, 256, 512, 32, dict(extend=("streaming", "streaming"))),
         "f32_decode_rope_infllm": (5, 2, 1, 1536, 4, 2, 32, tiny, 16, 256, 512, 32,
@@ -242,6 +283,8 @@ def main():
         if only and name not in only:
             continue
         make_paged_api_case(name, *spec)
+    if not only or "metadata_pool_layout" in only:
+        make_pool_layout_case("metadata_pool_layout", '{"metadata_cache_max_batch_size": 6, %s}' % layers, 8, 3, 32768)
 
 
 if __name__ == "__main__":

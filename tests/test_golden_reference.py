@@ -44,6 +44,13 @@ def load_case(path):
     return d, X, O.OArgs(**kw), dtype
 
 
+def _flags(d, name, suffix=""):
+    if f"{name}{suffix}" not in d.files:
+        return None
+    shape = tuple(int(x) for x in d[f"{name}_shape{suffix}"])
+    return np.unpackbits(d[f"{name}{suffix}"])[: int(np.prod(shape))].reshape(shape).astype(bool)
+
+
 def test_fixtures_are_present():
     names = {os.path.basename(f) for f in _ALL}
     assert {"reference_f32_prefill_tiny.npz", "reference_f32_prefill_gqa_ragged.npz", "reference_f32_decode_paged.npz",
@@ -63,6 +70,16 @@ def test_oracle_reproduces_the_reference_run(path):
     got = O.bf16_bits_to_f32(ctx) if dtype == "bf16" else ctx
     tol = 2e-2 if dtype == "bf16" else 5e-5
     assert np.abs(got - d["context"]).max() <= tol, np.abs(got - d["context"]).max()
+    # which key rows the mask estimation and the attention touched
+    for name, mine in (("mask_access", meta.mask_access), ("sa_access", meta.sa_access)):
+        want = _flags(d, name)
+        assert want is not None and want.shape == mine.shape
+        assert np.array_equal(mine > 0, want), f"{name}: {int(((mine > 0) != want).sum())} flags differ"
+    if "context_replay" in d.files:  # restart from the cached inputs of stage 1
+        part = O.OMetadata(None, None, None, None, stage_caches=list(meta.stage_caches[:2]))
+        ctx_r, meta_r = O.hip_attention_12(X, A, cached=part)
+        assert np.array_equal(meta_r.indices, d["indices_replay"])
+        assert np.abs(ctx_r - d["context_replay"]).max() <= tol
 
 
 @pytest.mark.gpu
@@ -79,6 +96,10 @@ def test_gpu_reproduces_the_reference_run(path):
     assert np.array_equal(meta.ks_start_end.cpu().numpy(), d["ks_start_end"])
     want = O.f32_to_bf16_bits(d["context"]) if dtype == "bf16" else d["context"]
     assert_context_close(ctx, want, dtype)
+    for name, st in (("mask_access", meta.mask_cache_statistics), ("sa_access", meta.sa_cache_statistics)):
+        flags = _flags(d, name)
+        got = st.access_counter.cpu().numpy() > 0
+        assert got.shape == flags.shape and np.array_equal(got, flags), name
 
 
 # ---------------------------------------------------------------- forward_paged_hip (paged_hip.py:35-320)
@@ -137,6 +158,9 @@ def test_oracle_reproduces_the_serving_entry_point(path):
         assert np.array_equal(meta.indices, d[f"indices_{layer_id}"])
         assert np.array_equal(meta.ks, d[f"ks_{layer_id}"])
         assert np.abs(ctx - want).max() <= 5e-5, np.abs(ctx - want).max()
+        for name, mine in (("mask_access", meta.mask_access), ("sa_access", meta.sa_access)):
+            flags = _flags(d, name, f"_{layer_id}")  # of the last call
+            assert flags.shape == mine.shape and np.array_equal(mine > 0, flags), name
         if TQ == 1:
             ctx2, _ = O.hip_attention_12(X, A, cached=meta)
             assert np.abs(ctx2 - d[f"o_cached_{layer_id}"].reshape(B, 1, H, D)).max() <= 5e-5
@@ -170,6 +194,34 @@ def test_gpu_reproduces_the_serving_entry_point(path):
         assert np.array_equal(meta.indices.cpu().numpy(), d[f"indices_{layer_id}"])
         assert np.array_equal(meta.ks.cpu().numpy(), d[f"ks_{layer_id}"])
         assert_context_close(o.reshape(B, TQ, H, D), d[f"o_{layer_id}"].reshape(B, TQ, H, D), "f32")
+        for name, st in (("mask_access", meta.mask_cache_statistics), ("sa_access", meta.sa_cache_statistics)):
+            flags = _flags(d, name, f"_{layer_id}")
+            got = st.access_counter.cpu().numpy() > 0
+            assert got.shape == flags.shape and np.array_equal(got, flags), name
         if TQ == 1:
             o2, _ = forward_paged_hip(q.reshape(B * TQ, H, D), layer_id=int(layer_id), cached_metadata=meta, **kw)
             assert_context_close(o2.reshape(B, TQ, H, D), d[f"o_cached_{layer_id}"].reshape(B, TQ, H, D), "f32")
+
+
+def test_metadata_pool_layout_equals_the_reference_pool():
+    """Buffer names, shapes, storage and view dtypes and batch formats of ``HiPMetadataCachePool`` as the reference's
+    class allocates them for the same configuration (hip_memory_pool.py:55-222)."""
+    import json
+
+    import torch
+
+    from hip_attn import HiPAttentionConfig, HiPMetadataCachePool
+
+    with open(os.path.join(HERE, "golden", "reference_metadata_pool_layout.json")) as f:
+        ref = json.load(f)
+    pool = HiPMetadataCachePool(max_total_num_tokens=1 << 20, query_head_num=ref["heads"], layer_num=ref["layers"],
+                                context_length=ref["context_length"], device="cpu",
+                                hip_config=HiPAttentionConfig(json_or_path=ref["spec"]))
+    assert len(pool.cache) == len(ref["layout"])
+    for mine, theirs in zip(pool.cache, ref["layout"]):
+        assert set(mine) == set(theirs)
+        for name, want in theirs.items():
+            b = mine[name]
+            got = dict(shape=list(b.buffer.shape), store=str(b.buffer.dtype), dtype=str(b.dtype), format=b.batch_format)
+            assert got == want, name
+    assert pool.allocated_gpu_bytes == ref["allocated_bytes"]
