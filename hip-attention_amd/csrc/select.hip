@@ -146,11 +146,13 @@ __device__ __forceinline__ SegScan selection_scan(const uint32_t *s_keys, int n,
 __global__ __launch_bounds__(SEL_THREADS) void select_stage_kernel(const float *scores, const int32_t *chunk_left,
                                                                   int bs_in, int bs_out, int row_rep, int HEAD, int hg,
                                                                   int n, int k, int sub_chunk, int splits,
-                                                                  int32_t *next_left) {
+                                                                  int32_t *next_left, int64_t *left64,
+                                                                  int64_t *right64) {
     __shared__ uint32_t s_keys[SEL_MAX_N];
     __shared__ int s_hist[256];
     __shared__ int s_misc[2];
     __shared__ int s_tmp[SEL_THREADS / 64];
+    int *s_sel = reinterpret_cast<int *>(s_keys);  // reused after selection: positions of selected chunks
 
     const int hgi = blockIdx.x % hg;
     const int o = (blockIdx.x / hg) % bs_out;
@@ -159,7 +161,7 @@ __global__ __launch_bounds__(SEL_THREADS) void select_stage_kernel(const float *
     const int nheads = HEAD / hg;
     const float *srow = scores + (((int64_t)b * bs_in + i) * HEAD + (int64_t)hgi * nheads) * n;
     const int32_t *lrow = chunk_left + (((int64_t)b * bs_in + i) * hg + hgi) * n;
-    int32_t *orow = next_left + (((int64_t)b * bs_out + o) * hg + hgi) * ((int64_t)k * splits);
+    const int64_t obase = (((int64_t)b * bs_out + o) * hg + hgi) * ((int64_t)k * splits);
 
     uint32_t thr;
     int need;
@@ -172,7 +174,10 @@ __global__ __launch_bounds__(SEL_THREADS) void select_stage_kernel(const float *
         topk_threshold(srow, nheads, n, k, s_keys, s_hist, s_misc, &thr, &need);
     }
     SegScan sc = selection_scan(s_keys, n, thr, need, s_tmp);
+    // each thread notes which entries of its segment are selected (keys are still being read by others), then the
+    // positions are listed in output order
     int out = sc.out_base, eqr = sc.eq_base;
+    unsigned long long selbits = 0ull;  // seg <= 64 since n <= 16384
     for (int c = sc.begin; c < sc.end; c++) {
         uint32_t key = s_keys[c];
         bool sel = key > thr;
@@ -180,10 +185,22 @@ __global__ __launch_bounds__(SEL_THREADS) void select_stage_kernel(const float *
             sel = eqr < need;
             eqr++;
         }
-        if (sel) {
-            const int left = lrow[c];
-            for (int j = 0; j < splits; j++) orow[(int64_t)out * splits + j] = left + j * sub_chunk;
-            out++;
+        if (sel) selbits |= 1ull << (c - sc.begin);
+    }
+    __syncthreads();
+    for (int c = sc.begin; c < sc.end; c++) {
+        if ((selbits >> (c - sc.begin)) & 1ull) s_sel[out++] = c;
+    }
+    __syncthreads();
+    // exactly k entries are selected (k <= n); every thread emits sub-chunks of its own, all loads independent
+    const int total = k * splits;
+    for (int idx = threadIdx.x; idx < total; idx += SEL_THREADS) {
+        const int e = idx / splits, j = idx - e * splits;
+        const int left = lrow[s_sel[e]] + j * sub_chunk;
+        next_left[obase + idx] = left;
+        if (left64) {  // the same list as the next stage's cached inputs: int64 edges (left, left + chunk)
+            left64[obase + idx] = left;
+            right64[obase + idx] = (int64_t)left + sub_chunk;
         }
     }
 }
@@ -292,8 +309,10 @@ using namespace hipattn;
 extern "C" int hipattn_select_stage(const float *scores, const int32_t *chunk_left, int32_t B, int32_t bs_in,
                                     int32_t bs_out, int32_t row_rep, int32_t HEAD, int32_t hg, int32_t n,
                                     int32_t k, int32_t chunk_size, int32_t splits, int32_t *next_left,
-                                    void *stream) {
+                                    int64_t *next_left64, int64_t *next_right64, void *stream) {
     HIPATTN_CHECK_ARG(scores && chunk_left && next_left, HIPATTN_E_ARG, "select stage: null pointer");
+    HIPATTN_CHECK_ARG((next_left64 == nullptr) == (next_right64 == nullptr), HIPATTN_E_ARG,
+                      "select stage: give both 64-bit outputs or neither");
     HIPATTN_CHECK_ARG(B > 0 && bs_in > 0 && bs_out > 0 && row_rep > 0 && HEAD > 0 && n > 0 && k > 0 && splits > 0,
                       HIPATTN_E_ARG, "select stage: non-positive size");
     HIPATTN_CHECK_ARG(hg == 1 || hg == HEAD, HIPATTN_E_ARG, "select stage: hg must be 1 or HEAD");
@@ -303,7 +322,7 @@ extern "C" int hipattn_select_stage(const float *scores, const int32_t *chunk_le
     HIPATTN_CHECK_ARG(n <= SEL_MAX_N, HIPATTN_E_UNSUPPORTED, "select stage: %d chunks exceed the limit %d", n, SEL_MAX_N);
     dim3 grid((unsigned)(B * bs_out * hg)), block(SEL_THREADS);
     hipLaunchKernelGGL(select_stage_kernel, grid, block, 0, (hipStream_t)stream, scores, chunk_left, bs_in, bs_out,
-                       row_rep, HEAD, hg, n, k, chunk_size / splits, splits, next_left);
+                       row_rep, HEAD, hg, n, k, chunk_size / splits, splits, next_left, next_left64, next_right64);
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
 }

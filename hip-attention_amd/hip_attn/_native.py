@@ -317,12 +317,14 @@ def mask_stage(qs, kvs, chunk_left, hg, n, chunk, right_clamp, bs, bq, stride_q,
     check(rc, "hipattn_mask_stage")
 
 
-def select_stage(scores, chunk_left, B, bs_in, bs_out, row_rep, HEAD, hg, n, k, chunk, splits, next_left, device):
+def select_stage(scores, chunk_left, B, bs_in, bs_out, row_rep, HEAD, hg, n, k, chunk, splits, next_left, device,
+                 left64=None, right64=None):
     with _timed("select_stage"):
       rc = lib().hipattn_select_stage(
         _p(scores), _p(chunk_left), ctypes.c_int32(B), ctypes.c_int32(bs_in), ctypes.c_int32(bs_out),
         ctypes.c_int32(row_rep), ctypes.c_int32(HEAD), ctypes.c_int32(hg), ctypes.c_int32(n), ctypes.c_int32(k),
-        ctypes.c_int32(chunk), ctypes.c_int32(splits), _p(next_left), stream_ptr(device))
+        ctypes.c_int32(chunk), ctypes.c_int32(splits), _p(next_left), _p(left64), _p(right64),
+        stream_ptr(device))
     check(rc, "hipattn_select_stage")
 
 

@@ -189,15 +189,32 @@ def _initial_chunks(chunk_count: int, chunk_size: int, sink: int, B: int, bs: in
     return hit
 
 
-def _stage_cache_views(chunk_left: Tensor, HEAD: int, chunk: int) -> HiPAttentionStageInputCache:
-    """Reference-layout view of a stage's inputs: int64 left/right and the reset scores."""
+_RESET_SCORE: dict = {}
+
+
+def _reset_scores(device, shape) -> Tensor:
+    """The scores a stage starts from (-32000 everywhere) as a view of one element kept per device."""
+    key = (device.type, device.index)
+    one = _RESET_SCORE.get(key)
+    if one is None:
+        one = torch.full((1, 1, 1, 1), -32000.0, dtype=torch.float32, device=device)
+        if not (device.type == "cuda" and torch.cuda.is_current_stream_capturing()):
+            _RESET_SCORE[key] = one  # an allocation made during graph capture belongs to that graph: not kept
+    return one.expand(*shape)
+
+
+def _stage_cache_views(chunk_left: Tensor, HEAD: int, chunk: int, left64: Optional[Tensor] = None,
+                       right64: Optional[Tensor] = None) -> HiPAttentionStageInputCache:
+    """Reference-layout view of a stage's inputs: int64 left/right and the reset scores.  ``left64 / right64``:
+    the same list already written as int64 by the selection kernel."""
     B, BS, hg, n = chunk_left.shape
-    left = chunk_left.to(torch.int64)
+    left = left64 if left64 is not None else chunk_left.to(torch.int64)
+    right = right64 if right64 is not None else left + chunk
     if hg == 1:
         left = left.expand(B, BS, HEAD, n)
-    right = left + chunk
-    scores = torch.full((1, 1, 1, 1), -32000.0, dtype=torch.float32, device=chunk_left.device).expand(B, BS, HEAD, n)
-    return HiPAttentionStageInputCache(indices_left=left, indices_right=right, out_scores=scores)
+        right = right.expand(B, BS, HEAD, n)
+    return HiPAttentionStageInputCache(indices_left=left, indices_right=right,
+                                       out_scores=_reset_scores(chunk_left.device, (B, BS, HEAD, n)))
 
 
 def _chunk_list_from_cache(cache: HiPAttentionStageInputCache, hg: int) -> Tensor:
@@ -307,6 +324,7 @@ def dual_stage_quadratic_hip_attention(
         scores = None
         left_out = None
         prev_n = None
+        left64 = right64 = None
         n_cached = len(stage_caches) if stage_caches is not None else 0
         for i_stage, stage in enumerate(stages):
             if i_stage < n_cached - 1:
@@ -346,9 +364,14 @@ def dual_stage_quadratic_hip_attention(
                 assert (chunk_size % stage.stage_chunk_size) == 0
                 splits = chunk_size // stage.stage_chunk_size
                 next_left = torch.empty((BSZ, bs_out, hg, keep * splits), dtype=torch.int32, device=device)
+                left64 = right64 = None
                 if keep > 0:
+                    if (stage_caches is not None) and (i_stage >= len(stage_caches)):
+                        # the list is also handed out as this stage's cached inputs: written once, in both widths
+                        left64 = torch.empty(next_left.shape, dtype=torch.int64, device=device)
+                        right64 = torch.empty(next_left.shape, dtype=torch.int64, device=device)
                     N.select_stage(scores, chunk_left, BSZ, bs_in, bs_out, row_rep, scores.shape[2], hg, prev_n, keep,
-                                   chunk_size, splits, next_left, device)
+                                   chunk_size, splits, next_left, device, left64=left64, right64=right64)
                 chunk_left = next_left
                 right_clamp = _BIG
             else:
@@ -360,7 +383,7 @@ def dual_stage_quadratic_hip_attention(
                 if i_stage == 0:
                     stage_caches.append(HiPAttentionStageInputCache(None, None, None))
                 else:
-                    stage_caches.append(_stage_cache_views(chunk_left, HEAD, stage.stage_chunk_size))
+                    stage_caches.append(_stage_cache_views(chunk_left, HEAD, stage.stage_chunk_size, left64, right64))
 
             chunk_size = stage.stage_chunk_size
             chunk_count = chunk_left.shape[-1]

@@ -167,11 +167,14 @@ int hipattn_prescale_k_rope(const void *k, int64_t stride0, int64_t stride1, int
  *   next_left   int32 [B, BS_out, HG, k*splits]; chunk j of a kept parent starts at
  *               left + j*(chunk_size/splits)
  *   output row o reads input row (o + row_rep*BS_in - BS_out) / row_rep
- *   (repeat_interleave(row_rep, 1)[:, -BS_out:], :2092-2123). */
+ *   (repeat_interleave(row_rep, 1)[:, -BS_out:], :2092-2123).
+ *   next_left64 / next_right64: NULL, or int64 buffers of next_left's shape that receive the same list as
+ *   (left, left + chunk_size/splits), the layout of HiPAttentionStageInputCache.indices_left / indices_right
+ *   (src/hip_attn/v1_2/attention_metadata.py:111-115). */
 int hipattn_select_stage(const float *scores, const int32_t *chunk_left, int32_t B, int32_t bs_in,
                          int32_t bs_out, int32_t row_rep, int32_t HEAD, int32_t hg, int32_t n,
                          int32_t k, int32_t chunk_size, int32_t splits, int32_t *next_left,
-                         void *stream);
+                         int64_t *next_left64, int64_t *next_right64, void *stream);
 
 /* After the last stage: top-K chunks, block alignment, de-duplication, active count, in the
  * reference's metadata layout.  Replaces src/hip_attn/v1_2/attention_extend.py:2757-2776 and

@@ -102,16 +102,21 @@ def access_flags(md, suffix):
 
 
 def make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, dtype=torch.float32,
-              lens=None, page_size=0, extend=None, softcap=None, block_size_k=64, replay=False):
+              lens=None, page_size=0, extend=None, softcap=None, block_size_k=64, replay=False, exact=False):
     """One call of the reference operator; ``lens`` (decode: TQ == 1) places each sequence's query at lens[b] - 1;
     ``page_size`` > 0 moves K/V into a paged cache behind a shuffled block table; ``extend`` = (scan rule, sa rule)
     turns on RoPE applied on load."""
     g = torch.Generator().manual_seed(seed)
     # values with 8 significant bits, so that the files can hold q, k, v as 16-bit patterns
     short = lambda t: t.to(torch.bfloat16).to(dtype)  # noqa: E731
-    q = short(torch.randn((B, TQ, H, D), generator=g, dtype=torch.float32) * 0.5)
-    k = short(torch.randn((B, TK, HKV, D), generator=g, dtype=torch.float32))
-    v = short(torch.randn((B, TK, HKV, D), generator=g, dtype=torch.float32))
+    if exact:  # full float32 draws, v = k: stored as float32, v not stored
+        q = torch.randn((B, TQ, H, D), generator=g, dtype=torch.float32)
+        k = torch.randn((B, TK, HKV, D), generator=g, dtype=torch.float32)
+        v = k.clone()
+    else:
+        q = short(torch.randn((B, TQ, H, D), generator=g, dtype=torch.float32) * 0.5)
+        k = short(torch.randn((B, TK, HKV, D), generator=g, dtype=torch.float32))
+        v = short(torch.randn((B, TK, HKV, D), generator=g, dtype=torch.float32))
     if lens is None:
         pos = (torch.arange(TQ) + TK - TQ)[None].expand(B, TQ).contiguous()
     else:
@@ -164,10 +169,12 @@ def make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, sec
     path = os.path.join(HERE, f"reference_{name}.npz")
     if page_size > 0:  # the cache and the block table hold the same rows
         extra.update(max_tsrc=TK)
+    elif exact:
+        extra.update(k=k.numpy(), v_is_k=1)
     else:
         extra.update(k=bits16(k), v=bits16(v))
     np.savez_compressed(
-        path, q=bits16(q), pos=pos.numpy(),
+        path, q=q.numpy() if exact else bits16(q), pos=pos.numpy(),
         context=ctx.float().numpy(), indices=md.indices.numpy(), ks=md.ks.numpy(), ks_start_end=md.ks_start_end.numpy(),
         stages=np.array([[-1 if x is None else x for x in s] for s in stages], dtype=np.int64),
         sink=sink, sw=sw, second_k=second_k, bsbq=bsbq, bf16=int(dtype == torch.bfloat16), block_size_k=block_size_k,
@@ -261,6 +268,8 @@ def main():
         "f32_prefill_rope_streaming": (4, 1, 64, 1024, 2, 1, 32, tiny, 16, 256, 512, 32, dict(extend=("streaming", "streaming"))),
         "f32_decode_rope_infllm": (5, 2, 1, 1536, 4, 2, 32, tiny, 16, 256, 512, 32,
                                    dict(lens=[1536, 1100], extend=("infllm", "infllm"))),
+        # the smallest benchmark configuration: 512 queries against 4096 keys, 4 heads over 1, head dim 64, float32
+        "f32_smallest_benchmark_prefill": (0, 1, 512, 4096, 4, 1, 64, tiny, 16, 256, 512, 32, dict(exact=True)),
         "f32_prefill_stride_d64": (8, 1, 128, 2048, 4, 2, 64, strided, 32, 128, 256, 32, {}),
         "f32_decode_default_stages": (9, 1, 1, 8192, 2, 1, 32, default, 256, 512, 2048, 64, {}),
         # Not generated: Triton's interpreter has no bfloat16 constants (``get_bf16``) and cannot call

@@ -24,7 +24,8 @@ def load_case(path):
     bf16 = bool(int(d["bf16"]))
     dtype = "bf16" if bf16 else "f32"
     # q, k, v are stored as the upper 16 bits of their float32 patterns (the lower 16 are zero)
-    conv = (lambda a: a) if bf16 else (lambda a: (a.astype(np.uint32) << 16).view(np.float32))
+    conv = (lambda a: a) if bf16 else (
+        lambda a: np.ascontiguousarray(a) if a.dtype == np.float32 else (a.astype(np.uint32) << 16).view(np.float32))
     stages = [O.OStage(int(a), int(b), int(c), None if e < 0 else int(e), int(f)) for a, b, c, e, f in d["stages"]]
     kw = dict(sink_token_size=int(d["sink"]), sliding_window_size=int(d["sw"]), second_stage_k=int(d["second_k"]),
               block_sparse_block_size_q=int(d["bsbq"]), stages=stages, block_size_k=int(d["block_size_k"]))
@@ -34,7 +35,7 @@ def load_case(path):
                       block_table=d["block_table"].astype(np.int64), cache_seq_lens=d["cache_seq_lens"].astype(np.int64))
         kw["extend_context_length"] = int(d["max_tsrc"])
     else:
-        X = O.OInputs(dtype, conv(d["q"]), pos, k=conv(d["k"]), v=conv(d["v"]))
+        X = O.OInputs(dtype, conv(d["q"]), pos, k=conv(d["k"]), v=conv(d["k" if "v_is_k" in d.files else "v"]))
     if "rope_cos" in d.files:
         X.rope_cos, X.rope_sin = d["rope_cos"].astype(np.float32), d["rope_sin"].astype(np.float32)
         kw.update(using_extend=True, need_apply_rope=True, scan_extend_backend=str(d["scan_backend"]),
@@ -57,6 +58,7 @@ def test_fixtures_are_present():
             "reference_f32_prefill_rope_relative.npz", "reference_f32_prefill_rope_streaming.npz",
             "reference_f32_decode_rope_infllm.npz", "reference_f32_prefill_stride_d64.npz",
             "reference_f32_decode_default_stages.npz", "reference_f32_paged_api_prefill.npz",
+            "reference_f32_smallest_benchmark_prefill.npz",
             "reference_f32_paged_api_decode_rope.npz"} <= names
 
 
