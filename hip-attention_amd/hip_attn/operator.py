@@ -124,13 +124,25 @@ def _kv_struct(args: HiPAttentionArgs, k: Optional[Tensor], v: Optional[Tensor],
     return st, keep
 
 
+_ZERO_FLAG: dict = {}
+
+
 def _new_statistics(args: HiPAttentionArgs, B: int, head_kv: int, pages: int, device):
-    """Zeroed ``int32 [B, HEAD_KV, pages]`` access and miss flags (attention_extend.py:1994-2006)."""
+    """Zeroed ``int32 [B, HEAD_KV, pages]`` access and miss flags (attention_extend.py:1994-2006).  Without an
+    offload cache nothing can miss: the miss flags are then a read-only view of one zero kept per device, which
+    saves clearing ``B * HEAD_KV * pages`` words per call."""
     if not args.require_cache_statistics:
         return HiPAttentionCacheAccessStatistics(None, None)
-    return HiPAttentionCacheAccessStatistics(
-        torch.zeros((B, head_kv, pages), dtype=torch.int32, device=device),
-        torch.zeros((B, head_kv, pages), dtype=torch.int32, device=device))
+    access = torch.zeros((B, head_kv, pages), dtype=torch.int32, device=device)
+    if args.offload_cache is not None:
+        return HiPAttentionCacheAccessStatistics(access, torch.zeros_like(access))
+    key = (device.type, device.index)
+    zero = _ZERO_FLAG.get(key)
+    if zero is None:
+        zero = torch.zeros((1, 1, 1), dtype=torch.int32, device=device)
+        if not (device.type == "cuda" and torch.cuda.is_current_stream_capturing()):
+            _ZERO_FLAG[key] = zero  # an allocation made during graph capture belongs to that graph: not kept
+    return HiPAttentionCacheAccessStatistics(access, zero.expand(B, head_kv, pages))
 
 
 def _mask_kv(args: HiPAttentionArgs, k_mask: Optional[Tensor], max_tsrc: int, q: Tensor, programs_rows: int,
