@@ -342,7 +342,14 @@ def dual_stage_quadratic_hip_attention(
             if i_stage < n_cached - 1:
                 continue
             elif i_stage == n_cached - 1:
-                pass
+                # The reference enters a restarted stage with stage 0's query block size and stage stride (:1960-1965;
+                # they are switched, :2092-2124, only on the way into a stage that is not restarted), and its restart
+                # test keeps them equal over all stages.  Where they differ its result is not the fresh run's; that
+                # state is refused rather than guessed at.
+                if i_stage > 0 and ((stage.stage_block_size_q, stage.stage_stride)
+                                    != (stages[0].stage_block_size_q, stages[0].stage_stride)):
+                    raise NotImplementedError("restart from cached stage inputs at a stage whose stage_block_size_q or "
+                                              "stage_stride differs from the first stage's is not built")
             elif i_stage > 0:
                 # truncate / realign / sort / re-tile / split (:2072-2165) folded into one selection pass
                 assert isinstance(stage, (ScanStage, NopStage)), f"stage type {type(stage).__name__} is not executable"

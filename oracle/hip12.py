@@ -401,7 +401,12 @@ def hip_attention_12(X: OInputs, A: OArgs, cached: Optional[OMetadata] = None):
             if i < len(stage_caches) - 1:
                 continue
             elif i == len(stage_caches) - 1:
-                pass
+                # The reference enters a restarted stage with the query block size and stage stride of stage 0
+                # (:1960-1965; the code that switches them, :2092-2124, runs only for stages that are not restarted).
+                # Its own restart test keeps them equal over all stages (tests/v1_2/test_gen3_stage_caching.py); a
+                # restart at a stage where they differ is not modelled.
+                if i > 0 and (st.stage_block_size_q, st.stage_stride) != (stages[0].stage_block_size_q, stages[0].stage_stride):
+                    raise NotImplementedError("restart at a stage whose block size or stride differs from stage 0's")
             elif i > 0:
                 assert st.stage_k % chunk == 0
                 kk = st.stage_k // chunk

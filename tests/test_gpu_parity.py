@@ -126,6 +126,24 @@ def test_stage_cache_replay_reproduces_output():
         assert np.array_equal(sc.out_scores.cpu().numpy(), osc.out_scores)
 
 
+def test_restart_at_a_stage_with_another_block_size_is_refused():
+    """The reference runs a restarted stage with the first stage's query block size and stride, so where they differ
+    its restart is not its fresh run; that state raises here instead of returning something else."""
+    _case("stage cache restart, block size changes at the restarted stage")
+    from hip_attn import HiPAttentionOutputMetadata12
+
+    X = make_inputs(6, B=1, TQ=128, TK=2048, H=2, HKV=1, D=64, dtype="f32")
+    A = tiny_args(stages=[O.OStage(64, 2, 64, None, 1), O.OStage(32, 2, 16, 1024, 1), O.OStage(32, 1, 2, 1024, 1)])
+    ctx, meta = run_product(X, A)
+    part = HiPAttentionOutputMetadata12(None, None, None, None, None, None, list(meta.stage_caches[:2]))
+    with pytest.raises(NotImplementedError):
+        run_product(X, A, cached=part)
+    # stage 2 also runs with blocks of 32 against the first stage's 64: a restart there is refused as well
+    part = HiPAttentionOutputMetadata12(None, None, None, None, None, None, list(meta.stage_caches[:3]))
+    with pytest.raises(NotImplementedError):
+        run_product(X, A, cached=part)
+
+
 def test_head_reduce_off_matches_oracle(monkeypatch):
     _case("head reduce off")
     monkeypatch.setenv("HIP_HEAD_REDUCE", "0")

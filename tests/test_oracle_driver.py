@@ -132,3 +132,14 @@ def test_decode_shape_and_flashdecode_head_sharing_is_neutral_under_head_reduce(
     ctx2, meta2 = O.hip_attention_12(X, A)
     assert np.array_equal(meta.indices, meta2.indices)
     assert np.abs(O.bf16_bits_to_f32(ctx) - O.bf16_bits_to_f32(ctx2)).max() > 0.02
+
+
+def test_restart_at_a_stage_with_another_block_size_is_refused():
+    import pytest
+
+    X = make_inputs(2, B=1, TQ=128, TK=2048, H=2, HKV=1, D=32, dtype="f32")
+    A = tiny_args(stages=[O.OStage(64, 2, 64, None, 1), O.OStage(32, 2, 16, 1024, 1), O.OStage(32, 1, 2, 1024, 1)])
+    ctx, meta = O.hip_attention_12(X, A)
+    part = O.OMetadata(None, None, None, None, stage_caches=list(meta.stage_caches[:2]))
+    with pytest.raises(NotImplementedError):
+        O.hip_attention_12(X, A, cached=part)
