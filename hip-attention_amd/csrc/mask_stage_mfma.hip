@@ -433,7 +433,11 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
     const bool two_sided = p.rope.cos != nullptr && prescaled;
     const int nb = rope ? 1 : nb0;
     const int nsub = (BC / 16) / nb;
-    bool via_lds = g_mask_via_lds == 2 ? !wide : (g_mask_via_lds == 1);
+    // narrow launches: chunks of up to 32 tokens keep a search inside a few KB that the heads of a group share
+    // through L1, and direct loads win (decode at 1M keys: 31 / 22 us against 38 / 28 us for the 32- and 8-token
+    // stages); wide chunks scatter the samples of a search, and rows fetched coalesced through LDS win (124 against
+    // 182 us for the 256-token stage)
+    bool via_lds = g_mask_via_lds == 2 ? (!wide && p.chunk > 32) : (g_mask_via_lds == 1);
     if (((p.kx.extended() || two_sided) && nb == 2) || rope) via_lds = false;
     const bool ext = rope || two_sided || p.kx.extended() || (wide && !two && !via_lds);
     const int hpw = (via_lds || two) ? 1 : (p.G < 4 ? p.G : 4);
