@@ -288,6 +288,17 @@ def main():
         "f32_paged_api_prefill": (20, 1, 192, 2048, 4, 2, 32, [2048], '{"using_extend": false, %s}' % layers, [7], 4096, False),
         "f32_paged_api_decode_rope": (21, 2, 1, 3072, 4, 2, 32, [3072, 2000], "{%s}" % layers, [0, 5], 131072, True),
     }
+    layers2 = ('"dense_layers": [0, 3], "layers": [{"second_stage_k": 256, "sliding_window_size": 256, '
+               '"sink_token_size": 64}, {"second_stage_k": 128, "sliding_window_size": 128}], "prefill_layers": '
+               '[{"second_stage_k": 256, "sliding_window_size": 256}, {"second_stage_k": 128, '
+               '"sliding_window_size": 512, "sink_token_size": 32}]')
+    api_cases.update({
+        # two sequences of different lengths, 100 new tokens each (one call per layer), per-layer sink sizes
+        "f32_paged_api_prefill_ragged": (30, 2, 100, 2048, 4, 2, 32, [2048, 1500],
+                                         '{"using_extend": false, %s}' % layers2, [3, 2], 8192, False),
+        # 130 new tokens with RoPE on load: the last 64 go through the second call
+        "f32_paged_api_prefill_rope_split": (33, 1, 130, 2048, 4, 1, 64, [1700], "{%s}" % layers2, [5], 2048, True),
+    })
     for name, spec in api_cases.items():
         if only and name not in only:
             continue

@@ -126,7 +126,8 @@ def _api_oracle_inputs(d, layer_id):
                   v_cache=np.ascontiguousarray(vc[:, None]),
                   block_table=d["req_to_tokens"][d["req_pool_indices"]].astype(np.int64),
                   cache_seq_lens=d["seq_lens"].astype(np.int64))
-    kw = dict(sliding_window_size=layer["sliding_window_size"], second_stage_k=layer["second_stage_k"],
+    kw = dict(sliding_window_size=layer.get("sliding_window_size", 1024), second_stage_k=layer.get("second_stage_k", 2048),
+              sink_token_size=layer.get("sink_token_size", 256),
               extend_context_length=int(d["max_context_len"]), model_context_length=int(d["orig_context_len"]),
               disable_flashdecode=TQ != 1)
     if spec.get("using_extend", True):
