@@ -5,6 +5,8 @@
 // compaction in position order: no sort is needed.  The top-k set is found by an exact radix
 // select on order-preserving integer keys; ties at the threshold are broken by position, which
 // is the fixed tie-break rule (score descending, position ascending).
+#include <stdlib.h>
+
 #include "common.hpp"
 
 namespace hipattn {
@@ -205,6 +207,154 @@ __global__ __launch_bounds__(SEL_THREADS) void select_stage_kernel(const float *
     }
 }
 
+// The same selection for launches of a few workgroups (decode: one per sequence), where the time is the length of the
+// dependent chain and not the work: 1024 threads hold ITEMS consecutive keys (and chunk edges) each in registers, so
+// the radix passes re-read nothing, the output ranks come from one block scan of packed counts, and every selected
+// entry is written by the thread that owns it.  Keys whose low 16 bits follow from their sign (scores that were
+// rounded to bf16) need two radix passes instead of four.
+constexpr int FAST_THREADS = 1024;
+
+template <int ITEMS>
+__global__ __launch_bounds__(FAST_THREADS) void select_stage_fast_kernel(const float *scores, const int32_t *chunk_left,
+                                                                        int bs_in, int bs_out, int row_rep, int HEAD,
+                                                                        int hg, int n, int k, int sub_chunk, int splits,
+                                                                        int32_t *next_left, int64_t *left64,
+                                                                        int64_t *right64) {
+    __shared__ int s_hist[256];
+    __shared__ int s_misc[2];
+    __shared__ uint32_t s_wave[FAST_THREADS / 64];
+
+    const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+    const int hgi = blockIdx.x % hg;
+    const int o = (blockIdx.x / hg) % bs_out;
+    const int b = blockIdx.x / (hg * bs_out);
+    const int i_in = (o + row_rep * bs_in - bs_out) / row_rep;
+    const int nheads = HEAD / hg;
+    const float *srow = scores + (((int64_t)b * bs_in + i_in) * HEAD + (int64_t)hgi * nheads) * n;
+    const int32_t *lrow = chunk_left + (((int64_t)b * bs_in + i_in) * hg + hgi) * n;
+    const int64_t obase = (((int64_t)b * bs_out + o) * hg + hgi) * ((int64_t)k * splits);
+
+    uint32_t key[ITEMS];
+    int left[ITEMS];
+    const int c0 = tid * ITEMS;
+    bool plain_low = true;  // low 16 bits are all zero (positive) / all one (negative) in every key
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) {
+        const int c = c0 + i;
+        key[i] = 0u;
+        left[i] = 0;
+        if (c < n) {
+            float m = srow[c];
+            for (int hh = 1; hh < nheads; hh++) m = fmaxf(m, srow[(int64_t)hh * n + c]);
+            key[i] = score_key(m);
+            left[i] = lrow[c];
+            plain_low = plain_low && ((key[i] & 0xffffu) == ((key[i] >> 31) ? 0u : 0xffffu));
+        }
+    }
+    uint32_t prefix = 0, mask = 0;
+    int need = k;
+    if (k < n) {
+        const int last_shift = __syncthreads_and(plain_low ? 1 : 0) ? 16 : 0;
+        for (int shift = 24; shift >= last_shift; shift -= 8) {
+            if (tid < 256) s_hist[tid] = 0;
+            __syncthreads();
+            {
+                int cur = -1, cnt = 0;
+#pragma unroll
+                for (int i = 0; i < ITEMS; i++) {
+                    if (c0 + i < n && (key[i] & mask) == prefix) {
+                        const int bin = (int)((key[i] >> shift) & 255u);
+                        if (bin == cur) {
+                            cnt++;
+                        } else {
+                            if (cnt) atomicAdd(&s_hist[cur], cnt);
+                            cur = bin;
+                            cnt = 1;
+                        }
+                    }
+                }
+                if (cnt) atomicAdd(&s_hist[cur], cnt);
+            }
+            __syncthreads();
+            if (tid < 64) {  // lane l owns bins 255-4l .. 252-4l; a prefix sum from the top finds the need-th largest
+                int hv[4];
+                int mine = 0;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    hv[j] = s_hist[255 - 4 * tid - j];
+                    mine += hv[j];
+                }
+                int incl = mine;
+#pragma unroll
+                for (int off = 1; off < 64; off <<= 1) {
+                    const int up = __shfl_up(incl, off);
+                    if (tid >= off) incl += up;
+                }
+                int cum = incl - mine;
+                if (cum < need && need <= incl) {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        if (cum < need && need <= cum + hv[j]) {
+                            s_misc[0] = 255 - 4 * tid - j;
+                            s_misc[1] = need - cum;
+                        }
+                        cum += hv[j];
+                    }
+                }
+            }
+            __syncthreads();
+            prefix |= ((uint32_t)s_misc[0]) << shift;
+            mask |= 255u << shift;
+            need = s_misc[1];
+        }
+    } else {
+        need = 0;  // everything is selected: no key equals the (empty) threshold, every key is above it
+    }
+    // ranks: entries above the threshold always, entries equal to it in position order until `need` are taken
+    const bool all = k >= n;
+    uint32_t packed = 0;  // low half: entries above the threshold, high half: entries equal to it
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) {
+        if (c0 + i < n) {
+            const uint32_t mk = key[i] & mask;
+            packed += all ? 1u : ((mk > prefix ? 1u : 0u) + (mk == prefix ? 0x10000u : 0u));
+        }
+    }
+    uint32_t incl = packed;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t up = __shfl_up(incl, off);
+        if (lane >= off) incl += up;
+    }
+    if (lane == 63) s_wave[wid] = incl;
+    __syncthreads();
+    uint32_t before = incl - packed;
+    for (int w = 0; w < wid; w++) before += s_wave[w];
+    int gt_before = (int)(before & 0xffffu), eq_before = (int)(before >> 16);
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) {
+        if (c0 + i >= n) continue;
+        const uint32_t mk = key[i] & mask;
+        const bool gt = all || mk > prefix;
+        const bool eq = !all && mk == prefix;
+        const bool sel = gt || (eq && eq_before < need);
+        if (sel) {
+            const int e = gt_before + (eq_before < need ? eq_before : need);
+            for (int j = 0; j < splits; j++) {
+                const int v = left[i] + j * sub_chunk;
+                const int64_t at = obase + (int64_t)e * splits + j;
+                next_left[at] = v;
+                if (left64) {
+                    left64[at] = v;
+                    right64[at] = (int64_t)v + sub_chunk;
+                }
+            }
+        }
+        gt_before += gt ? 1 : 0;
+        eq_before += eq ? 1 : 0;
+    }
+}
+
 __global__ __launch_bounds__(SEL_THREADS) void finalize_kernel(const float *scores, const int32_t *left_out,
                                                                const int64_t *pos, int64_t pos_sb, int64_t pos_st,
                                                                int bs, int bdst, int scan_stride, int HEAD,
@@ -321,6 +471,24 @@ extern "C" int hipattn_select_stage(const float *scores, const int32_t *chunk_le
     HIPATTN_CHECK_ARG(bs_out <= row_rep * bs_in, HIPATTN_E_ARG, "select stage: bs_out > row_rep*bs_in");
     HIPATTN_CHECK_ARG(n <= SEL_MAX_N, HIPATTN_E_UNSUPPORTED, "select stage: %d chunks exceed the limit %d", n, SEL_MAX_N);
     dim3 grid((unsigned)(B * bs_out * hg)), block(SEL_THREADS);
+    static int fast = -1;  // HIPATTN_SELECT_FAST=0 keeps the throughput kernel everywhere (cross-checking aid)
+    if (fast < 0) {
+        const char *e = getenv("HIPATTN_SELECT_FAST");
+        fast = (e && e[0] == '0') ? 0 : 1;
+    }
+    if (fast && grid.x <= 64) {  // a few workgroups: the latency kernel
+        dim3 fblock(FAST_THREADS);
+#define SEL_FAST(IT)                                                                                                  \
+    hipLaunchKernelGGL(select_stage_fast_kernel<IT>, grid, fblock, 0, (hipStream_t)stream, scores, chunk_left, bs_in, \
+                       bs_out, row_rep, HEAD, hg, n, k, chunk_size / splits, splits, next_left, next_left64,          \
+                       next_right64)
+        if (n <= FAST_THREADS) SEL_FAST(1);
+        else if (n <= 4 * FAST_THREADS) SEL_FAST(4);
+        else SEL_FAST(16);
+#undef SEL_FAST
+        HIPATTN_CHECK_HIP(hipGetLastError());
+        return 0;
+    }
     hipLaunchKernelGGL(select_stage_kernel, grid, block, 0, (hipStream_t)stream, scores, chunk_left, bs_in, bs_out,
                        row_rep, HEAD, hg, n, k, chunk_size / splits, splits, next_left, next_left64, next_right64);
     HIPATTN_CHECK_HIP(hipGetLastError());
