@@ -144,6 +144,19 @@ def test_restart_at_a_stage_with_another_block_size_is_refused():
         run_product(X, A, cached=part)
 
 
+def test_many_query_blocks_use_the_throughput_selection_kernel():
+    """More than 64 scan rows: the selection runs in the 256-thread kernel (launches of up to 64 workgroups take the
+    1024-thread one, which every small case above exercises)."""
+    _case("prefill with 70 query blocks")
+    X = make_inputs(17, B=1, TQ=2240, TK=4096, H=2, HKV=1, D=64, dtype="bf16")
+    A = tiny_args()
+    octx, ometa = O.hip_attention_12(X, A)
+    assert ometa.indices.shape[1] == 70
+    ctx, meta = run_product(X, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, "bf16")
+
+
 def test_head_reduce_off_matches_oracle(monkeypatch):
     _case("head reduce off")
     monkeypatch.setenv("HIP_HEAD_REDUCE", "0")
