@@ -70,8 +70,8 @@ int make_kv_view(const hipattn_kv_t *kv, int B, int HID, int dtype, KVView *o, K
     HIPATTN_CHECK_ARG(kv && kv->k, HIPATTN_E_ARG, "kv: null K pointer");
     HIPATTN_CHECK_ARG(kv->HKV > 0, HIPATTN_E_ARG, "kv: HKV <= 0");
     if (kv->fp8) {
-        HIPATTN_CHECK_ARG(dtype == HIPATTN_BF16 && kv->paged && !kv->cache, HIPATTN_E_UNSUPPORTED,
-                          "kv: fp8 storage needs a bf16 query, a paged cache and no offload cache");
+        HIPATTN_CHECK_ARG(dtype == HIPATTN_BF16 && kv->paged, HIPATTN_E_UNSUPPORTED,
+                          "kv: fp8 storage needs a bf16 query and the paged view");
         HIPATTN_CHECK_ARG(HID % 32 == 0, HIPATTN_E_UNSUPPORTED, "kv: fp8 storage needs a head dim that is a multiple of 32");
     }
     const int esz = kv->fp8 ? 1 : (dtype == HIPATTN_BF16 ? 2 : 4);

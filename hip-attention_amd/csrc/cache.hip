@@ -470,19 +470,23 @@ __global__ void pool_read_rows_kernel(const char *pool, int64_t stride_row_b, in
     *reinterpret_cast<uint4 *>(dst + i * dst_row_b + (int64_t)h * row_bytes + piece * 16) = v;
 }
 
+// bytes per stored element; 0 for a dtype code that is not a storage format
+static int storage_esz(int dtype) {
+    return dtype == HIPATTN_F32 ? 4 : dtype == HIPATTN_BF16 ? 2 : dtype == HIPATTN_FP8_E5M2 ? 1 : 0;
+}
+
 static int tiles_of(int64_t n) { return (int)((n + CT_TILE - 1) / CT_TILE); }
 
 static int check_desc(const hipattn_cache_desc_t *d, int64_t max_fetch, int *shift_out) {
     HIPATTN_CHECK_ARG(d, HIPATTN_E_ARG, "cache: null descriptor");
-    HIPATTN_CHECK_ARG(d->dtype == HIPATTN_F32 || d->dtype == HIPATTN_BF16, HIPATTN_E_UNSUPPORTED, "cache: dtype %d",
-                      d->dtype);
+    HIPATTN_CHECK_ARG(storage_esz(d->dtype) > 0, HIPATTN_E_UNSUPPORTED, "cache: dtype %d", d->dtype);
     HIPATTN_CHECK_ARG(d->HKV > 0 && d->HID > 0 && d->pool_rows > 0 && d->slots > 0 && max_fetch > 0, HIPATTN_E_ARG,
                       "cache: non-positive size");
     int shift = -1;
     for (int s = 0; s <= 6; s++)
         if (d->block_tokens == (1 << s)) shift = s;
     HIPATTN_CHECK_ARG(shift >= 0, HIPATTN_E_ARG, "cache: block_tokens %d is not a power of two in 1..64", d->block_tokens);
-    const int esz = d->dtype == HIPATTN_BF16 ? 2 : 4;
+    const int esz = storage_esz(d->dtype);
     HIPATTN_CHECK_ARG(((int64_t)d->HID * esz) % 16 == 0, HIPATTN_E_ALIGN, "cache: rows must be whole 16-byte packs");
     const int64_t n_blocks = (d->pool_rows + d->block_tokens - 1) / d->block_tokens;
     HIPATTN_CHECK_ARG(n_blocks * d->HKV < 0x7fffffffLL && d->slots < 0x7fffffffLL && max_fetch < 0x7fffffffLL,
@@ -522,7 +526,8 @@ static int launch_fill(int32_t *p, int64_t n, int32_t value, hipStream_t st) {
 
 int cache_view_for(const hipattn_cache *c, const hipattn_kv_t *kv, const KVView *o, int HID, int dtype, KVExt *x) {
     HIPATTN_CHECK_ARG(kv->paged, HIPATTN_E_ARG, "kv: an offload cache needs the paged view");
-    HIPATTN_CHECK_ARG(c->d.dtype == dtype && c->d.HID == HID && c->d.HKV == kv->HKV, HIPATTN_E_ARG,
+    const int stored = kv->fp8 ? HIPATTN_FP8_E5M2 : dtype;
+    HIPATTN_CHECK_ARG(c->d.dtype == stored && c->d.HID == HID && c->d.HKV == kv->HKV, HIPATTN_E_ARG,
                       "kv: cache was built for dtype %d, head dim %d, %d kv heads", c->d.dtype, c->d.HID, c->d.HKV);
     HIPATTN_CHECK_ARG(kv->k == c->d.host_k && (!c->d.with_v || !kv->v || kv->v == c->d.host_v), HIPATTN_E_ARG,
                       "kv: K/V pointers differ from the pools the cache was built over");
@@ -556,7 +561,7 @@ extern "C" int hipattn_cache_sizes(const hipattn_cache_desc_t *d, int64_t max_fe
     int rc = check_desc(d, max_fetch, &shift);
     if (rc) return rc;
     HIPATTN_CHECK_ARG(out, HIPATTN_E_ARG, "cache: null output");
-    const int esz = d->dtype == HIPATTN_BF16 ? 2 : 4;
+    const int esz = storage_esz(d->dtype);
     const int64_t n_blocks = (d->pool_rows + d->block_tokens - 1) / d->block_tokens;
     out->n_blocks = n_blocks;
     out->bank_bytes = d->slots * (1 + (d->with_v ? 1 : 0)) * d->block_tokens * (int64_t)d->HID * esz;
@@ -577,7 +582,7 @@ extern "C" int hipattn_cache_create(const hipattn_cache_desc_t *d, int64_t max_f
     HIPATTN_CHECK_ARG(d->host_k && d->bank && d->table && d->last_use && d->backref && d->miss && d->workspace &&
                           (!d->with_v || d->host_v),
                       HIPATTN_E_ARG, "cache: null buffer");
-    const int esz = d->dtype == HIPATTN_BF16 ? 2 : 4;
+    const int esz = storage_esz(d->dtype);
     const int64_t al = 16 / esz;
     HIPATTN_CHECK_ARG(aligned16(d->host_k) && aligned16(d->host_v) && aligned16(d->bank) && aligned16(d->workspace) &&
                           d->host_stride_row % al == 0 && d->host_stride_h % al == 0,
@@ -684,8 +689,8 @@ extern "C" int hipattn_pool_write_rows(void *pool, int64_t stride_row, int64_t s
                                        int32_t dtype, const int64_t *rows, int64_t n, const void *src, void *stream) {
     if (n == 0) return 0;
     HIPATTN_CHECK_ARG(pool && rows && src && n > 0 && HKV > 0 && HID > 0, HIPATTN_E_ARG, "pool write: bad argument");
-    HIPATTN_CHECK_ARG(dtype == HIPATTN_F32 || dtype == HIPATTN_BF16, HIPATTN_E_UNSUPPORTED, "pool write: dtype %d", dtype);
-    const int esz = dtype == HIPATTN_BF16 ? 2 : 4;
+    HIPATTN_CHECK_ARG(storage_esz(dtype) > 0, HIPATTN_E_UNSUPPORTED, "pool write: dtype %d", dtype);
+    const int esz = storage_esz(dtype);
     HIPATTN_CHECK_ARG(aligned16(pool) && aligned16(src) && (stride_row * esz) % 16 == 0 && (stride_h * esz) % 16 == 0 &&
                           ((int64_t)HID * esz) % 16 == 0,
                       HIPATTN_E_ALIGN, "pool write: rows must be whole, aligned 16-byte packs");
@@ -703,8 +708,8 @@ extern "C" int hipattn_pool_read_rows(const void *pool, int64_t stride_row, int6
                                       void *stream) {
     if (n == 0) return 0;
     HIPATTN_CHECK_ARG(pool && rows && dst && n > 0 && HKV > 0 && HID > 0, HIPATTN_E_ARG, "pool read: bad argument");
-    HIPATTN_CHECK_ARG(dtype == HIPATTN_F32 || dtype == HIPATTN_BF16, HIPATTN_E_UNSUPPORTED, "pool read: dtype %d", dtype);
-    const int esz = dtype == HIPATTN_BF16 ? 2 : 4;
+    HIPATTN_CHECK_ARG(storage_esz(dtype) > 0, HIPATTN_E_UNSUPPORTED, "pool read: dtype %d", dtype);
+    const int esz = storage_esz(dtype);
     HIPATTN_CHECK_ARG(aligned16(pool) && aligned16(dst) && (stride_row * esz) % 16 == 0 && (stride_h * esz) % 16 == 0 &&
                           (dst_stride_row * esz) % 16 == 0 && ((int64_t)HID * esz) % 16 == 0 &&
                           dst_stride_row >= (int64_t)HKV * HID,

@@ -127,12 +127,20 @@ def check(rc: int, what: str):
         raise HipAttnError(f"{what}: {kind} {rc}: {msg}")
 
 
+FP8_E5M2 = 2  # storage only: offload pools and their caches
+
+
 def dtype_code(t: torch.Tensor) -> int:
     if t.dtype == torch.bfloat16:
         return BF16
     if t.dtype == torch.float32:
         return F32
     raise HipAttnError(f"unsupported dtype {t.dtype}: the kernels take float32 or bfloat16")
+
+
+def storage_code(t: torch.Tensor) -> int:
+    """Code of a K/V storage tensor: float32, bfloat16, or fp8 (e5m2) bytes held as uint8 / float8_e5m2."""
+    return FP8_E5M2 if t.dtype in _FP8_DTYPES else dtype_code(t)
 
 
 def stream_ptr(device) -> ctypes.c_void_p:

@@ -9,8 +9,9 @@ them with blocking copies, another thread per asynchronous ``set_kv_buffer`` dow
 poll and sleep.  Here the device reads and writes the pinned pools itself, so both directions are kernels on one side
 stream ordered with events; no thread, no host wait, and ``on_layer_end`` has nothing to synchronise.
 
-Not built: the validation pool (``HIP_OFFLOAD_CACHE_VALIDATION``), in-kernel cache updates (``DEBUG_ONLINE``) and fp8
-pools.
+fp8 (e5m2) pools hold bytes, as the reference's do (``model_offload_cache.py:39-41``); the prefetched prefix comes back
+as ``float8_e5m2`` tensors.  Not built: the validation pool (``HIP_OFFLOAD_CACHE_VALIDATION``) and in-kernel cache
+updates (``DEBUG_ONLINE``).
 """
 from __future__ import annotations
 
@@ -37,11 +38,11 @@ class HiPModelOffloadCache:
     def __init__(self, max_token_size: int, max_mask_cache_token_size: int, max_sa_cache_token_size: int,
                  dtype: torch.dtype, head_num: int, head_dim: int, layer_num: int, device: torch.device, hip_config):
         assert isinstance(device, torch.device) and device.index is not None
-        if dtype not in (torch.bfloat16, torch.float32):
-            raise NotImplementedError(f"offload pools of dtype {dtype} are not built (bf16 and f32 are)")
+        if dtype not in (torch.bfloat16, torch.float32, torch.float8_e5m2):
+            raise NotImplementedError(f"offload pools of dtype {dtype} are not built (bf16, f32 and float8_e5m2 are)")
         self.size = max_token_size
         self.dtype = dtype
-        self.store_dtype = dtype
+        self.store_dtype = torch.uint8 if dtype == torch.float8_e5m2 else dtype
         self.device = device
         self.head_num, self.head_dim, self.layer_num = head_num, head_dim, layer_num
         self.max_mask_cache_token_size = max_mask_cache_token_size * head_num
@@ -131,6 +132,8 @@ class HiPModelOffloadCache:
             if layer.pending_write is not None:
                 stream.wait_event(layer.pending_write)
             k, v = layer.gather_rows(table[:prefix_seq_len], extra_rows=fresh)
+            if self.store_dtype != self.dtype:
+                k, v = k.view(self.dtype), v.view(self.dtype)
             done = torch.cuda.Event()
             done.record(stream)
         self.prefetched_kv[handle] = (k.unsqueeze(0), v.unsqueeze(0), prefix_seq_len, table, done)

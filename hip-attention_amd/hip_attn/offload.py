@@ -24,13 +24,24 @@ from torch import Tensor
 from . import _native as N
 
 
+def _as_stored(rows: Tensor, pool_dtype: torch.dtype) -> Tensor:
+    """Rows in a pool's storage format; a byte pool takes float8_e5m2 values (rounded from wider inputs)."""
+    if pool_dtype == torch.uint8:
+        if rows.dtype not in (torch.uint8, torch.float8_e5m2):
+            rows = rows.to(torch.float8_e5m2)
+        return rows.contiguous().view(torch.uint8)
+    return rows.to(pool_dtype).contiguous()
+
+
 class UVMCache:
     """Host pool ``[max_token_size, head_num, head_dim]`` in pinned memory (``uvm_gpu_cache.py:72-117``)."""
 
     def __init__(self, layer_id: int, max_token_size: int, head_num: int, head_dim: int, dtype: torch.dtype,
                  device: torch.device):
-        if dtype not in (torch.bfloat16, torch.float32):
-            raise NotImplementedError(f"offload pool dtype {dtype}: only bfloat16 and float32 are built")
+        if dtype not in (torch.bfloat16, torch.float32, torch.float8_e5m2, torch.uint8):
+            raise NotImplementedError(f"offload pool dtype {dtype}: bfloat16, float32 and float8_e5m2 are built")
+        if dtype == torch.float8_e5m2:
+            dtype = torch.uint8  # fp8 (e5m2) rows are held as bytes, as the reference does (model_offload_cache.py:39-41)
         self.layer_id = layer_id
         self.max_token_size = max_token_size
         self.head_num = head_num
@@ -67,7 +78,7 @@ class GPUCache:
         self.max_fetch = int(max_fetch if max_fetch is not None else min(self.slots, 65536))
 
         d = N.CacheDesc()
-        d.dtype = N.dtype_code(k_uvm.bank_cpu)
+        d.dtype = N.storage_code(k_uvm.bank_cpu)
         d.HKV, d.HID = k_uvm.head_num, k_uvm.head_dim
         d.block_tokens = block_tokens
         d.with_v = int(self.kv_packed)
@@ -137,8 +148,8 @@ class GPUCache:
         """Resident blocks receive freshly written rows (``uvm_gpu_cache.py:548-563``)."""
         self.wait()
         rows = table.reshape(-1).to(device=self.device, dtype=torch.int64).contiguous()
-        k_rows = cache_k.to(self.device).contiguous()
-        v_rows = cache_v.to(self.device).contiguous() if (self.kv_packed and cache_v is not None) else None
+        k_rows = _as_stored(cache_k.to(self.device), self.k_uvm.dtype)
+        v_rows = _as_stored(cache_v.to(self.device), self.k_uvm.dtype) if (self.kv_packed and cache_v is not None) else None
         N.cache_write_rows(self.handle, rows, k_rows, v_rows, self.device)
 
     def statistics(self) -> dict:
@@ -197,6 +208,7 @@ class HiPOffloadCache:
         s.page_size = 1
         s.HKV = self.head_kv
         s.cache = cache.handle
+        s.fp8 = int(kb.dtype == torch.uint8)
         return s
 
     # ------------------------------------------------------------------ reference methods
@@ -214,7 +226,7 @@ class HiPOffloadCache:
         for pool in (self.k_uvm, self.v_uvm):
             dst = torch.empty((n + extra_rows, self.head_kv, self.head_dim), dtype=pool.bank_cpu.dtype, device=self.device)
             N.pool_read_rows(pool.device_ptr, pool.bank_cpu.stride(0), pool.bank_cpu.stride(1), self.head_kv,
-                             self.head_dim, N.dtype_code(pool.bank_cpu), rows, dst, self.device)
+                             self.head_dim, N.storage_code(pool.bank_cpu), rows, dst, self.device)
             out.append(dst)
         return out[0], out[1]
 
@@ -223,14 +235,14 @@ class HiPOffloadCache:
         assert table.device == cache_k.device and cache_v.device == cache_k.device
         if cache_k.device.type == "cpu":
             idx = table.reshape(-1).to(torch.int64)
-            self.k_uvm.bank_cpu.index_copy_(0, idx, cache_k.reshape(-1, self.head_kv, self.head_dim))
-            self.v_uvm.bank_cpu.index_copy_(0, idx, cache_v.reshape(-1, self.head_kv, self.head_dim))
+            self.k_uvm.bank_cpu.index_copy_(0, idx, _as_stored(cache_k.reshape(-1, self.head_kv, self.head_dim), self.k_uvm.dtype))
+            self.v_uvm.bank_cpu.index_copy_(0, idx, _as_stored(cache_v.reshape(-1, self.head_kv, self.head_dim), self.v_uvm.dtype))
         else:
             rows = table.reshape(-1).to(torch.int64).contiguous()
             for pool, src in ((self.k_uvm, cache_k), (self.v_uvm, cache_v)):
-                src = src.reshape(-1, self.head_kv, self.head_dim).to(pool.dtype).contiguous()
+                src = _as_stored(src.reshape(-1, self.head_kv, self.head_dim), pool.dtype)
                 N.pool_write_rows(pool.device_ptr, pool.bank_cpu.stride(0), pool.bank_cpu.stride(1), self.head_kv,
-                                  self.head_dim, N.dtype_code(pool.bank_cpu), rows, src, self.device)
+                                  self.head_dim, N.storage_code(pool.bank_cpu), rows, src, self.device)
         self.mask_k_cache.on_set_kv_buffer(table_gpu, cache_k, None)
         self.sa_kv_cache.on_set_kv_buffer(table_gpu, cache_k, cache_v)
         idx_gpu = table_gpu.reshape(-1).to(torch.int64)

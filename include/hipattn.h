@@ -22,6 +22,7 @@ extern "C" {
 
 #define HIPATTN_F32 0
 #define HIPATTN_BF16 1
+#define HIPATTN_FP8_E5M2 2 /* storage only (offload pools and caches): K / V bytes that kernels widen to bf16 on load */
 
 #define HIPATTN_E_ARG (-1)       /* null pointer / negative size / inconsistent shapes */
 #define HIPATTN_E_UNSUPPORTED (-2) /* valid request the kernels do not cover (head dim, limits) */
@@ -254,7 +255,7 @@ int hipattn_bsa_decode_merge(const void *workspace, int32_t B, int32_t HEAD, int
 typedef struct hipattn_cache hipattn_cache_t;
 
 typedef struct hipattn_cache_desc {
-    int32_t dtype;        /* HIPATTN_F32 / HIPATTN_BF16 */
+    int32_t dtype;        /* HIPATTN_F32 / HIPATTN_BF16 / HIPATTN_FP8_E5M2 (with hipattn_kv_t.fp8 and bf16 queries) */
     int32_t HKV, HID;
     int32_t block_tokens; /* power of two, 1..64 */
     int32_t with_v;       /* 0: K only (mask estimation cache), 1: K and V per slot (attention cache) */

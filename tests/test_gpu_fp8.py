@@ -107,3 +107,48 @@ def test_portable_attention_kernel_on_fp8_cache():
                                      rows_shared=True)
         torch.cuda.synchronize()
         assert_context_close(out, ref, "bf16")
+
+
+@pytest.mark.parametrize("TQ,sa_tokens", [(1, 1 << 20), (96, 1 << 20), (1, 1024)])
+def test_fp8_pools_behind_the_offload_cache(TQ, sa_tokens):
+    """fp8 rows in pinned host pools behind the device block caches (``model_offload_cache.py:39-41``): the same
+    kernels read the same bytes, so the offloaded run equals the resident fp8 run bit for bit, hit or miss, and both
+    match the oracle on the widened values."""
+    from hip_attn import HiPOffloadCache, hip_attention_12
+
+    print(f"[case] fp8 offload TQ={TQ} sa_tokens={sa_tokens}", flush=True)
+    B, TK, H, HKV, D = 2, 2048, 8, 2, 128
+    lens = np.array([2048, 1500])
+    pos = np.stack([np.arange(TQ) + l - TQ for l in lens])
+    X = make_inputs(60 + TQ, B=B, TQ=TQ, TK=TK, H=H, HKV=HKV, D=D, dtype="bf16", pos=pos, scale=0.5)
+    XQ, kc, vc = _quantise(to_paged(X, 1, seed=12, seq_lens=lens))
+    A = O.OArgs(sliding_window_size=256, second_stage_k=512, extend_context_length=TK,
+                stages=[O.OStage(64, 4, 64, None, 1), O.OStage(64, 4, 16, 1024, 1), O.OStage(64, 1, 8, 512, 1)])
+    octx, ometa = O.hip_attention_12(XQ, A)
+    ctx_res, meta_res = _run(XQ, A, kc, vc, True)
+    assert_metadata_equal(meta_res, ometa)
+    assert_context_close(ctx_res, octx, "bf16")
+
+    rows = kc.shape[0]
+    cache = HiPOffloadCache(0, rows, 1 << 20, sa_tokens, HKV, D, torch.float8_e5m2, torch.device("cuda"))
+    assert cache.k_uvm.bank_cpu.dtype == torch.uint8
+    table = torch.arange(rows, dtype=torch.int64)
+    cache.set_kv_buffer(table, table.cuda(), kc[:, 0], vc[:, 0])  # float8_e5m2 rows from the host
+    hits = 0
+    for step in range(3):
+        args = product_args(A, XQ)
+        args.k_cache = args.v_cache = None
+        args.offload_cache = cache
+        ctx, meta = hip_attention_12(to_torch(XQ.q, "bf16"), None, None, args)
+        torch.cuda.synchronize()
+        assert_metadata_equal(meta, ometa)
+        assert torch.equal(ctx.view(torch.int16), ctx_res.view(torch.int16)), f"step {step}: offloaded != resident"
+        cache.handle_cache_miss(meta)
+        hits += cache.sa_kv_cache.statistics()["last_hit"]
+    assert hits > 0  # later steps were served from the device cache
+    # rows written from the device in a wider dtype are rounded to e5m2 on the way in
+    new = torch.randn((4, HKV, D), device="cuda", dtype=torch.bfloat16)
+    at = torch.tensor([5, 6, 7, 8], device="cuda")
+    cache.set_kv_buffer(at, at, new, new)
+    torch.cuda.synchronize()
+    assert torch.equal(cache.k_uvm.bank_cpu[5:9], new.to(torch.float8_e5m2).view(torch.uint8).cpu())

@@ -276,3 +276,37 @@ def test_model_level_manager_prefetches_prefixes_and_orders_async_stores():
     out_res, meta_res = hip_attention_12(q, ks[1][None], vs[1][None], HiPAttentionArgs12(stages=stages, **common))
     assert torch.equal(meta_off.indices, meta_res.indices)
     assert torch.equal(out_off, out_res)
+
+
+def test_model_level_manager_with_fp8_pools():
+    """float8_e5m2 pools are held as bytes (model_offload_cache.py:39-41); stores round wider rows to e5m2 and the
+    prefetched prefix comes back as float8_e5m2 with the new chunk's rows behind it."""
+    from hip_attn import HiPAttentionConfig, HiPModelOffloadCache
+
+    print("[case] model-level offload manager, fp8 pools", flush=True)
+    dev = torch.device("cuda", 0)
+    L, HKV, D, T = 2, 2, 64, 1024
+    mgr = HiPModelOffloadCache(max_token_size=T + 8, max_mask_cache_token_size=512, max_sa_cache_token_size=512,
+                               dtype=torch.float8_e5m2, head_num=HKV, head_dim=D, layer_num=L, device=dev,
+                               hip_config=HiPAttentionConfig())
+    assert mgr.store_dtype == torch.uint8 and mgr.layer_buffer[0].k_uvm.bank_cpu.dtype == torch.uint8
+    g = torch.Generator().manual_seed(9)
+    perm = (torch.randperm(T + 4, generator=g)[:T] + 1).to(dev)
+    ks = [torch.randn((T, HKV, D), generator=g).to(torch.bfloat16).to(dev) for _ in range(L)]
+    vs = [torch.randn((T, HKV, D), generator=g).to(torch.bfloat16).to(dev) for _ in range(L)]
+    prefix, fresh = 768, 256
+    for layer in range(L):
+        mgr.set_kv_buffer(layer, perm[:prefix], ks[layer][:prefix], vs[layer][:prefix], async_copy=(layer == 1))
+    req_to_token = torch.zeros((1, T), dtype=torch.int64, device=dev)
+    req_to_token[0] = perm
+    hooks = dict(batch_size=1, req_to_token=req_to_token, req_pool_indices=torch.tensor([0], device=dev),
+                 extend_prefix_lens_cpu=np.array([prefix]), extend_seq_lens_cpu=np.array([fresh]))
+    mgr.on_model_start(True, **hooks)
+    for layer in range(L):
+        mgr.on_layer_start(layer, True, **hooks)
+        k, v, _ = mgr.get_fetched_prefix_kv_buffer(layer, 0, ks[layer][None, prefix:], vs[layer][None, prefix:])
+        assert k.dtype == torch.float8_e5m2 and k.shape == (1, T, HKV, D)
+        assert torch.equal(k[0].view(torch.uint8), ks[layer].to(torch.float8_e5m2).view(torch.uint8))
+        assert torch.equal(v[0].view(torch.uint8), vs[layer].to(torch.float8_e5m2).view(torch.uint8))
+        mgr.on_layer_end(layer, True)
+    mgr.on_model_end(True)
