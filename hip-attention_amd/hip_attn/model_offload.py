@@ -10,12 +10,15 @@ poll and sleep.  Here the device reads and writes the pinned pools itself, so bo
 stream ordered with events; no thread, no host wait, and ``on_layer_end`` has nothing to synchronise.
 
 fp8 (e5m2) pools hold bytes, as the reference's do (``model_offload_cache.py:39-41``); the prefetched prefix comes back
-as ``float8_e5m2`` tensors.  Not built: the validation pool (``HIP_OFFLOAD_CACHE_VALIDATION``) and in-kernel cache
-updates (``DEBUG_ONLINE``).
+as ``float8_e5m2`` tensors.  ``HIP_OFFLOAD_CACHE_VALIDATION=1`` keeps a resident copy of every layer's rows
+(``:117-128``): stores go to both, the prefetched prefix is compared with the copy, and ``get_kv_buffer`` /
+``get_fetched_prefix_kv_buffer`` hand the copy out as the third value for ``forward_paged_hip(offloading_metadata=...)``.
+Not built: in-kernel cache updates (``DEBUG_ONLINE``).
 """
 from __future__ import annotations
 
 import logging
+import os
 from typing import Any, Dict, Optional, Tuple
 
 import torch
@@ -63,12 +66,20 @@ class HiPModelOffloadCache:
         # (layer, batch item) -> (k, v, prefix length, table, event recorded after the gather)
         self.prefetched_kv: Dict[Tuple[int, int], Tuple[Tensor, Tensor, int, Tensor, torch.cuda.Event]] = {}
         self.enable_async = True
+        self.require_validation = os.getenv("HIP_OFFLOAD_CACHE_VALIDATION", "0") == "1"
         self.validation_cache = None
+        if self.require_validation:  # resident copies [tokens + 1, heads, dim] per layer, K and V
+            shape = (max_token_size + 1, head_num, head_dim)
+            self.validation_cache = [(torch.zeros(shape, dtype=self.store_dtype, device=device),
+                                      torch.zeros(shape, dtype=self.store_dtype, device=device))
+                                     for _ in range(layer_num)]
 
     def is_online_cache_update_enabled(self) -> bool:
         return self.online_update_cache
 
     def get_kv_buffer(self, layer_id: int) -> Tuple[HiPOffloadCache, Any]:
+        if self.require_validation:
+            return self.layer_buffer[layer_id], self.validation_cache[layer_id]
         return self.layer_buffer[layer_id], None
 
     # ------------------------------------------------------------------ writes
@@ -79,6 +90,11 @@ class HiPModelOffloadCache:
         layer = self.layer_buffer[layer_id]
         if cache_k.dtype != self.dtype:
             cache_k, cache_v = cache_k.to(self.dtype), cache_v.to(self.dtype)
+        if self.require_validation:
+            rows = table.reshape(-1).to(self.device, dtype=torch.int64)
+            k_valid, v_valid = self.validation_cache[layer_id]
+            k_valid[rows] = cache_k.to(self.device).reshape(-1, self.head_num, self.head_dim).view(self.store_dtype)
+            v_valid[rows] = cache_v.to(self.device).reshape(-1, self.head_num, self.head_dim).view(self.store_dtype)
         if not (async_copy and self.enable_async and cache_k.is_cuda):
             layer.set_kv_buffer(table=table, table_gpu=table, cache_k=cache_k, cache_v=cache_v)
             return
@@ -152,6 +168,13 @@ class HiPModelOffloadCache:
         v.record_stream(current)
         k[:, prefix_seq_len:] = cache_k.to(self.dtype)
         v[:, prefix_seq_len:] = cache_v.to(self.dtype)
+        if self.require_validation:  # the gathered prefix must be what the resident copy holds (:211-226)
+            k_valid, v_valid = self.validation_cache[layer_id]
+            rows = table[:prefix_seq_len].to(self.device, dtype=torch.int64)
+            for got, want, name in ((k, k_valid, "K"), (v, v_valid, "V")):
+                err = float(((got[0, :prefix_seq_len].float() - want[rows].view(self.dtype).float()) ** 2).sum())
+                assert err < 1e-5, f"prefetched {name} prefix of layer {layer_id} differs from the validation pool: {err}"
+            return k, v, (k_valid, v_valid)
         return k, v, None
 
     def _synchronize(self):

@@ -22,7 +22,7 @@ from .memory_pool import cuda_graph_capture_configs  # noqa: F401  (paged_hip.py
 _LAST_DENSE = 64  # trailing prefill queries served with an (effectively) dense window, paged_hip.py:462
 
 
-def forward_paged_hip(
+def _forward_paged_hip(
     query: torch.Tensor,
     sm_scale: float,
     batch_size: int,
@@ -45,7 +45,6 @@ def forward_paged_hip(
     k: Optional[torch.Tensor] = None,
     v: Optional[torch.Tensor] = None,
     online_update_cache: bool = False,
-    offloading_metadata=None,
     is_decode: bool = False,
     query_for_mask: Optional[torch.Tensor] = None,
     diag_sliding_window_indices: Optional[torch.Tensor] = None,
@@ -148,3 +147,73 @@ def forward_paged_hip(
         context = torch.cat([sparse_ctx.to(query.dtype), dense_ctx.to(query.dtype)], dim=1)
 
     return context.view(N, num_heads, hidden), metadata
+
+
+def _sse(a: torch.Tensor, b: torch.Tensor) -> float:
+    return float(((a.float() - b.float()) ** 2).sum())
+
+
+def forward_paged_hip(
+    query: torch.Tensor,
+    sm_scale: float,
+    batch_size: int,
+    k_cache: Optional[torch.Tensor],
+    v_cache: Optional[torch.Tensor],
+    offload_cache,
+    positions: torch.Tensor,
+    seq_lens: torch.Tensor,
+    req_to_tokens: torch.Tensor,
+    req_pool_indices: torch.Tensor,
+    rope_cos: Optional[torch.Tensor],
+    rope_sin: Optional[torch.Tensor],
+    layer_id: int,
+    logit_cap: float,
+    orig_context_len: int,
+    max_context_len: int,
+    is_prefill: bool,
+    hip_config: HiPAttentionConfig,
+    cached_metadata: Optional[HiPAttentionOutputMetadata] = None,
+    k: Optional[torch.Tensor] = None,
+    v: Optional[torch.Tensor] = None,
+    online_update_cache: bool = False,
+    offloading_metadata=None,
+    is_decode: bool = False,
+    query_for_mask: Optional[torch.Tensor] = None,
+    diag_sliding_window_indices: Optional[torch.Tensor] = None,
+) -> Tuple[torch.Tensor, HiPAttentionOutputMetadata]:
+    """The serving entry point (``paged_hip.py:35-320``): ``query [N, H, D]`` -> ``(context [N, H, D], metadata)``.
+
+    ``offloading_metadata`` turns on the reference's self-check of an offloaded run (``:95-320``): it is the resident
+    copy of the K / V token pools that ``HiPModelOffloadCache`` keeps under ``HIP_OFFLOAD_CACHE_VALIDATION=1``.  The
+    call is repeated on that copy and the two outputs must agree (squared error below 1e-6 for prefill, 1e-7 for
+    decode); for decode the host pools are compared with the copy as well.
+    """
+    common = dict(sm_scale=sm_scale, batch_size=batch_size, positions=positions, seq_lens=seq_lens,
+                  req_to_tokens=req_to_tokens, req_pool_indices=req_pool_indices, rope_cos=rope_cos, rope_sin=rope_sin,
+                  layer_id=layer_id, logit_cap=logit_cap, orig_context_len=orig_context_len,
+                  max_context_len=max_context_len, is_prefill=is_prefill, hip_config=hip_config,
+                  cached_metadata=cached_metadata, k=k, v=v, online_update_cache=online_update_cache,
+                  is_decode=is_decode, query_for_mask=query_for_mask,
+                  diag_sliding_window_indices=diag_sliding_window_indices)
+    o, metadata = _forward_paged_hip(query, k_cache=k_cache, v_cache=v_cache, offload_cache=offload_cache, **common)
+    if offloading_metadata is None:
+        return o, metadata
+    k_valid, v_valid = offloading_metadata
+    if is_prefill:
+        o_valid, _ = _forward_paged_hip(query, k_cache=k_valid, v_cache=v_valid, offload_cache=offload_cache, **common)
+        err = _sse(o, o_valid)
+        assert err < 1e-6, f"prefill on the validation pools differs: sse={err}"
+        return o, metadata
+    o_valid, metadata_valid = _forward_paged_hip(query, k_cache=k_valid, v_cache=v_valid, offload_cache=None, **common)
+    err = _sse(o, o_valid)
+    if err >= 1e-7:
+        pool_k, pool_v = offload_cache.k_uvm.bank_cpu, offload_cache.v_uvm.bank_cpu
+        n = min(pool_k.shape[0], k_valid.shape[0])
+        wide = (lambda t: t.view(torch.float8_e5m2) if t.dtype == torch.uint8 else t)
+        err_k = _sse(wide(pool_k[:n]).to(k_valid.device), wide(k_valid[:n]))
+        err_v = _sse(wide(pool_v[:n]).to(v_valid.device), wide(v_valid[:n]))
+        same_mask = (metadata.indices is not None and metadata_valid.indices is not None
+                     and torch.equal(metadata.indices, metadata_valid.indices))
+        raise AssertionError(f"decode on the offload cache differs from the validation pools: sse={err}, "
+                             f"pool K / V against the copy: {err_k} / {err_v}, same block indices: {same_mask}")
+    return o, metadata

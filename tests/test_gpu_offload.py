@@ -310,3 +310,53 @@ def test_model_level_manager_with_fp8_pools():
         assert torch.equal(v[0].view(torch.uint8), vs[layer].to(torch.float8_e5m2).view(torch.uint8))
         mgr.on_layer_end(layer, True)
     mgr.on_model_end(True)
+
+
+def test_validation_pools_catch_a_corrupted_host_row(monkeypatch):
+    """``HIP_OFFLOAD_CACHE_VALIDATION=1``: the manager keeps a resident copy of every layer, checks prefetched prefixes
+    against it and hands it to ``forward_paged_hip(offloading_metadata=...)``, which repeats the call on the copy
+    (model_offload_cache.py:117-128,211-226, paged_hip.py:95-320)."""
+    from hip_attn import HiPAttentionConfig, HiPModelOffloadCache, forward_paged_hip
+
+    print("[case] offload validation pools", flush=True)
+    monkeypatch.setenv("HIP_OFFLOAD_CACHE_VALIDATION", "1")
+    dev = torch.device("cuda", 0)
+    L, HKV, H, D, T = 1, 2, 8, 64, 2048
+    cfg = HiPAttentionConfig(json_or_path='{"using_extend": false, "layers": [{"second_stage_k": 256, '
+                             '"sliding_window_size": 256}, {"second_stage_k": 256, "sliding_window_size": 256}]}')
+    mgr = HiPModelOffloadCache(max_token_size=T + 8, max_mask_cache_token_size=T, max_sa_cache_token_size=T,
+                               dtype=torch.bfloat16, head_num=HKV, head_dim=D, layer_num=L, device=dev, hip_config=cfg)
+    assert mgr.require_validation
+    g = torch.Generator().manual_seed(3)
+    perm = (torch.randperm(T + 4, generator=g)[:T] + 1).to(dev)
+    ks = torch.randn((T, HKV, D), generator=g).to(torch.bfloat16).to(dev)
+    vs = torch.randn((T, HKV, D), generator=g).to(torch.bfloat16).to(dev)
+    mgr.set_kv_buffer(0, perm, ks, vs)
+    cache, valid = mgr.get_kv_buffer(0)
+    assert torch.equal(valid[0][perm], ks) and torch.equal(valid[1][perm], vs)
+    # the prefix check of a prefill pass
+    req_to_token = perm[None].to(torch.int64).contiguous()
+    hooks = dict(batch_size=1, req_to_token=req_to_token, req_pool_indices=torch.tensor([0], device=dev),
+                 extend_prefix_lens_cpu=np.array([T - 128]), extend_seq_lens_cpu=np.array([128]))
+    mgr.on_model_start(True, **hooks)
+    k, v, extra = mgr.get_fetched_prefix_kv_buffer(0, 0, ks[None, T - 128:], vs[None, T - 128:])
+    assert extra is not None and torch.equal(k[0], ks)
+    mgr.on_model_end(True)
+    # a decode step validated against the copy
+    q = (torch.randn((1, H, D), generator=g) * 0.5).to(torch.bfloat16).to(dev)
+    call = dict(sm_scale=D ** -0.5, batch_size=1, k_cache=None, v_cache=None, offload_cache=cache,
+                positions=torch.tensor([T - 1], device=dev), seq_lens=torch.tensor([T], device=dev),
+                req_to_tokens=req_to_token, req_pool_indices=torch.tensor([0], device=dev), rope_cos=None, rope_sin=None,
+                layer_id=0, logit_cap=0.0, orig_context_len=131072, max_context_len=T, is_prefill=False, hip_config=cfg,
+                is_decode=True)
+    out, meta = forward_paged_hip(q, offloading_metadata=valid, **call)
+    out_plain, _ = forward_paged_hip(q, **call)
+    assert torch.equal(out, out_plain)
+    # corrupt rows of the host pool inside the sliding window: the validated call must notice
+    torch.cuda.synchronize()
+    cache.k_uvm.bank_cpu[perm[T - 64:].cpu()] = 0
+    cache.v_uvm.bank_cpu[perm[T - 64:].cpu()] = 0
+    cache.mask_k_cache.flush()
+    cache.sa_kv_cache.flush()
+    with pytest.raises(AssertionError):
+        forward_paged_hip(q, offloading_metadata=valid, **call)
