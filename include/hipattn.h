@@ -292,7 +292,8 @@ int hipattn_cache_commit(hipattn_cache_t *cache, void *stream);
 int hipattn_cache_write_rows(hipattn_cache_t *cache, const int64_t *rows, int64_t n, const void *k_rows,
                              const void *v_rows, void *stream);
 /* Scatter device rows src[n, HKV, HID] (contiguous) into a pinned host pool at int64 rows[n] -- the GPU-side
- * store of HiPOffloadCache.set_kv_buffer (src/hip_attn/v1_2/uvm_gpu_cache.py:665-668). */
+ * store of HiPOffloadCache.set_kv_buffer (src/hip_attn/v1_2/uvm_gpu_cache.py:665-668).  dtype is the pool's storage
+ * format (HIPATTN_F32 / HIPATTN_BF16 / HIPATTN_FP8_E5M2); rows are copied as stored, strides are in elements. */
 int hipattn_pool_write_rows(void *pool, int64_t stride_row, int64_t stride_h, int32_t HKV, int32_t HID,
                             int32_t dtype, const int64_t *rows, int64_t n, const void *src, void *stream);
 /* The gather in the other direction: dst[i, h, :] = pool[rows[i], h, :] for int64 rows[n] (negative: zero row); dst is
