@@ -59,10 +59,11 @@ class _Tensors(ctypes.Structure):
         ("scan_backend", ctypes.c_int),
         ("sa_backend", ctypes.c_int),
         ("logit_softcap", ctypes.c_float),
+        ("model_context_length", ctypes.c_int64),
     ]
 
 
-EXTEND_BACKENDS = {None: 0, "relative": 1, "streaming": 2, "infllm": 3}
+EXTEND_BACKENDS = {None: 0, "relative": 1, "streaming": 2, "infllm": 3, "dynamic_extend": 4}  # 4: mask stage only
 
 
 def build(force: bool = False) -> str:
@@ -167,6 +168,7 @@ class OInputs:
     access: Optional[np.ndarray] = None  # int32 [B,HKV,pages]: flags set by every key row the kernels fetch
     rope_cos: Optional[np.ndarray] = None  # float32 [L,HID] (values of the tables' own dtype, widened)
     rope_sin: Optional[np.ndarray] = None
+    model_context_length: int = 131072  # only the "dynamic_extend" rule of the mask stage reads it
     scan_backend: Optional[str] = None  # rotation rule of the mask stage / of sparse attention; None = no RoPE
     sa_backend: Optional[str] = None
     logit_softcap: float = 0.0
@@ -207,6 +209,7 @@ class OInputs:
             S.cache_seq_lens = arr(self.cache_seq_lens, np.int64)
         S.MAX_TSRC = max_tsrc
         S.logit_softcap = float(self.logit_softcap or 0.0)
+        S.model_context_length = int(self.model_context_length)
         if self.access is not None:
             assert self.access.dtype == np.int32 and self.access.flags.c_contiguous and self.access.ndim == 3
             S.access = self.access.ctypes.data
@@ -365,6 +368,7 @@ def hip_attention_12(X: OInputs, A: OArgs, cached: Optional[OMetadata] = None):
         assert A.need_apply_rope, "only keys stored without rotation are modelled"
         assert X.rope_cos is not None and X.rope_sin is not None
         X.scan_backend, X.sa_backend = A.scan_extend_backend, A.sa_extend_backend
+        X.model_context_length = A.model_context_length
     else:
         X.scan_backend = X.sa_backend = None
 

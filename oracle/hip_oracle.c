@@ -51,6 +51,7 @@
 #define HIPO_EXT_RELATIVE 1
 #define HIPO_EXT_STREAMING 2
 #define HIPO_EXT_INFLLM 3
+#define HIPO_EXT_DYNAMIC 4 /* mask stage only */
 
 typedef struct {
     int dtype;               /* HIPO_F32 / HIPO_BF16 (q, k, v, caches all share it) */
@@ -81,9 +82,12 @@ typedef struct {
     int scan_backend;        /* HIPO_EXT_* for the mask stage */
     int sa_backend;          /* HIPO_EXT_* for block sparse attention */
     float logit_softcap;     /* 0 = off; attention logits become tanh(qk / cap) * cap (attention_extend_bsa.py:507-508) */
+    int64_t model_context_length; /* HiPAttentionArgs.model_context_length (the "dynamic_extend" rule needs it) */
 } hipo_tensors_t;
 
 /* ---------------------------------------------------------------- scalar helpers */
+
+static int64_t dynamic_extend_pos(int64_t t, int64_t pmin, int64_t pmax, int64_t model_ctx);
 
 static inline float bf16_bits_to_f32(uint16_t h) {
     uint32_t u = (uint32_t)h << 16;
@@ -352,6 +356,7 @@ int hipo_mask_stage(const hipo_tensors_t *X, int64_t *left, int64_t *right, floa
                     int64_t p = X->pos[(int64_t)b * TDST + it];
                     if (X->scan_backend == HIPO_EXT_RELATIVE) qpos = 1 + (int64_t)sw_eff;
                     else if (X->scan_backend == HIPO_EXT_INFLLM) qpos = sw_eff;
+                    else if (X->scan_backend == HIPO_EXT_DYNAMIC) qpos = p; /* :635-636 */
                     else qpos = p < (int64_t)n + sw_eff ? p : (int64_t)n + sw_eff;
                 }
                 for (int o = 0; o < stride_q; o++) {
@@ -404,6 +409,10 @@ int hipo_mask_stage(const hipo_tensors_t *X, int64_t *left, int64_t *right, floa
                         int64_t kposL = 0, kposR = 0;
                         if (X->scan_backend == HIPO_EXT_RELATIVE) kposR = 1;
                         else if (X->scan_backend == HIPO_EXT_STREAMING) kposL = kposR = c;
+                        else if (X->scan_backend == HIPO_EXT_DYNAMIC) {
+                            kposL = dynamic_extend_pos(tl_, pmin, pmin + nvalid, X->model_context_length);
+                            kposR = dynamic_extend_pos(tr_, pmin, pmin + nvalid, X->model_context_length);
+                        }
                         scaled_key_at(X, b, tl_, h / G, c_k, kposL, kbuf);
                         for (int j = 0; j < nrows; j++) {
                             if (!rowvalid[j]) continue;
@@ -434,6 +443,24 @@ int hipo_mask_stage(const hipo_tensors_t *X, int64_t *left, int64_t *right, floa
         free(qhat); free(kbuf); free(qsum); free(rowvalid); free(l); free(r); free(sc);
     }
     return 0;
+}
+
+/* Rotated position of a sampled key under the "dynamic_extend" rule (attention_extend.py:254-274): a query block
+ * that reaches beyond the model's context squeezes the keys older than a quarter of that context into what is left
+ * of it, linearly, in float32; pmin is the position of the block's first (strided) row, pmax = pmin + the number of
+ * valid strided rows (:249). */
+static int64_t dynamic_extend_pos(int64_t t, int64_t pmin, int64_t pmax, int64_t model_ctx) {
+    const int64_t window = model_ctx / 4;
+    int64_t pos;
+    if (t >= pmax - window || pmax <= model_ctx) {
+        pos = t;
+    } else {
+        const float off = (float)t - (float)(pmin - window);
+        const float ratio = (float)(model_ctx - window) / (float)(pmin - window);
+        pos = (int64_t)(int32_t)(off * ratio) + (pmin - window);
+    }
+    const int64_t floor_ = pmax - model_ctx;
+    return pos > floor_ ? pos : floor_;
 }
 
 /* ---------------------------------------------------------------- block sparse attention

@@ -26,7 +26,7 @@ rng = np.random.default_rng(int(sys.argv[1]) if len(sys.argv) > 1 else 0)
 N = int(sys.argv[2]) if len(sys.argv) > 2 else 10
 
 def one(case):
-    B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, lens, page, extend, bk_arg, early = case
+    B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, lens, page, extend, bk_arg, early, mctx = case
     g = torch.Generator().manual_seed(int(rng.integers(1 << 30)))
     short = lambda t: t.to(torch.bfloat16).float()
     q = short(torch.randn((B, TQ, H, D), generator=g) * 0.5); k = short(torch.randn((B, TK, HKV, D), generator=g)); v = short(torch.randn((B, TK, HKV, D), generator=g))
@@ -34,9 +34,11 @@ def one(case):
     else: pos = (torch.tensor(lens, dtype=torch.int64)[:, None] - TQ + torch.arange(TQ)[None]).contiguous()
     kw = dict(sink_token_size=sink, sliding_window_size=sw, second_stage_k=second_k, block_sparse_block_size_q=bsbq,
               stages=[meta.ScanStage(stage_block_size_q=a, stage_block_stride_q=b, stage_chunk_size=c, stage_k=d, stage_stride=e) for (a, b, c, d, e) in stages],
-              require_cache_statistics=True, position_ids=pos, block_size_k=bk_arg, stage_early_terminate=early)
+              require_cache_statistics=True, position_ids=pos, block_size_k=bk_arg, stage_early_terminate=early,
+              model_context_length=mctx)
     okw = dict(sink_token_size=sink, sliding_window_size=sw, second_stage_k=second_k, block_sparse_block_size_q=bsbq,
-               stages=[O.OStage(*s) for s in stages], block_size_k=bk_arg, stage_early_terminate=early)
+               stages=[O.OStage(*s) for s in stages], block_size_k=bk_arg, stage_early_terminate=early,
+               model_context_length=mctx)
     X = None
     if extend is not None:
         cos, sin = G.rope_tables(2 * TK, D); cos, sin = short(cos), short(sin)
@@ -101,10 +103,11 @@ def rand_case():
     page = int(rng.choice([0, 0, 1, 4, 16]))
     extend = None
     if rng.random() < 0.4:
-        extend = (str(rng.choice(["relative", "streaming", "infllm"])), str(rng.choice(["streaming", "infllm"])))
+        extend = (str(rng.choice(["relative", "streaming", "infllm", "dynamic_extend"])), str(rng.choice(["streaming", "infllm"])))
     bk_arg = int(rng.choice([32, 64]))
     early = int(rng.choice([1, 1, 2, 4]))
-    return (B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, lens, page, extend, bk_arg, early)
+    mctx = int(rng.choice([131072, 1024, 512]))  # small values put the queries beyond the model's context
+    return (B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, lens, page, extend, bk_arg, early, mctx)
 
 for i in range(N):
     case = rand_case()
