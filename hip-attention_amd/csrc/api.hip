@@ -62,6 +62,10 @@ int make_rope_view(const hipattn_q_t *q, unsigned allowed, const char *who, Rope
     HIPATTN_CHECK_ARG(q->HID % 32 == 0, HIPATTN_E_UNSUPPORTED, "%s: rope needs a head dim that is a multiple of 32", who);
     o->cos = r->cos; o->sin = r->sin; o->stride_t = r->stride_t; o->len = r->len; o->backend = r->backend;
     o->k_side_delta = r->k_side_delta;
+    o->model_ctx = r->model_context_length;
+    HIPATTN_CHECK_ARG(r->backend != HIPATTN_EXTEND_DYNAMIC || r->model_context_length >= 512, HIPATTN_E_ARG,
+                      "%s: the dynamic rule needs model_context_length >= 512 (got %lld)", who,
+                      (long long)r->model_context_length);
     return 0;
 }
 

@@ -348,11 +348,29 @@ struct RopeView {
     int64_t stride_t, len;
     int backend;  // HIPATTN_EXTEND_*
     int64_t k_side_delta;  // prescaled RELATIVE scan: offset of the position-1 copy of the keys
+    int64_t model_ctx;     // DYNAMIC rule: the model's context length
     __device__ __forceinline__ int64_t clamp(int64_t pos) const { return pos < 0 ? 0 : (pos >= len ? len - 1 : pos); }
     __device__ __forceinline__ int64_t row(int64_t pos) const {  // element offset of the table row of a position
         return clamp(pos) * stride_t;
     }
 };
+
+// Position the sampled key at token t is rotated to under the DYNAMIC rule (attention_extend.py:254-274): a query
+// block that reaches beyond the model's context squeezes the keys older than a quarter of that context into the
+// rest of it, linearly and in float32.  pmin: position of the block's first strided row; pmax = pmin + its number
+// of valid strided rows.  The host refuses model_ctx < 512, which keeps pmin - window positive wherever the
+// quotient is used (pmax > model_ctx and at most 64 rows).
+__device__ __forceinline__ int64_t dynamic_extend_pos(int64_t t, int64_t pmin, int64_t pmax, int64_t model_ctx) {
+    const int64_t window = model_ctx / 4;
+    int64_t pos = t;
+    if (!(t >= pmax - window || pmax <= model_ctx)) {
+        const float off = __fsub_rn((float)t, (float)(pmin - window));
+        const float ratio = __fdiv_rn((float)(model_ctx - window), (float)(pmin - window));
+        pos = (int64_t)(int)__fmul_rn(off, ratio) + (pmin - window);
+    }
+    const int64_t lowest = pmax - model_ctx;
+    return pos > lowest ? pos : lowest;
+}
 
 // One element of a rotated row: x*c + o*s with `o` the partner element, already signed (-x[i + HID/2] in the
 // lower half, +x[i - HID/2] in the upper); both products and the sum are rounded to T, never fused.

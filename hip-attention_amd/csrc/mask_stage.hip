@@ -56,13 +56,15 @@ __device__ __forceinline__ float reduce16(const float (&part)[ROWS], int dl) {
 __device__ __forceinline__ int64_t mask_rope_qpos(const RopeView &r, long long pos, int n, int sw_eff) {
     if (r.backend == HIPATTN_EXTEND_RELATIVE) return 1 + (int64_t)sw_eff;
     if (r.backend == HIPATTN_EXTEND_INFLLM) return sw_eff;
+    if (r.backend == HIPATTN_EXTEND_DYNAMIC) return pos;
     const long long cap = (long long)n + sw_eff;
     return pos < cap ? pos : cap;
 }
-// Position the sampled key of chunk `c` is rotated to (attention_extend.py:289-298)
-__device__ __forceinline__ int64_t mask_rope_kpos(const RopeView &r, int c, int side) {
+// Position the sampled key of chunk `c`, token `t`, is rotated to (attention_extend.py:254-298)
+__device__ __forceinline__ int64_t mask_rope_kpos(const RopeView &r, int c, int side, int t, int64_t pmin, int64_t pmax) {
     if (r.backend == HIPATTN_EXTEND_RELATIVE) return side;
     if (r.backend == HIPATTN_EXTEND_STREAMING) return c;
+    if (r.backend == HIPATTN_EXTEND_DYNAMIC) return dynamic_extend_pos(t, pmin, pmax, r.model_ctx);
     return 0;
 }
 
@@ -72,6 +74,7 @@ __global__ __launch_bounds__(64) void mask_stage_kernel(MaskParams p) {
     constexpr int HALF = HID / 2;
     __shared__ int64_t s_koff[128];
     __shared__ float s_sc[128];
+    __shared__ int s_kt[ROPE ? 128 : 1];  // token of each sample (the DYNAMIC rule rotates by it)
     __shared__ __align__(16) T s_q[MAXROWS * HID];
 
     const int lane = threadIdx.x;
@@ -198,6 +201,10 @@ __global__ __launch_bounds__(64) void mask_stage_kernel(MaskParams p) {
             }
             s_koff[2 * lane] = o0;
             s_koff[2 * lane + 1] = o1;
+            if constexpr (ROPE) {
+                s_kt[2 * lane] = (l + c) >> 1;
+                s_kt[2 * lane + 1] = (c + r) >> 1;
+            }
             s_sc[2 * lane] = -INFINITY;
             s_sc[2 * lane + 1] = -INFINITY;
         }
@@ -224,7 +231,8 @@ __global__ __launch_bounds__(64) void mask_stage_kernel(MaskParams p) {
                         if constexpr (ROPE) {
                             // lanes dl and dl ^ 8 of a row group hold the two halves of the row
                             const int krow = (cs + st) * 4 + sub;
-                            const int64_t tr = p.rope.row(mask_rope_kpos(p.rope, g * BC + (krow >> 1), krow & 1)) + (dl & 7) * SEG;
+                            const int64_t tr = p.rope.row(mask_rope_kpos(p.rope, g * BC + (krow >> 1), krow & 1, s_kt[krow], pmin,
+                                                                      pmin + __popcll(rowmask))) + (dl & 7) * SEG;
                             float rc[SEG], rsn[SEG];
                             load_elems<T, SEG>(reinterpret_cast<const T *>(p.rope.cos) + tr, rc);
                             load_elems<T, SEG>(reinterpret_cast<const T *>(p.rope.sin) + tr, rsn);
@@ -328,7 +336,8 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
     MaskParams p;
     rc = make_kv_view(kv, q->B, q->HID, q->dtype, &p.kv, &p.kx);
     if (rc) return rc;
-    rc = make_rope_view(q, (1u << HIPATTN_EXTEND_RELATIVE) | (1u << HIPATTN_EXTEND_STREAMING) | (1u << HIPATTN_EXTEND_INFLLM),
+    rc = make_rope_view(q, (1u << HIPATTN_EXTEND_RELATIVE) | (1u << HIPATTN_EXTEND_STREAMING) | (1u << HIPATTN_EXTEND_INFLLM) |
+                               (1u << HIPATTN_EXTEND_DYNAMIC),
                         "mask stage", &p.rope);
     if (rc) return rc;
     HIPATTN_CHECK_ARG(!(p.rope.cos && k_prescaled) || p.rope.backend == HIPATTN_EXTEND_RELATIVE ||

@@ -47,6 +47,7 @@ __device__ __forceinline__ uint32_t scale_pack(uint32_t w, float c) {
 __device__ __forceinline__ int64_t rope_qpos(const RopeView &r, long long pos, int n, int sw_eff) {
     if (r.backend == HIPATTN_EXTEND_RELATIVE) return 1 + (int64_t)sw_eff;
     if (r.backend == HIPATTN_EXTEND_INFLLM) return sw_eff;
+    if (r.backend == HIPATTN_EXTEND_DYNAMIC) return pos;
     const long long cap = (long long)n + sw_eff;
     return pos < cap ? pos : cap;
 }
@@ -58,8 +59,9 @@ __device__ __forceinline__ int64_t rope_kpos(const RopeView &r, int c, int side)
 
 // RMODE = 1 (direct path, one token block per wave, extended parameter block): every sampled key row is rotated
 // before it is scaled.  The two halves of a row sit in the two half-waves (lane and lane ^ 32) at the same k-step,
-// and the rotated position of a lane's key never changes over the iterations, so its cos/sin entries are loaded
-// once and stay in registers.
+// and under the RELATIVE, STREAMING and INFLLM rules the rotated position of a lane's key never changes over the
+// iterations, so its cos/sin entries are loaded once and stay in registers.  The DYNAMIC rule rotates by the
+// sampled token itself (attention_extend.py:254-274) and reloads them with every sample.
 // RMODE = 2 (prescaled keys, extended parameter block): the keys were rotated and scaled ahead of the scan, one
 // copy per sample side; right-hand samples read the copy k_side_delta elements further on.
 // KV8 = true (extended parameter block, unscaled keys): key rows are fp8 (e5m2) bytes, widened on load.
@@ -236,6 +238,16 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
                 off = kv_k_row<EXT, NB == 2>(p.kv, kx, b, t, kvh, seqlen, hh == 0);
                 if constexpr (RMODE == 2) {
                     if (side && off != NO_ROW) off += p.rope.k_side_delta;
+                }
+                if constexpr (ROPE) {
+                    if (p.rope.backend == HIPATTN_EXTEND_DYNAMIC) {
+                        const int64_t tr = p.rope.row(dynamic_extend_pos(t, pmin, pmin + __popcll(rowmask), p.rope.model_ctx));
+#pragma unroll
+                        for (int ks = 0; ks < KS; ks++) {
+                            rcos[tb][ks] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr + ks * 8);
+                            rsin[tb][ks] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr + ks * 8);
+                        }
+                    }
                 }
             }
             if constexpr (VIA_LDS) {

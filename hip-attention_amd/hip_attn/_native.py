@@ -42,10 +42,11 @@ class RopeStruct(ctypes.Structure):
         ("stride_t", ctypes.c_int64), ("len", ctypes.c_int64),
         ("backend", ctypes.c_int32),
         ("k_side_delta", ctypes.c_int64),
+        ("model_context_length", ctypes.c_int64),
     ]
 
 
-EXTEND_BACKENDS = {"relative": 1, "streaming": 2, "infllm": 3}
+EXTEND_BACKENDS = {"relative": 1, "streaming": 2, "infllm": 3, "dynamic_extend": 4}  # the last: mask stage only
 
 
 class KVStruct(ctypes.Structure):
@@ -151,10 +152,14 @@ def _p(t: Optional[torch.Tensor]):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
 
 
-def make_rope(cos: torch.Tensor, sin: torch.Tensor, backend: str, k_side_delta: int = 0) -> RopeStruct:
-    """Describe RoPE tables ``[len, >= HID/2]`` (q's dtype, unit inner stride) and the rotation rule of one call."""
-    if backend not in EXTEND_BACKENDS:
-        raise NotImplementedError(f"extend backend {backend!r} is not built (built: {sorted(EXTEND_BACKENDS)})")
+def make_rope(cos: torch.Tensor, sin: torch.Tensor, backend: str, k_side_delta: int = 0,
+              model_context_length: int = 0, attention: bool = False) -> RopeStruct:
+    """Describe RoPE tables ``[len, >= HID/2]`` (q's dtype, unit inner stride) and the rotation rule of one call.
+    ``attention`` marks a call of block sparse attention, which knows fewer rules than the mask stage."""
+    built = [b for b in EXTEND_BACKENDS if not (attention and b in ("relative", "dynamic_extend"))]
+    if backend not in built:
+        where = "block sparse attention" if attention else "the mask stage"
+        raise NotImplementedError(f"extend backend {backend!r} is not built for {where} (built: {sorted(built)})")
     assert cos.ndim == 2 and sin.shape == cos.shape and cos.stride(1) == 1 and sin.stride(1) == 1
     assert cos.stride(0) == sin.stride(0) and cos.dtype == sin.dtype
     r = RopeStruct()
@@ -162,6 +167,7 @@ def make_rope(cos: torch.Tensor, sin: torch.Tensor, backend: str, k_side_delta: 
     r.stride_t, r.len = cos.stride(0), cos.shape[0]
     r.backend = EXTEND_BACKENDS[backend]
     r.k_side_delta = k_side_delta
+    r.model_context_length = int(model_context_length)
     return r
 
 

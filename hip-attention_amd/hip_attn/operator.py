@@ -426,7 +426,7 @@ def dual_stage_quadratic_hip_attention(
                     if rope_tabs is not None:  # :2200-2204
                         backend = stage.stage_extend_backend or args.scan_extend_backend
                         use_pre = use_pre and backend in ("relative", "infllm")  # key positions fixed per sample side
-                        rope = N.make_rope(*rope_tabs, backend, k_side_delta if use_pre else 0)
+                        rope = N.make_rope(*rope_tabs, backend, k_side_delta if use_pre else 0, args.model_context_length)
                     qs = N.make_q(qq, position_ids, rope)
                     N.mask_stage(qs, mask_kv_pre if use_pre else mask_kv, chunk_left, hg, chunk_count, chunk_size,
                                  right_clamp, bs, BLOCK_SIZE_Q, stage.stage_block_stride_q, BLOCK_CHUNK, STAGE_STRIDE,
@@ -563,7 +563,7 @@ def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], 
     kvs, keep = _kv_struct(args, k, v, max_tsrc, masking=False, stats=stats)
     if position_ids.dtype != torch.int64:
         position_ids = position_ids.to(torch.int64)
-    rope = N.make_rope(*rope_tables, args.sa_extend_backend) if rope_tables is not None else None
+    rope = N.make_rope(*rope_tables, args.sa_extend_backend, attention=True) if rope_tables is not None else None
     qs = N.make_q(qq, position_ids, rope, args.logit_softcap)
     if rope is not None or args.logit_softcap is not None:
         khat = None

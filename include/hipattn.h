@@ -42,11 +42,17 @@ extern "C" {
  *                          slot = token for sink tokens, (j + sink / block_size_k) * block_size_k + e for
  *                          element e of index entry j; pmin = smallest position in the query block
  *                INFLLM    max(0, pmin - sliding_window)
- * Positions are clamped into [0, len).  The reference's "dynamic_extend" and "self_extend" rules and the mode
- * that re-rotates keys stored WITH rotation (need_apply_rope = False) are not built. */
+ *   DYNAMIC (mask stage only, attention_extend.py:249-274, :635-636): the query at its own position; with
+ *                pmax = pmin + the number of valid strided query rows, W = model_context_length / 4, the sampled
+ *                key at token t keeps position t when t >= pmax - W or pmax <= model_context_length, else it moves
+ *                to int32((float(t) - float(pmin - W)) * (float(model_context_length - W) / float(pmin - W)))
+ *                + (pmin - W), all in float32; the result is raised to at least pmax - model_context_length
+ * Positions are clamped into [0, len).  The reference's "self_extend" rule, "dynamic_extend" inside block sparse
+ * attention and the mode that re-rotates keys stored WITH rotation (need_apply_rope = False) are not built. */
 #define HIPATTN_EXTEND_RELATIVE 1
 #define HIPATTN_EXTEND_STREAMING 2
 #define HIPATTN_EXTEND_INFLLM 3
+#define HIPATTN_EXTEND_DYNAMIC 4
 
 typedef struct hipattn_rope {
     const void *cos; /* [len, >= HID/2], q's dtype, 16-byte aligned rows; column i = frequency i */
@@ -58,6 +64,9 @@ typedef struct hipattn_rope {
      * and scaled (hipattn_prescale_k_rope), and the copy rotated to position 1, which the right-hand samples
      * read, starts this many elements behind it.  INFLLM needs the position-0 copy only.  Unused otherwise. */
     int64_t k_side_delta;
+    /* HiPAttentionArgs.model_context_length (attention_extend.py:250); read by the DYNAMIC rule only, which needs
+     * at least 512 */
+    int64_t model_context_length;
 } hipattn_rope_t;
 
 /* Query tensor q[B, TDST, HEAD, HID] and its token positions (0-based, int64)

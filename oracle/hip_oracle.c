@@ -31,7 +31,8 @@
  * are pinned by closed forms and brute-force checks in tests/ (see each function's comment)
  * and, for float32 inputs, by executions of the reference's own kernels under Triton's CPU
  * interpreter (tests/golden/reference_*.npz, tests/test_golden_reference.py): multi-level scans,
- * selection, both attention kernels, decode, RoPE on load.  Parity unpinned against the running
+ * selection, both attention kernels, decode, RoPE on load (relative, streaming, infllm, and dynamic_extend in
+ * the mask stage, whose squeeze branch the reference_*_rope_dynamic vectors exercise).  Parity unpinned against the running
  * reference: bfloat16 arithmetic (the interpreter has no bfloat16; the order of accumulation here is
  * MI355X's, not NVIDIA's) and logit_softcap (the interpreter cannot call libdevice.tanh).
  */

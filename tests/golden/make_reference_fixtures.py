@@ -102,10 +102,11 @@ def access_flags(md, suffix):
 
 
 def make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, dtype=torch.float32,
-              lens=None, page_size=0, extend=None, softcap=None, block_size_k=64, replay=False, exact=False):
+              lens=None, page_size=0, extend=None, softcap=None, block_size_k=64, replay=False, exact=False,
+              model_ctx=None):
     """One call of the reference operator; ``lens`` (decode: TQ == 1) places each sequence's query at lens[b] - 1;
     ``page_size`` > 0 moves K/V into a paged cache behind a shuffled block table; ``extend`` = (scan rule, sa rule)
-    turns on RoPE applied on load."""
+    turns on RoPE applied on load; ``model_ctx`` sets model_context_length (the dynamic_extend rule reads it)."""
     g = torch.Generator().manual_seed(seed)
     # values with 8 significant bits, so that the files can hold q, k, v as 16-bit patterns
     short = lambda t: t.to(torch.bfloat16).to(dtype)  # noqa: E731
@@ -132,6 +133,9 @@ def make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, sec
                   scan_extend_backend=extend[0], sa_extend_backend=extend[1])
         extra.update(rope_cos=cos.to(dtype).float().numpy(), rope_sin=sin.to(dtype).float().numpy(),
                      scan_backend=extend[0], sa_backend=extend[1])
+    if model_ctx is not None:
+        kw.update(model_context_length=model_ctx)
+        extra.update(model_context_length=model_ctx)
     if softcap is not None:
         kw.update(logit_softcap=softcap)
         extra.update(softcap=softcap)
@@ -272,6 +276,11 @@ def main():
         "f32_smallest_benchmark_prefill": (0, 1, 512, 4096, 4, 1, 64, tiny, 16, 256, 512, 32, dict(exact=True)),
         "f32_prefill_stride_d64": (8, 1, 128, 2048, 4, 2, 64, strided, 32, 128, 256, 32, {}),
         "f32_decode_default_stages": (9, 1, 1, 8192, 2, 1, 32, default, 256, 512, 2048, 64, {}),
+        # dynamic_extend in the scan: the context reaches beyond the model's, so old keys are squeezed into it
+        "f32_prefill_rope_dynamic": (10, 1, 64, 2048, 2, 1, 32, tiny, 16, 256, 512, 32,
+                                     dict(extend=("dynamic_extend", "streaming"), model_ctx=1024)),
+        "f32_decode_rope_dynamic": (11, 2, 1, 2048, 4, 2, 32, tiny, 16, 256, 512, 32,
+                                    dict(lens=[2048, 1500], page_size=8, extend=("dynamic_extend", "infllm"), model_ctx=512)),
         # Not generated: Triton's interpreter has no bfloat16 constants (``get_bf16``) and cannot call
         # ``libdevice.tanh`` (logit_softcap) outside a compiled kernel, so bfloat16 inputs and soft-capped logits
         # have no vectors from the reference.

@@ -40,6 +40,8 @@ def load_case(path):
         X.rope_cos, X.rope_sin = d["rope_cos"].astype(np.float32), d["rope_sin"].astype(np.float32)
         kw.update(using_extend=True, need_apply_rope=True, scan_extend_backend=str(d["scan_backend"]),
                   sa_extend_backend=str(d["sa_backend"]))
+    if "model_context_length" in d.files:
+        kw["model_context_length"] = int(d["model_context_length"])
     if "softcap" in d.files:
         kw["logit_softcap"] = float(d["softcap"])
     return d, X, O.OArgs(**kw), dtype
@@ -57,6 +59,7 @@ def test_fixtures_are_present():
     assert {"reference_f32_prefill_tiny.npz", "reference_f32_prefill_gqa_ragged.npz", "reference_f32_decode_paged.npz",
             "reference_f32_prefill_rope_relative.npz", "reference_f32_prefill_rope_streaming.npz",
             "reference_f32_decode_rope_infllm.npz", "reference_f32_prefill_stride_d64.npz",
+            "reference_f32_prefill_rope_dynamic.npz", "reference_f32_decode_rope_dynamic.npz",
             "reference_f32_decode_default_stages.npz", "reference_f32_paged_api_prefill.npz",
             "reference_f32_smallest_benchmark_prefill.npz",
             "reference_f32_paged_api_decode_rope.npz"} <= names

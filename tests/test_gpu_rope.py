@@ -1,4 +1,5 @@
-"""GPU parity of RoPE applied on load (the "extend" modes): mask stage rules relative / streaming / infllm, sparse
+"""GPU parity of RoPE applied on load (the "extend" modes): mask stage rules relative / streaming / infllm /
+dynamic_extend, sparse
 attention rules streaming / infllm, through every kernel that loads query or key rows (scan on the matrix cores and
 portable scan, tile kernel, portable attention kernel, decode kernel).
 
@@ -29,6 +30,32 @@ def test_prefill_with_rope_matches_oracle(dtype, scan):
     A = _ext(scan_extend_backend=scan, sa_extend_backend="streaming")
     octx, ometa = O.hip_attention_12(X, A)
     ctx, meta = run_product(X, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, dtype)
+
+
+@pytest.mark.parametrize("dtype,D", [("f32", 64), ("bf16", 64), ("bf16", 128)])
+@pytest.mark.parametrize("model_ctx", [1024, 131072])
+def test_dynamic_extend_scan_prefill_and_paged_decode(dtype, D, model_ctx):
+    """The dynamic_extend rule of the scan: queries beyond model_context_length squeeze the keys older than a quarter
+    of it into the rest (1024 against 3000 keys); below it (131072) every key keeps its own position."""
+    print(f"[case] rope dynamic_extend {dtype} D={D} model_ctx={model_ctx}", flush=True)
+    X = with_rope(make_inputs(51, B=2, TQ=200, TK=3000, H=4, HKV=2, D=D, dtype=dtype, scale=0.5), 4096)
+    A = _ext(scan_extend_backend="dynamic_extend", sa_extend_backend="streaming", model_context_length=model_ctx)
+    octx, ometa = O.hip_attention_12(X, A)
+    ctx, meta = run_product(X, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, dtype)
+    if model_ctx == 1024:  # the squeeze really changes what is selected
+        _, plain = O.hip_attention_12(X, _ext(scan_extend_backend="dynamic_extend", sa_extend_backend="streaming"))
+        assert not np.array_equal(plain.indices, ometa.indices)
+    lens = np.array([3000, 1777])
+    XD = make_inputs(52, B=2, TQ=1, TK=3000, H=4, HKV=2, D=D, dtype=dtype, pos=(lens - 1)[:, None], scale=0.5)
+    XP = with_rope(to_paged(XD, 16, seed=5, seq_lens=lens), 4096)
+    A = _ext(scan_extend_backend="dynamic_extend", sa_extend_backend="infllm", model_context_length=model_ctx,
+             extend_context_length=3072)
+    octx, ometa = O.hip_attention_12(XP, A)
+    ctx, meta = run_product(XP, A)
     assert_metadata_equal(meta, ometa)
     assert_context_close(ctx, octx, dtype)
 
@@ -115,9 +142,13 @@ def test_unbuilt_rules_fail_loudly():
     print("[case] rope unbuilt rules", flush=True)
     X = with_rope(make_inputs(36, B=1, TQ=32, TK=512, H=2, HKV=1, D=32, dtype="f32"), 1024)
     with pytest.raises(NotImplementedError):
-        run_product(X, _ext(scan_extend_backend="dynamic_extend"))
-    with pytest.raises((N.HipAttnError, NotImplementedError)):
+        run_product(X, _ext(scan_extend_backend="self_extend"))
+    with pytest.raises(NotImplementedError):
         run_product(X, _ext(sa_extend_backend="relative"))
+    with pytest.raises(NotImplementedError):
+        run_product(X, _ext(sa_extend_backend="dynamic_extend"))
+    with pytest.raises(N.HipAttnError):  # the squeeze divides by pmin - model_context_length / 4: tiny lengths are refused
+        run_product(X, _ext(scan_extend_backend="dynamic_extend", model_context_length=64))
     with pytest.raises(NotImplementedError):
         run_product(X, tiny_args(using_extend=True, need_apply_rope=False))
 
