@@ -48,11 +48,14 @@ def cdiv(a, b):
 
 
 def mask_stage_bytes(B, TDST, HEAD, HID, esz, stage_shapes):
-    """Algorithmic bytes of mask estimation: every sampled key row, per (batch, q-block, head, chunk, iteration)."""
+    """Algorithmic bytes of mask estimation: the key rows a search has to read, per (batch, q-block, head, chunk).
+    A search over a chunk of 2^k tokens runs k + 1 iterations of two samples; the last two iterations sample three
+    tokens again whose rows (and scores) the search already holds, so 2 (k + 1) - 3 rows are distinct."""
     out = []
     for (bq, n, chunk) in stage_shapes:
         iters = chunk.bit_length()  # floor(log2(chunk)) + 1
-        rows = B * cdiv(TDST, bq) * HEAD * n * iters * 2
+        per_search = 2 * iters - 3 if iters >= 2 else 2
+        rows = B * cdiv(TDST, bq) * HEAD * n * per_search
         out.append(rows * HID * esz)
     return out
 

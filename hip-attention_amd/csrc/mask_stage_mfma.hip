@@ -221,18 +221,42 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
     }
 
     const int lrow = lane / PPR, lpos = lane % PPR;  // loader role: row within an instruction, piece slot
+    // The last iterations of a search sample tokens again: in a range of two tokens one of the samples is the winner
+    // of the iteration before, in a range of one both are.  A lane keeps its previous sample (token, score) and
+    // takes a repeated token's score from there, or from its partner of the other side, instead of loading the row
+    // and multiplying again; the score of a token depends on nothing else.  Under the relative rule (and with keys
+    // rotated ahead per side) the rotation follows the side, so only the lane's own side counts there.
+    bool cross_side = RMODE != 2;
+    if constexpr (ROPE) cross_side = p.rope.backend != HIPATTN_EXTEND_RELATIVE;
+    int ptok[NB];
+    float pscore[NB];
+#pragma unroll
+    for (int tb = 0; tb < NB; tb++) {
+        ptok[tb] = -1;
+        pscore[tb] = 0.0f;
+    }
     while (width >= p.terminate) {
         width *= 0.5f;
-        bool active[NB];
-        int ctr[NB];
+        bool active[NB], reuse[NB], fresh[NB];
+        int ctr[NB], tok[NB];
+        float rscore[NB];
         uint4 raw[VIA_LDS ? 1 : NB][VIA_LDS ? 1 : KS];
 #pragma unroll
         for (int tb = 0; tb < NB; tb++) {
             active[tb] = real[tb] && (cl[tb] < cr[tb]) && (cl[tb] <= lim) && (cl[tb] >= 0);
             ctr[tb] = (cl[tb] + cr[tb]) >> 1;
+            tok[tb] = side ? ((ctr[tb] + cr[tb]) >> 1) : ((cl[tb] + ctr[tb]) >> 1);
+            {
+                const int otok = __shfl_xor(ptok[tb], 1);
+                const float oscore = __shfl_xor(pscore[tb], 1);
+                const bool mine = tok[tb] == ptok[tb];
+                reuse[tb] = active[tb] && (mine || (cross_side && tok[tb] == otok));
+                rscore[tb] = mine ? pscore[tb] : oscore;
+            }
+            fresh[tb] = __any(active[tb] && !reuse[tb]) != 0;
             int64_t off = NO_ROW;
-            if (active[tb]) {
-                const int t = side ? ((ctr[tb] + cr[tb]) >> 1) : ((cl[tb] + ctr[tb]) >> 1);
+            if (active[tb] && !reuse[tb]) {
+                const int t = tok[tb];
                 // access flags: wide launches (prefill) revisit rows constantly, so they look before they store;
                 // narrow ones (decode) touch mostly fresh rows and store blindly
                 off = kv_k_row<EXT, NB == 2>(p.kv, kx, b, t, kvh, seqlen, hh == 0);
@@ -260,7 +284,10 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
                 }
             }
         }
-        if constexpr (VIA_LDS) {
+        bool any_fresh = false;  // uniform over the wave, and the LDS path's workgroups are one wave
+#pragma unroll
+        for (int tb = 0; tb < NB; tb++) any_fresh = any_fresh || fresh[tb];
+        if (VIA_LDS && any_fresh) {
             __syncthreads();
             // coalesced fetch: PPR lanes cover one row; piece q of row r is parked at slot q ^ swz(r)
 #pragma unroll
@@ -282,6 +309,8 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
         }
 #pragma unroll
         for (int tb = 0; tb < NB; tb++) {
+            float v = -INFINITY;
+            if (fresh[tb]) {
             f32x16 acc[MB];
 #pragma unroll
             for (int mb = 0; mb < MB; mb++)
@@ -315,7 +344,6 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
                 for (int mb = 0; mb < MB; mb++)
                     acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qf[mb][ks].v, kf.v, acc[mb], 0, 0, 0);
             }
-            float v = -INFINITY;
             if (fast_rows == 16) {
 #pragma unroll
                 for (int i = 0; i < 8; i++) v = fmaxf(v, acc[0][i]);
@@ -335,6 +363,12 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
             }
             v = fmaxf(v, __shfl_xor(v, 32));
             v = round_bf16(v);
+            }
+            if (reuse[tb]) v = rscore[tb];
+            if (active[tb]) {
+                ptok[tb] = tok[tb];
+                pscore[tb] = v;
+            }
             const float other = __shfl_xor(v, 1);
             const float sL = side ? other : v;
             const float sR = side ? v : other;
@@ -430,7 +464,7 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
         const char *e = getenv("HIPATTN_MASK_NB");
         env_nb = e ? atoi(e) : 0;
     }
-    const int nb0 = (env_nb == 2 && BC >= 32) ? 2 : (wide ? 2 : 1);
+    const int nb0 = (env_nb == 2 && BC >= 32) ? 2 : (env_nb == 1 ? 1 : (wide ? 2 : 1));
     // LDS path: one wave per workgroup (it uses workgroup barriers); direct path: up to 4 heads per workgroup
     // (measured: sharing pays with one query-row block per program, not with two)
     if (g_mask_via_lds < 0) {
