@@ -33,13 +33,13 @@ HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 # HBM bytes per launch of the prefill kernels, from two rocprofv3 --pmc runs of this file (FETCH_SIZE, then
-# WRITE_SIZE, KiB per dispatch).  A 268 435 456-byte device copy reads 131 094 KiB of FETCH_SIZE and 262 144 KiB of
+# WRITE_SIZE, KiB per dispatch).  A 268 435 456-byte device copy reads 131 095 KiB of FETCH_SIZE and 262 144 KiB of
 # WRITE_SIZE in the same runs, so FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0.
 MEASURED_TRAFFIC_BYTES = {
-    "mask_stage[n=507,chunk=256,rows=16]": 2.0 * 772743.5 * 1024 + 53366.8 * 1024,
-    "mask_stage[n=1024,chunk=32,rows=16]": 2.0 * 2149794.1 * 1024 + 65683.6 * 1024,
-    "mask_stage[n=1024,chunk=8,rows=64]": 2.0 * 3694235.9 * 1024 + 131098.5 * 1024,
-    "bsa_prefill": 2.0 * 1831309.1 * 1024 + 262144.0 * 1024,
+    "mask_stage[n=507,chunk=256,rows=16]": 2.0 * 805247.5 * 1024 + 52370.1 * 1024,
+    "mask_stage[n=1024,chunk=32,rows=16]": 2.0 * 2158640.2 * 1024 + 65683.5 * 1024,
+    "mask_stage[n=1024,chunk=8,rows=64]": 2.0 * 3778523.6 * 1024 + 131098.2 * 1024,
+    "bsa_prefill": 2.0 * 1857323.1 * 1024 + 262144.8 * 1024,
 }
 
 

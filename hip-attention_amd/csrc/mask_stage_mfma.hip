@@ -486,7 +486,13 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
     bool via_lds = g_mask_via_lds == 2 ? (!wide && p.chunk > 32) : (g_mask_via_lds == 1);
     if (((p.kx.extended() || two_sided) && nb == 2) || rope) via_lds = false;
     const bool ext = rope || two_sided || p.kx.extended() || (wide && !two && !via_lds);
-    const int hpw = (via_lds || two) ? 1 : (p.G < 4 ? p.G : 4);
+    static int env_hpw2 = -1;
+    if (env_hpw2 < 0) {
+        const char *e = getenv("HIPATTN_MASK_HPW_TWO");
+        env_hpw2 = e ? atoi(e) : 1;
+    }
+    const int hpw_two = env_hpw2 < p.G ? env_hpw2 : p.G;
+    const int hpw = via_lds ? 1 : two ? hpw_two : (p.G < 4 ? p.G : 4);
     const int hblocks = (p.G + hpw - 1) / hpw;
     p.total = (long long)p.B * p.kv.HKV * hblocks * p.BS * p.ngroups * nsub;
     if (p.total >= 0x7fffffffLL) {
