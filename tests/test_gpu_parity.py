@@ -157,6 +157,26 @@ def test_many_query_blocks_use_the_throughput_selection_kernel():
     assert_context_close(ctx, octx, "bf16")
 
 
+@pytest.mark.parametrize("case", ["chunks 48/12/4", "early terminate 2", "chunks 40/8", "early terminate 4, f32"])
+def test_uneven_chunk_sizes_and_early_termination(case):
+    """Chunk sizes that are no powers of two make searches of uneven length (ranges of 3, 5, 6 tokens ...), and
+    stage_early_terminate cuts the last rounds off: both change which samples of a search repeat, which the scan
+    kernel on the matrix cores serves from the round before instead of loading the row again."""
+    _case(f"scan {case}")
+    dtype = "f32" if "f32" in case else "bf16"
+    X = make_inputs(61, B=1, TQ=100, TK=3000, H=4, HKV=2, D=64, dtype=dtype)
+    if case == "chunks 48/12/4":
+        A = tiny_args(stages=[O.OStage(32, 2, 48, None, 1), O.OStage(32, 2, 12, 1536, 1), O.OStage(32, 1, 4, 768, 1)])
+    elif case == "chunks 40/8":
+        A = tiny_args(stages=[O.OStage(32, 2, 40, None, 1), O.OStage(32, 1, 8, 1000, 1)], second_stage_k=600)
+    else:
+        A = tiny_args(stage_early_terminate=4 if "4" in case else 2)
+    octx, ometa = O.hip_attention_12(X, A)
+    ctx, meta = run_product(X, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, dtype)
+
+
 def test_head_reduce_off_matches_oracle(monkeypatch):
     _case("head reduce off")
     monkeypatch.setenv("HIP_HEAD_REDUCE", "0")
