@@ -19,6 +19,7 @@ struct MaskParamsBase {
     int B, TDST, HEAD, G, BS, BDST, BQ, stride_q, nrows, block_chunk, scan_stride, sw_eff;
     float terminate;
     int ngroups;
+    int group_reps;  // bf16 path: consecutive chunk groups walked by one wave (set by its launcher)
     long long total;
     float c_q, c_k;
     float *scores;

@@ -97,8 +97,10 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
     L /= nsub;
     const int s = (int)(L % p.BS);
     L /= p.BS;
-    const int g = (int)(L % p.ngroups);
-    L /= p.ngroups;
+    const int group_reps = MB == 2 ? p.group_reps : 1;
+    const int groups_outer = (p.ngroups + group_reps - 1) / group_reps;
+    const int g0 = (int)(L % groups_outer) * group_reps;
+    L /= groups_outer;
     const int kvh = (int)(L % p.kv.HKV);
     const int b = (int)(L / p.kv.HKV);
     const int h = kvh * p.G + hin;
@@ -109,6 +111,46 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
     const int64_t row_out = (((int64_t)b * p.BS + s) * p.HEAD + h) * p.n;
     const int64_t red_out = ((int64_t)b * p.BS + s) * p.n;
 
+    // ---- rows of this program
+    const long long qb = (long long)(p.BDST - 1) - (long long)(p.BS - 1) * p.scan_stride + (long long)s * p.scan_stride;
+    const long long myrow = qb * p.BQ + (long long)lane * p.stride_q;
+    const bool rv = (lane < p.nrows) && (myrow >= 0) && (myrow < p.TDST);
+    const unsigned long long rowmask = __ballot(rv);
+    const long long mypos = rv ? p.pos[(int64_t)b * p.pos_sb + myrow * p.pos_st] : 0x7fffffffffffffffLL;
+    const long long pmin = wave_min_ll(mypos);
+
+    // ---- Q^ fragments: lane (row = mb*32 + n, half hh) holds elements hh*HALF + ks*8 .. +8.
+    // Rows were averaged, rounded and scaled once per stage by qhat_kernel: [B, BS, HEAD, nrows, HID].
+    // They are fetched when the first chunk group of this wave has work and then serve all of its groups.
+    BFrag qf[MB][KS];
+    bool q_loaded = false;
+    // which of this lane's accumulator elements belong to valid query rows:
+    // element (mb, i) <-> row mb*32 + (i/4)*8 + hh*4 + i%4
+    unsigned vm[MB];
+    bool all_rows = true;
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+        vm[mb] = 0;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int j = mb * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
+            if ((j < p.nrows) && ((rowmask >> j) & 1ull)) vm[mb] |= 1u << i;
+        }
+    }
+    // fast paths: exactly the first 16 / 32 / 64 rows valid
+    const int fast_rows = (p.nrows == 16 && rowmask == 0xffffull) ? 16
+                        : (p.nrows == 32 && rowmask == 0xffffffffull) ? 32
+                        : (MB == 2 && p.nrows == 64 && rowmask == ~0ull) ? 64 : 0;
+    (void)all_rows;
+
+    const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
+    // ---- a wave walks p.group_reps consecutive chunk groups of its (scan row, head) with the same Q^ fragments
+    // (only the 64-row variant: with 16 or 32 rows the fragments are a tenth of the traffic, and the loop costs the
+    // registers of a third wave per SIMD)
+    const int reps = MB == 2 ? p.group_reps : 1;
+    for (int rep = 0; rep < reps; rep++) {
+    const int g = g0 + rep;
+    if (g >= p.ngroups) break;
     // ---- program-level quantities over the whole group of BC chunks
     int gl = (int)p.kv.max_tsrc, gr = (int)p.kv.max_tsrc;
     {
@@ -138,14 +180,6 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
         score[tb] = -32000.0f;
     }
 
-    // ---- rows of this program
-    const long long qb = (long long)(p.BDST - 1) - (long long)(p.BS - 1) * p.scan_stride + (long long)s * p.scan_stride;
-    const long long myrow = qb * p.BQ + (long long)lane * p.stride_q;
-    const bool rv = (lane < p.nrows) && (myrow >= 0) && (myrow < p.TDST);
-    const unsigned long long rowmask = __ballot(rv);
-    const long long mypos = rv ? p.pos[(int64_t)b * p.pos_sb + myrow * p.pos_st] : 0x7fffffffffffffffLL;
-    const long long pmin = wave_min_ll(mypos);
-
     bool run = (rowmask != 0ull) && (pmin >= 0);
     int lim = 0;
     float width = 0.0f;
@@ -167,13 +201,11 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
     };
     if (!run || !(width >= p.terminate)) {
         store_out();
-        return;
+        continue;
     }
 
-    // ---- Q^ fragments: lane (row = mb*32 + n, half hh) holds elements hh*HALF + ks*8 .. +8.
-    // Rows were averaged, rounded and scaled once per stage by qhat_kernel: [B, BS, HEAD, nrows, HID].
-    BFrag qf[MB][KS];
-    {
+    if (!q_loaded) {
+        q_loaded = true;
         const uint16_t *qh = p.qhat + ((((int64_t)b * p.BS + s) * p.HEAD + h) * p.nrows) * HID;
 #pragma unroll
         for (int mb = 0; mb < MB; mb++) {
@@ -186,26 +218,6 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
             }
         }
     }
-    // which of this lane's accumulator elements belong to valid query rows:
-    // element (mb, i) <-> row mb*32 + (i/4)*8 + hh*4 + i%4
-    unsigned vm[MB];
-    bool all_rows = true;
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++) {
-        vm[mb] = 0;
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int j = mb * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
-            if ((j < p.nrows) && ((rowmask >> j) & 1ull)) vm[mb] |= 1u << i;
-        }
-    }
-    // fast paths: exactly the first 16 / 32 / 64 rows valid
-    const int fast_rows = (p.nrows == 16 && rowmask == 0xffffull) ? 16
-                        : (p.nrows == 32 && rowmask == 0xffffffffull) ? 32
-                        : (MB == 2 && p.nrows == 64 && rowmask == ~0ull) ? 64 : 0;
-    (void)all_rows;
-
-    const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
 
     uint4 rcos[ROPE ? NB : 1][ROPE ? KS : 1], rsin[ROPE ? NB : 1][ROPE ? KS : 1];
     if constexpr (ROPE) {
@@ -380,6 +392,7 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
         }
     }
     store_out();
+    }
 }
 
 // Q^ rows of every scan program: strided mean of stride_q query rows in f32, rounded to bf16, scaled
@@ -494,7 +507,18 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
     const int hpw_two = env_hpw2 < p.G ? env_hpw2 : p.G;
     const int hpw = via_lds ? 1 : two ? hpw_two : (p.G < 4 ? p.G : 4);
     const int hblocks = (p.G + hpw - 1) / hpw;
-    p.total = (long long)p.B * p.kv.HKV * hblocks * p.BS * p.ngroups * nsub;
+    // wide launches with 64 query rows: a wave keeps its Q^ fragments for several chunk groups (they are 16 KB
+    // against the 40 KB of key rows that 32 searches over 8 tokens read; cfg-2-like prefill: 4.9 ms for one group
+    // per wave, 4.3 / 4.0 / 3.9 ms for 2 / 4 / 8)
+    static int env_reps = -1;
+    if (env_reps < 0) {
+        const char *e = getenv("HIPATTN_MASK_GROUP_REPS");
+        env_reps = e ? atoi(e) : 0;
+    }
+    p.group_reps = !two ? 1 : env_reps > 0 ? env_reps : (wide ? 8 : 1);
+    if (p.group_reps > p.ngroups) p.group_reps = p.ngroups;
+    const int groups_outer = (p.ngroups + p.group_reps - 1) / p.group_reps;
+    p.total = (long long)p.B * p.kv.HKV * hblocks * p.BS * groups_outer * nsub;
     if (p.total >= 0x7fffffffLL) {
         set_error("mask stage: grid too large");
         return HIPATTN_E_UNSUPPORTED;
