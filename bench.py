@@ -36,10 +36,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # WRITE_SIZE, KiB per dispatch).  A 268 435 456-byte device copy reads 131 095 KiB of FETCH_SIZE and 262 144 KiB of
 # WRITE_SIZE in the same runs, so FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0.
 MEASURED_TRAFFIC_BYTES = {
-    "mask_stage[n=507,chunk=256,rows=16]": 2.0 * 805247.5 * 1024 + 52370.1 * 1024,
-    "mask_stage[n=1024,chunk=32,rows=16]": 2.0 * 2158640.2 * 1024 + 65683.5 * 1024,
-    "mask_stage[n=1024,chunk=8,rows=64]": 2.0 * 3778523.6 * 1024 + 131098.2 * 1024,
-    "bsa_prefill": 2.0 * 1857323.1 * 1024 + 262144.8 * 1024,
+    "mask_stage[n=507,chunk=256,rows=16]": 2.0 * 815547.2 * 1024 + 52343.8 * 1024,
+    "mask_stage[n=1024,chunk=32,rows=16]": 2.0 * 2162302.3 * 1024 + 65683.4 * 1024,
+    "mask_stage[n=1024,chunk=8,rows=64]": 2.0 * 2738474.5 * 1024 + 131105.2 * 1024,
+    "bsa_prefill": 2.0 * 1857880.6 * 1024 + 262145.5 * 1024,
 }
 
 
