@@ -25,7 +25,7 @@ struct MaskParamsBase {
     float *scores;
     int reduce_heads;  // scores is [B, BS, 1, n], pre-filled with -inf, and receives the max over heads
     int32_t *left_out;
-    const uint16_t *qhat;  // bf16 path: workspace [B, BS, HEAD, nrows, HID] filled by the entry point
+    const uint16_t *qhat;  // bf16 path: workspace [B, BS, HEAD][nrows * HID] filled by the entry point (fragment order)
 };
 
 // the extended kernels (statistics, offload cache) take the same block with the extras appended

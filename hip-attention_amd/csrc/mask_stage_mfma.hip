@@ -120,7 +120,8 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
     const long long pmin = wave_min_ll(mypos);
 
     // ---- Q^ fragments: lane (row = mb*32 + n, half hh) holds elements hh*HALF + ks*8 .. +8.
-    // Rows were averaged, rounded and scaled once per stage by qhat_kernel: [B, BS, HEAD, nrows, HID].
+    // Rows were averaged, rounded and scaled once per stage by qhat_kernel: [B, BS, HEAD] blocks of nrows * HID
+    // elements, laid out by (k-step, row half, row) so that the lanes of a load instruction read consecutive pieces.
     // They are fetched when the first chunk group of this wave has work and then serve all of its groups.
     BFrag qf[MB][KS];
     bool q_loaded = false;
@@ -214,7 +215,7 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
 #pragma unroll
             for (int ks = 0; ks < KS; ks++) {
                 qf[mb][ks].q = make_uint4(0, 0, 0, 0);
-                if (jv) qf[mb][ks].q = *reinterpret_cast<const uint4 *>(qh + (int64_t)j * HID + hh * HALF + ks * 8);
+                if (jv) qf[mb][ks].q = *reinterpret_cast<const uint4 *>(qh + ((int64_t)(ks * 2 + hh) * p.nrows + j) * 8);
             }
         }
     }
@@ -459,7 +460,14 @@ __global__ void qhat_kernel(MaskParams p, int hid, uint16_t *out) {
         }
         o = make_uint4(ow[0], ow[1], ow[2], ow[3]);
     }
-    *reinterpret_cast<uint4 *>(out + gid * 8) = o;
+    // stored in the order the scan kernel's lanes fetch them: per (b, s, h) the 16-byte piece of k-step ks, row half hh
+    // and row j sits at ((ks * 2 + hh) * nrows + j), so one load instruction of a wave reads consecutive pieces
+    {
+        const int half_pieces = per_row / 2;
+        const int hh = piece / half_pieces, ks = piece % half_pieces;
+        const long long base = (gid / per_row / p.nrows) * (long long)p.nrows * hid;
+        *reinterpret_cast<uint4 *>(out + base + ((long long)(ks * 2 + hh) * p.nrows + j) * 8) = o;
+    }
 }
 
 static int g_mask_via_lds = -1;  // -1: decide per shape; 0 / 1: forced through HIPATTN_MASK_VIA_LDS (tuning aid)
