@@ -48,14 +48,21 @@ def _stage0(TK, sink, sw_eff, chunk, B, BS, H):
     return left, right, scores
 
 
-@pytest.mark.parametrize("backend", ["relative", "streaming", "infllm"])
+@pytest.mark.parametrize("backend", ["relative", "streaming", "infllm", "dynamic_extend", "dynamic_extend squeezed"])
 def test_mask_stage_chunk_size_one_scores(backend):
     # Chunks of one token: the scan evaluates token t once as the "left" and once as the "right" candidate and
     # keeps the larger score.  relative: key at 0 (left) or 1 (right), query at 1 + window; streaming: key at its
-    # chunk number, query at min(position, chunks + window); infllm: key at 0, query at the window.
+    # chunk number, query at min(position, chunks + window); infllm: key at 0, query at the window; dynamic_extend:
+    # every query row at its own position, and the key at its own token while the block ends inside the model's
+    # context -- plain rotary scores -- or, beyond it (model context 32 against positions 48..63), keys older than
+    # a quarter of that context squeezed linearly into the rest (attention_extend.py:249-274).
     D, BQ, sink, sw_eff = 32, 8, 4, 6
     X = make_inputs(11, B=1, TQ=16, TK=64, H=2, HKV=1, D=D, dtype="f32")
+    squeezed = backend.endswith("squeezed")
+    backend = backend.split()[0]
     X = with_rope(X, 256, scan_backend=backend)
+    if squeezed:
+        X.model_context_length = 32
     left, right, scores = _stage0(64, sink, sw_eff, 1, 1, 2, 2)
     l_in = left.copy()
     n = left.shape[-1]
@@ -72,6 +79,14 @@ def test_mask_stage_chunk_size_one_scores(backend):
                 qpos, kpos = np.full(BQ, 1 + sw_eff), (lambda c: (0, 1))
             elif backend == "infllm":
                 qpos, kpos = np.full(BQ, sw_eff), (lambda c: (0, 0))
+            elif backend == "dynamic_extend":
+                def kpos(c, t, pmin=int(p.min()), pmax=int(p.min()) + BQ, ctx=int(X.model_context_length)):
+                    w = ctx // 4
+                    if t >= pmax - w or pmax <= ctx:
+                        return (t, t)
+                    moved = int((np.float32(t) - np.float32(pmin - w)) * (np.float32(ctx - w) / np.float32(pmin - w)))
+                    return (max(pmax - ctx, moved + pmin - w),) * 2
+                qpos = p
             else:
                 qpos, kpos = np.minimum(p, n + sw_eff), (lambda c: (c, c))
             qr = _rot(q[0, rows, h], qpos, D) * cq
@@ -80,7 +95,10 @@ def test_mask_stage_chunk_size_one_scores(backend):
                 if t > p.min() - sw_eff:
                     assert scores[0, qb, h, c] == -32000.0
                     continue
-                best = max(float((qr @ (_rot(k[0, t, 0], kp, D) * ck)).max()) for kp in kpos(c))
+                kps = kpos(c, t) if backend == "dynamic_extend" else kpos(c)
+                if squeezed and t < 40:
+                    assert kps[0] != t  # the squeeze really moves these keys
+                best = max(float((qr @ (_rot(k[0, t, 0], kp, D) * ck)).max()) for kp in kps)
                 assert abs(scores[0, qb, h, c] - best) <= 2e-5 * max(1.0, abs(best)), (backend, h, qb, c)
                 checked += 1
     assert checked > 50
