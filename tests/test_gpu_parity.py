@@ -177,6 +177,22 @@ def test_uneven_chunk_sizes_and_early_termination(case):
     assert_context_close(ctx, octx, dtype)
 
 
+def test_wide_scan_with_64_query_rows_walks_chunk_groups_in_a_loop():
+    """16384 and more scan programs with 64 query rows: a wave of the scan kernel keeps its query fragments and walks
+    eight chunk groups; 2050 chunks make 33 groups of 64, so the last wave of a row walks one group that holds two
+    chunks.  (The oracle needs about 20 s of CPU time for this shape.)"""
+    _case("wide scan, 64 rows, 33 chunk groups")
+    TK = 16 + 128 + 2050 * 4
+    X = make_inputs(71, B=1, TQ=2048, TK=TK, H=16, HKV=4, D=32, dtype="bf16")
+    A = tiny_args(stages=[O.OStage(64, 1, 4, None, 1)], sliding_window_size=128, second_stage_k=256,
+                  block_sparse_block_size_q=64)
+    octx, ometa = O.hip_attention_12(X, A)
+    print("  oracle done", flush=True)
+    ctx, meta = run_product(X, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, "bf16")
+
+
 def test_head_reduce_off_matches_oracle(monkeypatch):
     _case("head reduce off")
     monkeypatch.setenv("HIP_HEAD_REDUCE", "0")
