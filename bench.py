@@ -35,12 +35,16 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the prefill kernels, from two rocprofv3 --pmc runs of this file (FETCH_SIZE, then
 # WRITE_SIZE, KiB per dispatch).  A 268 435 456-byte device copy reads 131 095 KiB of FETCH_SIZE and 262 144 KiB of
 # WRITE_SIZE in the same runs, so FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0.
+TRAFFIC_SOURCE = "recorded: profiles/prefill_hbm_traffic_pmc.md (not measured in this run)"
 MEASURED_TRAFFIC_BYTES = {
     "mask_stage[n=507,chunk=256,rows=16]": 2.0 * 815547.2 * 1024 + 52343.8 * 1024,
     "mask_stage[n=1024,chunk=32,rows=16]": 2.0 * 2162302.3 * 1024 + 65683.4 * 1024,
     "mask_stage[n=1024,chunk=8,rows=64]": 2.0 * 2738474.5 * 1024 + 131105.2 * 1024,
     "bsa_prefill": 2.0 * 1857880.6 * 1024 + 262145.5 * 1024,
 }
+
+
+SAMPLE_QUERIES = 512  # the last queries of the prefill workload that the CPU oracle recomputes
 
 
 def cdiv(a, b):
@@ -111,20 +115,35 @@ def run_prefill(args, device):
     rooflines = []
     for nm, by in zip(names, stage_bytes):
         if nm in kern:
+            # The scan's sampled rows are served by the L1 / L2 gather path, not by HBM (the keys of a kv head are
+            # re-read by every query block), so the rows it reads per second are reported as what they are, logical
+            # bytes, with no roof; the fraction of the HBM peak is taken from the recorded HBM counters.
             gbs = by / (kern[nm] * 1e-3) / 1e9
-            rooflines.append({"kernel": nm, "bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                              "frac": gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(nm), "ms": kern[nm],
-                              "algorithmic_bytes": by})
+            traffic = MEASURED_TRAFFIC_BYTES.get(nm)
+            hbm_gbs = traffic / (kern[nm] * 1e-3) / 1e9 if traffic else None
+            rooflines.append({"kernel": nm, "bound": "l2-gather", "achieved": gbs, "peak": None, "unit": "GB/s",
+                              "frac": None, "logical_GBps": gbs, "traffic": traffic, "traffic_source": TRAFFIC_SOURCE,
+                              "hbm_counter_GBps": hbm_gbs,
+                              "frac_hbm_counter": hbm_gbs / HBM_PEAK_GBS if hbm_gbs else None,
+                              "ms": kern[nm], "algorithmic_bytes": by})
     if "bsa_prefill" in kern:
         tf = bsa_flops / (kern["bsa_prefill"] * 1e-3) / 1e12
         rooflines.append({"kernel": "bsa_prefill", "bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS,
                           "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS,
-                          "traffic": MEASURED_TRAFFIC_BYTES.get("bsa_prefill"),
+                          "traffic": MEASURED_TRAFFIC_BYTES.get("bsa_prefill"), "traffic_source": TRAFFIC_SOURCE,
                           "ms": kern["bsa_prefill"], "algorithmic_flops": bsa_flops})
-    dominant = max(rooflines, key=lambda r: r["ms"]) if rooflines else None
+    # headline: the kernel of this step that sits under a hardware roof, the sparse attention kernel (matrix cores)
+    roofed = [r for r in rooflines if r["frac"] is not None]
+    dominant = max(roofed, key=lambda r: r["ms"]) if roofed else None
+    # the last query blocks of the timed call's result, for the comparison with the oracle in the cpu_baseline leg
+    nb = SAMPLE_QUERIES // 64
+    sample = {"indices": meta.indices[:, -nb:].cpu().numpy(), "ks": meta.ks[:, -nb:].cpu().numpy(),
+              "ks_start_end": meta.ks_start_end[:, -nb:].cpu().numpy(),
+              "context": ctx[:, -SAMPLE_QUERIES:].float().cpu().numpy()}
     del q, k, v, ctx, meta
     torch.cuda.empty_cache()
     return {
+        "sample": sample,
         "ms_per_step": ms_per_step,
         "tok_per_s": TQ / (ms_per_step * 1e-3),
         "kernels_ms": kern,
@@ -189,9 +208,25 @@ def _time_decode(step, steps, refresh_every):
     with torch.cuda.graph(g_cached, pool=g_refresh.pool()):
         out_c, _ = step(meta_r)
     torch.cuda.synchronize()
-    us_mixed = timed(steps, lambda i: (g_refresh if i % refresh_every == 0 else g_cached).replay())
-    us_refresh = timed(16, lambda i: g_refresh.replay())
-    us_cached = timed(64, lambda i: g_cached.replay())
+    # One replay of the cached step is two kernels (about 16 us): the host cannot always enqueue graphs that fast, so
+    # timing back-to-back replays of it measures the host as often as the GPU.  The GPU time of a step is therefore
+    # taken from a graph that holds 16 steps, median of 9 timings; the one-step-per-replay figure stays beside it.
+    g_cached16 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g_cached16, pool=g_refresh.pool()):
+        for _ in range(16):
+            out_c16, _ = step(meta_r)
+    torch.cuda.synchronize()
+
+    def median(xs):
+        xs = sorted(xs)
+        return xs[len(xs) // 2]
+
+    us_mixed = median([timed(steps, lambda i: (g_refresh if i % refresh_every == 0 else g_cached).replay())
+                       for _ in range(5)])
+    us_refresh = median([timed(16, lambda i: g_refresh.replay()) for _ in range(9)])
+    us_cached_single = median([timed(64, lambda i: g_cached.replay()) for _ in range(9)])
+    us_cached = median([timed(4, lambda i: g_cached16.replay()) / 16 for _ in range(9)])
+    del g_cached16, out_c16
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
@@ -210,7 +245,7 @@ def _time_decode(step, steps, refresh_every):
     with torch.cuda.graph(g_plain, pool=g_refresh.pool()):
         out_p, _ = step(None, False)
     torch.cuda.synchronize()
-    us_refresh_plain = timed(16, lambda i: g_plain.replay())
+    us_refresh_plain = median([timed(16, lambda i: g_plain.replay()) for _ in range(9)])
     del g_plain, out_p
     N.profile_begin()
     _, meta_last = step(None)
@@ -219,7 +254,8 @@ def _time_decode(step, steps, refresh_every):
     return {
         "launch": "hip graph replay (one graph per step kind)",
         "us_per_step_mixed": us_mixed, "us_per_step_refresh": us_refresh,
-        "us_per_step_cached": us_cached, "wall_us_per_step_mixed": wall_us, "refresh_every": refresh_every,
+        "us_per_step_cached": us_cached, "us_per_step_cached_one_graph_per_step": us_cached_single,
+        "wall_us_per_step_mixed": wall_us, "refresh_every": refresh_every,
         "us_per_step_refresh_without_statistics": us_refresh_plain,
         "graph_replay_matches_eager": graph_matches,
         "eager": {"us_per_step_mixed": eager_mixed, "us_per_step_refresh": eager_refresh,
@@ -263,8 +299,11 @@ def run_decode(args, device, TK=1 << 20, steps=64, refresh_every=8, needles=64):
     chunk = 1 << 17
     for s in range(0, TK, chunk):
         k[:, s:s + chunk] = torch.randn((1, chunk, HKV, D), generator=g, dtype=torch.float32).to(torch.bfloat16).to(device)
-    # needles: 8-token blocks at seeded positions whose component along a unit direction u is set to +12;
-    # the decode query is noise + 12 u, so a needle token scores ~144 against ~N(0, 17^2) for ordinary keys
+    # needles: 8-token blocks at seeded positions whose component along a unit direction u is set to +12, where an
+    # ordinary N(0,1) key has a component of about +-1 and never more than 4 or 5 (the workload description speaks of
+    # blocks "scaled x4 along a query-aligned direction"; scaling a random component by 4 would leave its sign to
+    # chance and half of the needles anti-aligned, so the component is set to 4 x 3 sigma instead).  The decode query
+    # is noise + 12 u, so a needle token scores ~144 against ~N(0, 17^2) for ordinary keys.
     u = torch.randn((D,), generator=g, dtype=torch.float32)
     u = u / u.norm()
     starts = (torch.randperm((TK - 4096) // 8, generator=g)[:needles] * 8 + 2048).sort().values
@@ -306,6 +345,26 @@ def run_decode(args, device, TK=1 << 20, steps=64, refresh_every=8, needles=64):
                 "needle_recall_any_head": float(found.any(dim=0).float().mean()),
                 "prefill_chunks_ms": [round(x, 1) for x in prefill_ms],
                 "prefill_tok_per_s": TK / (sum(prefill_ms) * 1e-3)})
+    if not args.skip_cpu:
+        # the oracle on the same decode query and keys: a search samples midpoints only, so recall below 1 is the
+        # algorithm's; what must hold is that the kernels select exactly what the oracle selects
+        import numpy as np
+        from oracle import hip12 as O
+
+        kb = k.cpu().view(torch.int16).numpy().view(np.uint16)
+        qb = q.cpu().view(torch.int16).numpy().view(np.uint16)
+        X = O.OInputs("bf16", qb, np.array([[TK - 1]], dtype=np.int64), k=kb, v=kb)
+        octx, ometa = O.hip_attention_12(X, O.OArgs(sliding_window_size=1024))
+        ofound = (ometa.indices[:, 0, :, None] == starts.numpy()[None, None, :]).any(axis=1)
+        out_gpu, _ = step(meta)
+        ref = O.bf16_bits_to_f32(octx)
+        err = np.abs(out_gpu.float().cpu().numpy() - ref)
+        res.update({"oracle_needle_recall_mean_over_heads": float(ofound.mean()),
+                    "oracle_needle_recall_any_head": float(ofound.any(axis=0).mean()),
+                    "indices_equal_oracle": bool(np.array_equal(meta.indices.cpu().numpy(), ometa.indices)
+                                                 and np.array_equal(meta.ks.cpu().numpy(), ometa.ks)),
+                    "context_within_tolerance_of_oracle": bool((err <= 2e-2 + 1e-2 * np.abs(ref)).all())})
+        del kb, X
     refresh_bytes, attn_bytes = _decode_bytes([TK], H, HKV, D)
     del k, v
     torch.cuda.empty_cache()
@@ -506,14 +565,16 @@ def run_offload(args, device, TK=3_000_000, warm_steps=4, drift_steps=12):
     return res
 
 
-def run_cpu_baseline(args):
-    """The CPU oracle on a bounded sample of the prefill workload: last 128 queries, all heads, full keys."""
+def run_cpu_baseline(args, sample=None):
+    """The CPU oracle on a bounded sample of the prefill workload: the last 512 queries, all heads, full keys.
+    With ``sample`` (the same query blocks of the timed GPU call) the two results are compared: indices, ``ks`` and
+    ``ks_start_end`` bit for bit, context within the bf16 tolerance (2e-2 abs + 1e-2 rel)."""
     import numpy as np
     import torch
     from oracle import hip12 as O
 
     TQ_full, TK, H, HKV, D = 32768, 131072, 32, 8, 128
-    TQs = 512
+    TQs = SAMPLE_QUERIES
     g = torch.Generator(device="cpu").manual_seed(1)
     q = torch.randn((1, TQ_full, H, D), generator=g, dtype=torch.float32).to(torch.bfloat16)[:, -TQs:]
     k = torch.randn((1, TK, HKV, D), generator=g, dtype=torch.float32).to(torch.bfloat16)
@@ -524,11 +585,23 @@ def run_cpu_baseline(args):
     A = O.OArgs(sliding_window_size=1024)
     threads = O.lib().hipo_num_threads()
     t0 = time.perf_counter()
-    O.hip_attention_12(X, A)
+    octx, ometa = O.hip_attention_12(X, A)
     dt = time.perf_counter() - t0
+    parity = None
+    if sample is not None:
+        ref = O.bf16_bits_to_f32(octx)
+        err = np.abs(sample["context"] - ref)
+        parity = {
+            "indices_equal": bool(np.array_equal(sample["indices"], ometa.indices)),
+            "ks_equal": bool(np.array_equal(sample["ks"], ometa.ks)
+                             and np.array_equal(sample["ks_start_end"], ometa.ks_start_end)),
+            "context_within_tolerance": bool((err <= 2e-2 + 1e-2 * np.abs(ref)).all()),
+            "context_max_abs_err": float(err.max()),
+        }
     return {"value": TQs / dt, "unit": "tok/s", "cores": int(threads), "kind": "port",
             "sample": f"last {TQs} of 32768 queries ({TQs // 64} query blocks) x 32 heads against all 131072 keys, "
-                      f"{dt:.1f} s of CPU time; throughput is per query token, so it compares directly"}
+                      f"{dt:.1f} s of CPU time; throughput is per query token, so it compares directly",
+            "parity": parity}
 
 
 def main():
@@ -558,7 +631,8 @@ def main():
     dec = run_decode(args, device) if (want("decode") and not args.skip_decode) else None
     bdec = run_batched_decode(args, device) if (want("batched_decode") and not args.skip_decode) else None
     off = run_offload(args, device) if (want("offload") and not args.skip_offload) else None
-    cpu = run_cpu_baseline(args) if (want("cpu") and not args.skip_cpu) else None
+    cpu = run_cpu_baseline(args, pre.get("sample")) if (want("cpu") and not args.skip_cpu) else None
+    par = (cpu or {}).get("parity")
     dom = pre["dominant"] or {}
     line = {
         "metric": "prefill tok/s at 128k KV (hip_attention_12, mask estimation + block-sparse attention)",
@@ -583,6 +657,9 @@ def main():
         "batched_decode": bdec,
         "offload": off,
         "cpu_baseline": cpu,
+        # the timed prefill's last 512 queries against the oracle's run on the same inputs (null: a leg was skipped)
+        "parity_on_sample": (None if par is None else
+                             bool(par["indices_equal"] and par["ks_equal"] and par["context_within_tolerance"])),
     }
     print(json.dumps(line))
 

@@ -65,7 +65,8 @@ class HiPModelOffloadCache:
         self.copy_stream = torch.cuda.Stream(device=device)
         # (layer, batch item) -> (k, v, prefix length, table, event recorded after the gather)
         self.prefetched_kv: Dict[Tuple[int, int], Tuple[Tensor, Tensor, int, Tensor, torch.cuda.Event]] = {}
-        self.enable_async = True
+        # the reference's switch, spelled as it spells it (model_offload_cache.py:108)
+        self.enable_async = os.getenv("HIP_DISABLE_AYSNC", "0") == "0"
         self.require_validation = os.getenv("HIP_OFFLOAD_CACHE_VALIDATION", "0") == "1"
         self.validation_cache = None
         if self.require_validation:  # resident copies [tokens + 1, heads, dim] per layer, K and V

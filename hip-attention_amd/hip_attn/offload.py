@@ -190,8 +190,7 @@ class HiPOffloadCache:
         """Paged (page size 1) description of the host pools with the cache that serves this phase."""
         cache = self.mask_k_cache if masking else self.sa_kv_cache
         cache.wait()
-        if self.pending_write is not None:
-            torch.cuda.current_stream(self.device).wait_event(self.pending_write)
+        self._wait_pending_write()
         kb, vb = self.k_uvm.bank_cpu, self.v_uvm.bank_cpu
         s = N.KVStruct()
         s.k, s.v = self.k_uvm.device_ptr, self.v_uvm.device_ptr
@@ -249,12 +248,21 @@ class HiPOffloadCache:
         for pool in (self.k_uvm, self.v_uvm):
             pool.metadata.index_put_((idx_gpu,), torch.index_select(pool.metadata, 0, idx_gpu) + 1)
 
+    def _wait_pending_write(self, stream: Optional[torch.cuda.Stream] = None):
+        """Order ``stream`` (default: the current one) after a store into the pools issued on another stream: a fetch
+        that ran beside the store could copy a pool row's old bytes into a block that the store's write-through
+        had just found absent."""
+        if self.pending_write is not None:
+            (stream or torch.cuda.current_stream(self.device)).wait_event(self.pending_write)
+
     def handle_cache_miss(self, metadata=None):
         stats_m = getattr(metadata, "mask_cache_statistics", None)
         stats_s = getattr(metadata, "sa_cache_statistics", None)
+        self._wait_pending_write(self.miss_stream)
         self.mask_k_cache.handle_cache_miss(metadata=metadata, stats=stats_m, stream=self.miss_stream)
         self.sa_kv_cache.handle_cache_miss(metadata=metadata, stats=stats_s, stream=self.miss_stream)
 
     def flush(self):
+        self._wait_pending_write()
         self.mask_k_cache.flush()
         self.sa_kv_cache.flush()

@@ -62,6 +62,36 @@ def _reject_unsupported(args: HiPAttentionArgs):
 
 
 _ROPE_TABLES = {}  # (cos ptr, sin ptr, versions, dtype) -> (cos, sin) in the compute dtype; tiny, most recent last
+_ROPE_TABLES_PINNED = {}  # entries handed out while a stream was capturing: a graph holds their addresses, never freed
+
+
+def _capturing(device) -> bool:
+    return device.type == "cuda" and torch.cuda.is_current_stream_capturing()
+
+
+def _cached_for_graphs(cache: dict, pinned: dict, key, build, limit: int, device):
+    """Look up or build a small read-only helper tensor that later calls share.
+
+    A HIP graph records the address of every tensor its kernels read, so an entry that was handed out while a stream
+    was capturing must live as long as the process: it moves to ``pinned`` and is never evicted.  An entry built
+    during a capture belongs to that graph's memory pool and is not kept at all.  Only entries no graph has seen
+    take part in the oldest-first eviction.
+    """
+    hit = pinned.get(key)
+    if hit is not None:
+        return hit
+    capturing = _capturing(device)
+    hit = cache.get(key)
+    if hit is None:
+        hit = build()
+        if capturing:
+            return hit
+        if len(cache) >= limit:
+            cache.pop(next(iter(cache)))
+        cache[key] = hit
+    elif capturing:
+        pinned[key] = cache.pop(key)
+    return hit
 
 
 def _rope_tables(args: HiPAttentionArgs, dtype: torch.dtype):
@@ -81,13 +111,44 @@ def _rope_tables(args: HiPAttentionArgs, dtype: torch.dtype):
     if usable(cos) and usable(sin) and cos.stride(0) == sin.stride(0):
         return cos, sin
     key = (cos.data_ptr(), sin.data_ptr(), cos._version, sin._version, tuple(cos.shape), dtype)
-    hit = _ROPE_TABLES.get(key)
-    if hit is None:
-        hit = (cos.to(dtype).contiguous(), sin.to(dtype).contiguous())
-        if len(_ROPE_TABLES) >= 8:
-            _ROPE_TABLES.pop(next(iter(_ROPE_TABLES)))
-        _ROPE_TABLES[key] = hit
-    return hit
+    return _cached_for_graphs(_ROPE_TABLES, _ROPE_TABLES_PINNED, key,
+                              lambda: (cos.to(dtype).contiguous(), sin.to(dtype).contiguous()), 8, cos.device)
+
+
+def _check_operands(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], args: HiPAttentionArgs):
+    """Refuse K/V storage the kernels would misread.
+
+    The C side derives the element size of every K / V row from q's dtype alone (fp8 caches aside), and takes every
+    pointer for memory of q's device: a key tensor of another dtype would be read at the wrong byte offsets, past
+    its end.  The reference's Triton kernels cast on load instead; here the caller converts.
+    """
+    dev, dt = q.device, q.dtype
+
+    def same(name, t, fp8_ok=False):
+        if t is None:
+            return
+        if t.device != dev:
+            raise N.HipAttnError(f"{name} is on {t.device}, q is on {dev}: every operand must live on q's device")
+        if t.dtype != dt and not (fp8_ok and dt == torch.bfloat16 and t.dtype in N._FP8_DTYPES):
+            what = "q's dtype" + (" (or fp8 e5m2 bytes under a bfloat16 q)" if fp8_ok else "")
+            raise N.HipAttnError(f"{name} has dtype {t.dtype} but q has {dt}: {name} must have {what}")
+
+    def on_device(name, t):
+        if t is not None and t.device != dev:
+            raise N.HipAttnError(f"{name} is on {t.device}, q is on {dev}: every operand must live on q's device")
+
+    same("k", k)
+    same("v", v)
+    same("args.q_mask", args.q_mask)
+    same("args.k_mask", args.k_mask)
+    same("args.k_cache", args.k_cache, fp8_ok=True)
+    same("args.v_cache", args.v_cache, fp8_ok=True)
+    on_device("args.block_table", args.block_table)
+    on_device("args.cache_seq_lens", args.cache_seq_lens)
+    on_device("args.position_ids", args.position_ids)
+    if args.using_extend and args.need_apply_rope:
+        on_device("args.rope_cos", args.rope_cos)
+        on_device("args.rope_sin", args.rope_sin)
 
 
 def _kv_struct(args: HiPAttentionArgs, k: Optional[Tensor], v: Optional[Tensor], max_tsrc: int,
@@ -180,6 +241,7 @@ def _mask_kv(args: HiPAttentionArgs, k_mask: Optional[Tensor], max_tsrc: int, q:
 
 
 _INITIAL_CHUNKS = {}  # read-only stage-0 chunk lists, keyed by their shape parameters
+_INITIAL_CHUNKS_PINNED = {}  # those a captured graph reads: kept for the life of the process
 
 
 def _initial_chunks(chunk_count: int, chunk_size: int, sink: int, B: int, bs: int, hg: int, device) -> Tensor:
@@ -187,18 +249,12 @@ def _initial_chunks(chunk_count: int, chunk_size: int, sink: int, B: int, bs: in
     Nothing writes to a chunk list, so the tensor is built once per shape and shared by later calls (a decode loop
     would otherwise pay four small launches per mask refresh for it)."""
     key = (chunk_count, chunk_size, sink, B, bs, hg, str(device))
-    hit = _INITIAL_CHUNKS.get(key)
-    if hit is None:
-        if torch.cuda.is_current_stream_capturing():
-            # a tensor created inside a capture lives in the graph's pool; build it the plain way and do not keep it
-            row = torch.arange(0, chunk_count, device=device, dtype=torch.int32) * chunk_size + sink
-            return row[None, None, None, :].expand(B, bs, hg, chunk_count).contiguous()
+
+    def build():
         row = torch.arange(0, chunk_count, device=device, dtype=torch.int32) * chunk_size + sink
-        hit = row[None, None, None, :].expand(B, bs, hg, chunk_count).contiguous()
-        if len(_INITIAL_CHUNKS) >= 16:
-            _INITIAL_CHUNKS.pop(next(iter(_INITIAL_CHUNKS)))
-        _INITIAL_CHUNKS[key] = hit
-    return hit
+        return row[None, None, None, :].expand(B, bs, hg, chunk_count).contiguous()
+
+    return _cached_for_graphs(_INITIAL_CHUNKS, _INITIAL_CHUNKS_PINNED, key, build, 16, device)
 
 
 _RESET_SCORE: dict = {}
@@ -256,6 +312,7 @@ def dual_stage_quadratic_hip_attention(
     if not q.is_cuda:
         raise N.HipAttnError("hip_attention_12 runs on the GPU only: q must be a device tensor")
     _reject_unsupported(args)
+    _check_operands(q, k, v, args)
     device = q.device
 
     q_bsa = q
@@ -559,6 +616,9 @@ def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], 
     turns on rotation on load under ``args.sa_extend_backend``.
     """
     device = q.device
+    if not q.is_cuda:
+        raise N.HipAttnError("block_sparse_attention runs on the GPU only: q must be a device tensor")
+    _check_operands(q, k, v, args)
     qq = q if q.stride(-1) == 1 else q.contiguous()
     kvs, keep = _kv_struct(args, k, v, max_tsrc, masking=False, stats=stats)
     if position_ids.dtype != torch.int64:

@@ -103,10 +103,11 @@ def access_flags(md, suffix):
 
 def make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, dtype=torch.float32,
               lens=None, page_size=0, extend=None, softcap=None, block_size_k=64, replay=False, exact=False,
-              model_ctx=None):
+              model_ctx=None, early=None):
     """One call of the reference operator; ``lens`` (decode: TQ == 1) places each sequence's query at lens[b] - 1;
     ``page_size`` > 0 moves K/V into a paged cache behind a shuffled block table; ``extend`` = (scan rule, sa rule)
-    turns on RoPE applied on load; ``model_ctx`` sets model_context_length (the dynamic_extend rule reads it)."""
+    turns on RoPE applied on load; ``model_ctx`` sets model_context_length (the dynamic_extend rule reads it);
+    ``early`` sets stage_early_terminate."""
     g = torch.Generator().manual_seed(seed)
     # values with 8 significant bits, so that the files can hold q, k, v as 16-bit patterns
     short = lambda t: t.to(torch.bfloat16).to(dtype)  # noqa: E731
@@ -121,7 +122,7 @@ def make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, sec
     if lens is None:
         pos = (torch.arange(TQ) + TK - TQ)[None].expand(B, TQ).contiguous()
     else:
-        pos = (torch.tensor(lens, dtype=torch.int64) - 1)[:, None]
+        pos = (torch.tensor(lens, dtype=torch.int64)[:, None] - TQ + torch.arange(TQ)[None]).contiguous()
     kw = dict(sink_token_size=sink, sliding_window_size=sw, second_stage_k=second_k, block_sparse_block_size_q=bsbq,
               stages=[meta.ScanStage(stage_block_size_q=a, stage_block_stride_q=b, stage_chunk_size=c, stage_k=d,
                                      stage_stride=e) for (a, b, c, d, e) in stages],
@@ -139,6 +140,9 @@ def make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, sec
     if softcap is not None:
         kw.update(logit_softcap=softcap)
         extra.update(softcap=softcap)
+    if early is not None:
+        kw.update(stage_early_terminate=early)
+        extra.update(stage_early_terminate=early)
     if page_size > 0:
         per = -(-TK // page_size)
         npages = B * per + 4
@@ -184,6 +188,47 @@ def make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, sec
         sink=sink, sw=sw, second_k=second_k, bsbq=bsbq, bf16=int(dtype == torch.bfloat16), block_size_k=block_size_k,
         **extra)
     print("wrote", path, "context", tuple(ctx.shape), "indices", tuple(md.indices.shape), flush=True)
+
+
+def sweep_case(seed):
+    """A random small configuration, drawn from ``seed``: batch, lengths, head counts, head dim, three scan stages
+    (block sizes, strides, chunk sizes, stage_k, stage stride), sink, window, second_stage_k, stage_early_terminate,
+    the attention block size, dense or paged keys and, sometimes, RoPE on load.  Prefixes stay long enough for every
+    stage to score more chunks than it keeps (with fewer, the reference's ``torch.topk`` chooses among never-scored
+    chunks of equal score, arbitrarily on the CPU), stage_early_terminate stays at or below the last chunk size (a
+    stage whose chunks are narrower is not scored at all, which leaves the same arbitrary choice), and a decode case
+    keeps a sink (the reference's decode launcher divides by its number of sink programs)."""
+    rng = np.random.default_rng(seed)
+    D = int(rng.choice([32, 64])); HKV = int(rng.choice([1, 2])); H = HKV * int(rng.choice([1, 2, 4]))
+    B = int(rng.choice([1, 2]))
+    decode = rng.random() < 0.4
+    TK = int(rng.choice([1536, 2048]))
+    TQ = 1 if decode else int(rng.choice([32, 48, 64, 100, 128]))
+    c0 = int(rng.choice([32, 64])); c1 = int(rng.choice([8, 16])); c2 = min(c1, int(rng.choice([1, 2, 4, 8])))
+    bq0 = int(rng.choice([32, 64])); bq2 = int(rng.choice([16, 32])) if bq0 == 32 else int(rng.choice([32, 64]))
+    bq1 = bq0 if rng.random() < 0.5 else bq2
+    sq0 = min(int(rng.choice([1, 2, 4])), bq0 // 16); sq1 = min(int(rng.choice([1, 2])), bq1 // 16)
+    sq2 = min(int(rng.choice([1, 2])), bq2 // 16)
+    k1 = int(rng.choice([4, 8])) * c0; k2 = int(rng.choice([8, 16, 32])) * c1
+    stages = [(bq0, sq0, c0, None, int(rng.choice([1, 1, 2]))), (bq1, sq1, c1, k1, 1), (bq2, sq2, c2, k2, 1)]
+    sink = int(rng.choice([4, 16, 32, 100] if decode else [0, 4, 16, 32, 100]))
+    sw = max(int(rng.choice([64, 128, 256])), 2 * c0)
+    second_k = min(int(rng.choice([16, 32, 64])) * c2, k2)
+    bsbq = int(rng.choice([16, 32, 64]))
+    if rng.random() < 0.7:
+        bsbq = min(bsbq, bq2)
+    lens = None
+    if decode or rng.random() < 0.4:
+        lens = [int(rng.integers(int(0.75 * TK), TK + 1)) for _ in range(B)]
+    extra = dict(lens=lens, page_size=int(rng.choice([0, 0, 1, 4, 16])), block_size_k=int(rng.choice([32, 64])),
+                 early=min(c2, int(rng.choice([1, 1, 2, 4]))), model_ctx=int(rng.choice([131072, 1024, 512])))
+    if rng.random() < 0.4:
+        extra["extend"] = (str(rng.choice(["relative", "streaming", "infllm", "dynamic_extend"])),
+                           str(rng.choice(["streaming", "infllm"])))
+    return (int(rng.integers(1 << 30)), B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, extra)
+
+
+SWEEP_SEEDS = (101, 102, 103, 104, 105, 106, 107, 108)  # committed witnesses of the random sweep
 
 
 def make_paged_api_case(name, seed, B, TQ, TK, H, HKV, D, lens, spec, layer_ids, orig_context_len, rope):
@@ -285,6 +330,8 @@ def main():
         # ``libdevice.tanh`` (logit_softcap) outside a compiled kernel, so bfloat16 inputs and soft-capped logits
         # have no vectors from the reference.
     }
+    for sd in SWEEP_SEEDS:
+        cases[f"f32_sweep_{sd}"] = sweep_case(sd)
     for name, (seed, B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, extra) in cases.items():
         if only and name not in only:
             continue

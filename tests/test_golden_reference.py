@@ -44,6 +44,8 @@ def load_case(path):
         kw["model_context_length"] = int(d["model_context_length"])
     if "softcap" in d.files:
         kw["logit_softcap"] = float(d["softcap"])
+    if "stage_early_terminate" in d.files:
+        kw["stage_early_terminate"] = int(d["stage_early_terminate"])
     return d, X, O.OArgs(**kw), dtype
 
 

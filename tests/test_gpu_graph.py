@@ -67,3 +67,41 @@ def test_decode_step_replays_from_a_graph(refresh):
         if refresh:
             assert torch.equal(meta_static.indices, meta_e.indices), f"replay {it}: indices differ"
             assert torch.equal(meta_static.ks, meta_e.ks)
+
+
+def test_graph_survives_many_other_shapes():
+    """A captured refresh step reads the cached stage-0 chunk list; calls with more than sixteen other shapes after
+    the capture must not free it (the list was handed out during the capture and is therefore kept for good)."""
+    from hip_attn import HiPAttentionArgs12, hip_attention_12
+
+    print("[case] graph replay after many other shapes", flush=True)
+    B, TK, H, HKV, D = 1, 4096, 8, 2, 128
+    X = make_inputs(91, B=B, TQ=1, TK=TK, H=H, HKV=HKV, D=D, dtype="bf16", pos=np.array([[TK - 1]]))
+    XP = to_paged(X, 16, seed=4, seq_lens=np.array([TK]))
+    kc, vc = to_torch(XP.k_cache, "bf16"), to_torch(XP.v_cache, "bf16")
+    bt = torch.from_numpy(XP.block_table).cuda()
+    sl = torch.from_numpy(XP.cache_seq_lens).cuda()
+    pos = torch.from_numpy(np.ascontiguousarray(XP.pos)).cuda()
+
+    def make_args(sink=256):
+        return HiPAttentionArgs12(sliding_window_size=512, second_stage_k=1024, sink_token_size=sink, k_cache=kc,
+                                  v_cache=vc, block_table=bt, cache_seq_lens=sl, position_ids=pos,
+                                  extend_context_length=TK, require_cache_statistics=False)
+
+    q_static = to_torch(X.q, "bf16")
+    hip_attention_12(q_static, None, None, make_args())  # warm-up: builds and keeps the chunk list
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_static, meta_static = hip_attention_12(q_static, None, None, make_args())
+    torch.cuda.synchronize()
+    eager, meta_e = hip_attention_12(q_static, None, None, make_args())
+    for sink in range(16, 16 + 16 * 24, 16):  # 24 other stage-0 lists
+        hip_attention_12(q_static, None, None, make_args(sink))
+    junk = [torch.full((n,), 0x7FFFFFF, dtype=torch.int32, device="cuda") for n in (4, 8, 16, 32, 64) for _ in range(8)]
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    del junk
+    assert torch.equal(meta_static.indices, meta_e.indices)
+    assert torch.equal(_bits(out_static), _bits(eager))

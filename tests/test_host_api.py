@@ -141,3 +141,63 @@ def test_metadata_cache_pool_round_trip_on_cpu():
         pool.get_buffer(1, "stage_1_indices_left", cfg.metadata_cache_max_batch_size + 1)
     with pytest.raises(KeyError):
         pool.get_buffer(1, "nope", 1)
+
+
+def test_operands_of_another_dtype_or_device_are_refused():
+    # the C side sizes every K / V row from q's dtype: a mismatch must never reach a kernel
+    import torch
+    from hip_attn import HiPAttentionArgs12
+    from hip_attn._native import HipAttnError
+    from hip_attn.operator import _check_operands, dual_stage_quadratic_hip_attention
+
+    q = torch.zeros((1, 4, 4, 64), dtype=torch.float32)
+    k = torch.zeros((1, 64, 1, 64), dtype=torch.float32)
+    _check_operands(q, k, k, HiPAttentionArgs12())
+    for bad in (k.to(torch.bfloat16), k.to(torch.float16), k.to(torch.float64)):
+        with pytest.raises(HipAttnError, match="dtype"):
+            _check_operands(q, bad, k, HiPAttentionArgs12())
+        with pytest.raises(HipAttnError, match="dtype"):
+            _check_operands(q, k, bad, HiPAttentionArgs12())
+    kc = torch.zeros((8, 16, 1, 64), dtype=torch.bfloat16)
+    with pytest.raises(HipAttnError, match="k_cache"):
+        _check_operands(q, None, None, HiPAttentionArgs12(k_cache=kc, v_cache=kc))
+    qb = q.to(torch.bfloat16)
+    _check_operands(qb, None, None, HiPAttentionArgs12(k_cache=kc, v_cache=kc))
+    _check_operands(qb, None, None, HiPAttentionArgs12(k_cache=kc.view(torch.uint8)[..., :64], v_cache=kc.view(torch.uint8)[..., :64]))
+    with pytest.raises(HipAttnError, match="k_cache"):  # fp8 bytes need bf16 queries
+        _check_operands(q, None, None, HiPAttentionArgs12(k_cache=kc.view(torch.uint8), v_cache=kc.view(torch.uint8)))
+    with pytest.raises(HipAttnError, match="q_mask"):
+        _check_operands(q, k, k, HiPAttentionArgs12(q_mask=qb))
+    meta = torch.zeros((1, 64, 1, 64), dtype=torch.float32, device="meta")
+    with pytest.raises(HipAttnError, match="device"):
+        _check_operands(q, meta, k, HiPAttentionArgs12())
+    with pytest.raises(HipAttnError, match="block_table"):
+        _check_operands(qb, None, None, HiPAttentionArgs12(
+            k_cache=kc, v_cache=kc, block_table=torch.zeros((1, 8), dtype=torch.int64, device="meta")))
+    with pytest.raises(HipAttnError, match="GPU only"):
+        dual_stage_quadratic_hip_attention(q, k, k, HiPAttentionArgs12())
+
+
+def test_helper_tensors_a_graph_has_seen_are_never_evicted(monkeypatch):
+    # a captured graph records addresses: what was handed out during a capture must outlive every eviction
+    import torch
+    from hip_attn import operator as op
+
+    cache, pinned, capturing = {}, {}, [False]
+    monkeypatch.setattr(op, "_capturing", lambda device: capturing[0])
+    dev = torch.device("cpu")
+    built = []
+
+    def get(key):
+        return op._cached_for_graphs(cache, pinned, key, lambda: built.append(key) or torch.full((1,), key), 4, dev)
+
+    a = get(0)                       # eager warm-up builds and keeps it
+    capturing[0] = True
+    assert get(0) is a and 0 in pinned and 0 not in cache   # the capture sees the kept tensor: pinned from now on
+    b = get(100)                     # built inside a capture: the graph's pool owns it, not kept
+    assert 100 not in cache and 100 not in pinned and get(100) is not b
+    capturing[0] = False
+    for key in range(1, 40):         # far more shapes than the limit
+        get(key)
+    assert len(cache) == 4 and get(0) is a and built.count(0) == 1
+    assert 1 not in cache and get(1) is not None and built.count(1) == 2   # unpinned entries are evicted oldest first
