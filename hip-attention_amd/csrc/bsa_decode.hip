@@ -7,6 +7,8 @@
 // states of a workgroup are merged through LDS before the partial is written.
 #include <stdlib.h>
 
+#include <atomic>
+
 #include "bsa.hpp"
 
 namespace hipattn {
@@ -412,4 +414,58 @@ extern "C" int hipattn_bsa_decode_merge(const void *workspace, int32_t B, int32_
 #undef MERGE_CASE
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Decode attention for callers that cannot allocate: the split partials live in a device array that is
+// part of the library's code object instead of a caller-allocated workspace.  Every GPU the library runs
+// on holds its own copy of the array at its own address for the life of the process.
+namespace hipattn {
+
+constexpr size_t DECODE_SCRATCH_BYTES = HIPATTN_DECODE_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[DECODE_SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+static std::atomic<void *> g_scratch_ptr[MAX_DEVICES];
+
+// Device address of `scratch` on the current device, looked up once per device.  The array's name is only a
+// host-side handle: kernels and stream operations must be given this address, never the name.
+static int decode_scratch(void **out) {
+    int dev = -1;
+    HIPATTN_CHECK_HIP(hipGetDevice(&dev));
+    HIPATTN_CHECK_ARG(dev >= 0 && dev < MAX_DEVICES, HIPATTN_E_UNSUPPORTED, "decode (static scratch): device %d", dev);
+    void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        HIPATTN_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        HIPATTN_CHECK_ARG(ptr != nullptr, HIPATTN_E_UNSUPPORTED, "decode (static scratch): no device address");
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // every thread that looks it up gets the same address
+    }
+    *out = ptr;
+    return 0;
+}
+
+}  // namespace hipattn
+
+extern "C" int hipattn_bsa_decode_static(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t *indices,
+                                         const int32_t *ks_start_end, int32_t idx_rows, int32_t BK,
+                                         int32_t block_size_k, int32_t sliding_window, int32_t sink,
+                                         int32_t second_stage_k, int32_t nsplits, void *out, int64_t out_stride_b,
+                                         int64_t out_stride_h, void *stream) {
+    HIPATTN_CHECK_ARG(q && kv && out, HIPATTN_E_ARG, "decode (static scratch): null pointer");
+    HIPATTN_CHECK_ARG(q->B > 0 && q->HEAD > 0 && q->HID > 0, HIPATTN_E_ARG, "decode (static scratch): non-positive size");
+    if (nsplits <= 0) nsplits = hipattn_bsa_decode_default_splits(q->B, kv->HKV, BK * block_size_k + sink + sliding_window + 1);
+    const int64_t need = hipattn_bsa_decode_workspace_bytes(q->B, q->HEAD, q->HID, nsplits);
+    HIPATTN_CHECK_ARG(need > 0 && (uint64_t)need <= DECODE_SCRATCH_BYTES, HIPATTN_E_UNSUPPORTED,
+                      "decode (static scratch): B %d x HEAD %d x nsplits %d x (HID %d + 4) floats = %lld bytes of partials "
+                      "exceed the %lld-byte scratch array; use hipattn_bsa_decode_partial with a workspace",
+                      q->B, q->HEAD, nsplits, q->HID, (long long)need, (long long)DECODE_SCRATCH_BYTES);
+    void *ws = nullptr;
+    int rc = decode_scratch(&ws);
+    if (rc) return rc;
+    // every (sequence, head, split) row of the partials is written by the first launch before the second reads it,
+    // so nothing left over from the call before can be seen and nothing needs clearing
+    rc = hipattn_bsa_decode_partial(q, kv, indices, ks_start_end, idx_rows, BK, block_size_k, sliding_window, sink,
+                                    second_stage_k, nsplits, ws, stream);
+    if (rc) return rc;
+    return hipattn_bsa_decode_merge(ws, q->B, q->HEAD, q->HID, nsplits, q->dtype, out, out_stride_b, out_stride_h, stream);
 }

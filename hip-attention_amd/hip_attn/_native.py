@@ -110,6 +110,7 @@ def lib():
         L.hipattn_bsa_decode_default_splits.restype = ctypes.c_int32
         for name in ("hipattn_mask_stage", "hipattn_prescale_k", "hipattn_select_stage", "hipattn_finalize_indices",
                      "hipattn_bsa_prefill", "hipattn_bsa_decode_partial", "hipattn_bsa_decode_merge",
+                     "hipattn_bsa_decode_static",
                      "hipattn_cache_sizes", "hipattn_cache_create", "hipattn_cache_flush",
                      "hipattn_cache_lookup_and_schedule", "hipattn_cache_commit", "hipattn_cache_write_rows",
                      "hipattn_cache_stats", "hipattn_pool_write_rows", "hipattn_host_device_pointer",
@@ -393,6 +394,20 @@ def bsa_decode(qs, kvs, indices, ks_start_end, BK, bk, sw, sink, out, device, ns
         stream_ptr(device))
     check(rc, "hipattn_bsa_decode_merge")
     return workspace
+
+
+def bsa_decode_static(qs, kvs, indices, ks_start_end, BK, bk, sw, sink, out, device, nsplits=0, second_stage_k=0):
+    """Decode attention through ``hipattn_bsa_decode_static``: the split partials live in a device array inside the
+    library, so the call allocates nothing (for callers that cannot: graph capture, tight serving loops)."""
+    assert indices.dtype == torch.int64 and indices.is_contiguous()
+    assert ks_start_end.dtype == torch.int32 and ks_start_end.is_contiguous()
+    with _timed("bsa_decode"):
+      rc = lib().hipattn_bsa_decode_static(
+        ctypes.byref(qs), ctypes.byref(kvs), _p(indices), _p(ks_start_end), ctypes.c_int32(indices.shape[1]),
+        ctypes.c_int32(BK), ctypes.c_int32(bk), ctypes.c_int32(sw), ctypes.c_int32(sink),
+        ctypes.c_int32(second_stage_k), ctypes.c_int32(nsplits), _p(out), ctypes.c_int64(out.stride(0)),
+        ctypes.c_int64(out.stride(2)), stream_ptr(device))
+    check(rc, "hipattn_bsa_decode_static")
 
 
 # ------------------------------------------------------------------ offload cache

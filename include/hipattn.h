@@ -243,6 +243,23 @@ int hipattn_bsa_decode_merge(const void *workspace, int32_t B, int32_t HEAD, int
                              int32_t nsplits, int32_t dtype, void *out, int64_t out_stride_b,
                              int64_t out_stride_h, void *stream);
 
+/* Decode attention that allocates nothing and needs no workspace: hipattn_bsa_decode_partial followed by
+ * hipattn_bsa_decode_merge with the split partials kept in a device array inside the library.  It has no
+ * counterpart in the reference; it is for callers that cannot allocate device memory around the call: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Arguments as for the two calls it
+ * combines; nsplits <= 0 picks hipattn_bsa_decode_default_splits.
+ *   Limit: B * HEAD * nsplits * (HID + 4) * 4 bytes of partials must fit HIPATTN_DECODE_SCRATCH_BYTES, otherwise
+ *   HIPATTN_E_UNSUPPORTED (the batched 16-sequence decode with 32 heads, head dim 128 and 9 splits needs 2.4 MB, one
+ *   sequence with 64 splits 1.1 MB).  Each GPU the library runs on holds the array until the process ends.
+ *   The first call on a device looks the array's address up (make it outside a graph capture).  All calls on one
+ *   GPU share the array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream, or
+ *   ordered by events, do not.  No hipMalloc, hipFree or allocating library call is made. */
+#define HIPATTN_DECODE_SCRATCH_BYTES (4 * 1024 * 1024)
+int hipattn_bsa_decode_static(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t *indices,
+                              const int32_t *ks_start_end, int32_t idx_rows, int32_t BK, int32_t block_size_k,
+                              int32_t sliding_window, int32_t sink, int32_t second_stage_k, int32_t nsplits,
+                              void *out, int64_t out_stride_b, int64_t out_stride_h, void *stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Offload cache: K (and V) of a layer live in pinned host memory as a pool [pool_rows, HKV, HID]
  * addressed through the paged view (row = page * page_size + offset); a block cache in device
