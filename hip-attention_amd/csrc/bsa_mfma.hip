@@ -57,7 +57,9 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
     extern __shared__ __align__(16) unsigned char smem_raw[];
     MfmaSmem<HID> &sm = *reinterpret_cast<MfmaSmem<HID> *>(smem_raw);
 
-    const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+    // wave-uniform quantities are marked as such (readfirstlane), so that the tile loop and its branches run on the
+    // scalar unit instead of under execution masks
+    const int tid = threadIdx.x, lane = tid & 63, wid = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, hh = lane >> 5;
     const int whead = wid >> 1, half = wid & 1;
 
@@ -94,8 +96,8 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
             long long w2 = __shfl_xor(mn, o);
             mn = w2 < mn ? w2 : mn;
         }
-        pmax_blk = (int)cur;
-        pmin_blk = (int)mn;
+        pmax_blk = __builtin_amdgcn_readfirstlane((int)cur);
+        pmin_blk = __builtin_amdgcn_readfirstlane((int)mn);
     }
     const int myj = half * 32 + col;                       // this lane's query row inside the block
     const long long myit = (long long)qb * p.bq + myj;
@@ -300,8 +302,8 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
         const bool window = tile >= tiles_sel + tiles_sink;
 
         // tile summary (token range, all valid?) posted by wave 0
-        const int tmin = mt.tmin, tmax = mt.tmax;
-        const bool all_valid = mt.all_valid != 0;
+        const int tmin = __builtin_amdgcn_readfirstlane(mt.tmin), tmax = __builtin_amdgcn_readfirstlane(mt.tmax);
+        const bool all_valid = __builtin_amdgcn_readfirstlane(mt.all_valid) != 0;
         bool full;  // every (valid row, token) pair of the tile is attended
         if (!window) full = all_valid && ((long long)tmax + p.sw <= pmin_blk);
         else full = all_valid && (tmax <= pmin_blk) && ((long long)pmax_blk < (long long)tmin + p.sw);
