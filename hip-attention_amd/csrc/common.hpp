@@ -447,6 +447,27 @@ __device__ __forceinline__ uint32_t swap_halves(uint32_t x) {
 }
 __device__ __forceinline__ float swap_halves(float x) { return __uint_as_float(swap_halves(__float_as_uint(x))); }
 
+// ---------------------------------------------------------------- direct global -> LDS loads
+// 16 bytes per lane from global memory straight into LDS (global_load_lds_dwordx4): lane i's piece lands at
+// lds_base + 16 * i, lds_base being wave-uniform; each lane supplies its own global address.  No registers and no
+// LDS stores are spent on staging.  Written as an asm statement: the compiler would order every later LDS read,
+// also of other buffers, behind a full wait on the vector-memory counter.  A kernel that uses it waits itself
+// (wait_vmcnt, then the workgroup barrier) before anything reads the buffer the loads fill.  A load cannot be
+// predicated into writing zeros: rows that do not exist are fetched from a row of zeros in device memory.
+__device__ __forceinline__ void load_to_lds16(const void *gsrc, void *lds_base) {
+    const uint32_t base = (uint32_t)(uintptr_t)lds_base;  // LDS addresses are the low 32 bits of the flat pointer
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(gsrc), "s"(__builtin_amdgcn_readfirstlane(base))
+                 : "memory", "m0");
+}
+// wait until at most N vector-memory operations of this wave are outstanding (they complete in order)
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));  // expcnt and lgkmcnt left at their maxima
+}
+
 // XCD-aware remap: consecutive workgroup ids are dealt round-robin to the 8 XCDs (each with its
 // own L2), so give every XCD one contiguous range of logical work ids.
 __device__ __forceinline__ long long xcd_remap(long long bid, long long total) {

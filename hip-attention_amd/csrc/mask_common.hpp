@@ -50,6 +50,11 @@ __device__ __forceinline__ void store_score(const MaskParamsBase &p, int64_t row
     else atomicMin(reinterpret_cast<unsigned int *>(a), __float_as_uint(v));
 }
 
+// bf16, prescaled keys, chunks of 2 .. 16 tokens on wide launches: every token of every chunk is scored once per
+// GQA group and the searches are replayed on the scores (mask_stage_dense.hip).  Expects p.qhat filled.  Returns
+// HIPATTN_E_UNSUPPORTED (no error text) when the launch is not one it covers.
+int mask_stage_dense_launch(const MaskParams &p, int HID, int rows_eff, hipStream_t st);
+
 // bf16 path on the matrix cores (mask_stage_mfma.hip)
 int mask_stage_mfma_launch(const MaskParams &p, int HID, int rows_eff, int prescaled, hipStream_t st);
 

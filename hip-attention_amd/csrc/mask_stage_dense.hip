@@ -1,0 +1,322 @@
+// Mask-estimation scan stage for small chunks on wide launches: score every token once, replay the searches.
+//
+// A binary search over a chunk of 2^k tokens samples 2 (k + 1) - 3 distinct tokens; the four heads of a GQA group
+// search the same chunks of the same keys and part ways after the first rounds, so together they load about
+// 4 * (2 (k + 1) - 3) key rows per chunk through the gather path, two cache lines per row and one row per lane.
+// For chunks of 8 tokens that is 20 rows where the chunk holds 8.  The score of a token,
+//     s[t] = bf16(max over the block's query rows of q^ . k^[t]),
+// depends on nothing but the token, so this kernel loads every token of every chunk once per (query block, kv head)
+// into LDS, fully coalesced and straight from global memory, lets each head of the group score all of them on the
+// matrix cores, and then walks the reference's search (attention_extend.py:736-745, 1183-1215) on the scores held
+// in registers: the samples, comparisons, winners, chunk score and refined left edge are those of the sampling
+// kernel, bit for bit, because every score is produced by the same chain of matrix instructions in the same order
+// (mask_stage_mfma.hip).  Access flags are set for the tokens the search samples, not for the tokens loaded.
+//
+// Workgroup = (batch, kv head, scan row) x up to four heads of the group, one wave per head; the wave keeps its Q^
+// fragments (A operand) in registers and consumes tiles of 64 tokens (B operand) from LDS.
+#include <stdlib.h>
+
+#include "mask_common.hpp"
+
+namespace hipattn {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 md_bf16x8;
+typedef __attribute__((ext_vector_type(16))) float md_f32x16;
+
+union MdFrag {
+    md_bf16x8 v;
+    uint4 q;
+};
+
+constexpr int MD_TN = 64;              // tokens per tile
+constexpr int MD_DIST = 2;             // tiles whose loads are issued ahead of the tile being consumed
+constexpr int MD_NBUF = MD_DIST + 1;   // the buffer refilled at tile t is the one tile t - 1 was read from
+constexpr int MD_MAX_CHUNKS = 2048;    // chunk list kept in LDS
+constexpr int MD_PASS = 8;             // tiles between two replays of the searches
+
+static __device__ __align__(16) uint16_t md_zero_row[256];
+
+// HPW = waves (heads) per workgroup; MB = 32-row blocks of query rows per program (1: up to 32 rows, 2: up to 64)
+template <int HID, int MB, int HPW, bool EXT>
+__global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFor<EXT> p, long long total_wg) {
+    constexpr int NT = 64 * HPW;
+    constexpr int KS = HID / 16;
+    constexpr int PPR = HID / 8;               // 16-byte pieces per key row
+    constexpr int CPT = MD_TN * PPR / NT;      // pieces a thread moves per tile = its load instructions per tile
+    static_assert((MD_DIST - 1) * CPT < 64, "in-flight loads must fit the counter");
+    const KVExt *kx = nullptr;
+    if constexpr (EXT) kx = &p.kx;
+    // rows of exactly HID elements, the 16-byte pieces of row r permuted by r (piece q sits at q ^ (r % PPR)): the
+    // lanes of a fragment read (consecutive rows, same piece) then hit different bank groups
+    __shared__ __align__(16) uint16_t s_rows[MD_NBUF][MD_TN][HID];
+    // The chunk list of this (batch, scan row), read from global memory once: a vector-memory load inside the tile
+    // loop would make the compiler wait for everything in flight, the tile loads included, before it uses the value.
+    __shared__ int s_left[MD_MAX_CHUNKS];
+    __shared__ float s_gwidth[MD_MAX_CHUNKS / 16];       // per group of block_chunk chunks: widest chunk, 0 = not searched
+    __shared__ float s_score[HPW][MD_PASS * MD_TN];      // per head: scores of the tokens of the last MD_PASS tiles
+
+    const int tid = threadIdx.x, lane = tid & 63, wid = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 31, hh = lane >> 5;
+
+    long long L = xcd_remap((long long)blockIdx.x, total_wg);
+    const int hblocks = (p.G + HPW - 1) / HPW;
+    const int hin = (int)(L % hblocks) * HPW + wid;
+    L /= hblocks;
+    const int s = (int)(L % p.BS);
+    L /= p.BS;
+    const int kvh = (int)(L % p.kv.HKV);
+    const int b = (int)(L / p.kv.HKV);
+    const bool head_ok = hin < p.G;
+    const int h = kvh * p.G + (head_ok ? hin : 0);
+
+    const int BC = p.block_chunk;
+    const int CH = p.chunk;                       // power of two, 2 .. 16
+    const int ch_shift = __builtin_ctz(CH);
+    const int64_t row_in = ((int64_t)b * p.BS + s) * p.n;  // one chunk list for all heads (hg == 1)
+    const int64_t row_out = (((int64_t)b * p.BS + s) * p.HEAD + h) * p.n;
+    const int64_t red_out = ((int64_t)b * p.BS + s) * p.n;
+
+    // ---- rows of this program (as in the sampling kernel)
+    const long long qb = (long long)(p.BDST - 1) - (long long)(p.BS - 1) * p.scan_stride + (long long)s * p.scan_stride;
+    const long long myrow = qb * p.BQ + (long long)lane * p.stride_q;
+    const bool rv = (lane < p.nrows) && (myrow >= 0) && (myrow < p.TDST);
+    const unsigned long long rowmask = __ballot(rv);
+    const long long mypos = rv ? p.pos[(int64_t)b * p.pos_sb + myrow * p.pos_st] : 0x7fffffffffffffffLL;
+    const long long pmin = wave_min_ll(mypos);
+    unsigned vm[MB];  // which accumulator elements belong to valid rows: element (mb, i) <-> row mb*32 + (i/4)*8 + hh*4 + i%4
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+        vm[mb] = 0;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int j = mb * 32 + (i >> 2) * 8 + hh * 4 + (i & 3);
+            if ((j < p.nrows) && ((rowmask >> j) & 1ull)) vm[mb] |= 1u << i;
+        }
+    }
+    const int fast_rows = (p.nrows == 16 && rowmask == 0xffffull) ? 16
+                        : (p.nrows == 32 && rowmask == 0xffffffffull) ? 32
+                        : (MB == 2 && p.nrows == 64 && rowmask == ~0ull) ? 64 : 0;
+    const bool any_rows = (rowmask != 0ull) && (pmin >= 0);
+    int lim = 0;
+    if (any_rows) {
+        const long long lm = pmin - p.sw_eff;
+        lim = (int)(lm < 0 ? 0 : lm);
+    }
+    const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
+    for (int i = tid; i < p.n; i += NT) s_left[i] = p.chunk_left[row_in + i];
+
+    // ---- Q^ fragments, in the order qhat_kernel stores them (k-step, row half, row)
+    MdFrag qf[MB][KS];
+    {
+        const uint16_t *qh = p.qhat + ((((int64_t)b * p.BS + s) * p.HEAD + h) * p.nrows) * HID;
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) {
+            const int j = mb * 32 + n;
+            const bool jv = head_ok && (j < p.nrows) && ((rowmask >> j) & 1ull);
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                qf[mb][ks].q = make_uint4(0, 0, 0, 0);
+                if (jv) qf[mb][ks].q = *reinterpret_cast<const uint4 *>(qh + ((int64_t)(ks * 2 + hh) * p.nrows + j) * 8);
+            }
+        }
+    }
+
+    // ---- tiles: tile x holds the tokens of chunks x * (64 / CH) ... in list order, CH consecutive slots per chunk
+    const int cpt_shift = 6 - ch_shift;  // log2(chunks per tile)
+    const int ntiles = (p.n + (1 << cpt_shift) - 1) >> cpt_shift;
+    // piece slot c = tid + NT * j of a tile is position c % PPR of token slot c / PPR; one load instruction of a wave
+    // fills 64 consecutive piece slots
+    auto prefetch = [&](int tile) {
+        const int buf = tile % MD_NBUF;
+#pragma unroll
+        for (int j = 0; j < CPT; j++) {
+            const int c = tid + NT * j;
+            const int slot = c / PPR, pos = c % PPR;
+            const int ci = (tile << cpt_shift) + (slot >> ch_shift);
+            const uint16_t *src = md_zero_row;
+            if (ci < p.n) {
+                const int cl = s_left[ci];
+                const int64_t rr = (int64_t)cl + CH;
+                const int cr = (int)(rr < p.right_clamp ? rr : p.right_clamp);
+                const int t = cl + (slot & (CH - 1));
+                // a chunk that starts beyond the block's reach is never searched (its left edge only moves right)
+                if (t < cr && cl <= lim && cl >= 0 && any_rows) {
+                    // dense keys only (the launcher sees to it): the row address is plain arithmetic; rows at or
+                    // beyond the end of the tensor read as zeros
+                    if (t < p.kv.tsrc)
+                        src = reinterpret_cast<const uint16_t *>(p.kv.k) + (int64_t)b * p.kv.k_stride_b +
+                              (int64_t)t * p.kv.k_stride_t + (int64_t)kvh * p.kv.k_stride_h + ((pos ^ slot) & (PPR - 1)) * 8;
+                }
+            }
+            load_to_lds16(src, &s_rows[buf][0][0] + (wid * 64 + NT * j) * 8);
+        }
+    };
+    __syncthreads();  // s_left visible (the loads above are complete: their values were stored)
+    for (int x = 0; x < MD_DIST && x < ntiles; x++) prefetch(x);
+
+    // ---- program-level gate and iteration count of the reference, per group of block_chunk chunks, once
+    for (int g = tid; g < p.ngroups; g += NT) {
+        int glmin = 0x7fffffff, wmax = -0x7fffffff;
+        for (int i = 0; i < BC; i++) {
+            const int ci = g * BC + i;
+            int gl = (int)p.kv.max_tsrc, gr = (int)p.kv.max_tsrc;  // padding entries of a short last group
+            if (ci < p.n) {
+                gl = s_left[ci];
+                const int64_t rr = (int64_t)gl + CH;
+                gr = (int)(rr < p.right_clamp ? rr : p.right_clamp);
+            }
+            glmin = gl < glmin ? gl : glmin;
+            wmax = (gr - gl) > wmax ? (gr - gl) : wmax;
+        }
+        const bool run = any_rows && (pmin + (long long)p.BQ * p.scan_stride >= (long long)glmin);
+        s_gwidth[g] = (run && (float)wmax >= p.terminate) ? (float)wmax : 0.0f;  // 0: the group is not searched
+    }
+    __syncthreads();
+
+    // The searches are replayed once per PASS tiles, one lane per chunk, on the scores the tiles left in LDS: replaying
+    // them tile by tile would keep 64 lanes busy with the four or eight chunks of a block.
+    float *my_scores = &s_score[wid][0];
+    auto replay = [&](int first_tile, int last_tile) {  // chunks of tiles [first_tile, last_tile]
+        const int c_begin = first_tile << cpt_shift;
+        int c_end = (last_tile + 1) << cpt_shift;
+        c_end = c_end < p.n ? c_end : p.n;
+        for (int cidx = c_begin + lane; cidx < c_end; cidx += 64) {
+            int cl = s_left[cidx];
+            const int64_t rr = (int64_t)cl + CH;
+            int cr = (int)(rr < p.right_clamp ? rr : p.right_clamp);
+            const int cl0 = cl;
+            float score = -32000.0f;
+            float width = s_gwidth[cidx / BC];
+            const float *sc = my_scores + ((cidx - c_begin) << ch_shift);  // s[cl0 + e] at sc[e]
+            unsigned touched = 0;  // bit e: the search sampled token cl0 + e
+            while (width >= p.terminate) {
+                width *= 0.5f;
+                const bool active = (cl < cr) && (cl <= lim) && (cl >= 0);
+                if (active) {
+                    const int ctr = (cl + cr) >> 1;
+                    const int eL = ((cl + ctr) >> 1) - cl0, eR = ((ctr + cr) >> 1) - cl0;
+                    const float sL = sc[eL], sR = sc[eR];
+                    touched |= (1u << eL) | (1u << eR);
+                    const bool win = sL > sR;
+                    if (win) cr = ctr; else cl = ctr;
+                    score = fmaxf(score, win ? sL : sR);
+                }
+            }
+            if constexpr (EXT) {
+                // access flags for the rows the sampling kernel would have loaded, stored without looking first
+                for (int e = 0; e < CH; e++)
+                    if ((touched >> e) & 1u) kv_k_row<true, false>(p.kv, kx, b, cl0 + e, kvh, seqlen, true);
+            }
+            store_score(p, row_out, red_out, cidx, score);
+            if (p.left_out) p.left_out[row_out + cidx] = cl;
+        }
+    };
+
+    for (int tile = 0; tile < ntiles; tile++) {
+        const int buf = tile % MD_NBUF;
+        // this wave's loads of the tile have landed (those of later tiles may still be in flight); after the barrier
+        // everyone's have, and everyone is done with the buffer of the tile before, which the next loads overwrite
+        const int newer = ntiles - 1 - tile;
+        if (newer >= MD_DIST - 1) wait_vmcnt<(MD_DIST - 1) * CPT>();
+        else if (newer == 1 && MD_DIST > 2) wait_vmcnt<CPT>();
+        else wait_vmcnt<0>();
+        __syncthreads();
+        if (tile + MD_DIST < ntiles) prefetch(tile + MD_DIST);
+        if (!head_ok) continue;
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++) {
+            const int c0 = ((tile * 2 + nb) * 32) >> ch_shift;  // first chunk of this block of 32 tokens
+            // a block of 32 tokens lies inside one group (block_chunk * CH is a multiple of 32)
+            const bool searched = c0 < p.n && __builtin_amdgcn_readfirstlane(__float_as_int(s_gwidth[c0 / BC])) != 0;
+            if (!searched) continue;
+            // ---- s[token] for the 32 tokens of the block
+            md_f32x16 acc[MB];
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) acc[mb][i] = 0.0f;
+            const int r = nb * 32 + n;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                MdFrag kf;
+                kf.q = *reinterpret_cast<const uint4 *>(&s_rows[buf][r][(((hh * (PPR / 2) + ks) ^ r) & (PPR - 1)) * 8]);
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++)
+                    acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qf[mb][ks].v, kf.v, acc[mb], 0, 0, 0);
+            }
+            float v = -INFINITY;
+            if (fast_rows == 16) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) v = fmaxf(v, acc[0][i]);
+            } else if (fast_rows == 32) {
+#pragma unroll
+                for (int i = 0; i < 16; i++) v = fmaxf(v, acc[0][i]);
+            } else if (fast_rows == 64) {
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) v = fmaxf(v, acc[mb][i]);
+            } else {
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) v = fmaxf(v, ((vm[mb] >> i) & 1u) ? acc[mb][i] : -INFINITY);
+            }
+            v = fmaxf(v, swap_halves(v));
+            if (hh == 0) my_scores[(tile % MD_PASS) * MD_TN + r] = round_bf16(v);
+        }
+        if ((tile % MD_PASS) == MD_PASS - 1 || tile == ntiles - 1) replay(tile - (tile % MD_PASS), tile);  // the wave's own LDS writes
+    }
+}
+
+template <int HID, int MB, int HPW>
+static int launch_dense(const MaskParams &p, hipStream_t st) {
+    const int hblocks = (p.G + HPW - 1) / HPW;
+    const long long total = (long long)p.B * p.kv.HKV * p.BS * hblocks;
+    if (total >= 0x7fffffffLL) return HIPATTN_E_UNSUPPORTED;
+    dim3 grid((unsigned)total), block(64 * HPW);
+    if (p.kx.extended()) {
+        hipLaunchKernelGGL((mask_stage_dense_kernel<HID, MB, HPW, true>), grid, block, 0, st, p, total);
+    } else {
+        const MaskParamsBase &pb = p;
+        hipLaunchKernelGGL((mask_stage_dense_kernel<HID, MB, HPW, false>), grid, block, 0, st, pb, total);
+    }
+    HIPATTN_CHECK_HIP(hipGetLastError());
+    return 0;
+}
+
+template <int HID>
+static int launch_dense_hid(const MaskParams &p, int rows_eff, hipStream_t st) {
+    const bool two = rows_eff > 32;
+    if (p.G >= 4) return two ? launch_dense<HID, 2, 4>(p, st) : launch_dense<HID, 1, 4>(p, st);
+    if (p.G >= 2) return two ? launch_dense<HID, 2, 2>(p, st) : launch_dense<HID, 1, 2>(p, st);
+    return HIPATTN_E_UNSUPPORTED;  // one head per group: nothing to share, the sampling kernel reads fewer rows
+}
+
+int mask_stage_dense_launch(const MaskParams &p, int HID, int rows_eff, hipStream_t st) {
+    // HIPATTN_MASK_DENSE: 0 = never, 1 = where it pays (default), 2 = wherever the kernel applies (testing)
+    const char *e = getenv("HIPATTN_MASK_DENSE");  // read on every call: tests switch it inside one process
+    const int mode = e ? atoi(e) : 1;
+    if (mode == 0) return HIPATTN_E_UNSUPPORTED;
+    const int CH = p.chunk;
+    if (CH < 2 || CH > 16 || (CH & (CH - 1)) != 0) return HIPATTN_E_UNSUPPORTED;
+    if (p.hg != 1 || p.rope.cos || p.kx.cached || p.kx.kv8) return HIPATTN_E_UNSUPPORTED;
+    if (p.nrows > 64 || p.n > MD_MAX_CHUNKS) return HIPATTN_E_UNSUPPORTED;
+    // paged keys need a page lookup per token, a vector-memory load the tile loop cannot afford (see s_left)
+    if (p.kv.paged) return HIPATTN_E_UNSUPPORTED;
+    if (mode == 1) {
+        // pays when the group's searches together load more rows than the chunks hold, on launches wide enough to
+        // keep the chip busy with one workgroup per (batch, kv head, scan row)
+        const int iters = 32 - __builtin_clz((unsigned)CH);  // floor(log2(CH)) + 1
+        const int per_search = 2 * iters - 3;
+        const long long wgs = (long long)p.B * p.kv.HKV * p.BS;
+        if (!(per_search * p.G >= 2 * CH) || wgs < 1024 || p.n < 64) return HIPATTN_E_UNSUPPORTED;
+    }
+    switch (HID) {
+        case 64: return launch_dense_hid<64>(p, rows_eff, st);
+        case 128: return launch_dense_hid<128>(p, rows_eff, st);
+    }
+    return HIPATTN_E_UNSUPPORTED;
+}
+
+}  // namespace hipattn

@@ -536,6 +536,11 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
         const long long blocks = (work + 255) / 256;
         hipLaunchKernelGGL(qhat_kernel, dim3((unsigned)blocks), dim3(256), 0, st, p, HID, const_cast<uint16_t *>(p.qhat));
     }
+    if (prescaled && !two_sided) {
+        // small chunks on wide launches: every token scored once per GQA group, searches replayed on the scores
+        const int rc = mask_stage_dense_launch(p, HID, rows_eff, st);
+        if (rc != HIPATTN_E_UNSUPPORTED) return rc;
+    }
     dim3 grid((unsigned)p.total), block(64 * hpw);
     const MaskParamsBase &pb = p;  // the plain kernels take the block without the extras
 #define MS_LAUNCH(MBv, NBv, PSv, VLv)                                                                                 \

@@ -241,3 +241,45 @@ def test_head_dim_256_with_softcap_like_gemma2():
     ctx, meta = run_product(X, A)
     assert_metadata_equal(meta, ometa)
     assert_context_close(ctx, octx, "bf16")
+
+
+DENSE_CASES = {
+    # name: (B, TQ, TK, H, HKV, D, stages, kwargs)
+    "chunks 64/16/2, 16 and 32 rows, G=4": (1, 200, 4096, 8, 2, 64,
+                                            [O.OStage(32, 2, 64, None, 1), O.OStage(32, 2, 16, 2048, 1), O.OStage(32, 1, 2, 1024, 1)], {}),
+    "chunks 256/32/8, 64 rows, D=128, G=4": (1, 300, 12288, 8, 2, 128,
+                                             [O.OStage(64, 4, 256, None, 1), O.OStage(64, 4, 32, 8192, 1), O.OStage(64, 1, 8, 2048, 1)],
+                                             dict(sliding_window_size=512, sink_token_size=64, second_stage_k=1024)),
+    "chunks 64/8/4, G=2, early terminate 2": (2, 100, 3000, 4, 2, 64,
+                                              [O.OStage(32, 1, 64, None, 1), O.OStage(32, 1, 8, 1024, 1), O.OStage(32, 1, 4, 512, 1)],
+                                              dict(stage_early_terminate=2, second_stage_k=256)),
+    "chunks 128/16/4 with 16 chunks per program": (1, 64, 2500, 4, 1, 128,
+                                                   [O.OStage(64, 1, 128, None, 1), O.OStage(64, 2, 16, 1024, 1), O.OStage(32, 1, 4, 256, 1)],
+                                                   dict(block_size_k=16, second_stage_k=128, sliding_window_size=256)),
+}
+
+
+@pytest.mark.parametrize("paged", [False, True])
+@pytest.mark.parametrize("case", list(DENSE_CASES))
+def test_small_chunk_stages_scored_densely(case, paged, monkeypatch):
+    """Stages with chunks of 2 .. 16 tokens on prescaled keys can score every token of every chunk once per GQA group
+    and replay the searches on the scores; forced here on small problems (the operator picks that kernel by itself
+    only on wide launches).  Indices, ks and the access flags must equal the oracle's, which samples."""
+    _case(f"dense scan: {case}, paged={paged}")
+    monkeypatch.setenv("HIPATTN_MASK_DENSE", "2")
+    monkeypatch.setenv("HIP_ATTN_PRESCALE_K", "1")
+    B, TQ, TK, H, HKV, D, stages, kw = DENSE_CASES[case]
+    X = make_inputs(500 + list(DENSE_CASES).index(case), B=B, TQ=TQ, TK=TK, H=H, HKV=HKV, D=D, dtype="bf16")
+    A = tiny_args(stages=stages, **kw)
+    if paged:
+        X = to_paged(X, 16, seed=7)
+        A.extend_context_length = TK
+    octx, ometa = O.hip_attention_12(X, A)
+    ctx, meta = run_product(X, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, "bf16")
+    # and the sampling kernels on the same input, for the access flags of a run that cannot be compared directly
+    monkeypatch.setenv("HIPATTN_MASK_DENSE", "0")
+    ctx2, meta2 = run_product(X, A)
+    assert torch.equal(meta2.indices, meta.indices)
+    assert torch.equal(meta2.mask_cache_statistics.access_counter, meta.mask_cache_statistics.access_counter)
