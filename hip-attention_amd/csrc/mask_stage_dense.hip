@@ -223,47 +223,63 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
         __syncthreads();
         if (tile + MD_DIST < ntiles) prefetch(tile + MD_DIST);
         if (!head_ok) continue;
+        // a block of 32 tokens lies inside one group (block_chunk * CH is a multiple of 32)
+        bool searched[2];
 #pragma unroll
         for (int nb = 0; nb < 2; nb++) {
             const int c0 = ((tile * 2 + nb) * 32) >> ch_shift;  // first chunk of this block of 32 tokens
-            // a block of 32 tokens lies inside one group (block_chunk * CH is a multiple of 32)
-            const bool searched = c0 < p.n && __builtin_amdgcn_readfirstlane(__float_as_int(s_gwidth[c0 / BC])) != 0;
-            if (!searched) continue;
-            // ---- s[token] for the 32 tokens of the block
-            md_f32x16 acc[MB];
+            searched[nb] = c0 < p.n && __builtin_amdgcn_readfirstlane(__float_as_int(s_gwidth[c0 / BC])) != 0;
+        }
+        if (!searched[0] && !searched[1]) continue;
+        // ---- s[token] for the 64 tokens of the tile: all K^ fragments of the tile are fetched from LDS first, then
+        // the four accumulation chains (two token blocks x two row blocks) keep the matrix unit fed back to back
+        MdFrag kf[2][KS];
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++) {
+            const int r = nb * 32 + n;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++)
+                kf[nb][ks].q = *reinterpret_cast<const uint4 *>(&s_rows[buf][r][(((hh * (PPR / 2) + ks) ^ r) & (PPR - 1)) * 8]);
+        }
+        // the compiler's scheduler would otherwise sink every fragment read to just before its first use and wait
+        // for it there, one LDS round trip per k-step
+        __builtin_amdgcn_sched_barrier(0);
+        md_f32x16 acc[2][MB];
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++)
 #pragma unroll
             for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-                for (int i = 0; i < 16; i++) acc[mb][i] = 0.0f;
-            const int r = nb * 32 + n;
+                for (int i = 0; i < 16; i++) acc[nb][mb][i] = 0.0f;
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) {
-                MdFrag kf;
-                kf.q = *reinterpret_cast<const uint4 *>(&s_rows[buf][r][(((hh * (PPR / 2) + ks) ^ r) & (PPR - 1)) * 8]);
+        for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+            for (int nb = 0; nb < 2; nb++)
 #pragma unroll
                 for (int mb = 0; mb < MB; mb++)
-                    acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qf[mb][ks].v, kf.v, acc[mb], 0, 0, 0);
-            }
+                    acc[nb][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qf[mb][ks].v, kf[nb][ks].v, acc[nb][mb], 0, 0, 0);
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++) {
             float v = -INFINITY;
             if (fast_rows == 16) {
 #pragma unroll
-                for (int i = 0; i < 8; i++) v = fmaxf(v, acc[0][i]);
+                for (int i = 0; i < 8; i++) v = fmaxf(v, acc[nb][0][i]);
             } else if (fast_rows == 32) {
 #pragma unroll
-                for (int i = 0; i < 16; i++) v = fmaxf(v, acc[0][i]);
+                for (int i = 0; i < 16; i++) v = fmaxf(v, acc[nb][0][i]);
             } else if (fast_rows == 64) {
 #pragma unroll
                 for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-                    for (int i = 0; i < 16; i++) v = fmaxf(v, acc[mb][i]);
+                    for (int i = 0; i < 16; i++) v = fmaxf(v, acc[nb][mb][i]);
             } else {
 #pragma unroll
                 for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-                    for (int i = 0; i < 16; i++) v = fmaxf(v, ((vm[mb] >> i) & 1u) ? acc[mb][i] : -INFINITY);
+                    for (int i = 0; i < 16; i++) v = fmaxf(v, ((vm[mb] >> i) & 1u) ? acc[nb][mb][i] : -INFINITY);
             }
             v = fmaxf(v, swap_halves(v));
-            if (hh == 0) my_scores[(tile % MD_PASS) * MD_TN + r] = round_bf16(v);
+            if (hh == 0 && searched[nb]) my_scores[(tile % MD_PASS) * MD_TN + nb * 32 + n] = round_bf16(v);
         }
         if ((tile % MD_PASS) == MD_PASS - 1 || tile == ntiles - 1) replay(tile - (tile % MD_PASS), tile);  // the wave's own LDS writes
     }
