@@ -64,6 +64,14 @@ __device__ __forceinline__ int64_t bsa_rope_far_pos(const RopeView &r, long long
     return v < 0 ? 0 : v;
 }
 
+// The "dynamic_extend" rule inside attention (attention_extend_bsa.py:271-292, :323-357): a sink or selected key is
+// rotated with a blend of two table rows, 0.75 of the row of its "streaming" position and 0.25 of the row of its own
+// position squeezed into the model's context (dynamic_extend_pos); both products and the sum are rounded to T.
+template <typename T>
+__device__ __forceinline__ float rope_blend(float stream, float dyn) {
+    return Elem<T>::round(__fadd_rn(Elem<T>::round(__fmul_rn(stream, 0.75f)), Elem<T>::round(__fmul_rn(dyn, 0.25f))));
+}
+
 // ---------------------------------------------------------------- pieces shared by the matrix-core attention kernels
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;

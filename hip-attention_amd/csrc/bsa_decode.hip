@@ -146,6 +146,17 @@ __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<E
             const int64_t tr = p.rope.row(rpos) + (dl & 7) * SEG;
             load_elems<T, SEG>(reinterpret_cast<const T *>(p.rope.cos) + tr, rc);
             load_elems<T, SEG>(reinterpret_cast<const T *>(p.rope.sin) + tr, rsn);
+            if (kind == 0 && p.rope.backend == HIPATTN_EXTEND_DYNAMIC) {  // one query row: pmax = its position + 1
+                float dc[SEG], ds[SEG];
+                const int64_t td = p.rope.row(dynamic_extend_pos(t, ppos, ppos + 1, p.rope.model_ctx)) + (dl & 7) * SEG;
+                load_elems<T, SEG>(reinterpret_cast<const T *>(p.rope.cos) + td, dc);
+                load_elems<T, SEG>(reinterpret_cast<const T *>(p.rope.sin) + td, ds);
+#pragma unroll
+                for (int e = 0; e < SEG; e++) {
+                    rc[e] = rope_blend<T>(rc[e], dc[e]);
+                    rsn[e] = rope_blend<T>(rsn[e], ds[e]);
+                }
+            }
 #pragma unroll
             for (int e = 0; e < SEG; e++) {
                 const float other = __shfl_xor(kh[e], 8);

@@ -378,6 +378,8 @@ static int pick_dec(const DecodeMfmaParams &dp, hipStream_t st) {
 
 int bsa_decode_mfma_launch(const BsaParams &p, int dtype, int HID, int nsplits, float *ws, hipStream_t st) {
     if (dtype != HIPATTN_BF16 || p.G > 8) return HIPATTN_E_UNSUPPORTED;
+    // the dynamic rule blends two table rows per key: served by the vector-unit kernel
+    if (p.rope.cos && p.rope.backend == HIPATTN_EXTEND_DYNAMIC) return HIPATTN_E_UNSUPPORTED;
     DecodeMfmaParams dp;
     dp.a = p;
     dp.nsplits = nsplits;

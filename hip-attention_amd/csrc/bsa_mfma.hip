@@ -498,6 +498,8 @@ static int launch_mfma(const BsaParams &p, hipStream_t st) {
 int bsa_mfma_launch(const BsaParams &p, int dtype, int HID, hipStream_t st) {
     if (dtype != HIPATTN_BF16) return HIPATTN_E_UNSUPPORTED;
     if (p.bq > 64) return HIPATTN_E_UNSUPPORTED;
+    // the dynamic rule blends two table rows per key: served by the portable kernel
+    if (p.rope.cos && p.rope.backend == HIPATTN_EXTEND_DYNAMIC) return HIPATTN_E_UNSUPPORTED;
     if ((p.o_st % 4) != 0 || (p.o_sh % 4) != 0 || (p.o_sb % 4) != 0) return HIPATTN_E_UNSUPPORTED;
     bool ext = p.kx.extended();
     BsaParams plain;

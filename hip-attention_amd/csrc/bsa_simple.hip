@@ -23,9 +23,11 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
 
     // CURR = largest position + 1 over the block's rows
     long long curr = 0, pmin = 0x7fffffffffffffffLL;
+    int nvalid = 0;  // valid rows of the block
     for (int j = lane; j < p.bq; j += 64) {
         long long it = (long long)qb * p.bq + j;
         if (it < p.TDST) {
+            nvalid++;
             long long sl = p.pos[(int64_t)b * p.pos_sb + it * p.pos_st] + 1;
             curr = sl > curr ? sl : curr;
             pmin = sl - 1 < pmin ? sl - 1 : pmin;
@@ -37,6 +39,7 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
         curr = w > curr ? w : curr;
         long long w2 = __shfl_xor(pmin, o);
         pmin = w2 < pmin ? w2 : pmin;
+        nvalid += __shfl_xor(nvalid, o);
     }
     int rs = p.kse[irow * 2 + 0], re = p.kse[irow * 2 + 1];
     const long long rope_shift = pmin - p.sw - p.sink - (long long)(re - rs) * p.bk + 1;
@@ -124,6 +127,17 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
                             const int64_t tr = p.rope.row(rpos) + d0 % HALF;
                             load_elems<T, CH>(reinterpret_cast<const T *>(p.rope.cos) + tr, rc);
                             load_elems<T, CH>(reinterpret_cast<const T *>(p.rope.sin) + tr, rsn);
+                            if (kind == 0 && p.rope.backend == HIPATTN_EXTEND_DYNAMIC) {
+                                float dc[CH], ds[CH];
+                                const int64_t td = p.rope.row(dynamic_extend_pos(t, pmin, pmin + nvalid, p.rope.model_ctx)) + d0 % HALF;
+                                load_elems<T, CH>(reinterpret_cast<const T *>(p.rope.cos) + td, dc);
+                                load_elems<T, CH>(reinterpret_cast<const T *>(p.rope.sin) + td, ds);
+#pragma unroll
+                                for (int e = 0; e < CH; e++) {
+                                    rc[e] = rope_blend<T>(rc[e], dc[e]);
+                                    rsn[e] = rope_blend<T>(rsn[e], ds[e]);
+                                }
+                            }
 #pragma unroll
                             for (int e = 0; e < CH; e++)
                                 kk[e] = rope_elem<T>(kk[e], d0 < HALF ? -other[e] : other[e], rc[e], rsn[e]);
@@ -200,7 +214,8 @@ int bsa_fill_params(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t 
     HIPATTN_CHECK_ARG(bq > 0 && bk > 0 && sw >= 0 && sink >= 0 && idx_rows > 0, HIPATTN_E_ARG, "bsa: bad sizes");
     rc = make_kv_view(kv, q->B, q->HID, q->dtype, &p->kv, &p->kx);
     if (rc) return rc;
-    rc = make_rope_view(q, (1u << HIPATTN_EXTEND_STREAMING) | (1u << HIPATTN_EXTEND_INFLLM), "bsa", &p->rope);
+    rc = make_rope_view(q, (1u << HIPATTN_EXTEND_STREAMING) | (1u << HIPATTN_EXTEND_INFLLM) | (1u << HIPATTN_EXTEND_DYNAMIC), "bsa",
+                        &p->rope);
     if (rc) return rc;
     HIPATTN_CHECK_ARG(q->logit_softcap >= 0.0f, HIPATTN_E_ARG, "bsa: negative logit_softcap");
     p->softcap = q->logit_softcap;

@@ -46,7 +46,7 @@ class RopeStruct(ctypes.Structure):
     ]
 
 
-EXTEND_BACKENDS = {"relative": 1, "streaming": 2, "infllm": 3, "dynamic_extend": 4}  # the last: mask stage only
+EXTEND_BACKENDS = {"relative": 1, "streaming": 2, "infllm": 3, "dynamic_extend": 4}
 
 
 class KVStruct(ctypes.Structure):
@@ -157,7 +157,7 @@ def make_rope(cos: torch.Tensor, sin: torch.Tensor, backend: str, k_side_delta: 
               model_context_length: int = 0, attention: bool = False) -> RopeStruct:
     """Describe RoPE tables ``[len, >= HID/2]`` (q's dtype, unit inner stride) and the rotation rule of one call.
     ``attention`` marks a call of block sparse attention, which knows fewer rules than the mask stage."""
-    built = [b for b in EXTEND_BACKENDS if not (attention and b in ("relative", "dynamic_extend"))]
+    built = [b for b in EXTEND_BACKENDS if not (attention and b == "relative")]
     if backend not in built:
         where = "block sparse attention" if attention else "the mask stage"
         raise NotImplementedError(f"extend backend {backend!r} is not built for {where} (built: {sorted(built)})")

@@ -623,7 +623,8 @@ def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], 
     kvs, keep = _kv_struct(args, k, v, max_tsrc, masking=False, stats=stats)
     if position_ids.dtype != torch.int64:
         position_ids = position_ids.to(torch.int64)
-    rope = N.make_rope(*rope_tables, args.sa_extend_backend, attention=True) if rope_tables is not None else None
+    rope = (N.make_rope(*rope_tables, args.sa_extend_backend, 0, args.model_context_length, attention=True)
+            if rope_tables is not None else None)
     qs = N.make_q(qq, position_ids, rope, args.logit_softcap)
     if rope is not None or args.logit_softcap is not None:
         khat = None

@@ -42,13 +42,18 @@ extern "C" {
  *                          slot = token for sink tokens, (j + sink / block_size_k) * block_size_k + e for
  *                          element e of index entry j; pmin = smallest position in the query block
  *                INFLLM    max(0, pmin - sliding_window)
- *   DYNAMIC (mask stage only, attention_extend.py:249-274, :635-636): the query at its own position; with
+ *   DYNAMIC, mask stage (attention_extend.py:249-274, :635-636): the query at its own position; with
  *                pmax = pmin + the number of valid strided query rows, W = model_context_length / 4, the sampled
  *                key at token t keeps position t when t >= pmax - W or pmax <= model_context_length, else it moves
  *                to int32((float(t) - float(pmin - W)) * (float(model_context_length - W) / float(pmin - W)))
  *                + (pmin - W), all in float32; the result is raised to at least pmax - model_context_length
- * Positions are clamped into [0, len).  The reference's "self_extend" rule, "dynamic_extend" inside block sparse
- * attention and the mode that re-rotates keys stored WITH rotation (need_apply_rope = False) are not built. */
+ *   DYNAMIC, attention (attention_extend_bsa.py:271-292, :323-357): sink and selected keys are rotated with a blend of
+ *                two table rows, 0.75 of the row of their STREAMING position and 0.25 of the row of the position
+ *                the mask-stage formula above gives for their token (pmin = smallest position of the query block,
+ *                pmax = pmin + its valid rows; decode: pmax = pmin + 1); both products and the sum are rounded to
+ *                the element type.  Served by the portable attention kernels.
+ * Positions are clamped into [0, len).  The reference's "self_extend" rule and the mode that re-rotates keys stored
+ * WITH rotation (need_apply_rope = False) are not built. */
 #define HIPATTN_EXTEND_RELATIVE 1
 #define HIPATTN_EXTEND_STREAMING 2
 #define HIPATTN_EXTEND_INFLLM 3

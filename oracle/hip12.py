@@ -63,7 +63,7 @@ class _Tensors(ctypes.Structure):
     ]
 
 
-EXTEND_BACKENDS = {None: 0, "relative": 1, "streaming": 2, "infllm": 3, "dynamic_extend": 4}  # 4: mask stage only
+EXTEND_BACKENDS = {None: 0, "relative": 1, "streaming": 2, "infllm": 3, "dynamic_extend": 4}
 
 
 def build(force: bool = False) -> str:
@@ -168,7 +168,7 @@ class OInputs:
     access: Optional[np.ndarray] = None  # int32 [B,HKV,pages]: flags set by every key row the kernels fetch
     rope_cos: Optional[np.ndarray] = None  # float32 [L,HID] (values of the tables' own dtype, widened)
     rope_sin: Optional[np.ndarray] = None
-    model_context_length: int = 131072  # only the "dynamic_extend" rule of the mask stage reads it
+    model_context_length: int = 131072  # only the "dynamic_extend" rules read it
     scan_backend: Optional[str] = None  # rotation rule of the mask stage / of sparse attention; None = no RoPE
     sa_backend: Optional[str] = None
     logit_softcap: float = 0.0

@@ -52,7 +52,7 @@
 #define HIPO_EXT_RELATIVE 1
 #define HIPO_EXT_STREAMING 2
 #define HIPO_EXT_INFLLM 3
-#define HIPO_EXT_DYNAMIC 4 /* mask stage only */
+#define HIPO_EXT_DYNAMIC 4
 
 typedef struct {
     int dtype;               /* HIPO_F32 / HIPO_BF16 (q, k, v, caches all share it) */
@@ -274,6 +274,28 @@ static void rope_rotate(const hipo_tensors_t *X, float *x, int64_t pos) {
     for (int d = 0; d < H2; d++) {
         float c = round_T(X->rope_cos[pos * HID + d], dt);
         float s = round_T(X->rope_sin[pos * HID + d], dt);
+        float lo = x[d], hi = x[d + H2];
+        float nlo = round_T(round_T(lo * c, dt) + round_T(-hi * s, dt), dt);
+        float nhi = round_T(round_T(hi * c, dt) + round_T(lo * s, dt), dt);
+        x[d] = nlo;
+        x[d + H2] = nhi;
+    }
+}
+
+/* The "dynamic_extend" rule inside block sparse attention (attention_extend_bsa.py:271-292, :323-357): the table row
+ * of the key's compressed position is blended with the row of its "streaming" position, 0.25 to 0.75, every product
+ * and the sum rounded to T, and the row is rotated with the blended cos / sin. */
+static void rope_rotate_blend(const hipo_tensors_t *X, float *x, int64_t pos_stream, int64_t pos_dyn) {
+    const int HID = X->HID, H2 = X->HID / 2, dt = X->dtype;
+    if (pos_stream < 0) pos_stream = 0;
+    if (pos_stream >= X->rope_len) pos_stream = X->rope_len - 1;
+    if (pos_dyn < 0) pos_dyn = 0;
+    if (pos_dyn >= X->rope_len) pos_dyn = X->rope_len - 1;
+    for (int d = 0; d < H2; d++) {
+        float cz = round_T(X->rope_cos[pos_stream * HID + d], dt), sz = round_T(X->rope_sin[pos_stream * HID + d], dt);
+        float cn = round_T(X->rope_cos[pos_dyn * HID + d], dt), sn = round_T(X->rope_sin[pos_dyn * HID + d], dt);
+        float c = round_T(round_T(cz * 0.75f, dt) + round_T(cn * 0.25f, dt), dt);
+        float s = round_T(round_T(sz * 0.75f, dt) + round_T(sn * 0.25f, dt), dt);
         float lo = x[d], hi = x[d + H2];
         float nlo = round_T(round_T(lo * c, dt) + round_T(-hi * s, dt), dt);
         float nhi = round_T(round_T(hi * c, dt) + round_T(lo * s, dt), dt);
@@ -530,9 +552,11 @@ int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_
             int hrow = share_first_head ? (h / G) * G : h;
             int64_t irow = ((int64_t)b * HEAD + hrow) * NBQ_rows + qb;
             int64_t curr = 0, pos_min = INT64_MAX;
+            int nvalid = 0; /* valid rows of the block (sum(mask_tdst), attention_extend_bsa.py:255) */
             for (int j = 0; j < block_size_q; j++) {
                 int64_t it = (int64_t)qb * block_size_q + j;
                 if (it < TDST) {
+                    nvalid++;
                     int64_t sl = X->pos[(int64_t)b * TDST + it] + 1;
                     if (sl > curr) curr = sl;
                     if (sl - 1 < pos_min) pos_min = sl - 1;
@@ -572,7 +596,15 @@ int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_
                     if (X->sa_backend == HIPO_EXT_INFLLM) rp = pos_min - sw;
                     if (rp < 0) rp = 0;
                 }
-                scaled_key_at(X, b, tok[i], kvh, c_k, rp, khat + (size_t)i * HID);
+                if (kind[i] == 0 && X->rope_cos && X->sa_backend == HIPO_EXT_DYNAMIC) {
+                    /* the key's own position squeezed into the model's context, blended with the streaming one */
+                    float *kr = khat + (size_t)i * HID;
+                    fetch_row(X, 0, b, tok[i], kvh, kr);
+                    rope_rotate_blend(X, kr, rp, dynamic_extend_pos(tok[i], pos_min, pos_min + nvalid, X->model_context_length));
+                    for (int d = 0; d < HID; d++) kr[d] = round_T(kr[d] * c_k, X->dtype);
+                } else {
+                    scaled_key_at(X, b, tok[i], kvh, c_k, rp, khat + (size_t)i * HID);
+                }
                 fetch_row(X, 1, b, tok[i], kvh, vrow + (size_t)i * HID);
             }
             for (int j = 0; j < block_size_q; j++) {

@@ -326,6 +326,11 @@ def main():
                                      dict(extend=("dynamic_extend", "streaming"), model_ctx=1024)),
         "f32_decode_rope_dynamic": (11, 2, 1, 2048, 4, 2, 32, tiny, 16, 256, 512, 32,
                                     dict(lens=[2048, 1500], page_size=8, extend=("dynamic_extend", "infllm"), model_ctx=512)),
+        # dynamic_extend inside block sparse attention: cos / sin of the squeezed position blended with the streaming ones
+        "f32_prefill_sa_rope_dynamic": (12, 1, 96, 2048, 4, 2, 32, tiny, 16, 256, 512, 32,
+                                        dict(extend=("relative", "dynamic_extend"), model_ctx=1024)),
+        "f32_decode_sa_rope_dynamic": (13, 2, 1, 2048, 4, 2, 32, tiny, 16, 256, 512, 32,
+                                       dict(lens=[2048, 1400], page_size=4, extend=("streaming", "dynamic_extend"), model_ctx=512)),
         # Not generated: Triton's interpreter has no bfloat16 constants (``get_bf16``) and cannot call
         # ``libdevice.tanh`` (logit_softcap) outside a compiled kernel, so bfloat16 inputs and soft-capped logits
         # have no vectors from the reference.

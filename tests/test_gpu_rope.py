@@ -137,6 +137,34 @@ def test_float32_tables_with_bf16_queries_are_cast_like_the_reference():
     assert_context_close(ctx, octx, "bf16")
 
 
+@pytest.mark.parametrize("dtype,D", [("f32", 64), ("bf16", 64), ("bf16", 128)])
+@pytest.mark.parametrize("model_ctx", [1024, 131072])
+def test_dynamic_extend_inside_attention_prefill_and_paged_decode(dtype, D, model_ctx):
+    """The dynamic_extend rule of block sparse attention: sink and selected keys are rotated with 0.75 of the table row
+    of their streaming position and 0.25 of the row of their own position squeezed into the model's context
+    (attention_extend_bsa.py:271-292, :323-357).  With model_ctx = 1024 the 3000-token context reaches beyond the
+    model's and the squeeze is active; with 131072 the second row is the key's own position."""
+    print(f"[case] rope dynamic_extend in attention {dtype} D={D} model_ctx={model_ctx}", flush=True)
+    X = with_rope(make_inputs(51, B=2, TQ=100, TK=3000, H=4, HKV=2, D=D, dtype=dtype, scale=0.5), 4096)
+    A = _ext(scan_extend_backend="relative", sa_extend_backend="dynamic_extend", model_context_length=model_ctx)
+    octx, ometa = O.hip_attention_12(X, A)
+    ctx, meta = run_product(X, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, dtype)
+    ref_stream, _ = O.hip_attention_12(X, _ext(scan_extend_backend="relative", sa_extend_backend="streaming"))
+    widen = O.bf16_bits_to_f32 if dtype == "bf16" else (lambda a: a)
+    assert np.abs(widen(octx) - widen(ref_stream)).max() > 0.05  # the rule really changes the result
+    lens = np.array([3000, 1400])
+    Xd = make_inputs(52, B=2, TQ=1, TK=3000, H=4, HKV=2, D=D, dtype=dtype, pos=(lens - 1)[:, None], scale=0.5)
+    XP = with_rope(to_paged(Xd, 8, seed=9, seq_lens=lens), 4096)
+    A = _ext(scan_extend_backend="streaming", sa_extend_backend="dynamic_extend", model_context_length=model_ctx,
+             extend_context_length=3000)
+    octx, ometa = O.hip_attention_12(XP, A)
+    ctx, meta = run_product(XP, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, dtype)
+
+
 def test_unbuilt_rules_fail_loudly():
     from hip_attn import _native as N
     print("[case] rope unbuilt rules", flush=True)
@@ -145,8 +173,6 @@ def test_unbuilt_rules_fail_loudly():
         run_product(X, _ext(scan_extend_backend="self_extend"))
     with pytest.raises(NotImplementedError):
         run_product(X, _ext(sa_extend_backend="relative"))
-    with pytest.raises(NotImplementedError):
-        run_product(X, _ext(sa_extend_backend="dynamic_extend"))
     with pytest.raises(N.HipAttnError):  # the squeeze divides by pmin - model_context_length / 4: tiny lengths are refused
         run_product(X, _ext(scan_extend_backend="dynamic_extend", model_context_length=64))
     with pytest.raises(NotImplementedError):
