@@ -530,6 +530,100 @@ def run_offload(args, device, TK=3_000_000, warm_steps=4, drift_steps=12):
     same = bool(torch.equal(out_res.view(torch.int16), out_cold.view(torch.int16)) and
                 torch.equal(out_res.view(torch.int16), out_warm.view(torch.int16)) and
                 torch.equal(meta_res.indices, meta.indices))
+    # --- overlap of the miss fetch with compute.  One layer alone has nothing to overlap a fetch with: the next call
+    # on the same layer needs the blocks.  In a model the fetch of layer L runs beside the attention of the layers
+    # after it, so each step here is followed by a refresh step and `filler` cached decode steps on resident KV that
+    # stand for them (one HIP graph).
+    # Three passes over the same fresh drifting queries: fetch on the side stream (cache.miss_stream), then the same
+    # queries again with everything resident (all hit), then, from the same start, fetch on the main stream.
+    overlap = None
+    if drift_steps >= 4:
+        filler = 8
+        side = torch.cuda.Stream(device=device)
+        fresh = [torch.randn((1, 1, H, D), generator=g, dtype=torch.float32) for _ in range(drift_steps)]
+        fresh_q = [blended(blend, nz) for nz in fresh]
+
+        # the stand-in layers as one HIP graph, so that the host enqueues them in a few microseconds
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                call(q, meta_res, resident=resident)
+                call(q, None, resident=resident)
+        torch.cuda.synchronize()
+        g_fill = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g_fill):
+            call(q, None, resident=resident)  # the next layer refreshes its mask on the same step
+            for _ in range(filler):
+                fill_out, _ = call(q, meta_res, resident=resident)
+        torch.cuda.synchronize()
+
+        def rewarm():
+            cache.miss_stream = None
+            cache.flush()
+            for _ in range(4):
+                _, m0 = call(q)
+                cache.handle_cache_miss(m0)
+            torch.cuda.synchronize()
+
+        def loop(stream):
+            cache.miss_stream = stream
+            per_step, fetch_us, call_us = [], [], []
+            for qd in fresh_q:
+                e0, e1, e2, e3 = (torch.cuda.Event(enable_timing=True) for _ in range(4))
+                torch.cuda.synchronize()
+                e0.record()
+                _, md = call(qd)
+                e1.record()
+                if stream is not None:
+                    # the next layers are enqueued first; the fetch waits for the step only (event e1)
+                    g_fill.replay()
+                    cache.handle_cache_miss(md, after=e1)
+                    torch.cuda.current_stream().wait_stream(stream)  # the step is over when both are done
+                else:
+                    cache.handle_cache_miss(md)
+                    e2.record()
+                    g_fill.replay()
+                e3.record()
+                torch.cuda.synchronize()
+                per_step.append(e0.elapsed_time(e3) * 1e3)
+                fetch_us.append(e1.elapsed_time(e2) * 1e3 if stream is None else 0.0)
+                call_us.append(e0.elapsed_time(e1) * 1e3)
+            cache.miss_stream = None
+            return per_step, fetch_us, call_us
+
+        fetched = lambda: cache.sa_kv_cache.statistics()["blocks_fetched"] + cache.mask_k_cache.statistics()["blocks_fetched"]  # noqa: E731
+        rewarm()
+        f0 = fetched()
+        t_async, _, c_async = loop(side)
+        f1 = fetched()
+        t_hit, idle_commit, c_hit = loop(None)       # everything resident now: every read hits
+        f2 = fetched()
+        rewarm()
+        f3 = fetched()
+        t_sync, t_fetch, _ = loop(None)
+        f4 = fetched()
+        us_fill, _ = timed(lambda: g_fill.replay(), 4)
+        med = lambda xs: sorted(xs)[len(xs) // 2]  # noqa: E731
+        m_async, m_hit, m_sync = med(t_async[2:]), med(t_hit[2:]), med(t_sync[2:])
+        m_fetch = med(t_fetch[2:]) - med(idle_commit[2:])  # the part of the commit that is the fetch itself
+        del g_fill, fill_out
+        overlap = {
+            "filler": f"one HIP graph: a refresh step and {filler} cached steps on resident KV", "steps": len(fresh_q) - 2,
+            "step_us_all_hit": m_hit, "step_us_miss_fetch_on_main_stream": m_sync,
+            "step_us_miss_fetch_on_side_stream": m_async,
+            "commit_us_with_misses": med(t_fetch[2:]), "commit_us_nothing_to_fetch": med(idle_commit[2:]),
+            "fetch_us": m_fetch,
+            "overlap_efficiency": 1.0 - (m_async - m_hit) / m_fetch if m_fetch > 0 else None,
+            # the same without what the step itself loses by reading the missed blocks from host memory
+            "host_read_penalty_us": med(c_async[2:]) - med(c_hit[2:]),
+            "fetch_fraction_hidden": (1.0 - (m_async - m_hit - (med(c_async[2:]) - med(c_hit[2:]))) / m_fetch
+                                      if m_fetch > 0 else None),
+            "overlap_efficiency_fetch_on_main_stream": 1.0 - (m_sync - m_hit) / m_fetch if m_fetch > 0 else None,
+            "blocks_fetched_side_stream_pass": f1 - f0, "blocks_fetched_all_hit_pass": f2 - f1,
+            "blocks_fetched_main_stream_pass": f4 - f3,
+            "filler_us": us_fill,
+            "definition": "1 - (step with misses - step all hit) / fetch time; the step with misses also reads the "
+                          "missed blocks from host memory inside its kernels, which no overlap removes",
+        }
     tail = drift[2:]
     block_bytes = 2 * BT * D * 2  # upper bound per fetched block (key-only blocks are half of it)
     res = {
@@ -559,6 +653,7 @@ def run_offload(args, device, TK=3_000_000, warm_steps=4, drift_steps=12):
             "output_equals_uncapped": capped_same,
         },
         "offloaded_equals_resident": same,
+        "overlap": overlap,
     }
     del cache, kres, resident
     torch.cuda.empty_cache()

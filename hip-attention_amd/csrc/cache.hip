@@ -13,6 +13,8 @@
 
 #include <new>
 
+#include <stdlib.h>
+
 #include "common.hpp"
 
 struct hipattn_cache {
@@ -374,17 +376,35 @@ __global__ __launch_bounds__(CT_THREADS) void cache_fetch_kernel(CacheDev c) {
         const int32_t slot = c.victim_list[i];
         const int64_t h = e / c.n_blocks, blk = e % c.n_blocks;
         char *dst = c.bank + (int64_t)slot * c.slot_bytes;
-        for (int w = threadIdx.x; w < total; w += CT_THREADS) {
-            const int part = w / (c.block_tokens * pieces_per_row);
-            const int r = (w / pieces_per_row) % c.block_tokens;
-            const int piece = w % pieces_per_row;
-            const int64_t row = (blk << c.shift) + r;
-            uint4 val = make_uint4(0, 0, 0, 0);
-            if (row < c.pool_rows) {
-                const char *src = (part ? c.host_v : c.host_k) + row * c.host_stride_row_b + h * c.host_stride_h_b;
-                val = *reinterpret_cast<const uint4 *>(src + piece * 16);
+        // four 16-byte pieces per thread in flight before the first is stored: the few workgroups of this kernel have
+        // to cover the latency of the host link with their own loads
+        for (int w0 = threadIdx.x; w0 < total; w0 += 4 * CT_THREADS) {
+            uint4 val[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int w = w0 + u * CT_THREADS;
+                val[u] = make_uint4(0, 0, 0, 0);
+                if (w < total) {
+                    const int part = w / (c.block_tokens * pieces_per_row);
+                    const int r = (w / pieces_per_row) % c.block_tokens;
+                    const int piece = w % pieces_per_row;
+                    const int64_t row = (blk << c.shift) + r;
+                    if (row < c.pool_rows) {
+                        const char *src = (part ? c.host_v : c.host_k) + row * c.host_stride_row_b + h * c.host_stride_h_b;
+                        val[u] = *reinterpret_cast<const uint4 *>(src + piece * 16);
+                    }
+                }
             }
-            *reinterpret_cast<uint4 *>(dst + ((int64_t)part * c.block_tokens + r) * c.row_bytes + piece * 16) = val;
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int w = w0 + u * CT_THREADS;
+                if (w < total) {
+                    const int part = w / (c.block_tokens * pieces_per_row);
+                    const int r = (w / pieces_per_row) % c.block_tokens;
+                    const int piece = w % pieces_per_row;
+                    *reinterpret_cast<uint4 *>(dst + ((int64_t)part * c.block_tokens + r) * c.row_bytes + piece * 16) = val[u];
+                }
+            }
         }
         if (threadIdx.x == 0) {
             const int32_t old = c.backref[slot];
@@ -654,8 +674,17 @@ extern "C" int hipattn_cache_commit(hipattn_cache_t *c, void *stream) {
     HIPATTN_CHECK_ARG(c, HIPATTN_E_ARG, "cache: null handle");
     hipStream_t st = (hipStream_t)stream;
     const CacheDev v = dev_of(c);
-    // a bounded grid walks the fetch list: how many blocks there are is only known on the device
-    const unsigned fetch_grid = (unsigned)(c->max_fetch < 4096 ? c->max_fetch : 4096);
+    // A bounded grid walks the fetch list: how many blocks there are is only known on the device.  Two workgroups
+    // per compute unit keep far more bytes in flight than the host link needs (4 MB against a few hundred KB) and
+    // leave the wave slots of the chip to whatever runs beside the fetch on another stream; a grid that fills every
+    // slot with waves waiting on the host link starves those kernels (measured: no overlap at all with 4096).
+    static int env_grid = -1;
+    if (env_grid < 0) {
+        const char *e = getenv("HIPATTN_CACHE_FETCH_GRID");  // tuning aid
+        env_grid = e ? atoi(e) : 0;
+    }
+    const long long want = env_grid > 0 ? env_grid : 64;
+    const unsigned fetch_grid = (unsigned)(c->max_fetch < want ? c->max_fetch : want);
     hipLaunchKernelGGL(cache_fetch_kernel, dim3(fetch_grid), dim3(CT_THREADS), 0, st, v);
     hipLaunchKernelGGL(cache_step_kernel, dim3(1), dim3(64), 0, st, v);
     HIPATTN_CHECK_HIP(hipGetLastError());

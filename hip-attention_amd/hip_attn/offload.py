@@ -16,6 +16,7 @@ methods, re-designed for this hardware:
 """
 from __future__ import annotations
 
+import os
 from typing import Optional, Tuple
 
 import torch
@@ -104,6 +105,10 @@ class GPUCache:
         self._desc = d
         self.handle = N.cache_create(d, self.max_fetch, dev)
         self._ready: Optional[torch.cuda.Event] = None
+        # schedule + commit are about twenty small launches whose enqueueing costs more host time than the kernels
+        # take when there is little to fetch: after a first eager run they are replayed from one HIP graph
+        self._miss_graph: Optional[torch.cuda.CUDAGraph] = None
+        self._miss_calls = 0
         self.allocated_gpu_bytes = sum(t.numel() * t.element_size() for t in (
             self.bank, self.table, self.last_use, self.backref, self.miss, self.workspace))
 
@@ -125,24 +130,50 @@ class GPUCache:
             torch.cuda.current_stream(self.device).wait_event(self._ready)
             self._ready = None
 
-    def handle_cache_miss(self, metadata=None, stats=None, stream: Optional[torch.cuda.Stream] = None):
+    def handle_cache_miss(self, metadata=None, stats=None, stream: Optional[torch.cuda.Stream] = None,
+                          after: Optional[torch.cuda.Event] = None):
         """Bring the blocks flagged during the last step into the cache (``uvm_gpu_cache.py:305-398``).
 
         ``metadata`` / ``stats`` are accepted for signature compatibility: the readers already recorded
         what missed.  With ``stream`` the work runs there, after everything enqueued so far on the current
-        stream; the next attention call waits for it.
+        stream, or, with ``after``, after that event only (recorded behind the step whose misses are fetched:
+        work enqueued on the current stream since then runs beside the fetch); the next attention call waits for it.
         """
         if stream is None:
             self.wait()
-            N.cache_schedule(self.handle, self.device)
-            N.cache_commit(self.handle, self.device)
+            self._schedule_and_commit()
             return
-        stream.wait_stream(torch.cuda.current_stream(self.device))
+        if after is not None:
+            stream.wait_event(after)
+        else:
+            stream.wait_stream(torch.cuda.current_stream(self.device))
         with torch.cuda.stream(stream):
-            N.cache_schedule(self.handle, self.device)
-            N.cache_commit(self.handle, self.device)
+            self._schedule_and_commit()
             self._ready = torch.cuda.Event()
             self._ready.record(stream)
+
+    def _schedule_and_commit(self):
+        """Enqueue the lookup and the fetch on the current stream: eagerly the first time and inside a caller's own
+        graph capture, otherwise as one replay of a graph captured on the second call (the kernels take the cache's
+        arrays by address and read every count on the device, so one recording serves every later call)."""
+        capturing = torch.cuda.is_current_stream_capturing()
+        use_graph = os.getenv("HIP_ATTN_CACHE_MISS_GRAPH", "1") == "1" and not capturing
+        self._miss_calls += 1
+        if use_graph and self._miss_graph is None and self._miss_calls >= 2:
+            current = torch.cuda.current_stream(self.device)
+            graph = torch.cuda.CUDAGraph()
+            cap = torch.cuda.Stream(device=self.device)
+            cap.wait_stream(current)
+            with torch.cuda.graph(graph, stream=cap):
+                N.cache_schedule(self.handle, self.device)
+                N.cache_commit(self.handle, self.device)
+            current.wait_stream(cap)
+            self._miss_graph = graph
+        if use_graph and self._miss_graph is not None:
+            self._miss_graph.replay()
+        else:
+            N.cache_schedule(self.handle, self.device)
+            N.cache_commit(self.handle, self.device)
 
     def on_set_kv_buffer(self, table: Tensor, cache_k: Tensor, cache_v: Optional[Tensor]):
         """Resident blocks receive freshly written rows (``uvm_gpu_cache.py:548-563``)."""
@@ -255,12 +286,14 @@ class HiPOffloadCache:
         if self.pending_write is not None:
             (stream or torch.cuda.current_stream(self.device)).wait_event(self.pending_write)
 
-    def handle_cache_miss(self, metadata=None):
+    def handle_cache_miss(self, metadata=None, after: Optional[torch.cuda.Event] = None):
+        """``after``: with ``miss_stream`` set, an event recorded behind the step whose misses are to be fetched; what
+        the caller has enqueued on the current stream since then (the next layers) runs beside the fetch."""
         stats_m = getattr(metadata, "mask_cache_statistics", None)
         stats_s = getattr(metadata, "sa_cache_statistics", None)
         self._wait_pending_write(self.miss_stream)
-        self.mask_k_cache.handle_cache_miss(metadata=metadata, stats=stats_m, stream=self.miss_stream)
-        self.sa_kv_cache.handle_cache_miss(metadata=metadata, stats=stats_s, stream=self.miss_stream)
+        self.mask_k_cache.handle_cache_miss(metadata=metadata, stats=stats_m, stream=self.miss_stream, after=after)
+        self.sa_kv_cache.handle_cache_miss(metadata=metadata, stats=stats_s, stream=self.miss_stream, after=after)
 
     def flush(self):
         self._wait_pending_write()
