@@ -18,26 +18,35 @@
 
 namespace hipattn {
 
+// a row of zeros in device memory: empty token slots of a tile are loaded from here, so that the loads of a tile
+// need no branches
+__device__ __align__(16) uint16_t g_zero_row[256];
+
 constexpr int TN = 64;        // tokens per tile
 constexpr int NTHREADS = 512;
 constexpr int MAX_LDS_IDX = 1024;  // selected-block starts kept in LDS
 
 // what wave 0 posts about the 64 token slots of a tile
 struct MfmaMeta {
-    long long ko[TN], vo[TN];  // K / V row offsets (NO_ROW: zero row)
+    long long ko[TN], vo[TN];  // addresses of the K / V rows (an empty slot: the row of zeros)
     int tok[TN];               // token, -1 for an empty slot
     int rp[TN];                // row of the RoPE tables the key is rotated with
     int tmin, tmax, all_valid; // smallest / largest token of the tile (tmax < 0: empty tile), no empty slot
     int pad_;
 };
 
+// Tiles are resolved in batches of META_BATCH, one batch ahead of their use: the ring holds two batches.
+template <int HID>
+constexpr int META_BATCH = HID <= 128 ? 16 : 4;
+
 template <int HID>
 struct MfmaSmem {
     uint16_t k[2][TN][HID + KPAD];
     uint16_t v[2][TN][HID + VPAD];
-    MfmaMeta meta[4];
+    MfmaMeta meta[2 * META_BATCH<HID>];
     int idx[MAX_LDS_IDX];
 };
+static_assert(sizeof(MfmaSmem<256>) <= 160 * 1024, "LDS of a compute unit");
 
 // ROPE = true (extended parameter block, unscaled keys): query rows and staged key rows are rotated on load.
 // A query lane holds both halves of its row (k-steps ks and ks + KS/2); the two halves of a staged key row are
@@ -167,16 +176,15 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
 
     const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
 
-    // ---- staging.  Wave 0 walks the token list: lane = token slot of a tile; it resolves the token, its K / V row
-    // offsets (page lookup, statistics, offload cache) and, with RoPE, its rotated position, one tile ahead of the
-    // loads, and posts them in LDS (four slots, so that a slot is rewritten only after every wave is done with it).
+    // ---- staging.  The token list is resolved a batch of tiles at a time, one tile per wave (lane = token slot of
+    // the tile): the token, its K / V row offsets (page lookup, statistics, offload cache) and, with RoPE, its rotated
+    // position are posted in LDS a batch ahead of the loads, so that no wave carries this work on every tile.
     // All threads then fetch rows by posted offset: chunk c = tid + NTHREADS*j is 16-byte piece c % (HID/8) of token
     // slot c / (HID/8).
-    long long m_ko = NO_ROW, m_vo = NO_ROW;
-    int m_t = -1, m_rp = 0, m_tmin = 0, m_tmax = -1, m_allv = 0;
+    constexpr int HB = META_BATCH<HID>;
     const int bk_shift = (p.bk & (p.bk - 1)) == 0 ? __builtin_ctz(p.bk) : -1;  // block sizes are usually powers of two
     const int tlimit = (int)(p.kv.max_tsrc < (long long)curr ? p.kv.max_tsrc : (long long)curr);
-    auto resolve = [&](int tile) {  // wave 0 only
+    auto resolve = [&](int tile) {  // one wave per tile
         int kind, base;  // kind 0 selected, 1 sink, 2 window
         if (tile < tiles_sel) { kind = 0; base = tile * TN; }
         else if (tile < tiles_sel + tiles_sink) { kind = 1; base = (tile - tiles_sel) * TN; }
@@ -210,45 +218,49 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
         }
         int64_t ko = NO_ROW, vo = NO_ROW;
         if (t >= 0) kv_rows<true, EXT>(p.kv, kx, b, t, kvh, seqlen, ko, vo, true);
-        m_ko = ko;
-        m_vo = vo;
-        m_t = t;
-        if constexpr (ROPE) m_rp = (int)p.rope.clamp(rpos);
+        MfmaMeta &mt = sm.meta[tile & (2 * HB - 1)];
+        constexpr int ESZ = KV8 ? 1 : 2;
+        mt.ko[lane] = ko != NO_ROW ? (long long)(reinterpret_cast<const char *>(p.kv.k) + ko * ESZ) : (long long)g_zero_row;
+        mt.vo[lane] = vo != NO_ROW ? (long long)(reinterpret_cast<const char *>(p.kv.v) + vo * ESZ) : (long long)g_zero_row;
+        mt.tok[lane] = t;
+        if constexpr (ROPE) mt.rp[lane] = (int)p.rope.clamp(rpos);
         // tile summary for the mask shortcut, once for the whole workgroup
-        m_tmin = wave_min_i(t < 0 ? 0x7fffffff : t);
-        m_tmax = wave_max_i(t);
-        m_allv = __all(t >= 0) ? 1 : 0;
-    };
-    auto post = [&](int tile) {  // wave 0 only
-        MfmaMeta &mt = sm.meta[tile & 3];
-        mt.ko[lane] = m_ko;
-        mt.vo[lane] = m_vo;
-        mt.tok[lane] = m_t;
-        if constexpr (ROPE) mt.rp[lane] = m_rp;
+        const int tmin = wave_min_i(t < 0 ? 0x7fffffff : t);
+        const int tmax = wave_max_i(t);
+        const int allv = __all(t >= 0) ? 1 : 0;
         if (lane == 0) {
-            mt.tmin = m_tmin;
-            mt.tmax = m_tmax;
-            mt.all_valid = m_allv;
+            mt.tmin = tmin;
+            mt.tmax = tmax;
+            mt.all_valid = allv;
         }
+    };
+    // tiles first .. first + HB - 1, spread over the waves
+    auto resolve_batch = [&](int first) {
+        for (int t = first + wid; t < first + HB && t < ntiles; t += NTHREADS / 64) resolve(t);
     };
     uint4 kreg[CPT], vreg[CPT];
     uint4 creg[ROPE ? CPT : 1], sreg[ROPE ? CPT : 1];  // cos / sin pieces of the staged key rows
     auto prefetch = [&](int tile) {
-        const MfmaMeta &mt = sm.meta[tile & 3];
+        const MfmaMeta &mt = sm.meta[tile & (2 * HB - 1)];
+        long long ka[CPT], va[CPT];
+        int rp[CPT];
 #pragma unroll
         for (int j = 0; j < CPT; j++) {
-            const int c = tid + NTHREADS * j;
-            const int slot = c / (HID / 8), piece = c % (HID / 8);
-            const long long ko = mt.ko[slot], vo = mt.vo[slot];
-            kreg[j] = make_uint4(0, 0, 0, 0);
-            vreg[j] = make_uint4(0, 0, 0, 0);
+            const int slot = (tid + NTHREADS * j) / (HID / 8);
+            ka[j] = mt.ko[slot];
+            va[j] = mt.vo[slot];
+            if constexpr (ROPE) rp[j] = mt.rp[slot];
+        }
+#pragma unroll
+        for (int j = 0; j < CPT; j++) {
+            const int piece = (tid + NTHREADS * j) % (HID / 8);
             if constexpr (ROPE) {
-                const int64_t tr = (int64_t)mt.rp[slot] * p.rope.stride_t + (piece % (HID / 16)) * 8;
+                const int64_t tr = (int64_t)rp[j] * p.rope.stride_t + (piece % (HID / 16)) * 8;
                 creg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr);
                 sreg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr);
             }
-            if (ko != NO_ROW) kreg[j] = load_kv_piece<KV8>(p.kv.k, ko + piece * 8);
-            if (vo != NO_ROW) vreg[j] = load_kv_piece<KV8>(p.kv.v, vo + piece * 8);
+            kreg[j] = load_kv_piece<KV8>((const void *)ka[j], piece * 8);
+            vreg[j] = load_kv_piece<KV8>((const void *)va[j], piece * 8);
         }
     };
     auto commit = [&](int buf) {
@@ -283,22 +295,19 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
     float l_run = 0.0f;
 
     if (ntiles > 0) {
-        if (wid == 0) {
-            resolve(0);
-            post(0);
-            if (ntiles > 1) resolve(1);
-        }
+        resolve_batch(0);
         __syncthreads();
         prefetch(0);
     }
     for (int tile = 0; tile < ntiles; tile++) {
         const int buf = tile & 1;
         commit(buf);
-        if (wid == 0 && tile + 1 < ntiles) post(tile + 1);
         __syncthreads();
         if (tile + 1 < ntiles) prefetch(tile + 1);
-        if (wid == 0 && tile + 2 < ntiles) resolve(tile + 2);
-        const MfmaMeta &mt = sm.meta[tile & 3];
+        // the next batch of tiles: its half of the ring was last read a batch ago, and the barrier of the next
+        // round stands between these writes and their first use
+        if (((tile + 2) & (HB - 1)) == 0 && tile + 2 < ntiles) resolve_batch(tile + 2);
+        const MfmaMeta &mt = sm.meta[tile & (2 * HB - 1)];
         const bool window = tile >= tiles_sel + tiles_sink;
 
         // tile summary (token range, all valid?) posted by wave 0
@@ -323,7 +332,6 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
             sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0.v, qf[ks].v, sacc[0], 0, 0, 0);
             sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1.v, qf[ks].v, sacc[1], 0, 0, 0);
         }
-
         if constexpr (CAP) {
             const float k2 = 2.0f * LOG2E / p.softcap;
 #pragma unroll
@@ -382,7 +390,6 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
                 }
         l_run = l_run * alpha + lsum;
         m_run = m_use;
-
         // ---- O^T += V^T P^T
         if (__any(alpha != 1.0f)) {
 #pragma unroll
