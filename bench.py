@@ -539,7 +539,8 @@ def run_offload(args, device, TK=3_000_000, warm_steps=4, drift_steps=12):
     overlap = None
     if drift_steps >= 4:
         filler = 8
-        side = torch.cuda.Stream(device=device)
+        from hip_attn.offload import concurrent_stream
+        side, side_beside = concurrent_stream(device)  # a stream on a hardware queue of its own
         fresh = [torch.randn((1, 1, H, D), generator=g, dtype=torch.float32) for _ in range(drift_steps)]
         fresh_q = [blended(blend, nz) for nz in fresh]
 
@@ -608,6 +609,7 @@ def run_offload(args, device, TK=3_000_000, warm_steps=4, drift_steps=12):
         del g_fill, fill_out
         overlap = {
             "filler": f"one HIP graph: a refresh step and {filler} cached steps on resident KV", "steps": len(fresh_q) - 2,
+            "side_stream_seen_running_beside_main": side_beside,
             "step_us_all_hit": m_hit, "step_us_miss_fetch_on_main_stream": m_sync,
             "step_us_miss_fetch_on_side_stream": m_async,
             "commit_us_with_misses": med(t_fetch[2:]), "commit_us_nothing_to_fetch": med(idle_commit[2:]),

@@ -34,6 +34,42 @@ def _as_stored(rows: Tensor, pool_dtype: torch.dtype) -> Tensor:
     return rows.to(pool_dtype).contiguous()
 
 
+def concurrent_stream(device, tries: int = 6):
+    """A side stream whose work really runs beside the current stream's, and whether the probe saw it do so.
+
+    A process has few hardware queues (four by default) and the runtime spreads its streams over them, so a new stream
+    may share the current stream's queue; work on it then waits for everything enqueued there before it, and a fetch
+    on such a stream overlaps nothing.  The probe puts about a millisecond of copies on the current stream and a
+    small fill on the candidate: a candidate on a queue of its own finishes first.  Streams tried and rejected are
+    kept alive, so that later streams do not take their place on the queues.  Called once, at set-up."""
+    device = torch.device(device)
+    main = torch.cuda.current_stream(device)
+    big = torch.empty(64 << 20, dtype=torch.float32, device=device)
+    small = torch.empty(1024, dtype=torch.float32, device=device)
+    cand = None
+    for _ in range(tries):
+        cand = torch.cuda.Stream(device=device)
+        _REJECTED_STREAMS.append(cand)
+        torch.cuda.synchronize(device)
+        done_main, done_side = torch.cuda.Event(), torch.cuda.Event()
+        for _ in range(8):
+            big.add_(1.0)
+        done_main.record(main)
+        with torch.cuda.stream(cand):
+            small.zero_()
+            done_side.record(cand)
+        done_side.synchronize()
+        beside = not done_main.query()
+        torch.cuda.synchronize(device)
+        if beside:
+            _REJECTED_STREAMS.pop()
+            return cand, True
+    return cand, False
+
+
+_REJECTED_STREAMS = []
+
+
 class UVMCache:
     """Host pool ``[max_token_size, head_num, head_dim]`` in pinned memory (``uvm_gpu_cache.py:72-117``)."""
 
@@ -278,6 +314,12 @@ class HiPOffloadCache:
         idx_gpu = table_gpu.reshape(-1).to(torch.int64)
         for pool in (self.k_uvm, self.v_uvm):
             pool.metadata.index_put_((idx_gpu,), torch.index_select(pool.metadata, 0, idx_gpu) + 1)
+
+    def enable_miss_stream(self) -> bool:
+        """Fetch missed blocks on a side stream from now on (``miss_stream``); returns whether that stream was seen to
+        run beside the current one (see ``concurrent_stream``)."""
+        self.miss_stream, beside = concurrent_stream(self.device)
+        return beside
 
     def _wait_pending_write(self, stream: Optional[torch.cuda.Stream] = None):
         """Order ``stream`` (default: the current one) after a store into the pools issued on another stream: a fetch
