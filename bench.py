@@ -405,7 +405,28 @@ def run_batched_decode(args, device, B=16, steps=64, refresh_every=8):
                                require_cache_statistics=(meta_in is None) if stats is None else stats)
         return hip_attention_12(q, None, None, a, cached_metadata=meta_in)
 
-    res, _ = _time_decode(step, steps, refresh_every)
+    res, meta = _time_decode(step, steps, refresh_every)
+    if not args.skip_cpu:
+        # the oracle on the shortest and the longest sequence of the batch, same paged cache and block table
+        import numpy as np
+        from oracle import hip12 as O
+
+        pick = [int(lens.argmin()), int(lens.argmax())]
+        kb = kc.cpu().view(torch.int16).numpy().view(np.uint16)
+        qb = q[pick].cpu().view(torch.int16).numpy().view(np.uint16)
+        X = O.OInputs("bf16", qb, pos[pick].cpu().numpy(), k_cache=kb, v_cache=kb,
+                      block_table=bt[pick].cpu().numpy().astype(np.int64),
+                      cache_seq_lens=lens[pick].numpy().astype(np.int64))
+        octx, ometa = O.hip_attention_12(X, O.OArgs(sliding_window_size=1024, extend_context_length=MAXLEN))
+        out_gpu, _ = step(meta)
+        rows = np.concatenate([np.arange(b * H, (b + 1) * H) for b in pick])
+        ref = O.bf16_bits_to_f32(octx)
+        err = np.abs(out_gpu[pick].float().cpu().numpy() - ref)
+        res.update({"oracle_checked_sequences": pick,
+                    "indices_equal_oracle": bool(np.array_equal(meta.indices.cpu().numpy()[rows], ometa.indices)
+                                                 and np.array_equal(meta.ks.cpu().numpy()[rows], ometa.ks)),
+                    "context_within_tolerance_of_oracle": bool((err <= 2e-2 + 1e-2 * np.abs(ref)).all())})
+        del kb, X
     # every sequence scans the chunk grid of the full 262144-token table (the reference sizes the first stage by
     # extend_context_length); chunks beyond a sequence's length end their search after the activity test
     refresh_bytes, attn_bytes = _decode_bytes([int(x) for x in lens], H, HKV, D)
