@@ -287,11 +287,11 @@ class _timed:
 def prescale_k(k: torch.Tensor, device, head_major: bool = False) -> torch.Tensor:
     """``bf16(k * c_k)`` for a whole 4-D bf16 key tensor (dense ``[B,T,HKV,D]`` or a paged cache).
 
-    ``head_major``: the copy of a dense tensor is laid out ``[B,HKV,T,D]`` in memory (and returned as a ``[B,T,HKV,D]``
-    view of it), so that consecutive tokens of a kv head are consecutive rows."""
+    ``head_major``: the copy is laid out ``[HKV, n0, n1, D]`` in memory (and returned as a view of the input's shape),
+    so that consecutive tokens of a kv head -- of a page, for a paged cache -- are consecutive rows."""
     assert k.ndim == 4 and k.dtype == torch.bfloat16 and k.stride(3) == 1
     if head_major:
-        return prescale_k(k.permute(0, 2, 1, 3), device).permute(0, 2, 1, 3)
+        return prescale_k(k.permute(2, 0, 1, 3), device).permute(1, 2, 0, 3)
     out = torch.empty(k.shape, dtype=k.dtype, device=k.device)
     with _timed("prescale_k"):
       rc = lib().hipattn_prescale_k(

@@ -225,10 +225,10 @@ def _mask_kv(args: HiPAttentionArgs, k_mask: Optional[Tensor], max_tsrc: int, q:
             if force == "1" or (force != "0" and sampled_rows >= 4 * rows_total):
                 delta = 0
                 if rope_tabs is None:
-                    # a dense tensor's copy is laid out [B, HKV, T, D]: with the rows of one kv head 2 KB apart, as in
-                    # [B, T, HKV, D], the workgroups that scan a head together keep hitting the same eighth of the
-                    # memory channels (cfg-2-like prefill: the 256- and 32-token stages 4.13 -> 3.77 and 5.19 -> 4.82 ms)
-                    khat = khat0 = N.prescale_k(src, device, head_major=k_mask is not None)
+                    # the copy is laid out with the kv head outermost: the rows a search samples then lie within a
+                    # few KB instead of spreading over HKV times as much (cfg-2-like prefill: the 256- and 32-token
+                    # stages 4.13 -> 3.77 and 5.19 -> 4.82 ms, the same from a page-16 cache)
+                    khat = khat0 = N.prescale_k(src, device, head_major=True)
                 else:
                     # rotated to position 0 (left samples, and everything under infllm) and 1 (right samples, relative)
                     khat = N.prescale_k_rope(src, rope_tabs[0], rope_tabs[1], (0, 1), device)
