@@ -11,6 +11,7 @@
 // in registers: the samples, comparisons, winners, chunk score and refined left edge are those of the sampling
 // kernel, bit for bit, because every score is produced by the same chain of matrix instructions in the same order
 // (mask_stage_mfma.hip).  Access flags are set for the tokens the search samples, not for the tokens loaded.
+// Keys come from a dense tensor or from a paged cache.
 //
 // Workgroup = (batch, kv head, scan row) x up to four heads of the group, one wave per head; the wave keeps its Q^
 // fragments (A operand) in registers and consumes tiles of 64 tokens (B operand) from LDS.
@@ -36,8 +37,9 @@ constexpr int MD_PASS = 8;             // tiles between two replays of the searc
 
 static __device__ __align__(16) uint16_t md_zero_row[256];
 
-// HPW = waves (heads) per workgroup; MB = 32-row blocks of query rows per program (1: up to 32 rows, 2: up to 64)
-template <int HID, int MB, int HPW, bool EXT>
+// HPW = waves (heads) per workgroup; MB = 32-row blocks of query rows per program (1: up to 32 rows, 2: up to 64);
+// PAGED: keys live in a paged cache, the page of every token slot is looked up a pass ahead (below)
+template <int HID, int MB, int HPW, bool EXT, bool PAGED>
 __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFor<EXT> p, long long total_wg) {
     constexpr int NT = 64 * HPW;
     constexpr int KS = HID / 16;
@@ -54,6 +56,10 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
     __shared__ int s_left[MD_MAX_CHUNKS];
     __shared__ float s_gwidth[MD_MAX_CHUNKS / 16];       // per group of block_chunk chunks: widest chunk, 0 = not searched
     __shared__ float s_score[HPW][MD_PASS * MD_TN];      // per head: scores of the tokens of the last MD_PASS tiles
+    // Paged keys: the pool page of every token slot of a pass of MD_PASS tiles (-1: slot not loaded), two passes.
+    // The block table is read with ordinary loads, which drain the tile loads in flight (see s_left), so it is read
+    // once per pass, for the whole next pass, instead of inside the prefetch of every tile.
+    __shared__ int s_page[PAGED ? 2 : 1][PAGED ? MD_PASS * MD_TN : 1];
 
     const int tid = threadIdx.x, lane = tid & 63, wid = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, hh = lane >> 5;
@@ -134,15 +140,23 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
             const int slot = c / PPR, pos = c % PPR;
             const int ci = (tile << cpt_shift) + (slot >> ch_shift);
             const uint16_t *src = md_zero_row;
-            if (ci < p.n) {
+            if constexpr (PAGED) {
+                const int pg = s_page[(tile / MD_PASS) & 1][(tile % MD_PASS) * MD_TN + slot];
+                if (pg >= 0) {
+                    const int t = s_left[ci] + (slot & (CH - 1));  // pg >= 0 implies ci < p.n
+                    src = reinterpret_cast<const uint16_t *>(p.kv.k) + (int64_t)pg * p.kv.k_stride_b +
+                          (int64_t)(t & (p.kv.page_size - 1)) * p.kv.k_stride_t + (int64_t)kvh * p.kv.k_stride_h +
+                          ((pos ^ slot) & (PPR - 1)) * 8;
+                }
+            } else if (ci < p.n) {
                 const int cl = s_left[ci];
                 const int64_t rr = (int64_t)cl + CH;
                 const int cr = (int)(rr < p.right_clamp ? rr : p.right_clamp);
                 const int t = cl + (slot & (CH - 1));
                 // a chunk that starts beyond the block's reach is never searched (its left edge only moves right)
                 if (t < cr && cl <= lim && cl >= 0 && any_rows) {
-                    // dense keys only (the launcher sees to it): the row address is plain arithmetic; rows at or
-                    // beyond the end of the tensor read as zeros
+                    // dense keys: the row address is plain arithmetic; rows at or beyond the end of the tensor read
+                    // as zeros
                     if (t < p.kv.tsrc)
                         src = reinterpret_cast<const uint16_t *>(p.kv.k) + (int64_t)b * p.kv.k_stride_b +
                               (int64_t)t * p.kv.k_stride_t + (int64_t)kvh * p.kv.k_stride_h + ((pos ^ slot) & (PPR - 1)) * 8;
@@ -151,7 +165,28 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
             load_to_lds16(src, &s_rows[buf][0][0] + (wid * 64 + NT * j) * 8);
         }
     };
+    // pages of the token slots of pass `pass` (tiles pass * MD_PASS ...), by all threads
+    auto lookup_pages = [&](int pass) {
+        if constexpr (PAGED) {
+            for (int i = tid; i < MD_PASS * MD_TN; i += NT) {
+                const int ci = ((pass * MD_PASS) << cpt_shift) + (i >> ch_shift);
+                int pg = -1;
+                if (ci < p.n) {
+                    const int cl = s_left[ci];
+                    const int64_t rr = (int64_t)cl + CH;
+                    const int cr = (int)(rr < p.right_clamp ? rr : p.right_clamp);
+                    const int t = cl + (i & (CH - 1));
+                    if (t < cr && cl <= lim && cl >= 0 && any_rows) pg = (int)p.kv.page_of(b, t, seqlen);
+                }
+                s_page[pass & 1][i] = pg;
+            }
+        }
+    };
     __syncthreads();  // s_left visible (the loads above are complete: their values were stored)
+    if constexpr (PAGED) {
+        lookup_pages(0);
+        __syncthreads();
+    }
     for (int x = 0; x < MD_DIST && x < ntiles; x++) prefetch(x);
 
     // ---- program-level gate and iteration count of the reference, per group of block_chunk chunks, once
@@ -205,7 +240,17 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
             if constexpr (EXT) {
                 // access flags for the rows the sampling kernel would have loaded, stored without looking first
                 for (int e = 0; e < CH; e++)
-                    if ((touched >> e) & 1u) kv_k_row<true, false>(p.kv, kx, b, cl0 + e, kvh, seqlen, true);
+                    if ((touched >> e) & 1u) {
+                        if constexpr (PAGED) {
+                            // paged flags are per pool page; the page was looked up with the slot
+                            const int pg = s_page[(first_tile / MD_PASS) & 1][((cidx - c_begin) << ch_shift) + e];
+                            if (kx->access_flags && pg >= 0)
+                                mark_flag<false>(kx->access_flags + (int64_t)b * kx->flags_stride_b +
+                                                 (int64_t)kvh * kx->flags_stride_h + pg);
+                        } else {
+                            kv_k_row<true, false>(p.kv, kx, b, cl0 + e, kvh, seqlen, true);
+                        }
+                    }
             }
             store_score(p, row_out, red_out, cidx, score);
             if (p.left_out) p.left_out[row_out + cidx] = cl;
@@ -222,6 +267,13 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
         else wait_vmcnt<0>();
         __syncthreads();
         if (tile + MD_DIST < ntiles) prefetch(tile + MD_DIST);
+        if constexpr (PAGED) {
+            // the next pass's pages: written here, made visible by the barrier of the next round, first read by the
+            // prefetch of the round after
+            static_assert(MD_PASS - MD_DIST - 2 >= 0, "room for the lookup before the first prefetch of a pass");
+            if ((tile % MD_PASS) == MD_PASS - MD_DIST - 2 && (tile / MD_PASS + 1) * MD_PASS < ntiles)
+                lookup_pages(tile / MD_PASS + 1);
+        }
         if (!head_ok) continue;
         // a block of 32 tokens lies inside one group (block_chunk * CH is a multiple of 32)
         bool searched[2];
@@ -291,11 +343,13 @@ static int launch_dense(const MaskParams &p, hipStream_t st) {
     const long long total = (long long)p.B * p.kv.HKV * p.BS * hblocks;
     if (total >= 0x7fffffffLL) return HIPATTN_E_UNSUPPORTED;
     dim3 grid((unsigned)total), block(64 * HPW);
+    const MaskParamsBase &pb = p;
     if (p.kx.extended()) {
-        hipLaunchKernelGGL((mask_stage_dense_kernel<HID, MB, HPW, true>), grid, block, 0, st, p, total);
+        if (p.kv.paged) hipLaunchKernelGGL((mask_stage_dense_kernel<HID, MB, HPW, true, true>), grid, block, 0, st, p, total);
+        else hipLaunchKernelGGL((mask_stage_dense_kernel<HID, MB, HPW, true, false>), grid, block, 0, st, p, total);
     } else {
-        const MaskParamsBase &pb = p;
-        hipLaunchKernelGGL((mask_stage_dense_kernel<HID, MB, HPW, false>), grid, block, 0, st, pb, total);
+        if (p.kv.paged) hipLaunchKernelGGL((mask_stage_dense_kernel<HID, MB, HPW, false, true>), grid, block, 0, st, pb, total);
+        else hipLaunchKernelGGL((mask_stage_dense_kernel<HID, MB, HPW, false, false>), grid, block, 0, st, pb, total);
     }
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
@@ -318,8 +372,6 @@ int mask_stage_dense_launch(const MaskParams &p, int HID, int rows_eff, hipStrea
     if (CH < 2 || CH > 16 || (CH & (CH - 1)) != 0) return HIPATTN_E_UNSUPPORTED;
     if (p.hg != 1 || p.rope.cos || p.kx.cached || p.kx.kv8) return HIPATTN_E_UNSUPPORTED;
     if (p.nrows > 64 || p.n > MD_MAX_CHUNKS) return HIPATTN_E_UNSUPPORTED;
-    // paged keys need a page lookup per token, a vector-memory load the tile loop cannot afford (see s_left)
-    if (p.kv.paged) return HIPATTN_E_UNSUPPORTED;
     if (mode == 1) {
         // pays when the group's searches together load more rows than the chunks hold, on launches wide enough to
         // keep the chip busy with one workgroup per (batch, kv head, scan row)

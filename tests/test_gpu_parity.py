@@ -259,7 +259,7 @@ DENSE_CASES = {
 }
 
 
-@pytest.mark.parametrize("paged", [False, True])
+@pytest.mark.parametrize("paged", [0, 16, 4, 1])
 @pytest.mark.parametrize("case", list(DENSE_CASES))
 def test_small_chunk_stages_scored_densely(case, paged, monkeypatch):
     """Stages with chunks of 2 .. 16 tokens on prescaled keys can score every token of every chunk once per GQA group
@@ -271,8 +271,8 @@ def test_small_chunk_stages_scored_densely(case, paged, monkeypatch):
     B, TQ, TK, H, HKV, D, stages, kw = DENSE_CASES[case]
     X = make_inputs(500 + list(DENSE_CASES).index(case), B=B, TQ=TQ, TK=TK, H=H, HKV=HKV, D=D, dtype="bf16")
     A = tiny_args(stages=stages, **kw)
-    if paged:
-        X = to_paged(X, 16, seed=7)
+    if paged:  # page size; the pages of the token slots are looked up a pass of tiles ahead
+        X = to_paged(X, paged, seed=7)
         A.extend_context_length = TK
     octx, ometa = O.hip_attention_12(X, A)
     ctx, meta = run_product(X, A)
