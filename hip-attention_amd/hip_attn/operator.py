@@ -654,11 +654,23 @@ def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], 
             if "is not built" not in str(e) or _decode_seams_overlap(args, BK):
                 raise
     ksrc = k if k is not None else args.k_cache
-    if khat is not None and (ksrc is None or khat.shape != ksrc.shape or khat.stride() != ksrc.stride()
-                             or kvs.cache):
+    if khat is not None and (ksrc is None or khat.shape != ksrc.shape or kvs.cache):
         khat = None
+    if khat is not None and impl != 1:
+        # The pre-scaled copy has its own layout (kv head outermost), so the tile kernel gets a description whose K
+        # side carries the copy's strides.  Only the tile kernel takes pre-scaled keys: where it does not apply, the
+        # call is repeated on the tensors as they are.
+        kvs_hat = type(kvs).from_buffer_copy(kvs)
+        kvs_hat.k_stride_b, kvs_hat.k_stride_t, kvs_hat.k_stride_h = khat.stride(0), khat.stride(1), khat.stride(2)
+        try:
+            N.bsa_prefill(qs, kvs_hat, indices, ks_start_end, BK, args.block_size_q, args.block_size_k,
+                          args.sliding_window_size, args.sink_token_size, decode or rows_shared, 2, out, device,
+                          k_prescaled=khat)
+            return out
+        except N.HipAttnError as e:
+            if "does not cover" not in str(e) or impl == 2:
+                raise
     N.bsa_prefill(qs, kvs, indices, ks_start_end, BK, args.block_size_q, args.block_size_k,
-                  args.sliding_window_size, args.sink_token_size, decode or rows_shared, impl, out, device,
-                  k_prescaled=khat)
+                  args.sliding_window_size, args.sink_token_size, decode or rows_shared, impl, out, device)
     del keep
     return out
