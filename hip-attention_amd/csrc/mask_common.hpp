@@ -51,9 +51,14 @@ __device__ __forceinline__ void store_score(const MaskParamsBase &p, int64_t row
 }
 
 // bf16, prescaled keys, chunks of 2 .. 16 tokens on wide launches: every token of every chunk is scored once per
-// GQA group and the searches are replayed on the scores (mask_stage_dense.hip).  Expects p.qhat filled.  Returns
-// HIPATTN_E_UNSUPPORTED (no error text) when the launch is not one it covers.
-int mask_stage_dense_launch(const MaskParams &p, int HID, int rows_eff, hipStream_t st);
+// GQA group and the searches are replayed on the scores (mask_stage_dense.hip).
+// mask_stage_dense_applies: is this launch one the kernel covers (and, by the default rule, worth it)?
+// mask_stage_dense_launch: expects the scores initialised (reduce_heads) and either p.qhat filled or, with
+// q_inline (stride_q == 1 only: a query row is its own mean), nothing: the kernel then scales the query rows itself.
+bool mask_stage_dense_applies(const MaskParams &p, int HID, int rows_eff);
+int mask_stage_dense_launch(const MaskParams &p, int HID, int rows_eff, bool q_inline, hipStream_t st);
+// -inf into the head-reduced scores of a stage (what the query preparation launch otherwise does on its way)
+void mask_stage_fill_scores(const MaskParams &p, hipStream_t st);
 
 // bf16 path on the matrix cores (mask_stage_mfma.hip)
 int mask_stage_mfma_launch(const MaskParams &p, int HID, int rows_eff, int prescaled, hipStream_t st);

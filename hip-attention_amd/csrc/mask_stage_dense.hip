@@ -37,9 +37,19 @@ constexpr int MD_PASS = 8;             // tiles between two replays of the searc
 
 static __device__ __align__(16) uint16_t md_zero_row[256];
 
+typedef __attribute__((ext_vector_type(2))) __bf16 md_bf16x2;
+typedef __attribute__((ext_vector_type(2))) float md_f32x2;
+// a packed pair of bf16, each times c, rounded to nearest even
+__device__ __forceinline__ uint32_t md_scale_pack(uint32_t w, float c) {
+    md_f32x2 v = {__uint_as_float(w << 16) * c, __uint_as_float(w & 0xffff0000u) * c};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, md_bf16x2));
+}
+
 // HPW = waves (heads) per workgroup; MB = 32-row blocks of query rows per program (1: up to 32 rows, 2: up to 64);
 // PAGED: keys live in a paged cache, the page of every token slot is looked up a pass ahead (below)
-template <int HID, int MB, int HPW, bool EXT, bool PAGED>
+// QINLINE: the programs' query rows are the tensor's own rows (stride_q == 1): scaled here instead of read from the
+// workspace that the query preparation launch would have filled
+template <int HID, int MB, int HPW, bool EXT, bool PAGED, bool QINLINE>
 __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFor<EXT> p, long long total_wg) {
     constexpr int NT = 64 * HPW;
     constexpr int KS = HID / 16;
@@ -113,7 +123,28 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
 
     // ---- Q^ fragments, in the order qhat_kernel stores them (k-step, row half, row)
     MdFrag qf[MB][KS];
-    {
+    if constexpr (QINLINE) {
+        // a row is its own mean: bf16(q * c_q), the k-step's eight elements at hh * HID/2 + ks * 8
+        const uint16_t *qbase = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) {
+            const int j = mb * 32 + n;
+            const bool jv = head_ok && (j < p.nrows) && ((rowmask >> j) & 1ull);
+            const long long it = qb * p.BQ + j;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                uint4 w = make_uint4(0, 0, 0, 0);
+                if (jv) {
+                    w = *reinterpret_cast<const uint4 *>(qbase + it * p.q_st + hh * (HID / 2) + ks * 8);
+                    w.x = md_scale_pack(w.x, p.c_q);
+                    w.y = md_scale_pack(w.y, p.c_q);
+                    w.z = md_scale_pack(w.z, p.c_q);
+                    w.w = md_scale_pack(w.w, p.c_q);
+                }
+                qf[mb][ks].q = w;
+            }
+        }
+    } else {
         const uint16_t *qh = p.qhat + ((((int64_t)b * p.BS + s) * p.HEAD + h) * p.nrows) * HID;
 #pragma unroll
         for (int mb = 0; mb < MB; mb++) {
@@ -337,7 +368,19 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
     }
 }
 
-template <int HID, int MB, int HPW>
+__global__ void md_fill_scores_kernel(float *scores, long long n) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
+        scores[i] = -INFINITY;
+}
+
+void mask_stage_fill_scores(const MaskParams &p, hipStream_t st) {
+    if (!p.reduce_heads) return;
+    const long long nscores = (long long)p.B * p.BS * p.n;
+    const long long blocks = (nscores + 255) / 256;
+    hipLaunchKernelGGL(md_fill_scores_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0, st, p.scores, nscores);
+}
+
+template <int HID, int MB, int HPW, bool QINLINE>
 static int launch_dense(const MaskParams &p, hipStream_t st) {
     const int hblocks = (p.G + HPW - 1) / HPW;
     const long long total = (long long)p.B * p.kv.HKV * p.BS * hblocks;
@@ -345,44 +388,54 @@ static int launch_dense(const MaskParams &p, hipStream_t st) {
     dim3 grid((unsigned)total), block(64 * HPW);
     const MaskParamsBase &pb = p;
     if (p.kx.extended()) {
-        if (p.kv.paged) hipLaunchKernelGGL((mask_stage_dense_kernel<HID, MB, HPW, true, true>), grid, block, 0, st, p, total);
-        else hipLaunchKernelGGL((mask_stage_dense_kernel<HID, MB, HPW, true, false>), grid, block, 0, st, p, total);
+        if (p.kv.paged) hipLaunchKernelGGL((mask_stage_dense_kernel<HID, MB, HPW, true, true, QINLINE>), grid, block, 0, st, p, total);
+        else hipLaunchKernelGGL((mask_stage_dense_kernel<HID, MB, HPW, true, false, QINLINE>), grid, block, 0, st, p, total);
     } else {
-        if (p.kv.paged) hipLaunchKernelGGL((mask_stage_dense_kernel<HID, MB, HPW, false, true>), grid, block, 0, st, pb, total);
-        else hipLaunchKernelGGL((mask_stage_dense_kernel<HID, MB, HPW, false, false>), grid, block, 0, st, pb, total);
+        if (p.kv.paged) hipLaunchKernelGGL((mask_stage_dense_kernel<HID, MB, HPW, false, true, QINLINE>), grid, block, 0, st, pb, total);
+        else hipLaunchKernelGGL((mask_stage_dense_kernel<HID, MB, HPW, false, false, QINLINE>), grid, block, 0, st, pb, total);
     }
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
 }
 
-template <int HID>
+template <int HID, bool QINLINE>
 static int launch_dense_hid(const MaskParams &p, int rows_eff, hipStream_t st) {
     const bool two = rows_eff > 32;
-    if (p.G >= 4) return two ? launch_dense<HID, 2, 4>(p, st) : launch_dense<HID, 1, 4>(p, st);
-    if (p.G >= 2) return two ? launch_dense<HID, 2, 2>(p, st) : launch_dense<HID, 1, 2>(p, st);
-    return HIPATTN_E_UNSUPPORTED;  // one head per group: nothing to share, the sampling kernel reads fewer rows
+    if (p.G >= 4) return two ? launch_dense<HID, 2, 4, QINLINE>(p, st) : launch_dense<HID, 1, 4, QINLINE>(p, st);
+    if (p.G >= 2) return two ? launch_dense<HID, 2, 2, QINLINE>(p, st) : launch_dense<HID, 1, 2, QINLINE>(p, st);
+    return HIPATTN_E_UNSUPPORTED;
 }
 
-int mask_stage_dense_launch(const MaskParams &p, int HID, int rows_eff, hipStream_t st) {
+bool mask_stage_dense_applies(const MaskParams &p, int HID, int rows_eff) {
     // HIPATTN_MASK_DENSE: 0 = never, 1 = where it pays (default), 2 = wherever the kernel applies (testing)
     const char *e = getenv("HIPATTN_MASK_DENSE");  // read on every call: tests switch it inside one process
     const int mode = e ? atoi(e) : 1;
-    if (mode == 0) return HIPATTN_E_UNSUPPORTED;
+    if (mode == 0) return false;
     const int CH = p.chunk;
-    if (CH < 2 || CH > 16 || (CH & (CH - 1)) != 0) return HIPATTN_E_UNSUPPORTED;
-    if (p.hg != 1 || p.rope.cos || p.kx.cached || p.kx.kv8) return HIPATTN_E_UNSUPPORTED;
-    if (p.nrows > 64 || p.n > MD_MAX_CHUNKS) return HIPATTN_E_UNSUPPORTED;
+    if (CH < 2 || CH > 16 || (CH & (CH - 1)) != 0) return false;
+    if (p.hg != 1 || p.rope.cos || p.kx.cached || p.kx.kv8) return false;
+    if (p.nrows > 64 || p.n > MD_MAX_CHUNKS) return false;
+    if (HID != 64 && HID != 128) return false;
+    if (p.G < 2) return false;  // one head per group: nothing to share, the sampling kernel reads fewer rows
     if (mode == 1) {
         // pays when the group's searches together load more rows than the chunks hold, on launches wide enough to
         // keep the chip busy with one workgroup per (batch, kv head, scan row)
         const int iters = 32 - __builtin_clz((unsigned)CH);  // floor(log2(CH)) + 1
         const int per_search = 2 * iters - 3;
         const long long wgs = (long long)p.B * p.kv.HKV * p.BS;
-        if (!(per_search * p.G >= 2 * CH) || wgs < 1024 || p.n < 64) return HIPATTN_E_UNSUPPORTED;
+        if (!(per_search * p.G >= 2 * CH) || wgs < 1024 || p.n < 64) return false;
     }
+    const int hpw = p.G >= 4 ? 4 : 2;
+    const long long total = (long long)p.B * p.kv.HKV * p.BS * ((p.G + hpw - 1) / hpw);
+    (void)rows_eff;
+    return total < 0x7fffffffLL;
+}
+
+int mask_stage_dense_launch(const MaskParams &p, int HID, int rows_eff, bool q_inline, hipStream_t st) {
+    if (q_inline && p.stride_q != 1) return HIPATTN_E_UNSUPPORTED;
     switch (HID) {
-        case 64: return launch_dense_hid<64>(p, rows_eff, st);
-        case 128: return launch_dense_hid<128>(p, rows_eff, st);
+        case 64: return q_inline ? launch_dense_hid<64, true>(p, rows_eff, st) : launch_dense_hid<64, false>(p, rows_eff, st);
+        case 128: return q_inline ? launch_dense_hid<128, true>(p, rows_eff, st) : launch_dense_hid<128, false>(p, rows_eff, st);
     }
     return HIPATTN_E_UNSUPPORTED;
 }

@@ -531,15 +531,21 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
         set_error("mask stage: grid too large");
         return HIPATTN_E_UNSUPPORTED;
     }
-    {
+    // small chunks on wide launches: every token scored once per GQA group, searches replayed on the scores
+    const bool dense = prescaled && !two_sided && mask_stage_dense_applies(p, HID, rows_eff);
+    // with stride_q == 1 a program's query rows are the tensor's own: that kernel scales them itself and the
+    // preparation launch (a pass over all of q) shrinks to the fill of the head-reduced scores
+    const bool q_inline = dense && p.stride_q == 1;
+    if (q_inline) {
+        mask_stage_fill_scores(p, st);
+    } else {
         const long long work = (long long)p.B * p.BS * p.HEAD * p.nrows * (HID / 8);
         const long long blocks = (work + 255) / 256;
         hipLaunchKernelGGL(qhat_kernel, dim3((unsigned)blocks), dim3(256), 0, st, p, HID, const_cast<uint16_t *>(p.qhat));
     }
-    if (prescaled && !two_sided) {
-        // small chunks on wide launches: every token scored once per GQA group, searches replayed on the scores
-        const int rc = mask_stage_dense_launch(p, HID, rows_eff, st);
-        if (rc != HIPATTN_E_UNSUPPORTED) return rc;
+    if (dense) {
+        const int rc = mask_stage_dense_launch(p, HID, rows_eff, q_inline, st);
+        if (rc != HIPATTN_E_UNSUPPORTED || q_inline) return rc;
     }
     dim3 grid((unsigned)p.total), block(64 * hpw);
     const MaskParamsBase &pb = p;  // the plain kernels take the block without the extras
