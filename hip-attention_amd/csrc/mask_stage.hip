@@ -362,7 +362,8 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
     HIPATTN_CHECK_ARG(p.total < 0x7fffffffLL, HIPATTN_E_UNSUPPORTED, "mask stage: grid too large");
     scale_constants(q->HID, q->dtype, &p.c_q, &p.c_k);
     p.scores = scores; p.left_out = left_out;
-    p.reduce_heads = reduce_heads ? 1 : 0;
+    HIPATTN_CHECK_ARG(reduce_heads >= 0 && reduce_heads <= 2, HIPATTN_E_ARG, "mask stage: reduce_heads %d not in {0, 1, 2}", reduce_heads);
+    p.reduce_heads = reduce_heads;  // 2: the scores were set to -inf by the caller
     HIPATTN_CHECK_ARG(!reduce_heads || hg == 1, HIPATTN_E_ARG, "mask stage: reduce_heads needs one shared chunk list (hg == 1)");
     int rows_max = (q->TDST + stride_q - 1) / stride_q;
     int rows_eff = p.nrows < rows_max ? p.nrows : rows_max;
@@ -379,7 +380,7 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
         return mask_stage_mfma_launch(p, q->HID, rows_eff, k_prescaled, st);
     } else if (q->dtype == HIPATTN_F32) {
         HIPATTN_CHECK_ARG(!k_prescaled, HIPATTN_E_ARG, "mask stage: prescaled keys are a bf16-only option");
-        if (p.reduce_heads) {
+        if (p.reduce_heads == 1) {
             const long long nscores = (long long)p.B * p.BS * p.n;
             hipLaunchKernelGGL(fill_scores_kernel, dim3((unsigned)((nscores + 255) / 256 < 4096 ? (nscores + 255) / 256 : 4096)),
                                dim3(256), 0, st, scores, nscores, -INFINITY);

@@ -374,7 +374,7 @@ __global__ void md_fill_scores_kernel(float *scores, long long n) {
 }
 
 void mask_stage_fill_scores(const MaskParams &p, hipStream_t st) {
-    if (!p.reduce_heads) return;
+    if (p.reduce_heads != 1) return;  // 0: plain stores; 2: the caller has initialised them
     const long long nscores = (long long)p.B * p.BS * p.n;
     const long long blocks = (nscores + 255) / 256;
     hipLaunchKernelGGL(md_fill_scores_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0, st, p.scores, nscores);

@@ -64,10 +64,14 @@ __device__ __forceinline__ int64_t rope_kpos(const RopeView &r, int c, int side)
 // sampled token itself (attention_extend.py:254-274) and reloads them with every sample.
 // RMODE = 2 (prescaled keys, extended parameter block): the keys were rotated and scaled ahead of the scan, one
 // copy per sample side; right-hand samples read the copy k_side_delta elements further on.
+// RMODE = 3 (no rotation, one token block per wave, a single query token): the one valid program row is that token's
+// row, which the kernel scales itself; no preparation launch is needed.
 // KV8 = true (extended parameter block, unscaled keys): key rows are fp8 (e5m2) bytes, widened on load.
 template <int HID, int MB, int NB, bool PRESCALED, bool VIA_LDS, bool EXT, int RMODE = 0, bool KV8 = false>
 __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     constexpr bool ROPE = RMODE == 1;
+    constexpr bool QINL = RMODE == 3;  // query rows scaled here instead of read from the prepared workspace
+    static_assert(!QINL || NB == 1, "inline query rows: the one-token-block variants only");
     static_assert(!KV8 || (EXT && !PRESCALED), "fp8 keys: extended build, scaled in the kernel");
     static_assert(!ROPE || (EXT && !VIA_LDS && !PRESCALED), "rope variant: direct path of the extended build");
     static_assert(RMODE != 2 || (EXT && PRESCALED), "two-sided prescaled keys: extended build of the prescaled path");
@@ -125,6 +129,30 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
     // They are fetched when the first chunk group of this wave has work and then serve all of its groups.
     BFrag qf[MB][KS];
     bool q_loaded = false;
+    if constexpr (QINL) {
+        // A single query token: row 0 of the program is that token's row of this head, scaled here; no preparation
+        // launch ran.  Every wave of the launch wants one of a handful of rows, so they are read through the
+        // scalar cache (uniform address, constant address space): as vector loads, thousands of waves queue up on
+        // the same few cache lines (1M-key decode: the 256-token stage 122 us against 116).
+        typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+        typedef const u32x4_t __attribute__((address_space(4))) *cptr_t;
+        const uint64_t qaddr = (uint64_t)(reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh);
+        const uint64_t qaddr_u = ((uint64_t)__builtin_amdgcn_readfirstlane((int)(qaddr >> 32)) << 32) |
+                                 (uint32_t)__builtin_amdgcn_readfirstlane((int)(qaddr & 0xffffffffu));
+        cptr_t qs = (cptr_t)qaddr_u;
+        const bool mine = (n == 0) && (rowmask & 1ull);
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                const u32x4_t lo = qs[ks], hi = qs[KS + ks];  // the k-step's pieces of the two halves of the row
+                uint32_t w[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) w[e] = (mb == 0 && mine) ? scale_pack(hh ? hi[e] : lo[e], p.c_q) : 0u;
+                qf[mb][ks].q = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+        q_loaded = true;
+    }
     // which of this lane's accumulator elements belong to valid query rows:
     // element (mb, i) <-> row mb*32 + (i/4)*8 + hh*4 + i%4
     unsigned vm[MB];
@@ -207,15 +235,17 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
 
     if (!q_loaded) {
         q_loaded = true;
-        const uint16_t *qh = p.qhat + ((((int64_t)b * p.BS + s) * p.HEAD + h) * p.nrows) * HID;
+        if constexpr (!QINL) {
+            const uint16_t *qh = p.qhat + ((((int64_t)b * p.BS + s) * p.HEAD + h) * p.nrows) * HID;
 #pragma unroll
-        for (int mb = 0; mb < MB; mb++) {
-            const int j = mb * 32 + n;
-            const bool jv = (j < p.nrows) && ((rowmask >> j) & 1ull);
+            for (int mb = 0; mb < MB; mb++) {
+                const int j = mb * 32 + n;
+                const bool jv = (j < p.nrows) && ((rowmask >> j) & 1ull);
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) {
-                qf[mb][ks].q = make_uint4(0, 0, 0, 0);
-                if (jv) qf[mb][ks].q = *reinterpret_cast<const uint4 *>(qh + ((int64_t)(ks * 2 + hh) * p.nrows + j) * 8);
+                for (int ks = 0; ks < KS; ks++) {
+                    qf[mb][ks].q = make_uint4(0, 0, 0, 0);
+                    if (jv) qf[mb][ks].q = *reinterpret_cast<const uint4 *>(qh + ((int64_t)(ks * 2 + hh) * p.nrows + j) * 8);
+                }
             }
         }
     }
@@ -402,7 +432,7 @@ __global__ void qhat_kernel(MaskParams p, int hid, uint16_t *out) {
     const int per_row = hid / 8;
     const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     const long long total = (long long)p.B * p.BS * p.HEAD * p.nrows * per_row;
-    if (p.reduce_heads) {
+    if (p.reduce_heads == 1) {
         // the scan folds the maximum over heads into scores [B, BS, 1, n]: start it at -inf here, in the launch that
         // precedes the scan on the stream anyway
         const long long nscores = (long long)p.B * p.BS * p.n;
@@ -533,9 +563,11 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
     }
     // small chunks on wide launches: every token scored once per GQA group, searches replayed on the scores
     const bool dense = prescaled && !two_sided && mask_stage_dense_applies(p, HID, rows_eff);
-    // with stride_q == 1 a program's query rows are the tensor's own: that kernel scales them itself and the
-    // preparation launch (a pass over all of q) shrinks to the fill of the head-reduced scores
-    const bool q_inline = dense && p.stride_q == 1;
+    // Where every program row is the mean of exactly one query row and is not rotated (the dense kernel with
+    // stride_q == 1; the narrow sampling kernels with a single query token), the kernels scale the rows themselves: the preparation launch
+    // (a pass over all of q) shrinks to the fill of the head-reduced scores, and to nothing when the caller has
+    // initialised those (reduce_heads == 2).
+    const bool q_inline = !rope && !two_sided && ((dense && p.stride_q == 1) || (!dense && p.TDST == 1 && nb == 1 && !p.kx.kv8));
     if (q_inline) {
         mask_stage_fill_scores(p, st);
     } else {
@@ -580,6 +612,23 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
     if (p.kx.kv8 && prescaled) {
         set_error("mask stage: prescaled keys cannot be combined with fp8 key storage");
         return HIPATTN_E_ARG;
+    }
+    if (q_inline) {  // narrow launch, one token block per wave, query rows scaled in the kernel
+#define MS_INLINE(MBv, PSv, VLv)                                                                                       \
+    do {                                                                                                              \
+        if (ext) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, 1, PSv, VLv, true, 3>), grid, block, 0, st, p, nsub, hpw); \
+        else hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, MBv, 1, PSv, VLv, false, 3>), grid, block, 0, st, pb, nsub, hpw);   \
+    } while (0)
+#define MS_INLINE_PICK(MBv)                                                                          \
+    do {                                                                                             \
+        if (prescaled) { if (via_lds) MS_INLINE(MBv, true, true); else MS_INLINE(MBv, true, false); } \
+        else { if (via_lds) MS_INLINE(MBv, false, true); else MS_INLINE(MBv, false, false); }         \
+    } while (0)
+        if (two) MS_INLINE_PICK(2); else MS_INLINE_PICK(1);
+#undef MS_INLINE_PICK
+#undef MS_INLINE
+        HIPATTN_CHECK_HIP(hipGetLastError());
+        return 0;
     }
     if (rope && p.kx.kv8) {
         if (two) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 2, 1, false, false, true, 1, true>), grid, block, 0, st, p, nsub, hpw);

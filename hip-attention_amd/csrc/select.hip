@@ -149,7 +149,7 @@ __global__ __launch_bounds__(SEL_THREADS) void select_stage_kernel(const float *
                                                                   int bs_in, int bs_out, int row_rep, int HEAD, int hg,
                                                                   int n, int k, int sub_chunk, int splits,
                                                                   int32_t *next_left, int64_t *left64,
-                                                                  int64_t *right64) {
+                                                                  int64_t *right64, float *next_scores) {
     __shared__ uint32_t s_keys[SEL_MAX_N];
     __shared__ int s_hist[256];
     __shared__ int s_misc[2];
@@ -200,6 +200,7 @@ __global__ __launch_bounds__(SEL_THREADS) void select_stage_kernel(const float *
         const int e = idx / splits, j = idx - e * splits;
         const int left = lrow[s_sel[e]] + j * sub_chunk;
         next_left[obase + idx] = left;
+        if (next_scores) next_scores[obase + idx] = -INFINITY;  // the next stage's head-reduced scores start here
         if (left64) {  // the same list as the next stage's cached inputs: int64 edges (left, left + chunk)
             left64[obase + idx] = left;
             right64[obase + idx] = (int64_t)left + sub_chunk;
@@ -219,7 +220,7 @@ __global__ __launch_bounds__(FAST_THREADS) void select_stage_fast_kernel(const f
                                                                         int bs_in, int bs_out, int row_rep, int HEAD,
                                                                         int hg, int n, int k, int sub_chunk, int splits,
                                                                         int32_t *next_left, int64_t *left64,
-                                                                        int64_t *right64) {
+                                                                        int64_t *right64, float *next_scores) {
     __shared__ int s_hist[256];
     __shared__ int s_misc[2];
     __shared__ uint32_t s_wave[FAST_THREADS / 64];
@@ -344,6 +345,7 @@ __global__ __launch_bounds__(FAST_THREADS) void select_stage_fast_kernel(const f
                 const int v = left[i] + j * sub_chunk;
                 const int64_t at = obase + (int64_t)e * splits + j;
                 next_left[at] = v;
+                if (next_scores) next_scores[at] = -INFINITY;
                 if (left64) {
                     left64[at] = v;
                     right64[at] = (int64_t)v + sub_chunk;
@@ -459,13 +461,14 @@ using namespace hipattn;
 extern "C" int hipattn_select_stage(const float *scores, const int32_t *chunk_left, int32_t B, int32_t bs_in,
                                     int32_t bs_out, int32_t row_rep, int32_t HEAD, int32_t hg, int32_t n,
                                     int32_t k, int32_t chunk_size, int32_t splits, int32_t *next_left,
-                                    int64_t *next_left64, int64_t *next_right64, void *stream) {
+                                    int64_t *next_left64, int64_t *next_right64, float *next_scores, void *stream) {
     HIPATTN_CHECK_ARG(scores && chunk_left && next_left, HIPATTN_E_ARG, "select stage: null pointer");
     HIPATTN_CHECK_ARG((next_left64 == nullptr) == (next_right64 == nullptr), HIPATTN_E_ARG,
                       "select stage: give both 64-bit outputs or neither");
     HIPATTN_CHECK_ARG(B > 0 && bs_in > 0 && bs_out > 0 && row_rep > 0 && HEAD > 0 && n > 0 && k > 0 && splits > 0,
                       HIPATTN_E_ARG, "select stage: non-positive size");
     HIPATTN_CHECK_ARG(hg == 1 || hg == HEAD, HIPATTN_E_ARG, "select stage: hg must be 1 or HEAD");
+    HIPATTN_CHECK_ARG(!next_scores || hg == 1, HIPATTN_E_ARG, "select stage: next_scores needs one shared chunk list (hg == 1)");
     HIPATTN_CHECK_ARG(k <= n, HIPATTN_E_ARG, "select stage: k %d > n %d", k, n);
     HIPATTN_CHECK_ARG(chunk_size % splits == 0, HIPATTN_E_ARG, "select stage: chunk %d %% splits %d", chunk_size, splits);
     HIPATTN_CHECK_ARG(bs_out <= row_rep * bs_in, HIPATTN_E_ARG, "select stage: bs_out > row_rep*bs_in");
@@ -481,7 +484,7 @@ extern "C" int hipattn_select_stage(const float *scores, const int32_t *chunk_le
 #define SEL_FAST(IT)                                                                                                  \
     hipLaunchKernelGGL(select_stage_fast_kernel<IT>, grid, fblock, 0, (hipStream_t)stream, scores, chunk_left, bs_in, \
                        bs_out, row_rep, HEAD, hg, n, k, chunk_size / splits, splits, next_left, next_left64,          \
-                       next_right64)
+                       next_right64, next_scores)
         if (n <= FAST_THREADS) SEL_FAST(1);
         else if (n <= 4 * FAST_THREADS) SEL_FAST(4);
         else SEL_FAST(16);
@@ -490,7 +493,8 @@ extern "C" int hipattn_select_stage(const float *scores, const int32_t *chunk_le
         return 0;
     }
     hipLaunchKernelGGL(select_stage_kernel, grid, block, 0, (hipStream_t)stream, scores, chunk_left, bs_in, bs_out,
-                       row_rep, HEAD, hg, n, k, chunk_size / splits, splits, next_left, next_left64, next_right64);
+                       row_rep, HEAD, hg, n, k, chunk_size / splits, splits, next_left, next_left64, next_right64,
+                       next_scores);
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
 }

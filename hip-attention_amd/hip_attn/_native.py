@@ -338,12 +338,14 @@ def mask_stage(qs, kvs, chunk_left, hg, n, chunk, right_clamp, bs, bq, stride_q,
 
 
 def select_stage(scores, chunk_left, B, bs_in, bs_out, row_rep, HEAD, hg, n, k, chunk, splits, next_left, device,
-                 left64=None, right64=None):
+                 left64=None, right64=None, next_scores=None):
+    """``next_scores``: the next stage's head-reduced scores (shape of ``next_left`` with ``hg == 1``), set to -inf here
+    so that ``mask_stage(..., reduce_heads=2)`` finds them initialised."""
     with _timed("select_stage"):
       rc = lib().hipattn_select_stage(
         _p(scores), _p(chunk_left), ctypes.c_int32(B), ctypes.c_int32(bs_in), ctypes.c_int32(bs_out),
         ctypes.c_int32(row_rep), ctypes.c_int32(HEAD), ctypes.c_int32(hg), ctypes.c_int32(n), ctypes.c_int32(k),
-        ctypes.c_int32(chunk), ctypes.c_int32(splits), _p(next_left), _p(left64), _p(right64),
+        ctypes.c_int32(chunk), ctypes.c_int32(splits), _p(next_left), _p(left64), _p(right64), _p(next_scores),
         stream_ptr(device))
     check(rc, "hipattn_select_stage")
 

@@ -399,6 +399,7 @@ def dual_stage_quadratic_hip_attention(
         left64 = right64 = None
         n_cached = len(stage_caches) if stage_caches is not None else 0
         for i_stage, stage in enumerate(stages):
+            prefilled_scores = None
             if i_stage < n_cached - 1:
                 continue
             elif i_stage == n_cached - 1:
@@ -449,8 +450,13 @@ def dual_stage_quadratic_hip_attention(
                         # the list is also handed out as this stage's cached inputs: written once, in both widths
                         left64 = torch.empty(next_left.shape, dtype=torch.int64, device=device)
                         right64 = torch.empty(next_left.shape, dtype=torch.int64, device=device)
+                    if hg == 1 and isinstance(stage, ScanStage):
+                        # the head-reduced scores of the stage that follows have the shape of its chunk list: the
+                        # selection pass starts them at -inf, which saves the scan a launch of its own for that
+                        prefilled_scores = torch.empty(next_left.shape, dtype=torch.float32, device=device)
                     N.select_stage(scores, chunk_left, BSZ, bs_in, bs_out, row_rep, scores.shape[2], hg, prev_n, keep,
-                                   chunk_size, splits, next_left, device, left64=left64, right64=right64)
+                                   chunk_size, splits, next_left, device, left64=left64, right64=right64,
+                                   next_scores=prefilled_scores)
                 chunk_left = next_left
                 right_clamp = _BIG
             else:
@@ -475,7 +481,10 @@ def dual_stage_quadratic_hip_attention(
             if isinstance(stage, ScanStage):
                 # one shared chunk list: the scan kernels fold the maximum over heads into their score store
                 reduce = hg == 1
-                if reduce:
+                if reduce and prefilled_scores is not None:
+                    assert prefilled_scores.shape == (BSZ, bs, 1, chunk_count)
+                    scores, reduce = prefilled_scores, 2  # already at -inf
+                elif reduce:
                     scores = torch.empty((BSZ, bs, 1, chunk_count), dtype=torch.float32, device=device)  # mask_stage fills it
                 else:
                     scores = torch.empty((BSZ, bs, HEAD, chunk_count), dtype=torch.float32, device=device)

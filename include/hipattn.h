@@ -140,8 +140,10 @@ const char *hipattn_last_error(void);
  *                                      scores are max-reduced over heads, else HEAD
  *   right = min(left + chunk_size, right_clamp)
  *   scores      f32   [B, BS, HEAD, n] written for every chunk (-32000 where not scored); with
- *                     reduce_heads != 0 (needs hg == 1): [B, BS, 1, n], set to -inf by the entry point and then
- *                     raised to the maximum over heads (the torch.max at :2566-2570 folded into the scan)
+ *                     reduce_heads != 0 (needs hg == 1): [B, BS, 1, n], set to -inf by the entry point
+ *                     (reduce_heads = 1) or already by the caller, e.g. through hipattn_select_stage's next_scores
+ *                     (reduce_heads = 2), and then raised to the maximum over heads (the torch.max at :2566-2570
+ *                     folded into the scan)
  *   left_out    int32 [B, BS, HEAD, n] refined left edge per head, or NULL
  *   block_chunk = chunks per reference program (16/32/64): fixes the program-level gate and
  *   iteration count (:595-601,736-737).
@@ -185,11 +187,14 @@ int hipattn_prescale_k_rope(const void *k, int64_t stride0, int64_t stride1, int
  *   (repeat_interleave(row_rep, 1)[:, -BS_out:], :2092-2123).
  *   next_left64 / next_right64: NULL, or int64 buffers of next_left's shape that receive the same list as
  *   (left, left + chunk_size/splits), the layout of HiPAttentionStageInputCache.indices_left / indices_right
- *   (src/hip_attn/v1_2/attention_metadata.py:111-115). */
+ *   (src/hip_attn/v1_2/attention_metadata.py:111-115).
+ *   next_scores: NULL, or (hg == 1 only) the next stage's head-reduced scores, f32 [B, BS_out, 1, k*splits]: every
+ *   entry is set to -inf, so that the next hipattn_mask_stage can be called with reduce_heads = 2 and needs no
+ *   launch of its own to initialise them. */
 int hipattn_select_stage(const float *scores, const int32_t *chunk_left, int32_t B, int32_t bs_in,
                          int32_t bs_out, int32_t row_rep, int32_t HEAD, int32_t hg, int32_t n,
                          int32_t k, int32_t chunk_size, int32_t splits, int32_t *next_left,
-                         int64_t *next_left64, int64_t *next_right64, void *stream);
+                         int64_t *next_left64, int64_t *next_right64, float *next_scores, void *stream);
 
 /* After the last stage: top-K chunks, block alignment, de-duplication, active count, in the
  * reference's metadata layout.  Replaces src/hip_attn/v1_2/attention_extend.py:2757-2776 and
