@@ -340,10 +340,11 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
                                (1u << HIPATTN_EXTEND_DYNAMIC),
                         "mask stage", &p.rope);
     if (rc) return rc;
-    HIPATTN_CHECK_ARG(!(p.rope.cos && k_prescaled) || p.rope.backend == HIPATTN_EXTEND_RELATIVE ||
+    HIPATTN_CHECK_ARG(k_prescaled >= 0 && k_prescaled <= 3, HIPATTN_E_ARG, "mask stage: k_prescaled %d not in 0..3", k_prescaled);
+    HIPATTN_CHECK_ARG(!(p.rope.cos && (k_prescaled & 1)) || p.rope.backend == HIPATTN_EXTEND_RELATIVE ||
                           p.rope.backend == HIPATTN_EXTEND_INFLLM,
                       HIPATTN_E_ARG, "mask stage: prescaled keys need a rule with fixed key positions (relative, infllm)");
-    if (p.rope.backend != HIPATTN_EXTEND_RELATIVE || !k_prescaled) p.rope.k_side_delta = 0;
+    if (p.rope.backend != HIPATTN_EXTEND_RELATIVE || !(k_prescaled & 1)) p.rope.k_side_delta = 0;
     HIPATTN_CHECK_ARG(p.rope.k_side_delta % 8 == 0, HIPATTN_E_ALIGN, "mask stage: k_side_delta must keep 16-byte alignment");
     HIPATTN_CHECK_ARG(q->HEAD % p.kv.HKV == 0, HIPATTN_E_ARG, "mask stage: HEAD %% HKV != 0");
     p.q = q->ptr; p.q_sb = q->stride_b; p.q_st = q->stride_t; p.q_sh = q->stride_h;
@@ -377,9 +378,9 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
         HIPATTN_CHECK_ARG(workspace && aligned16(workspace), HIPATTN_E_ARG,
                           "mask stage: bf16 inputs need a 16-byte aligned workspace (hipattn_mask_stage_workspace_bytes)");
         p.qhat = reinterpret_cast<const uint16_t *>(workspace);
-        return mask_stage_mfma_launch(p, q->HID, rows_eff, k_prescaled, st);
+        return mask_stage_mfma_launch(p, q->HID, rows_eff, k_prescaled, st);  // bit 0: keys, bit 1: query rows ready
     } else if (q->dtype == HIPATTN_F32) {
-        HIPATTN_CHECK_ARG(!k_prescaled, HIPATTN_E_ARG, "mask stage: prescaled keys are a bf16-only option");
+        HIPATTN_CHECK_ARG(!(k_prescaled & 1), HIPATTN_E_ARG, "mask stage: prescaled keys are a bf16-only option");
         if (p.reduce_heads == 1) {
             const long long nscores = (long long)p.B * p.BS * p.n;
             hipLaunchKernelGGL(fill_scores_kernel, dim3((unsigned)((nscores + 255) / 256 < 4096 ? (nscores + 255) / 256 : 4096)),

@@ -503,7 +503,9 @@ __global__ void qhat_kernel(MaskParams p, int hid, uint16_t *out) {
 static int g_mask_via_lds = -1;  // -1: decide per shape; 0 / 1: forced through HIPATTN_MASK_VIA_LDS (tuning aid)
 
 template <int HID>
-static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hipStream_t st) {
+static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStream_t st) {
+    const int prescaled = flags & 1;          // keys scaled (and rotated) ahead of the scan
+    const bool q_ready = (flags & 2) != 0;    // the workspace holds this stage's query rows already
     MaskParams p = p0;
     const int BC = p.block_chunk;
     const bool two = rows_eff > 32;
@@ -568,7 +570,7 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int prescaled, hi
     // (a pass over all of q) shrinks to the fill of the head-reduced scores, and to nothing when the caller has
     // initialised those (reduce_heads == 2).
     const bool q_inline = !rope && !two_sided && ((dense && p.stride_q == 1) || (!dense && p.TDST == 1 && nb == 1 && !p.kx.kv8));
-    if (q_inline) {
+    if (q_inline || q_ready) {
         mask_stage_fill_scores(p, st);
     } else {
         const long long work = (long long)p.B * p.BS * p.HEAD * p.nrows * (HID / 8);

@@ -320,21 +320,26 @@ def prescale_k_rope(k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, posit
 
 
 def mask_stage(qs, kvs, chunk_left, hg, n, chunk, right_clamp, bs, bq, stride_q, block_chunk, scan_stride,
-               sw_eff, terminate, scores, left_out, device, k_prescaled=False, reduce_heads=False):
-    need = lib().hipattn_mask_stage_workspace_bytes(
-        ctypes.c_int32(qs.dtype), ctypes.c_int32(qs.B), ctypes.c_int32(bs), ctypes.c_int32(qs.HEAD),
-        ctypes.c_int32(qs.HID), ctypes.c_int32(bq), ctypes.c_int32(stride_q))
-    workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=scores.device) if need > 0 else None
+               sw_eff, terminate, scores, left_out, device, k_prescaled=False, reduce_heads=False, workspace=None):
+    """``workspace``: the tensor an earlier call with the same query rows (same q, bs, bq, stride_q, scan_stride, no
+    rotation) returned; the rows it holds are used as they are.  Returns the workspace (None for f32)."""
+    q_ready = workspace is not None
+    if workspace is None:
+        need = lib().hipattn_mask_stage_workspace_bytes(
+            ctypes.c_int32(qs.dtype), ctypes.c_int32(qs.B), ctypes.c_int32(bs), ctypes.c_int32(qs.HEAD),
+            ctypes.c_int32(qs.HID), ctypes.c_int32(bq), ctypes.c_int32(stride_q))
+        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=scores.device) if need > 0 else None
     with _timed(f"mask_stage[n={n},chunk={chunk},rows={bq // stride_q}]"):
       rc = lib().hipattn_mask_stage(
         ctypes.byref(qs), ctypes.byref(kvs), _p(chunk_left), ctypes.c_int32(hg), ctypes.c_int32(n),
         ctypes.c_int32(chunk), ctypes.c_int64(right_clamp), ctypes.c_int32(bs), ctypes.c_int32(bq),
         ctypes.c_int32(stride_q), ctypes.c_int32(block_chunk), ctypes.c_int32(scan_stride),
-        ctypes.c_int32(sw_eff), ctypes.c_int32(terminate), ctypes.c_int32(int(k_prescaled)),
+        ctypes.c_int32(sw_eff), ctypes.c_int32(terminate), ctypes.c_int32(int(bool(k_prescaled)) | (2 if q_ready else 0)),
         ctypes.c_int32(int(reduce_heads)), _p(workspace),
         _p(scores),
         _p(left_out), stream_ptr(device))
     check(rc, "hipattn_mask_stage")
+    return workspace
 
 
 def select_stage(scores, chunk_left, B, bs_in, bs_out, row_rep, HEAD, hg, n, k, chunk, splits, next_left, device,

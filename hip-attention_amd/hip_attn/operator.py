@@ -398,6 +398,7 @@ def dual_stage_quadratic_hip_attention(
         prev_n = None
         left64 = right64 = None
         n_cached = len(stage_caches) if stage_caches is not None else 0
+        query_rows = {}
         for i_stage, stage in enumerate(stages):
             prefilled_scores = None
             if i_stage < n_cached - 1:
@@ -497,10 +498,17 @@ def dual_stage_quadratic_hip_attention(
                         use_pre = use_pre and backend in ("relative", "infllm")  # key positions fixed per sample side
                         rope = N.make_rope(*rope_tabs, backend, k_side_delta if use_pre else 0, args.model_context_length)
                     qs = N.make_q(qq, position_ids, rope)
-                    N.mask_stage(qs, mask_kv_pre if use_pre else mask_kv, chunk_left, hg, chunk_count, chunk_size,
-                                 right_clamp, bs, BLOCK_SIZE_Q, stage.stage_block_stride_q, BLOCK_CHUNK, STAGE_STRIDE,
-                                 sw_eff, args.stage_early_terminate, scores, left_out, device, k_prescaled=use_pre,
-                                 reduce_heads=reduce)
+                    # Stages that differ only in their chunks share their averaged, scaled query rows.  Only where a
+                    # row is a mean of several query rows: otherwise a kernel may scale its rows itself and leave the
+                    # workspace unwritten.
+                    shared = rope is None and stage.stage_block_stride_q > 1 and TDST > 1
+                    ws_key = (bs, BLOCK_SIZE_Q, stage.stage_block_stride_q, STAGE_STRIDE) if shared else None
+                    ws = N.mask_stage(qs, mask_kv_pre if use_pre else mask_kv, chunk_left, hg, chunk_count, chunk_size,
+                                      right_clamp, bs, BLOCK_SIZE_Q, stage.stage_block_stride_q, BLOCK_CHUNK, STAGE_STRIDE,
+                                      sw_eff, args.stage_early_terminate, scores, left_out, device, k_prescaled=use_pre,
+                                      reduce_heads=reduce, workspace=query_rows.get(ws_key))
+                    if ws_key is not None and ws is not None:
+                        query_rows[ws_key] = ws
             elif isinstance(stage, NopStage):
                 scores = torch.full((BSZ, bs, 1 if hg == 1 else HEAD, chunk_count), -32000.0, dtype=torch.float32,
                                     device=device)
