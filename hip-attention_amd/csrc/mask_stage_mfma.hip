@@ -64,6 +64,11 @@ __device__ __forceinline__ int64_t rope_kpos(const RopeView &r, int c, int side)
 // sampled token itself (attention_extend.py:254-274) and reloads them with every sample.
 // RMODE = 2 (prescaled keys, extended parameter block): the keys were rotated and scaled ahead of the scan, one
 // copy per sample side; right-hand samples read the copy k_side_delta elements further on.
+// RMODE = 4 (prescaled keys, one token block per wave, wide launches): the 32 sampled rows of an iteration are fetched
+// with eight direct-to-LDS load instructions in which sixteen consecutive lanes cover one 256-byte row (a lane reading
+// its own half row makes every load instruction touch 64 cache lines, and the address unit then passes one line per
+// clock: 9.5 TB/s over the chip on L2-resident rows where the coalesced shape reaches 30), into an 8 KB tile of the
+// wave with the 16-byte pieces of row r permuted by r, and read back in operand layout.
 // RMODE = 3 (no rotation, one token block per wave, a single query token): the one valid program row is that token's
 // row, which the kernel scales itself; no preparation launch is needed.
 // KV8 = true (extended parameter block, unscaled keys): key rows are fp8 (e5m2) bytes, widened on load.
@@ -72,6 +77,8 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
     constexpr bool ROPE = RMODE == 1;
     constexpr bool QINL = RMODE == 3;  // query rows scaled here instead of read from the prepared workspace
     static_assert(!QINL || NB == 1, "inline query rows: the one-token-block variants only");
+    constexpr bool DMA = RMODE == 4;   // rows fetched coalesced, straight into a per-wave LDS tile
+    static_assert(!DMA || (PRESCALED && !VIA_LDS && NB == 1), "coalesced direct-to-LDS rows: prescaled keys, one token block per wave");
     static_assert(!KV8 || (EXT && !PRESCALED), "fp8 keys: extended build, scaled in the kernel");
     static_assert(!ROPE || (EXT && !VIA_LDS && !PRESCALED), "rope variant: direct path of the extended build");
     static_assert(RMODE != 2 || (EXT && PRESCALED), "two-sided prescaled keys: extended build of the prescaled path");
@@ -84,7 +91,7 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
     constexpr int NROWS = NB * 32;                // sampled rows per iteration of this wave
     constexpr int SWZ = (PPR < 16 ? PPR : 16) - 1;
     constexpr int SWZ_DIV = PPR < 16 ? 16 / PPR : 1;
-    __shared__ __align__(16) uint4 s_rows[VIA_LDS ? NROWS * PPR : 1];
+    __shared__ __align__(16) uint4 s_rows[VIA_LDS ? NROWS * PPR : DMA ? 4 * 32 * PPR : 1];  // DMA: one tile per wave (up to four)
     __shared__ int64_t s_off[VIA_LDS ? NROWS : 1];
     // a workgroup holds `hpw` waves = `hpw` query heads of one GQA group working on the same chunks:
     // their early-iteration samples coincide, so they share cache lines in the CU's L1
@@ -101,7 +108,7 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
     L /= nsub;
     const int s = (int)(L % p.BS);
     L /= p.BS;
-    const int group_reps = MB == 2 ? p.group_reps : 1;
+    const int group_reps = (MB == 2 || RMODE == 4) ? p.group_reps : 1;
     const int groups_outer = (p.ngroups + group_reps - 1) / group_reps;
     const int g0 = (int)(L % groups_outer) * group_reps;
     L /= groups_outer;
@@ -176,7 +183,7 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
     // ---- a wave walks p.group_reps consecutive chunk groups of its (scan row, head) with the same Q^ fragments
     // (only the 64-row variant: with 16 or 32 rows the fragments are a tenth of the traffic, and the loop costs the
     // registers of a third wave per SIMD)
-    const int reps = MB == 2 ? p.group_reps : 1;
+    const int reps = (MB == 2 || DMA) ? p.group_reps : 1;
     for (int rep = 0; rep < reps; rep++) {
     const int g = g0 + rep;
     if (g >= p.ngroups) break;
@@ -283,7 +290,8 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
         bool active[NB], reuse[NB], fresh[NB];
         int ctr[NB], tok[NB];
         float rscore[NB];
-        uint4 raw[VIA_LDS ? 1 : NB][VIA_LDS ? 1 : KS];
+        uint4 raw[(VIA_LDS || DMA) ? 1 : NB][(VIA_LDS || DMA) ? 1 : KS];
+        int64_t offs[NB];
 #pragma unroll
         for (int tb = 0; tb < NB; tb++) {
             active[tb] = real[tb] && (cl[tb] < cr[tb]) && (cl[tb] <= lim) && (cl[tb] >= 0);
@@ -317,14 +325,35 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
                     }
                 }
             }
+            offs[tb] = off;
             if constexpr (VIA_LDS) {
                 if (hh == 0) s_off[tb * 32 + n] = off;
-            } else {
+            } else if constexpr (!DMA) {
 #pragma unroll
                 for (int ks = 0; ks < KS; ks++) {
                     raw[tb][ks] = make_uint4(0, 0, 0, 0);
                     if (off != NO_ROW) raw[tb][ks] = load_kv_piece<KV8>(p.kv.k, off + hh * HALF + ks * 8);
                 }
+            }
+        }
+        uint4 *my_tile = &s_rows[DMA ? (threadIdx.x >> 6) * 32 * PPR : 0];
+        if constexpr (DMA) {
+            if (fresh[0]) {
+                // instruction i fetches rows 4i .. 4i+3: lane l takes slot l % 16 of row 4i + l / 16, which holds the
+                // row's piece (l % 16) ^ (row % 16); the row's offset is held by the lane of that row.  Rows that are
+                // not sampled afresh are left as they are: a lane only ever looks at the column of its own row.
+                // (offsets are multiples of eight elements: they travel between lanes as 32-bit piece numbers)
+                const int my_piece0 = offs[0] == NO_ROW ? -1 : (int)(offs[0] >> 3);
+#pragma unroll
+                for (int i = 0; i < 32 * PPR / 64; i++) {
+                    const int r = i * (64 / PPR) + lane / PPR;
+                    const int o = __shfl(my_piece0, r);
+                    if (o >= 0) {
+                        const int q = (lane % PPR) ^ (r & (PPR - 1));
+                        load_to_lds16(reinterpret_cast<const uint4 *>(p.kv.k) + ((int64_t)o + q), my_tile + i * 64);
+                    }
+                }
+                wait_vmcnt<0>();
             }
         }
         bool any_fresh = false;  // uniform over the wave, and the LDS path's workgroups are one wave
@@ -366,6 +395,8 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
                 BFrag kf;
                 if constexpr (VIA_LDS) {
                     kf.q = s_rows[r * PPR + ((hh * (PPR / 2) + ks) ^ sw)];
+                } else if constexpr (DMA) {
+                    kf.q = my_tile[n * PPR + ((hh * (PPR / 2) + ks) ^ (n & (PPR - 1)))];
                 } else if constexpr (PRESCALED) {
                     kf.q = raw[tb][ks];
                 } else if constexpr (ROPE) {
@@ -517,7 +548,12 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
         const char *e = getenv("HIPATTN_MASK_NB");
         env_nb = e ? atoi(e) : 0;
     }
-    const int nb0 = (env_nb == 2 && BC >= 32) ? 2 : (env_nb == 1 ? 1 : (wide ? 2 : 1));
+    // HIPATTN_MASK_DMA: wide launches on prescaled keys fetch their rows coalesced, straight into LDS (default);
+    // 0 = each lane loads its own half row, as the other launches do (read on every call: tests switch it)
+    const char *e_dma = getenv("HIPATTN_MASK_DMA");
+    const bool dma = (e_dma ? atoi(e_dma) : 1) != 0 && wide && prescaled && p.rope.cos == nullptr && !p.kx.kv8 &&
+                     !p.kx.cached && HID <= 128 && env_nb != 2;
+    const int nb0 = dma ? 1 : (env_nb == 2 && BC >= 32) ? 2 : (env_nb == 1 ? 1 : (wide ? 2 : 1));
     // LDS path: one wave per workgroup (it uses workgroup barriers); direct path: up to 4 heads per workgroup
     // (measured: sharing pays with one query-row block per program, not with two)
     if (g_mask_via_lds < 0) {
@@ -536,7 +572,7 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
     // through L1, and direct loads win (decode at 1M keys: 31 / 22 us against 38 / 28 us for the 32- and 8-token
     // stages); wide chunks scatter the samples of a search, and rows fetched coalesced through LDS win (124 against
     // 182 us for the 256-token stage)
-    bool via_lds = g_mask_via_lds == 2 ? (!wide && p.chunk > 32) : (g_mask_via_lds == 1);
+    bool via_lds = dma ? false : g_mask_via_lds == 2 ? (!wide && p.chunk > 32) : (g_mask_via_lds == 1);
     if (((p.kx.extended() || two_sided) && nb == 2) || rope) via_lds = false;
     const bool ext = rope || two_sided || p.kx.extended() || (wide && !two && !via_lds);
     static int env_hpw2 = -1;
@@ -555,7 +591,7 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
         const char *e = getenv("HIPATTN_MASK_GROUP_REPS");
         env_reps = e ? atoi(e) : 0;
     }
-    p.group_reps = !two ? 1 : env_reps > 0 ? env_reps : (wide ? 8 : 1);
+    p.group_reps = (!two && !dma) ? 1 : env_reps > 0 ? env_reps : (wide ? (dma && !two ? 16 : 8) : 1);
     if (p.group_reps > p.ngroups) p.group_reps = p.ngroups;
     const int groups_outer = (p.ngroups + p.group_reps - 1) / p.group_reps;
     p.total = (long long)p.B * p.kv.HKV * hblocks * p.BS * groups_outer * nsub;
@@ -614,6 +650,14 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
     if (p.kx.kv8 && prescaled) {
         set_error("mask stage: prescaled keys cannot be combined with fp8 key storage");
         return HIPATTN_E_ARG;
+    }
+    if (dma && !q_inline) {
+        if constexpr (HID <= 128) {
+            if (two) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 2, 1, true, false, true, 4>), grid, block, 0, st, p, nsub, hpw);
+            else hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 4>), grid, block, 0, st, p, nsub, hpw);
+            HIPATTN_CHECK_HIP(hipGetLastError());
+            return 0;
+        }
     }
     if (q_inline) {  // narrow launch, one token block per wave, query rows scaled in the kernel
 #define MS_INLINE(MBv, PSv, VLv)                                                                                       \
