@@ -30,9 +30,9 @@ union MdFrag {
 };
 
 constexpr int MD_TN = 64;              // tokens per tile
-constexpr int MD_DIST = 2;             // tiles whose loads are issued ahead of the tile being consumed
+constexpr int MD_DIST = 3;             // tiles whose loads are issued ahead of the tile being consumed
 constexpr int MD_NBUF = MD_DIST + 1;   // the buffer refilled at tile t is the one tile t - 1 was read from
-constexpr int MD_MAX_CHUNKS = 2048;    // chunk list kept in LDS
+constexpr int MD_MAX_CHUNKS = 1024;    // chunk list kept in LDS
 constexpr int MD_PASS = 8;             // tiles between two replays of the searches
 
 static __device__ __align__(16) uint16_t md_zero_row[256];
@@ -65,7 +65,7 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
     // loop would make the compiler wait for everything in flight, the tile loads included, before it uses the value.
     __shared__ int s_left[MD_MAX_CHUNKS];
     __shared__ float s_gwidth[MD_MAX_CHUNKS / 16];       // per group of block_chunk chunks: widest chunk, 0 = not searched
-    __shared__ float s_score[HPW][MD_PASS * MD_TN];      // per head: scores of the tokens of the last MD_PASS tiles
+    __shared__ uint16_t s_score[HPW][MD_PASS * MD_TN];   // per head: scores (bf16 bits) of the tokens of the last MD_PASS tiles
     // Paged keys: the pool page of every token slot of a pass of MD_PASS tiles (-1: slot not loaded), two passes.
     // The block table is read with ordinary loads, which drain the tile loads in flight (see s_left), so it is read
     // once per pass, for the whole next pass, instead of inside the prefetch of every tile.
@@ -119,7 +119,7 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
         lim = (int)(lm < 0 ? 0 : lm);
     }
     const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
-    for (int i = tid; i < p.n; i += NT) s_left[i] = p.chunk_left[row_in + i];
+    for (int i = tid; i < MD_MAX_CHUNKS; i += NT) s_left[i] = i < p.n ? p.chunk_left[row_in + i] : -1;
 
     // ---- Q^ fragments, in the order qhat_kernel stores them (k-step, row half, row)
     MdFrag qf[MB][KS];
@@ -163,38 +163,49 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
     const int ntiles = (p.n + (1 << cpt_shift) - 1) >> cpt_shift;
     // piece slot c = tid + NT * j of a tile is position c % PPR of token slot c / PPR; one load instruction of a wave
     // fills 64 consecutive piece slots
+    const uint16_t *pf_base[CPT];
+    int pf_e[CPT];
+#pragma unroll
+    for (int j = 0; j < CPT; j++) {
+        const int c = tid + NT * j;
+        const int slot = c / PPR, pos = c % PPR;
+        pf_e[j] = slot & (CH - 1);
+        pf_base[j] = reinterpret_cast<const uint16_t *>(p.kv.k) + (int64_t)b * p.kv.k_stride_b +
+                     (int64_t)pf_e[j] * p.kv.k_stride_t + (int64_t)kvh * p.kv.k_stride_h + ((pos ^ slot) & (PPR - 1)) * 8;
+    }
+    const unsigned lim_u = any_rows ? (unsigned)lim : 0u;
+    const bool none_u = !any_rows;  // then even cl == 0 must fail
+    const int t_end = none_u ? -0x7fffffff : (int)(p.right_clamp < (int64_t)p.kv.tsrc ? p.right_clamp : (int64_t)p.kv.tsrc);
     auto prefetch = [&](int tile) {
         const int buf = tile % MD_NBUF;
+        // all addresses first, then the loads back to back: the load statements keep their order, so an LDS read
+        // between two of them would be waited for there
+        const uint16_t *src[CPT];
 #pragma unroll
         for (int j = 0; j < CPT; j++) {
-            const int c = tid + NT * j;
-            const int slot = c / PPR, pos = c % PPR;
+            const int slot = (tid + NT * j) / PPR, pos = (tid + NT * j) % PPR;
             const int ci = (tile << cpt_shift) + (slot >> ch_shift);
-            const uint16_t *src = md_zero_row;
+            src[j] = md_zero_row;
             if constexpr (PAGED) {
                 const int pg = s_page[(tile / MD_PASS) & 1][(tile % MD_PASS) * MD_TN + slot];
                 if (pg >= 0) {
                     const int t = s_left[ci] + (slot & (CH - 1));  // pg >= 0 implies ci < p.n
-                    src = reinterpret_cast<const uint16_t *>(p.kv.k) + (int64_t)pg * p.kv.k_stride_b +
-                          (int64_t)(t & (p.kv.page_size - 1)) * p.kv.k_stride_t + (int64_t)kvh * p.kv.k_stride_h +
-                          ((pos ^ slot) & (PPR - 1)) * 8;
+                    src[j] = reinterpret_cast<const uint16_t *>(p.kv.k) + (int64_t)pg * p.kv.k_stride_b +
+                             (int64_t)(t & (p.kv.page_size - 1)) * p.kv.k_stride_t + (int64_t)kvh * p.kv.k_stride_h +
+                             ((pos ^ slot) & (PPR - 1)) * 8;
                 }
-            } else if (ci < p.n) {
+            } else {
+                // Dense keys: the row address is plain arithmetic, and all of it but the chunk's left edge is the same
+                // for every tile (pf_base).  A chunk that starts beyond the block's reach is never searched (its left
+                // edge only moves right): 0 <= cl <= lim as one unsigned compare; entries of the list beyond its end
+                // hold -1.  Rows at or beyond the end of the chunk (right_clamp) or of the tensor read as zeros.
                 const int cl = s_left[ci];
-                const int64_t rr = (int64_t)cl + CH;
-                const int cr = (int)(rr < p.right_clamp ? rr : p.right_clamp);
-                const int t = cl + (slot & (CH - 1));
-                // a chunk that starts beyond the block's reach is never searched (its left edge only moves right)
-                if (t < cr && cl <= lim && cl >= 0 && any_rows) {
-                    // dense keys: the row address is plain arithmetic; rows at or beyond the end of the tensor read
-                    // as zeros
-                    if (t < p.kv.tsrc)
-                        src = reinterpret_cast<const uint16_t *>(p.kv.k) + (int64_t)b * p.kv.k_stride_b +
-                              (int64_t)t * p.kv.k_stride_t + (int64_t)kvh * p.kv.k_stride_h + ((pos ^ slot) & (PPR - 1)) * 8;
-                }
+                const int t = cl + pf_e[j];
+                if ((unsigned)cl <= lim_u && t < t_end) src[j] = pf_base[j] + (int64_t)cl * p.kv.k_stride_t;
             }
-            load_to_lds16(src, &s_rows[buf][0][0] + (wid * 64 + NT * j) * 8);
         }
+#pragma unroll
+        for (int j = 0; j < CPT; j++) load_to_lds16(src[j], &s_rows[buf][0][0] + (wid * 64 + NT * j) * 8);
     };
     // pages of the token slots of pass `pass` (tiles pass * MD_PASS ...), by all threads
     auto lookup_pages = [&](int pass) {
@@ -241,7 +252,7 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
 
     // The searches are replayed once per PASS tiles, one lane per chunk, on the scores the tiles left in LDS: replaying
     // them tile by tile would keep 64 lanes busy with the four or eight chunks of a block.
-    float *my_scores = &s_score[wid][0];
+    uint16_t *my_scores = &s_score[wid][0];
     auto replay = [&](int first_tile, int last_tile) {  // chunks of tiles [first_tile, last_tile]
         const int c_begin = first_tile << cpt_shift;
         int c_end = (last_tile + 1) << cpt_shift;
@@ -253,7 +264,7 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
             const int cl0 = cl;
             float score = -32000.0f;
             float width = s_gwidth[cidx / BC];
-            const float *sc = my_scores + ((cidx - c_begin) << ch_shift);  // s[cl0 + e] at sc[e]
+            const uint16_t *sc = my_scores + ((cidx - c_begin) << ch_shift);  // s[cl0 + e] at sc[e]
             unsigned touched = 0;  // bit e: the search sampled token cl0 + e
             while (width >= p.terminate) {
                 width *= 0.5f;
@@ -261,7 +272,7 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
                 if (active) {
                     const int ctr = (cl + cr) >> 1;
                     const int eL = ((cl + ctr) >> 1) - cl0, eR = ((ctr + cr) >> 1) - cl0;
-                    const float sL = sc[eL], sR = sc[eR];
+                    const float sL = __uint_as_float((uint32_t)sc[eL] << 16), sR = __uint_as_float((uint32_t)sc[eR] << 16);
                     touched |= (1u << eL) | (1u << eR);
                     const bool win = sL > sR;
                     if (win) cr = ctr; else cl = ctr;
@@ -362,7 +373,7 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
                     for (int i = 0; i < 16; i++) v = fmaxf(v, ((vm[mb] >> i) & 1u) ? acc[nb][mb][i] : -INFINITY);
             }
             v = fmaxf(v, swap_halves(v));
-            if (hh == 0 && searched[nb]) my_scores[(tile % MD_PASS) * MD_TN + nb * 32 + n] = round_bf16(v);
+            if (hh == 0 && searched[nb]) my_scores[(tile % MD_PASS) * MD_TN + nb * 32 + n] = (uint16_t)(__float_as_uint(round_bf16(v)) >> 16);
         }
         if ((tile % MD_PASS) == MD_PASS - 1 || tile == ntiles - 1) replay(tile - (tile % MD_PASS), tile);  // the wave's own LDS writes
     }

@@ -552,7 +552,7 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
     // 0 = each lane loads its own half row, as the other launches do (read on every call: tests switch it)
     const char *e_dma = getenv("HIPATTN_MASK_DMA");
     const bool dma = (e_dma ? atoi(e_dma) : 1) != 0 && wide && prescaled && p.rope.cos == nullptr && !p.kx.kv8 &&
-                     !p.kx.cached && HID <= 128 && env_nb != 2;
+                     !p.kx.cached && HID <= 128 && env_nb != 2 && !two;  // (64-row programs: 204 registers, 6.7 against 3.9 ms)
     const int nb0 = dma ? 1 : (env_nb == 2 && BC >= 32) ? 2 : (env_nb == 1 ? 1 : (wide ? 2 : 1));
     // LDS path: one wave per workgroup (it uses workgroup barriers); direct path: up to 4 heads per workgroup
     // (measured: sharing pays with one query-row block per program, not with two)
@@ -591,7 +591,7 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
         const char *e = getenv("HIPATTN_MASK_GROUP_REPS");
         env_reps = e ? atoi(e) : 0;
     }
-    p.group_reps = (!two && !dma) ? 1 : env_reps > 0 ? env_reps : (wide ? (dma && !two ? 16 : 8) : 1);
+    p.group_reps = (!two && !dma) ? 1 : env_reps > 0 ? env_reps : (wide ? (dma ? 16 : 8) : 1);
     if (p.group_reps > p.ngroups) p.group_reps = p.ngroups;
     const int groups_outer = (p.ngroups + p.group_reps - 1) / p.group_reps;
     p.total = (long long)p.B * p.kv.HKV * hblocks * p.BS * groups_outer * nsub;
@@ -653,8 +653,7 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
     }
     if (dma && !q_inline) {
         if constexpr (HID <= 128) {
-            if (two) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 2, 1, true, false, true, 4>), grid, block, 0, st, p, nsub, hpw);
-            else hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 4>), grid, block, 0, st, p, nsub, hpw);
+            hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 4>), grid, block, 0, st, p, nsub, hpw);
             HIPATTN_CHECK_HIP(hipGetLastError());
             return 0;
         }
