@@ -461,6 +461,13 @@ __device__ __forceinline__ void load_to_lds16(const void *gsrc, void *lds_base) 
                  : "v"(gsrc), "s"(__builtin_amdgcn_readfirstlane(base))
                  : "memory", "m0");
 }
+// the same with the LDS address given as a wave-uniform 32-bit value (kept in a scalar register by the caller)
+__device__ __forceinline__ void load_to_lds16_at(const void *gsrc, uint32_t lds_addr_uniform) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(gsrc), "s"(lds_addr_uniform)
+                 : "memory", "m0");
+}
 // wait until at most N vector-memory operations of this wave are outstanding (they complete in order)
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {

@@ -20,6 +20,7 @@
 #include "mask_common.hpp"
 
 namespace hipattn {
+static __device__ __align__(16) uint16_t g_scan_zero_row[256];
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
@@ -337,6 +338,7 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
             }
         }
         uint4 *my_tile = &s_rows[DMA ? (threadIdx.x >> 6) * 32 * PPR : 0];
+        const uint32_t tile_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)my_tile);  // LDS address: low 32 bits
         if constexpr (DMA) {
             if (fresh[0]) {
                 // instruction i fetches rows 4i .. 4i+3: lane l takes slot l % 16 of row 4i + l / 16, which holds the
@@ -344,15 +346,23 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
                 // not sampled afresh are left as they are: a lane only ever looks at the column of its own row.
                 // (offsets are multiples of eight elements: they travel between lanes as 32-bit piece numbers)
                 const int my_piece0 = offs[0] == NO_ROW ? -1 : (int)(offs[0] >> 3);
+                // all cross-lane reads first, then the loads back to back: the load statements keep their order, so a
+                // cross-lane read between two of them would be waited for there
+                // Rows that are not sampled afresh come from a row of zeros, so that no load sits in a branch.
+                constexpr int NI = 32 * PPR / 64;
+                int o[NI];
 #pragma unroll
-                for (int i = 0; i < 32 * PPR / 64; i++) {
+                for (int i = 0; i < NI; i++) o[i] = __shfl(my_piece0, i * (64 / PPR) + lane / PPR);
+                const uint4 *src[NI];
+#pragma unroll
+                for (int i = 0; i < NI; i++) {
                     const int r = i * (64 / PPR) + lane / PPR;
-                    const int o = __shfl(my_piece0, r);
-                    if (o >= 0) {
-                        const int q = (lane % PPR) ^ (r & (PPR - 1));
-                        load_to_lds16(reinterpret_cast<const uint4 *>(p.kv.k) + ((int64_t)o + q), my_tile + i * 64);
-                    }
+                    const int q = (lane % PPR) ^ (r & (PPR - 1));
+                    src[i] = o[i] >= 0 ? reinterpret_cast<const uint4 *>(p.kv.k) + ((int64_t)o[i] + q)
+                                       : reinterpret_cast<const uint4 *>(g_scan_zero_row) + (lane % PPR);
                 }
+#pragma unroll
+                for (int i = 0; i < NI; i++) load_to_lds16_at(src[i], tile_addr + i * 1024);
                 wait_vmcnt<0>();
             }
         }
@@ -455,6 +465,7 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
     }
     store_out();
     }
+
 }
 
 // Q^ rows of every scan program: strided mean of stride_q query rows in f32, rounded to bf16, scaled
