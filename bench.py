@@ -37,10 +37,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # WRITE_SIZE in the same runs, so FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0.
 TRAFFIC_SOURCE = "recorded: profiles/prefill_hbm_traffic_pmc.md (not measured in this run)"
 MEASURED_TRAFFIC_BYTES = {
-    "mask_stage[n=507,chunk=256,rows=16]": 2.0 * 792845.2 * 1024 + 51628.8 * 1024,
-    "mask_stage[n=1024,chunk=32,rows=16]": 2.0 * 2107565.4 * 1024 + 65683.5 * 1024,
-    "mask_stage[n=1024,chunk=8,rows=64]": 2.0 * 2207574.0 * 1024 + 220521.1 * 1024,
-    "bsa_prefill": 2.0 * 1861475.8 * 1024 + 262144.2 * 1024,
+    "mask_stage[n=507,chunk=256,rows=16]": 2.0 * 4469318.8 * 1024 + 419163.2 * 1024,
+    "mask_stage[n=1024,chunk=32,rows=16]": 2.0 * 6656534.2 * 1024 + 445547.4 * 1024,
+    "mask_stage[n=1024,chunk=8,rows=64]": 2.0 * 2162424.6 * 1024 + 218122.1 * 1024,
+    "bsa_prefill": 2.0 * 1861253.1 * 1024 + 262144.2 * 1024,
 }
 
 
