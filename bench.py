@@ -35,7 +35,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the prefill kernels, from two rocprofv3 --pmc runs of this file (FETCH_SIZE, then
 # WRITE_SIZE, KiB per dispatch).  A 268 435 456-byte device copy reads 131 095 KiB of FETCH_SIZE and 262 144 KiB of
 # WRITE_SIZE in the same runs, so FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0.
-TRAFFIC_SOURCE = "recorded: profiles/prefill_hbm_traffic_pmc.md (not measured in this run)"
+TRAFFIC_SOURCE = ("recorded: profiles/prefill_hbm_traffic_pmc.md (not measured in this run); FETCH_SIZE / WRITE_SIZE count bytes "
+                  "between the L2 caches and the memory side, served by the 256 MB memory-side cache or by HBM")
 MEASURED_TRAFFIC_BYTES = {
     "mask_stage[n=507,chunk=256,rows=16]": 2.0 * 4469318.8 * 1024 + 419163.2 * 1024,
     "mask_stage[n=1024,chunk=32,rows=16]": 2.0 * 6656534.2 * 1024 + 445547.4 * 1024,
