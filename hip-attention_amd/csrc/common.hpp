@@ -468,6 +468,14 @@ __device__ __forceinline__ void load_to_lds16_at(const void *gsrc, uint32_t lds_
                  : "v"(gsrc), "s"(lds_addr_uniform)
                  : "memory", "m0");
 }
+// the same with the global address given as a wave-uniform base (scalar register pair) plus a 32-bit byte offset per
+// lane: half the address registers, and no 64-bit additions per lane
+__device__ __forceinline__ void load_to_lds16_at_s(const void *gbase_uniform, uint32_t byte_off, uint32_t lds_addr_uniform) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(byte_off), "s"(gbase_uniform), "s"(lds_addr_uniform)
+                 : "memory", "m0");
+}
 // wait until at most N vector-memory operations of this wave are outstanding (they complete in order)
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {

@@ -74,11 +74,13 @@ __device__ __forceinline__ int64_t rope_kpos(const RopeView &r, int c, int side)
 // row, which the kernel scales itself; no preparation launch is needed.
 // KV8 = true (extended parameter block, unscaled keys): key rows are fp8 (e5m2) bytes, widened on load.
 template <int HID, int MB, int NB, bool PRESCALED, bool VIA_LDS, bool EXT, int RMODE = 0, bool KV8 = false>
-__global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
+__global__ __launch_bounds__(VIA_LDS ? 64 : 256) __attribute__((amdgpu_waves_per_eu((RMODE == 4 || RMODE == 5) ? 4 : 1)))
+void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     constexpr bool ROPE = RMODE == 1;
     constexpr bool QINL = RMODE == 3;  // query rows scaled here instead of read from the prepared workspace
     static_assert(!QINL || NB == 1, "inline query rows: the one-token-block variants only");
-    constexpr bool DMA = RMODE == 4;   // rows fetched coalesced, straight into a per-wave LDS tile
+    constexpr bool DMA = RMODE == 4 || RMODE == 5;  // rows fetched coalesced, straight into a per-wave LDS tile
+    constexpr bool OFF32 = RMODE == 5;  // their addresses: 32-bit byte offsets from the batch item's first key row
     static_assert(!DMA || (PRESCALED && !VIA_LDS && NB == 1), "coalesced direct-to-LDS rows: prescaled keys, one token block per wave");
     static_assert(!KV8 || (EXT && !PRESCALED), "fp8 keys: extended build, scaled in the kernel");
     static_assert(!ROPE || (EXT && !VIA_LDS && !PRESCALED), "rope variant: direct path of the extended build");
@@ -109,7 +111,7 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
     L /= nsub;
     const int s = (int)(L % p.BS);
     L /= p.BS;
-    const int group_reps = (MB == 2 || RMODE == 4) ? p.group_reps : 1;
+    const int group_reps = (MB == 2 || DMA) ? p.group_reps : 1;
     const int groups_outer = (p.ngroups + group_reps - 1) / group_reps;
     const int g0 = (int)(L % groups_outer) * group_reps;
     L /= groups_outer;
@@ -345,24 +347,40 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
                 // row's piece (l % 16) ^ (row % 16); the row's offset is held by the lane of that row.  Rows that are
                 // not sampled afresh are left as they are: a lane only ever looks at the column of its own row.
                 // (offsets are multiples of eight elements: they travel between lanes as 32-bit piece numbers)
-                const int my_piece0 = offs[0] == NO_ROW ? -1 : (int)(offs[0] >> 3);
+                const int64_t first_row = OFF32 ? (int64_t)b * p.kv.k_stride_b : 0;
+                const int my_piece0 = offs[0] == NO_ROW ? -1 : (int)((offs[0] - first_row) >> 3);
                 // all cross-lane reads first, then the loads back to back: the load statements keep their order, so a
                 // cross-lane read between two of them would be waited for there
-                // Rows that are not sampled afresh come from a row of zeros, so that no load sits in a branch.
                 constexpr int NI = 32 * PPR / 64;
                 int o[NI];
 #pragma unroll
                 for (int i = 0; i < NI; i++) o[i] = __shfl(my_piece0, i * (64 / PPR) + lane / PPR);
-                const uint4 *src[NI];
+                if constexpr (OFF32) {
+                    // Rows that are not sampled afresh are fetched from the batch item's first row (any row will do:
+                    // their products are not looked at), so that no load sits in a branch.
+                    const uint16_t *kb = reinterpret_cast<const uint16_t *>(p.kv.k) + first_row;
+                    uint32_t so[NI];
 #pragma unroll
-                for (int i = 0; i < NI; i++) {
-                    const int r = i * (64 / PPR) + lane / PPR;
-                    const int q = (lane % PPR) ^ (r & (PPR - 1));
-                    src[i] = o[i] >= 0 ? reinterpret_cast<const uint4 *>(p.kv.k) + ((int64_t)o[i] + q)
-                                       : reinterpret_cast<const uint4 *>(g_scan_zero_row) + (lane % PPR);
+                    for (int i = 0; i < NI; i++) {
+                        const int r = i * (64 / PPR) + lane / PPR;
+                        const int q = (lane % PPR) ^ (r & (PPR - 1));
+                        so[i] = o[i] >= 0 ? (uint32_t)(o[i] + q) << 4 : 0u;
+                    }
+#pragma unroll
+                    for (int i = 0; i < NI; i++) load_to_lds16_at_s(kb, so[i], tile_addr + i * 1024);
+                } else {
+                    // Rows that are not sampled afresh come from a row of zeros, so that no load sits in a branch.
+                    const uint4 *src[NI];
+#pragma unroll
+                    for (int i = 0; i < NI; i++) {
+                        const int r = i * (64 / PPR) + lane / PPR;
+                        const int q = (lane % PPR) ^ (r & (PPR - 1));
+                        src[i] = o[i] >= 0 ? reinterpret_cast<const uint4 *>(p.kv.k) + ((int64_t)o[i] + q)
+                                           : reinterpret_cast<const uint4 *>(g_scan_zero_row) + (lane % PPR);
+                    }
+#pragma unroll
+                    for (int i = 0; i < NI; i++) load_to_lds16_at(src[i], tile_addr + i * 1024);
                 }
-#pragma unroll
-                for (int i = 0; i < NI; i++) load_to_lds16_at(src[i], tile_addr + i * 1024);
                 wait_vmcnt<0>();
             }
         }
@@ -447,6 +465,9 @@ __global__ __launch_bounds__(VIA_LDS ? 64 : 256) void mask_stage_mfma_kernel(Mas
             }
             v = fmaxf(v, __shfl_xor(v, 32));
             v = round_bf16(v);
+            if constexpr (OFF32) {
+                if (offs[tb] == NO_ROW) v = 0.0f;  // a token without a row scores as a row of zeros
+            }
             }
             if (reuse[tb]) v = rscore[tb];
             if (active[tb]) {
@@ -664,7 +685,12 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
     }
     if (dma && !q_inline) {
         if constexpr (HID <= 128) {
-            hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 4>), grid, block, 0, st, p, nsub, hpw);
+            // a dense key tensor whose batch items span less than 4 GB: row addresses as 32-bit offsets
+            const long long item_bytes = 2LL * ((p.kv.tsrc - 1) * p.kv.k_stride_t + (long long)(p.kv.HKV - 1) * p.kv.k_stride_h + HID);
+            const bool off32 = !p.kv.paged && p.kv.k_stride_t >= 0 && p.kv.k_stride_h >= 0 && p.kv.k_stride_t % 8 == 0 &&
+                               p.kv.k_stride_h % 8 == 0 && p.kv.k_stride_b % 8 == 0 && item_bytes < (1LL << 32);
+            if (off32) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 5>), grid, block, 0, st, p, nsub, hpw);
+            else hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 4>), grid, block, 0, st, p, nsub, hpw);
             HIPATTN_CHECK_HIP(hipGetLastError());
             return 0;
         }
