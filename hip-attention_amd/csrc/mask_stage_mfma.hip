@@ -58,6 +58,13 @@ __device__ __forceinline__ int64_t rope_kpos(const RopeView &r, int c, int side)
     return 0;
 }
 
+// Waves per SIMD the register allocator is held to: the scans are chains of dependent round trips (token logic, row
+// loads, products, compares) that only other waves can fill, so a variant that drifts a few registers over the
+// boundary of its class loses a quarter of its throughput (the coalesced variant had grown to 144 registers).
+constexpr int mask_stage_waves(int HID, int MB, int NB, int RMODE) {
+    const int w = RMODE == 1 ? (MB == 2 ? 1 : 2) : (MB == 1 && NB == 1) ? 4 : (MB == 1 || (NB == 1 && RMODE == 3)) ? 3 : 2;
+    return HID > 128 ? (w + 1) / 2 : w;  // 256-element rows: twice the fragments
+}
 // RMODE = 1 (direct path, one token block per wave, extended parameter block): every sampled key row is rotated
 // before it is scaled.  The two halves of a row sit in the two half-waves (lane and lane ^ 32) at the same k-step,
 // and under the RELATIVE, STREAMING and INFLLM rules the rotated position of a lane's key never changes over the
@@ -74,7 +81,7 @@ __device__ __forceinline__ int64_t rope_kpos(const RopeView &r, int c, int side)
 // row, which the kernel scales itself; no preparation launch is needed.
 // KV8 = true (extended parameter block, unscaled keys): key rows are fp8 (e5m2) bytes, widened on load.
 template <int HID, int MB, int NB, bool PRESCALED, bool VIA_LDS, bool EXT, int RMODE = 0, bool KV8 = false>
-__global__ __launch_bounds__(VIA_LDS ? 64 : 256) __attribute__((amdgpu_waves_per_eu((RMODE == 4 || RMODE == 5) ? 4 : 1)))
+__global__ __launch_bounds__(VIA_LDS ? 64 : 256) __attribute__((amdgpu_waves_per_eu(mask_stage_waves(HID, MB, NB, RMODE))))
 void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     constexpr bool ROPE = RMODE == 1;
     constexpr bool QINL = RMODE == 3;  // query rows scaled here instead of read from the prepared workspace
@@ -332,10 +339,13 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
             if constexpr (VIA_LDS) {
                 if (hh == 0) s_off[tb * 32 + n] = off;
             } else if constexpr (!DMA) {
+                // no load in a branch of its own: lanes without a row read a row of zeros, so that the pieces of a
+                // row are requested back to back and arrive after one trip to memory, not one after the other
+                if (fresh[tb]) {
+                    const void *rbase = off != NO_ROW ? p.kv.k : static_cast<const void *>(g_scan_zero_row);
+                    const int64_t roff = off != NO_ROW ? off + hh * HALF : 0;
 #pragma unroll
-                for (int ks = 0; ks < KS; ks++) {
-                    raw[tb][ks] = make_uint4(0, 0, 0, 0);
-                    if (off != NO_ROW) raw[tb][ks] = load_kv_piece<KV8>(p.kv.k, off + hh * HALF + ks * 8);
+                    for (int ks = 0; ks < KS; ks++) raw[tb][ks] = load_kv_piece<KV8>(rbase, roff + ks * 8);
                 }
             }
         }
@@ -389,21 +399,33 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
         for (int tb = 0; tb < NB; tb++) any_fresh = any_fresh || fresh[tb];
         if (VIA_LDS && any_fresh) {
             __syncthreads();
-            // coalesced fetch: PPR lanes cover one row; piece q of row r is parked at slot q ^ swz(r)
+            // coalesced fetch: PPR lanes cover one row; piece q of row r is parked at slot q ^ swz(r).  Eight loads
+            // are requested before the first is used, and none sits in a branch (rows that are not sampled come
+            // from a row of zeros): one trip to memory per eight instead of one per load.
+            constexpr int NLOAD = NROWS / RPI;
+            constexpr int LB = NLOAD < 8 ? NLOAD : 8;
 #pragma unroll
-            for (int i = 0; i < NROWS / RPI; i++) {
-                const int r = i * RPI + lrow;
-                const int64_t off = s_off[r];
-                const int q = lpos ^ ((r / SWZ_DIV) & SWZ);
-                uint4 v = make_uint4(0, 0, 0, 0);
-                if (off != NO_ROW) v = load_kv_piece<KV8>(p.kv.k, off + q * 8);
-                if (!PRESCALED) {
-                    v.x = scale_pack(v.x, p.c_k);
-                    v.y = scale_pack(v.y, p.c_k);
-                    v.z = scale_pack(v.z, p.c_k);
-                    v.w = scale_pack(v.w, p.c_k);
+            for (int i0 = 0; i0 < NLOAD; i0 += LB) {
+                uint4 v[LB];
+#pragma unroll
+                for (int j = 0; j < LB; j++) {
+                    const int r = (i0 + j) * RPI + lrow;
+                    const int64_t off = s_off[r];
+                    const int q = lpos ^ ((r / SWZ_DIV) & SWZ);
+                    const void *rbase = off != NO_ROW ? p.kv.k : static_cast<const void *>(g_scan_zero_row);
+                    v[j] = load_kv_piece<KV8>(rbase, (off != NO_ROW ? off : 0) + q * 8);
                 }
-                s_rows[r * PPR + lpos] = v;
+#pragma unroll
+                for (int j = 0; j < LB; j++) {
+                    const int r = (i0 + j) * RPI + lrow;
+                    if (!PRESCALED) {
+                        v[j].x = scale_pack(v[j].x, p.c_k);
+                        v[j].y = scale_pack(v[j].y, p.c_k);
+                        v[j].z = scale_pack(v[j].z, p.c_k);
+                        v[j].w = scale_pack(v[j].w, p.c_k);
+                    }
+                    s_rows[r * PPR + lpos] = v[j];
+                }
             }
             __syncthreads();
         }
