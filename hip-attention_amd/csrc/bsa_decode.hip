@@ -218,46 +218,66 @@ __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<E
     }
 }
 
-// Merge of the per-split partials of one (batch, head): out = sum_s w_s x_s / sum_s w_s with w_s = 2^(lse_s - max lse),
-// summed in split order.  The partials were written by workgroups all over the chip, so every read is a long-latency
-// one: the rows are first pulled into LDS with all loads of a chunk in flight at once, then combined from there.
-constexpr int MERGE_THREADS = 256;
-constexpr int MERGE_CHUNK = 32;  // splits staged per round
+// Merge of the per-split partials of one (batch, head): out = sum_s w_s x_s / sum_s w_s with w_s = 2^(lse_s - max lse).
+// The partials were written by workgroups all over the chip, so every read is a long-latency one, and the launch is
+// small (one workgroup per head): what counts is the number of dependent trips to memory.  A workgroup's 1024 threads
+// are 1024 / HID parts x HID columns: a part takes every (1024 / HID)-th split and folds its partials into a running
+// (maximum, numerator, denominator), eight splits' loads in flight at a time and no pass over the log-sum-exps
+// beforehand; the parts are then folded through LDS (53 splits of 128 columns: one trip; it was three, 6.2 us).
+constexpr int MERGE_THREADS = 1024;
+constexpr int MERGE_BATCH = 8;
 
 template <typename T, int HID>
 __global__ __launch_bounds__(MERGE_THREADS) void bsa_decode_merge_kernel(const float *ws, int HEAD, int nsplits, T *out,
                                                                         int64_t o_sb, int64_t o_sh) {
     constexpr int ROW = HID + 4;
-    __shared__ __align__(16) float s_rows[MERGE_CHUNK * ROW];
-    __shared__ float s_red[MERGE_THREADS / 64];
+    constexpr int PARTS = MERGE_THREADS / HID;
+    __shared__ float s_m[PARTS][HID], s_num[PARTS][HID], s_den[PARTS][HID];
     const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    const int part = tid / HID, d = tid % HID;
     const float *base = ws + ((int64_t)b * HEAD + h) * nsplits * ROW;
-    // max of the log-sum-exps
-    float mm = -INFINITY;
-    for (int s = tid; s < nsplits; s += MERGE_THREADS) mm = fmaxf(mm, base[(int64_t)s * ROW + HID]);
-    mm = wave_max(mm);
-    if ((tid & 63) == 0) s_red[tid >> 6] = mm;
-    __syncthreads();
-    mm = s_red[0];
+    float m = -INFINITY, num = 0.0f, den = 0.0f;
+    for (int s0 = part; s0 < nsplits; s0 += PARTS * MERGE_BATCH) {
+        float lse[MERGE_BATCH], val[MERGE_BATCH];
 #pragma unroll
-    for (int w = 1; w < MERGE_THREADS / 64; w++) mm = fmaxf(mm, s_red[w]);
-    float num = 0.0f, den = 0.0f;
-    for (int s0 = 0; s0 < nsplits; s0 += MERGE_CHUNK) {
-        const int ns = nsplits - s0 < MERGE_CHUNK ? nsplits - s0 : MERGE_CHUNK;
-        __syncthreads();
-        const float4 *src = reinterpret_cast<const float4 *>(base + (int64_t)s0 * ROW);  // rows are 16-byte multiples
-        float4 *dst = reinterpret_cast<float4 *>(s_rows);
-        for (int i = tid; i < ns * ROW / 4; i += MERGE_THREADS) dst[i] = src[i];
-        __syncthreads();
-        if (tid < HID && mm > -INFINITY) {
-            for (int s = 0; s < ns; s++) {
-                const float w = exp2f(s_rows[s * ROW + HID] - mm);
-                num += w * s_rows[s * ROW + tid];
-                den += w;
+        for (int j = 0; j < MERGE_BATCH; j++) {
+            const int s = s0 + j * PARTS;
+            const bool ok = s < nsplits;
+            const float *row = base + (int64_t)(ok ? s : part) * ROW;
+            const float l = row[HID], v = row[d];
+            lse[j] = ok ? l : -INFINITY;
+            val[j] = v;
+        }
+#pragma unroll
+        for (int j = 0; j < MERGE_BATCH; j++) {
+            if (lse[j] > -INFINITY) {
+                const float mn = fmaxf(m, lse[j]);
+                const float keep = exp2f(m - mn), w = exp2f(lse[j] - mn);  // m = -inf: keep = 0
+                num = num * keep + w * val[j];
+                den = den * keep + w;
+                m = mn;
             }
         }
     }
-    if (tid < HID) out[(int64_t)b * o_sb + (int64_t)h * o_sh + tid] = Elem<T>::narrow(den > 0.0f ? num / den : 0.0f);
+    s_m[part][d] = m;
+    s_num[part][d] = num;
+    s_den[part][d] = den;
+    __syncthreads();
+    if (tid < HID) {
+        float mm = -INFINITY;
+#pragma unroll
+        for (int q = 0; q < PARTS; q++) mm = fmaxf(mm, s_m[q][tid]);
+        float n = 0.0f, dd = 0.0f;
+        if (mm > -INFINITY) {
+#pragma unroll
+            for (int q = 0; q < PARTS; q++) {
+                const float w = exp2f(s_m[q][tid] - mm);  // parts without a split: exp2(-inf) = 0
+                n += w * s_num[q][tid];
+                dd += w * s_den[q][tid];
+            }
+        }
+        out[(int64_t)b * o_sb + (int64_t)h * o_sh + tid] = Elem<T>::narrow(dd > 0.0f ? n / dd : 0.0f);
+    }
 }
 
 template <typename T, int HID>

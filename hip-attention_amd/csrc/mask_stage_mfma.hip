@@ -468,7 +468,9 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                 for (int mb = 0; mb < MB; mb++)
                     acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qf[mb][ks].v, kf.v, acc[mb], 0, 0, 0);
             }
-            if (fast_rows == 16) {
+            if constexpr (QINL) {
+                v = hh == 0 ? acc[0][0] : -INFINITY;  // the one valid row is row 0: element 0 of the lower half-wave
+            } else if (fast_rows == 16) {
 #pragma unroll
                 for (int i = 0; i < 8; i++) v = fmaxf(v, acc[0][i]);
             } else if (fast_rows == 32) {
