@@ -190,6 +190,16 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     (void)all_rows;
 
     const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
+    // OFF32 (dense keys, a batch item under 4 GB, no block cache): a row's place is a 32-bit number of 16-byte pieces
+    // from the item's first row, one 24-bit multiply per sample; the general routine's 64-bit products, its paged and
+    // cached branches and the scalar registers they pin (spilled and re-read in every iteration) stay out of the loop
+    const uint32_t piece_st = OFF32 ? (uint32_t)(p.kv.k_stride_t >> 3) : 0u;
+    const uint32_t piece_h = OFF32 ? (uint32_t)(((int64_t)kvh * p.kv.k_stride_h) >> 3) : 0u;
+    const int tsrc32 = OFF32 ? (int)p.kv.tsrc : 0;
+    int32_t *flag_row = nullptr;
+    if constexpr (OFF32) {
+        if (kx->access_flags) flag_row = kx->access_flags + (int64_t)b * kx->flags_stride_b + (int64_t)kvh * kx->flags_stride_h;
+    }
     // ---- a wave walks p.group_reps consecutive chunk groups of its (scan row, head) with the same Q^ fragments
     // (only the 64-row variant: with 16 or 32 rows the fragments are a tenth of the traffic, and the loop costs the
     // registers of a third wave per SIMD)
@@ -302,6 +312,7 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
         float rscore[NB];
         uint4 raw[(VIA_LDS || DMA) ? 1 : NB][(VIA_LDS || DMA) ? 1 : KS];
         int64_t offs[NB];
+        int pieces[NB];  // OFF32: the sampled row as a piece number, -1 = none
 #pragma unroll
         for (int tb = 0; tb < NB; tb++) {
             active[tb] = real[tb] && (cl[tb] < cr[tb]) && (cl[tb] <= lim) && (cl[tb] >= 0);
@@ -316,7 +327,16 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
             }
             fresh[tb] = __any(active[tb] && !reuse[tb]) != 0;
             int64_t off = NO_ROW;
-            if (active[tb] && !reuse[tb]) {
+            if constexpr (OFF32) {
+                pieces[tb] = -1;
+                if (active[tb] && !reuse[tb]) {
+                    const int t = tok[tb];
+                    if (t >= 0 && t < tsrc32) {
+                        pieces[tb] = (int)(__umul24((uint32_t)t, piece_st) + piece_h);
+                        if (flag_row && hh == 0) flag_row[t] = 1;
+                    }
+                }
+            } else if (active[tb] && !reuse[tb]) {
                 const int t = tok[tb];
                 // access flags: wide launches (prefill) revisit rows constantly, so they look before they store;
                 // narrow ones (decode) touch mostly fresh rows and store blindly
@@ -357,8 +377,7 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                 // row's piece (l % 16) ^ (row % 16); the row's offset is held by the lane of that row.  Rows that are
                 // not sampled afresh are left as they are: a lane only ever looks at the column of its own row.
                 // (offsets are multiples of eight elements: they travel between lanes as 32-bit piece numbers)
-                const int64_t first_row = OFF32 ? (int64_t)b * p.kv.k_stride_b : 0;
-                const int my_piece0 = offs[0] == NO_ROW ? -1 : (int)((offs[0] - first_row) >> 3);
+                const int my_piece0 = OFF32 ? pieces[0] : offs[0] == NO_ROW ? -1 : (int)(offs[0] >> 3);
                 // all cross-lane reads first, then the loads back to back: the load statements keep their order, so a
                 // cross-lane read between two of them would be waited for there
                 constexpr int NI = 32 * PPR / 64;
@@ -368,7 +387,7 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                 if constexpr (OFF32) {
                     // Rows that are not sampled afresh are fetched from the batch item's first row (any row will do:
                     // their products are not looked at), so that no load sits in a branch.
-                    const uint16_t *kb = reinterpret_cast<const uint16_t *>(p.kv.k) + first_row;
+                    const uint16_t *kb = reinterpret_cast<const uint16_t *>(p.kv.k) + (int64_t)b * p.kv.k_stride_b;
                     uint32_t so[NI];
 #pragma unroll
                     for (int i = 0; i < NI; i++) {
@@ -490,7 +509,7 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
             v = fmaxf(v, __shfl_xor(v, 32));
             v = round_bf16(v);
             if constexpr (OFF32) {
-                if (offs[tb] == NO_ROW) v = 0.0f;  // a token without a row scores as a row of zeros
+                if (pieces[tb] < 0) v = 0.0f;  // a token without a row scores as a row of zeros
             }
             }
             if (reuse[tb]) v = rscore[tb];
@@ -712,7 +731,8 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
             // a dense key tensor whose batch items span less than 4 GB: row addresses as 32-bit offsets
             const long long item_bytes = 2LL * ((p.kv.tsrc - 1) * p.kv.k_stride_t + (long long)(p.kv.HKV - 1) * p.kv.k_stride_h + HID);
             const bool off32 = !p.kv.paged && p.kv.k_stride_t >= 0 && p.kv.k_stride_h >= 0 && p.kv.k_stride_t % 8 == 0 &&
-                               p.kv.k_stride_h % 8 == 0 && p.kv.k_stride_b % 8 == 0 && item_bytes < (1LL << 32);
+                               p.kv.k_stride_h % 8 == 0 && p.kv.k_stride_b % 8 == 0 && item_bytes < (1LL << 32) &&
+                               p.kv.tsrc < (1LL << 24) && (p.kv.k_stride_t >> 3) < (1LL << 24);
             if (off32) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 5>), grid, block, 0, st, p, nsub, hpw);
             else hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 4>), grid, block, 0, st, p, nsub, hpw);
             HIPATTN_CHECK_HIP(hipGetLastError());
