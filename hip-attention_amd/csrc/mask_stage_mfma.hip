@@ -77,6 +77,8 @@ constexpr int mask_stage_waves(int HID, int MB, int NB, int RMODE) {
 // its own half row makes every load instruction touch 64 cache lines, and the address unit then passes one line per
 // clock: 9.5 TB/s over the chip on L2-resident rows where the coalesced shape reaches 30), into an 8 KB tile of the
 // wave with the 16-byte pieces of row r permuted by r, and read back in operand layout.
+// RMODE = 6: a single query token (as RMODE = 3) with the rows fetched as under RMODE = 4; keys prescaled or scaled
+// after the tile is read back.
 // RMODE = 3 (no rotation, one token block per wave, a single query token): the one valid program row is that token's
 // row, which the kernel scales itself; no preparation launch is needed.
 // KV8 = true (extended parameter block, unscaled keys): key rows are fp8 (e5m2) bytes, widened on load.
@@ -84,11 +86,12 @@ template <int HID, int MB, int NB, bool PRESCALED, bool VIA_LDS, bool EXT, int R
 __global__ __launch_bounds__(VIA_LDS ? 64 : 256) __attribute__((amdgpu_waves_per_eu(mask_stage_waves(HID, MB, NB, RMODE))))
 void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     constexpr bool ROPE = RMODE == 1;
-    constexpr bool QINL = RMODE == 3;  // query rows scaled here instead of read from the prepared workspace
+    constexpr bool QINL = RMODE == 3 || RMODE == 6;  // query rows scaled here instead of read from the prepared workspace
     static_assert(!QINL || NB == 1, "inline query rows: the one-token-block variants only");
-    constexpr bool DMA = RMODE == 4 || RMODE == 5;  // rows fetched coalesced, straight into a per-wave LDS tile
+    constexpr bool DMA = RMODE == 4 || RMODE == 5 || RMODE == 6;  // rows fetched coalesced, straight into a per-wave LDS tile
     constexpr bool OFF32 = RMODE == 5;  // their addresses: 32-bit byte offsets from the batch item's first key row
-    static_assert(!DMA || (PRESCALED && !VIA_LDS && NB == 1), "coalesced direct-to-LDS rows: prescaled keys, one token block per wave");
+    static_assert(!DMA || (!VIA_LDS && NB == 1 && !KV8), "coalesced direct-to-LDS rows: one token block per wave, bf16 keys");
+    static_assert((RMODE != 4 && RMODE != 5) || PRESCALED, "coalesced rows on wide launches: prescaled keys");
     static_assert(!KV8 || (EXT && !PRESCALED), "fp8 keys: extended build, scaled in the kernel");
     static_assert(!ROPE || (EXT && !VIA_LDS && !PRESCALED), "rope variant: direct path of the extended build");
     static_assert(RMODE != 2 || (EXT && PRESCALED), "two-sided prescaled keys: extended build of the prescaled path");
@@ -466,6 +469,10 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                     kf.q = s_rows[r * PPR + ((hh * (PPR / 2) + ks) ^ sw)];
                 } else if constexpr (DMA) {
                     kf.q = my_tile[n * PPR + ((hh * (PPR / 2) + ks) ^ (n & (PPR - 1)))];
+                    if constexpr (!PRESCALED) {  // the tile holds the rows as stored
+#pragma unroll
+                        for (int e = 0; e < 4; e++) kf.u[e] = scale_pack(kf.u[e], p.c_k);
+                    }
                 } else if constexpr (PRESCALED) {
                     kf.q = raw[tb][ks];
                 } else if constexpr (ROPE) {
@@ -628,7 +635,18 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
     const char *e_dma = getenv("HIPATTN_MASK_DMA");
     const bool dma = (e_dma ? atoi(e_dma) : 1) != 0 && wide && prescaled && p.rope.cos == nullptr && !p.kx.kv8 &&
                      !p.kx.cached && HID <= 128 && env_nb != 2 && !two;  // (64-row programs: 204 registers, 6.7 against 3.9 ms)
-    const int nb0 = dma ? 1 : (env_nb == 2 && BC >= 32) ? 2 : (env_nb == 1 ? 1 : (wide ? 2 : 1));
+    // small chunks on wide launches: every token scored once per GQA group, searches replayed on the scores
+    const bool dense = prescaled && p.rope.cos == nullptr && mask_stage_dense_applies(p, HID, rows_eff);
+    // HIPATTN_MASK_DMA_INLINE: launches with a single query token fetch their rows that way too, from keys as stored
+    // (1 = always, 0 = never, default: from 16384 waves on, e.g. a batch of sequences; a lone sequence's stages of
+    // small chunks are a few hundred workgroups whose searches share rows through L1)
+    const char *e_di = getenv("HIPATTN_MASK_DMA_INLINE");
+    const int di = e_di ? atoi(e_di) : 2;
+    const long long waves_one_block = (long long)p.B * p.HEAD * p.BS * p.ngroups * (BC / 16);
+    const bool dma_inline = (e_dma ? atoi(e_dma) : 1) != 0 && di != 0 && !dense && p.TDST == 1 && !two &&
+                            p.rope.cos == nullptr && !p.kx.kv8 && !p.kx.cached && HID <= 128 && env_nb != 2 &&
+                            (di == 1 || waves_one_block >= 16384);
+    const int nb0 = (dma || dma_inline) ? 1 : (env_nb == 2 && BC >= 32) ? 2 : (env_nb == 1 ? 1 : (wide ? 2 : 1));
     // LDS path: one wave per workgroup (it uses workgroup barriers); direct path: up to 4 heads per workgroup
     // (measured: sharing pays with one query-row block per program, not with two)
     if (g_mask_via_lds < 0) {
@@ -647,7 +665,7 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
     // through L1, and direct loads win (decode at 1M keys: 31 / 22 us against 38 / 28 us for the 32- and 8-token
     // stages); wide chunks scatter the samples of a search, and rows fetched coalesced through LDS win (124 against
     // 182 us for the 256-token stage)
-    bool via_lds = dma ? false : g_mask_via_lds == 2 ? (!wide && p.chunk > 32) : (g_mask_via_lds == 1);
+    bool via_lds = (dma || dma_inline) ? false : g_mask_via_lds == 2 ? (!wide && p.chunk > 32) : (g_mask_via_lds == 1);
     if (((p.kx.extended() || two_sided) && nb == 2) || rope) via_lds = false;
     const bool ext = rope || two_sided || p.kx.extended() || (wide && !two && !via_lds);
     static int env_hpw2 = -1;
@@ -674,8 +692,6 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
         set_error("mask stage: grid too large");
         return HIPATTN_E_UNSUPPORTED;
     }
-    // small chunks on wide launches: every token scored once per GQA group, searches replayed on the scores
-    const bool dense = prescaled && !two_sided && mask_stage_dense_applies(p, HID, rows_eff);
     // Where every program row is the mean of exactly one query row and is not rotated (the dense kernel with
     // stride_q == 1; the narrow sampling kernels with a single query token), the kernels scale the rows themselves: the preparation launch
     // (a pass over all of q) shrinks to the fill of the head-reduced scores, and to nothing when the caller has
@@ -735,6 +751,14 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
                                p.kv.tsrc < (1LL << 24) && (p.kv.k_stride_t >> 3) < (1LL << 24);
             if (off32) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 5>), grid, block, 0, st, p, nsub, hpw);
             else hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 4>), grid, block, 0, st, p, nsub, hpw);
+            HIPATTN_CHECK_HIP(hipGetLastError());
+            return 0;
+        }
+    }
+    if (dma_inline) {
+        if constexpr (HID <= 128) {
+            if (prescaled) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 6>), grid, block, 0, st, p, nsub, hpw);
+            else hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, false, false, true, 6>), grid, block, 0, st, p, nsub, hpw);
             HIPATTN_CHECK_HIP(hipGetLastError());
             return 0;
         }
