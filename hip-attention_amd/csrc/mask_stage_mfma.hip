@@ -632,8 +632,10 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
     }
     // HIPATTN_MASK_DMA: wide launches on prescaled keys fetch their rows coalesced, straight into LDS (default);
     // 0 = each lane loads its own half row, as the other launches do (read on every call: tests switch it)
+    // (2 = on every launch the variant can serve, however small: testing)
     const char *e_dma = getenv("HIPATTN_MASK_DMA");
-    const bool dma = (e_dma ? atoi(e_dma) : 1) != 0 && wide && prescaled && p.rope.cos == nullptr && !p.kx.kv8 &&
+    const int dma_mode = e_dma ? atoi(e_dma) : 1;
+    const bool dma = dma_mode != 0 && (wide || dma_mode == 2) && prescaled && p.rope.cos == nullptr && !p.kx.kv8 &&
                      !p.kx.cached && HID <= 128 && env_nb != 2 && !two;  // (64-row programs: 204 registers, 6.7 against 3.9 ms)
     // small chunks on wide launches: every token scored once per GQA group, searches replayed on the scores
     const bool dense = prescaled && p.rope.cos == nullptr && mask_stage_dense_applies(p, HID, rows_eff);
@@ -643,7 +645,7 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
     const char *e_di = getenv("HIPATTN_MASK_DMA_INLINE");
     const int di = e_di ? atoi(e_di) : 2;
     const long long waves_one_block = (long long)p.B * p.HEAD * p.BS * p.ngroups * (BC / 16);
-    const bool dma_inline = (e_dma ? atoi(e_dma) : 1) != 0 && di != 0 && !dense && p.TDST == 1 && !two &&
+    const bool dma_inline = dma_mode != 0 && di != 0 && !dense && p.TDST == 1 && !two &&
                             p.rope.cos == nullptr && !p.kx.kv8 && !p.kx.cached && HID <= 128 && env_nb != 2 &&
                             (di == 1 || waves_one_block >= 16384);
     const int nb0 = (dma || dma_inline) ? 1 : (env_nb == 2 && BC >= 32) ? 2 : (env_nb == 1 ? 1 : (wide ? 2 : 1));
@@ -684,7 +686,7 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
         const char *e = getenv("HIPATTN_MASK_GROUP_REPS");
         env_reps = e ? atoi(e) : 0;
     }
-    p.group_reps = (!two && !dma) ? 1 : env_reps > 0 ? env_reps : (wide ? (dma ? 16 : 8) : 1);
+    p.group_reps = (!two && !dma) ? 1 : env_reps > 0 ? env_reps : dma ? 16 : (wide ? 8 : 1);
     if (p.group_reps > p.ngroups) p.group_reps = p.ngroups;
     const int groups_outer = (p.ngroups + p.group_reps - 1) / p.group_reps;
     p.total = (long long)p.B * p.kv.HKV * hblocks * p.BS * groups_outer * nsub;

@@ -283,3 +283,52 @@ def test_small_chunk_stages_scored_densely(case, paged, monkeypatch):
     ctx2, meta2 = run_product(X, A)
     assert torch.equal(meta2.indices, meta.indices)
     assert torch.equal(meta2.mask_cache_statistics.access_counter, meta.mask_cache_statistics.access_counter)
+
+
+@pytest.mark.parametrize("layout", ["dense", "page 16", "page 1"])
+def test_single_token_scans_with_coalesced_row_fetch(layout, monkeypatch):
+    """Decode launches of many waves fetch the sampled rows coalesced, straight into LDS, from keys as stored; forced
+    here on a small batch (HIPATTN_MASK_DMA_INLINE=1).  Masks and access flags must equal the oracle's and those of
+    the launches that load a half row per lane."""
+    _case(f"coalesced single-token scans, {layout}")
+    lens = np.array([3000, 1777, 4096, 2500])
+    if layout == "dense":
+        X = make_inputs(14, B=2, TQ=1, TK=4096, H=8, HKV=2, D=128, dtype="bf16", pos=np.array([[4095], [4095]]))
+        A = O.OArgs(sliding_window_size=512)
+    else:
+        X = make_inputs(4, B=4, TQ=1, TK=4096, H=8, HKV=2, D=128, dtype="bf16", pos=(lens - 1)[:, None])
+        X = to_paged(X, int(layout.split()[1]), seed=5, seq_lens=lens)
+        A = O.OArgs(sliding_window_size=512, extend_context_length=4096)
+    octx, ometa = O.hip_attention_12(X, A)
+    monkeypatch.setenv("HIPATTN_MASK_DMA_INLINE", "1")
+    ctx, meta = run_product(X, A, require_cache_statistics=True)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, "bf16")
+    monkeypatch.setenv("HIPATTN_MASK_DMA_INLINE", "0")
+    ctx0, meta0 = run_product(X, A, require_cache_statistics=True)
+    assert torch.equal(meta0.indices, meta.indices)
+    assert torch.equal(meta0.mask_cache_statistics.access_counter, meta.mask_cache_statistics.access_counter)
+
+
+@pytest.mark.parametrize("paged", [0, 16])
+def test_prefill_scans_with_coalesced_row_fetch_on_a_small_launch(paged, monkeypatch):
+    """The coalesced fetch of the wide prefill launches (prescaled keys; 32-bit row offsets on a dense tensor, 64-bit
+    ones on a paged cache), forced on a launch of a few hundred programs (HIPATTN_MASK_DMA=2): ragged candidate
+    lists, a wave walking past the end of its chunk groups, statistics flags."""
+    _case(f"coalesced prefill scans on a small launch, paged={paged}")
+    monkeypatch.setenv("HIP_ATTN_PRESCALE_K", "1")
+    monkeypatch.setenv("HIPATTN_MASK_DENSE", "0")
+    X = make_inputs(15, B=2, TQ=300, TK=8192, H=8, HKV=2, D=128, dtype="bf16")
+    A = O.OArgs(sliding_window_size=512)
+    if paged:
+        X = to_paged(X, paged, seed=13)
+        A.extend_context_length = 8192
+    octx, ometa = O.hip_attention_12(X, A)
+    monkeypatch.setenv("HIPATTN_MASK_DMA", "2")
+    ctx, meta = run_product(X, A, require_cache_statistics=True)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, "bf16")
+    monkeypatch.setenv("HIPATTN_MASK_DMA", "0")
+    ctx0, meta0 = run_product(X, A, require_cache_statistics=True)
+    assert torch.equal(meta0.indices, meta.indices)
+    assert torch.equal(meta0.mask_cache_statistics.access_counter, meta.mask_cache_statistics.access_counter)
