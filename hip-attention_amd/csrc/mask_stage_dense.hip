@@ -176,17 +176,20 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
     const unsigned lim_u = any_rows ? (unsigned)lim : 0u;
     const bool none_u = !any_rows;  // then even cl == 0 must fail
     const int t_end = none_u ? -0x7fffffff : (int)(p.right_clamp < (int64_t)p.kv.tsrc ? p.right_clamp : (int64_t)p.kv.tsrc);
+    // the address of the row of zeros, formed once (the compiler would fetch it from the offset table at every use)
+    const uint16_t *zero_row = md_zero_row;
+    asm volatile("" : "+s"(zero_row));
     auto prefetch = [&](int tile) {
         const int buf = tile % MD_NBUF;
         // all addresses first, then the loads back to back: the load statements keep their order, so an LDS read
         // between two of them would be waited for there
         const uint16_t *src[CPT];
+        if constexpr (PAGED) {
 #pragma unroll
-        for (int j = 0; j < CPT; j++) {
-            const int slot = (tid + NT * j) / PPR, pos = (tid + NT * j) % PPR;
-            const int ci = (tile << cpt_shift) + (slot >> ch_shift);
-            src[j] = md_zero_row;
-            if constexpr (PAGED) {
+            for (int j = 0; j < CPT; j++) {
+                const int slot = (tid + NT * j) / PPR, pos = (tid + NT * j) % PPR;
+                const int ci = (tile << cpt_shift) + (slot >> ch_shift);
+                src[j] = zero_row;
                 const int pg = s_page[(tile / MD_PASS) & 1][(tile % MD_PASS) * MD_TN + slot];
                 if (pg >= 0) {
                     const int t = s_left[ci] + (slot & (CH - 1));  // pg >= 0 implies ci < p.n
@@ -194,14 +197,24 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
                              (int64_t)(t & (p.kv.page_size - 1)) * p.kv.k_stride_t + (int64_t)kvh * p.kv.k_stride_h +
                              ((pos ^ slot) & (PPR - 1)) * 8;
                 }
-            } else {
-                // Dense keys: the row address is plain arithmetic, and all of it but the chunk's left edge is the same
-                // for every tile (pf_base).  A chunk that starts beyond the block's reach is never searched (its left
-                // edge only moves right): 0 <= cl <= lim as one unsigned compare; entries of the list beyond its end
-                // hold -1.  Rows at or beyond the end of the chunk (right_clamp) or of the tensor read as zeros.
-                const int cl = s_left[ci];
-                const int t = cl + pf_e[j];
-                if ((unsigned)cl <= lim_u && t < t_end) src[j] = pf_base[j] + (int64_t)cl * p.kv.k_stride_t;
+            }
+        } else {
+            // Dense keys: the row address is plain arithmetic, and all of it but the chunk's left edge is the same
+            // for every tile (pf_base).  A chunk that starts beyond the block's reach is never searched (its left
+            // edge only moves right): 0 <= cl <= lim as one unsigned compare; entries of the list beyond its end
+            // hold -1.  Rows at or beyond the end of the chunk (right_clamp) or of the tensor read as zeros.
+            // The list entries of all loads are read from LDS together, and nothing below branches: the offset of a
+            // row from its chunk's left edge is one 24-bit multiply (the product fits 31 bits and its factors 24:
+            // checked before the launch).
+            int cl[CPT];
+#pragma unroll
+            for (int j = 0; j < CPT; j++) cl[j] = s_left[(tile << cpt_shift) + (((tid + NT * j) / PPR) >> ch_shift)];
+#pragma unroll
+            for (int j = 0; j < CPT; j++) {
+                const int t = cl[j] + pf_e[j];
+                const bool ok = ((unsigned)cl[j] <= lim_u) & (t < t_end);
+                const uint16_t *row = pf_base[j] + (int64_t)(int)__umul24((uint32_t)cl[j], (uint32_t)p.kv.k_stride_t);
+                src[j] = ok ? row : zero_row;
             }
         }
 #pragma unroll
@@ -290,7 +303,12 @@ __global__ __launch_bounds__(64 * HPW) void mask_stage_dense_kernel(MaskParamsFo
                                 mark_flag<false>(kx->access_flags + (int64_t)b * kx->flags_stride_b +
                                                  (int64_t)kvh * kx->flags_stride_h + pg);
                         } else {
-                            kv_k_row<true, false>(p.kv, kx, b, cl0 + e, kvh, seqlen, true);
+                            // (written out: the general routine's paged and cached branches hold loads, and a load
+                            // the compiler tracks anywhere in the tile loop makes it drain the tile loads in flight)
+                            const int t = cl0 + e;
+                            if (kx->access_flags && t >= 0 && t < p.kv.tsrc)
+                                mark_flag<false>(kx->access_flags + (int64_t)b * kx->flags_stride_b +
+                                                 (int64_t)kvh * kx->flags_stride_h + t);
                         }
                     }
             }
@@ -436,6 +454,10 @@ bool mask_stage_dense_applies(const MaskParams &p, int HID, int rows_eff) {
         const long long wgs = (long long)p.B * p.kv.HKV * p.BS;
         if (!(per_search * p.G >= 2 * CH) || wgs < 1024 || p.n < 64) return false;
     }
+    // dense keys: a row's offset from its chunk's left edge is formed with one 24-bit multiply
+    if (!p.kv.paged && !(p.kv.k_stride_t > 0 && p.kv.k_stride_t < (1 << 24) && p.kv.tsrc < (1 << 24) &&
+                         p.kv.tsrc * p.kv.k_stride_t < (1LL << 31)))
+        return false;
     const int hpw = p.G >= 4 ? 4 : 2;
     const long long total = (long long)p.B * p.kv.HKV * p.BS * ((p.G + hpw - 1) / hpw);
     (void)rows_eff;
