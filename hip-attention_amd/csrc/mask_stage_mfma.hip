@@ -380,7 +380,10 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                 // row's piece (l % 16) ^ (row % 16); the row's offset is held by the lane of that row.  Rows that are
                 // not sampled afresh are left as they are: a lane only ever looks at the column of its own row.
                 // (offsets are multiples of eight elements: they travel between lanes as 32-bit piece numbers)
-                const int my_piece0 = OFF32 ? pieces[0] : offs[0] == NO_ROW ? -1 : (int)(offs[0] >> 3);
+                // (OFF32: a lane without a fresh sample sends the first row of its kv head: any row will do, its
+                // products are not looked at, and no load needs a select or sits in a branch)
+                const int my_piece0 = OFF32 ? (pieces[0] < 0 ? (int)piece_h : pieces[0])
+                                            : offs[0] == NO_ROW ? -1 : (int)(offs[0] >> 3);
                 // all cross-lane reads first, then the loads back to back: the load statements keep their order, so a
                 // cross-lane read between two of them would be waited for there
                 constexpr int NI = 32 * PPR / 64;
@@ -388,15 +391,13 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
 #pragma unroll
                 for (int i = 0; i < NI; i++) o[i] = __shfl(my_piece0, i * (64 / PPR) + lane / PPR);
                 if constexpr (OFF32) {
-                    // Rows that are not sampled afresh are fetched from the batch item's first row (any row will do:
-                    // their products are not looked at), so that no load sits in a branch.
                     const uint16_t *kb = reinterpret_cast<const uint16_t *>(p.kv.k) + (int64_t)b * p.kv.k_stride_b;
                     uint32_t so[NI];
 #pragma unroll
                     for (int i = 0; i < NI; i++) {
                         const int r = i * (64 / PPR) + lane / PPR;
                         const int q = (lane % PPR) ^ (r & (PPR - 1));
-                        so[i] = o[i] >= 0 ? (uint32_t)(o[i] + q) << 4 : 0u;
+                        so[i] = (uint32_t)(o[i] + q) << 4;
                     }
 #pragma unroll
                     for (int i = 0; i < NI; i++) load_to_lds16_at_s(kb, so[i], tile_addr + i * 1024);
