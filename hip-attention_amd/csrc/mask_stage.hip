@@ -340,7 +340,7 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
                                (1u << HIPATTN_EXTEND_DYNAMIC),
                         "mask stage", &p.rope);
     if (rc) return rc;
-    HIPATTN_CHECK_ARG(k_prescaled >= 0 && k_prescaled <= 3, HIPATTN_E_ARG, "mask stage: k_prescaled %d not in 0..3", k_prescaled);
+    HIPATTN_CHECK_ARG(k_prescaled >= 0 && k_prescaled <= 7, HIPATTN_E_ARG, "mask stage: k_prescaled %d not in 0..7", k_prescaled);
     HIPATTN_CHECK_ARG(!(p.rope.cos && (k_prescaled & 1)) || p.rope.backend == HIPATTN_EXTEND_RELATIVE ||
                           p.rope.backend == HIPATTN_EXTEND_INFLLM,
                       HIPATTN_E_ARG, "mask stage: prescaled keys need a rule with fixed key positions (relative, infllm)");
@@ -378,7 +378,7 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
         HIPATTN_CHECK_ARG(workspace && aligned16(workspace), HIPATTN_E_ARG,
                           "mask stage: bf16 inputs need a 16-byte aligned workspace (hipattn_mask_stage_workspace_bytes)");
         p.qhat = reinterpret_cast<const uint16_t *>(workspace);
-        return mask_stage_mfma_launch(p, q->HID, rows_eff, k_prescaled, st);  // bit 0: keys, bit 1: query rows ready
+        return mask_stage_mfma_launch(p, q->HID, rows_eff, k_prescaled, st);  // bit 0: keys, bit 1: query rows ready, bit 2: rows beyond 32 GiB
     } else if (q->dtype == HIPATTN_F32) {
         HIPATTN_CHECK_ARG(!(k_prescaled & 1), HIPATTN_E_ARG, "mask stage: prescaled keys are a bf16-only option");
         if (p.reduce_heads == 1) {

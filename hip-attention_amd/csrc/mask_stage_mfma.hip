@@ -620,6 +620,9 @@ template <int HID>
 static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStream_t st) {
     const int prescaled = flags & 1;          // keys scaled (and rotated) ahead of the scan
     const bool q_ready = (flags & 2) != 0;    // the workspace holds this stage's query rows already
+    // key rows may lie 32 GiB or more beyond kv.k: the coalesced variants, whose lanes exchange the rows' places as
+    // 31-bit numbers of 16-byte pieces, are not used
+    const bool far_rows = (flags & 4) != 0;
     MaskParams p = p0;
     const int BC = p.block_chunk;
     const bool two = rows_eff > 32;
@@ -636,7 +639,7 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
     // (2 = on every launch the variant can serve, however small: testing)
     const char *e_dma = getenv("HIPATTN_MASK_DMA");
     const int dma_mode = e_dma ? atoi(e_dma) : 1;
-    const bool dma = dma_mode != 0 && (wide || dma_mode == 2) && prescaled && p.rope.cos == nullptr && !p.kx.kv8 &&
+    const bool dma = dma_mode != 0 && !far_rows && (wide || dma_mode == 2) && prescaled && p.rope.cos == nullptr && !p.kx.kv8 &&
                      !p.kx.cached && HID <= 128 && env_nb != 2 && !two;  // (64-row programs: 204 registers, 6.7 against 3.9 ms)
     // small chunks on wide launches: every token scored once per GQA group, searches replayed on the scores
     const bool dense = prescaled && p.rope.cos == nullptr && mask_stage_dense_applies(p, HID, rows_eff);
@@ -646,7 +649,7 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
     const char *e_di = getenv("HIPATTN_MASK_DMA_INLINE");
     const int di = e_di ? atoi(e_di) : 2;
     const long long waves_one_block = (long long)p.B * p.HEAD * p.BS * p.ngroups * (BC / 16);
-    const bool dma_inline = dma_mode != 0 && di != 0 && !dense && p.TDST == 1 && !two &&
+    const bool dma_inline = dma_mode != 0 && !far_rows && di != 0 && !dense && p.TDST == 1 && !two &&
                             p.rope.cos == nullptr && !p.kx.kv8 && !p.kx.cached && HID <= 128 && env_nb != 2 &&
                             (di == 1 || waves_one_block >= 16384);
     const int nb0 = (dma || dma_inline) ? 1 : (env_nb == 2 && BC >= 32) ? 2 : (env_nb == 1 ? 1 : (wide ? 2 : 1));

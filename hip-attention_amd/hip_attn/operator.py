@@ -243,6 +243,14 @@ def _mask_kv(args: HiPAttentionArgs, k_mask: Optional[Tensor], max_tsrc: int, q:
     return plain, None, keep, None, 0
 
 
+def _spans_32_gib(t: Optional[Tensor]) -> bool:
+    """Whether rows of ``t`` can lie 32 GiB or more beyond its first element (see ``hipattn_mask_stage``)."""
+    if t is None:
+        return False
+    span = sum((n - 1) * abs(s) for n, s in zip(t.shape, t.stride())) + 1
+    return span * t.element_size() >= (1 << 35)
+
+
 _INITIAL_CHUNKS = {}  # read-only stage-0 chunk lists, keyed by their shape parameters
 _INITIAL_CHUNKS_PINNED = {}  # those a captured graph reads: kept for the life of the process
 
@@ -506,7 +514,8 @@ def dual_stage_quadratic_hip_attention(
                     ws = N.mask_stage(qs, mask_kv_pre if use_pre else mask_kv, chunk_left, hg, chunk_count, chunk_size,
                                       right_clamp, bs, BLOCK_SIZE_Q, stage.stage_block_stride_q, BLOCK_CHUNK, STAGE_STRIDE,
                                       sw_eff, args.stage_early_terminate, scores, left_out, device, k_prescaled=use_pre,
-                                      reduce_heads=reduce, workspace=query_rows.get(ws_key))
+                                      reduce_heads=reduce, workspace=query_rows.get(ws_key),
+                                      far_rows=_spans_32_gib(khat if use_pre else (k_mask if k_mask is not None else args.k_cache)))
                     if ws_key is not None and ws is not None:
                         query_rows[ws_key] = ws
             elif isinstance(stage, NopStage):

@@ -149,7 +149,9 @@ const char *hipattn_last_error(void);
  *   iteration count (:595-601,736-737).
  *   k_prescaled: bit 0: kv->k already holds bf16(K * c_k) (see hipattn_prescale_k); bit 1: the workspace already
  *   holds the query rows of this stage, left there by an earlier call with the same q, bs, bq, stride_q, scan_stride
- *   and no rotation (stages that differ only in their chunks share them).
+ *   and no rotation (stages that differ only in their chunks share them); bit 2: key rows may lie 32 GiB or more
+ *   beyond kv->k (a paged pool of that size; a dense tensor's extent is known from its strides): the launches that
+ *   pass the places of rows between lanes as 31-bit numbers of 16-byte pieces are then not used.
  *   workspace: device scratch of hipattn_mask_stage_workspace_bytes(...) bytes. */
 int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, const int32_t *chunk_left,
                        int32_t hg, int32_t n, int32_t chunk_size, int64_t right_clamp,

@@ -201,3 +201,17 @@ def test_helper_tensors_a_graph_has_seen_are_never_evicted(monkeypatch):
         get(key)
     assert len(cache) == 4 and get(0) is a and built.count(0) == 1
     assert 1 not in cache and get(1) is not None and built.count(1) == 2   # unpinned entries are evicted oldest first
+
+
+def test_key_buffers_of_32_gib_are_reported_to_the_scan():
+    """Scan launches that pass the places of key rows between lanes as 31-bit piece numbers must be told when a
+    buffer is too large for that; the span counts strides, not elements."""
+    import torch
+    from hip_attn import operator as op
+
+    small = torch.empty((1, 1 << 20, 8, 128), dtype=torch.bfloat16, device="meta")
+    assert not op._spans_32_gib(small) and not op._spans_32_gib(None)
+    pool = torch.empty(((1 << 20) + 1, 16, 8, 128), dtype=torch.bfloat16, device="meta")  # 32 KiB pages: one more than 32 GiB
+    assert op._spans_32_gib(pool)
+    assert not op._spans_32_gib(pool[: 1 << 19])
+    assert op._spans_32_gib(pool[:: 1 << 19])  # three pages, 16 GiB apart
