@@ -77,6 +77,11 @@ constexpr int mask_stage_waves(int HID, int MB, int NB, int RMODE) {
 // its own half row makes every load instruction touch 64 cache lines, and the address unit then passes one line per
 // clock: 9.5 TB/s over the chip on L2-resident rows where the coalesced shape reaches 30), into an 8 KB tile of the
 // wave with the 16-byte pieces of row r permuted by r, and read back in operand layout.
+// RMODE = 7 / 8 (as 5 / 4, programs of up to 16 query rows): the products run on v_mfma_f32_16x16x32_bf16, whose four
+// groups of eight elements per instruction are given the order in which two steps of the 32x32x16 instruction take
+// theirs (k-step 2j lower half, 2j upper half, 2j + 1 lower, 2j + 1 upper): the accumulation chain of a score, and
+// with it every bit of the result, is the same (compared on 2M products of adversarial inputs, while any other order
+// of the groups differs in a quarter of them), at half the matrix cycles, 24 registers fewer and no rows of zeros.
 // RMODE = 6: a single query token (as RMODE = 3) with the rows fetched as under RMODE = 4; keys prescaled or scaled
 // after the tile is read back.
 // RMODE = 3 (no rotation, one token block per wave, a single query token): the one valid program row is that token's
@@ -88,10 +93,12 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     constexpr bool ROPE = RMODE == 1;
     constexpr bool QINL = RMODE == 3 || RMODE == 6;  // query rows scaled here instead of read from the prepared workspace
     static_assert(!QINL || NB == 1, "inline query rows: the one-token-block variants only");
-    constexpr bool DMA = RMODE == 4 || RMODE == 5 || RMODE == 6;  // rows fetched coalesced, straight into a per-wave LDS tile
-    constexpr bool OFF32 = RMODE == 5;  // their addresses: 32-bit byte offsets from the batch item's first key row
+    constexpr bool DMA = RMODE >= 4 && RMODE <= 8;  // rows fetched coalesced, straight into a per-wave LDS tile
+    constexpr bool OFF32 = RMODE == 5 || RMODE == 7;  // their addresses: 32-bit byte offsets from the batch item's first key row
+    constexpr bool M16 = RMODE == 7 || RMODE == 8;    // programs of up to 16 query rows on the 16x16x32 instruction
     static_assert(!DMA || (!VIA_LDS && NB == 1 && !KV8), "coalesced direct-to-LDS rows: one token block per wave, bf16 keys");
-    static_assert((RMODE != 4 && RMODE != 5) || PRESCALED, "coalesced rows on wide launches: prescaled keys");
+    static_assert(!DMA || RMODE == 6 || PRESCALED, "coalesced rows on wide launches: prescaled keys");
+    static_assert(!M16 || (MB == 1 && HID % 32 == 0), "16-row variant: one row block, head dim a multiple of 32");
     static_assert(!KV8 || (EXT && !PRESCALED), "fp8 keys: extended build, scaled in the kernel");
     static_assert(!ROPE || (EXT && !VIA_LDS && !PRESCALED), "rope variant: direct path of the extended build");
     static_assert(RMODE != 2 || (EXT && PRESCALED), "two-sided prescaled keys: extended build of the prescaled path");
@@ -147,7 +154,8 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     // Rows were averaged, rounded and scaled once per stage by qhat_kernel: [B, BS, HEAD] blocks of nrows * HID
     // elements, laid out by (k-step, row half, row) so that the lanes of a load instruction read consecutive pieces.
     // They are fetched when the first chunk group of this wave has work and then serve all of its groups.
-    BFrag qf[MB][KS];
+    BFrag qf[M16 ? 1 : MB][M16 ? 1 : KS];
+    BFrag qf16[M16 ? KS / 2 : 1];  // 16-row variant: lane (row l % 16, group l / 16) holds k-step 2j + (l / 32), half (l / 16) % 2
     bool q_loaded = false;
     if constexpr (QINL) {
         // A single query token: row 0 of the program is that token's row of this head, scaled here; no preparation
@@ -265,7 +273,17 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
 
     if (!q_loaded) {
         q_loaded = true;
-        if constexpr (!QINL) {
+        if constexpr (M16) {
+            const uint16_t *qh = p.qhat + ((((int64_t)b * p.BS + s) * p.HEAD + h) * p.nrows) * HID;
+            const int j16 = lane & 15, kb = lane >> 4;
+            const bool jv = (j16 < p.nrows) && ((rowmask >> j16) & 1ull);
+#pragma unroll
+            for (int j = 0; j < KS / 2; j++) {
+                const int ks = 2 * j + (kb >> 1), qhh = kb & 1;
+                qf16[j].q = make_uint4(0, 0, 0, 0);
+                if (jv) qf16[j].q = *reinterpret_cast<const uint4 *>(qh + ((int64_t)(ks * 2 + qhh) * p.nrows + j16) * 8);
+            }
+        } else if constexpr (!QINL) {
             const uint16_t *qh = p.qhat + ((((int64_t)b * p.BS + s) * p.HEAD + h) * p.nrows) * HID;
 #pragma unroll
             for (int mb = 0; mb < MB; mb++) {
@@ -455,7 +473,50 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
 #pragma unroll
         for (int tb = 0; tb < NB; tb++) {
             float v = -INFINITY;
-            if (fresh[tb]) {
+            if constexpr (M16) {
+                if (fresh[tb]) {
+                    // D[row, token]: lane (token c = l % 16 of a half, row group g = l / 16) holds rows 4g .. 4g + 3
+                    typedef __attribute__((ext_vector_type(4))) float f32x4;
+                    const int c = lane & 15, kb = lane >> 4;
+                    float vh[2];
+#pragma unroll
+                    for (int half = 0; half < 2; half++) {
+                        f32x4 acc4 = {0.0f, 0.0f, 0.0f, 0.0f};
+                        const int t = half * 16 + c;
+                        BFrag kf16[KS / 2];
+#pragma unroll
+                        for (int j = 0; j < KS / 2; j++) {
+                            const int piece = (kb & 1) * (PPR / 2) + 2 * j + (kb >> 1);
+                            kf16[j].q = my_tile[t * PPR + (piece ^ (t & (PPR - 1)))];
+                        }
+#pragma unroll
+                        for (int j = 0; j < KS / 2; j++)
+                            acc4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf16[j].v, kf16[j].v, acc4, 0, 0, 0);
+                        float m = -INFINITY;
+                        if (fast_rows == 16) {
+                            m = fmaxf(fmaxf(acc4[0], acc4[1]), fmaxf(acc4[2], acc4[3]));
+                        } else {
+#pragma unroll
+                            for (int r = 0; r < 4; r++) {
+                                const int row = kb * 4 + r;
+                                const bool ok = (row < p.nrows) && ((rowmask >> row) & 1ull);
+                                m = fmaxf(m, ok ? acc4[r] : -INFINITY);
+                            }
+                        }
+                        vh[half] = m;
+                    }
+                    // fold the four row groups: after the exchange over lane ^ 16 a lane holds its own token
+                    // (l % 32) over two groups, after lane ^ 32 over all four
+                    const bool upper = (lane & 16) != 0;
+                    const float keep = upper ? vh[1] : vh[0], send = upper ? vh[0] : vh[1];
+                    v = fmaxf(keep, __shfl_xor(send, 16));
+                    v = fmaxf(v, __shfl_xor(v, 32));
+                    v = round_bf16(v);
+                    if constexpr (OFF32) {
+                        if (pieces[tb] < 0) v = 0.0f;
+                    }
+                }
+            } else if (fresh[tb]) {
             f32x16 acc[MB];
 #pragma unroll
             for (int mb = 0; mb < MB; mb++)
@@ -755,6 +816,20 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
             const bool off32 = !p.kv.paged && p.kv.k_stride_t >= 0 && p.kv.k_stride_h >= 0 && p.kv.k_stride_t % 8 == 0 &&
                                p.kv.k_stride_h % 8 == 0 && p.kv.k_stride_b % 8 == 0 && item_bytes < (1LL << 32) &&
                                p.kv.tsrc < (1LL << 24) && (p.kv.k_stride_t >> 3) < (1LL << 24);
+            // HIPATTN_MASK_M16=1: programs of up to 16 query rows take the 16x16x32 form of the products.  Same bits,
+            // half the matrix cycles, 86 registers instead of 126 (five waves per SIMD), and the same time to within
+            // 2% (cfg-2-like prefill: 2.08 / 2.62 against 2.05 / 2.59 ms): these launches are held by the rate at
+            // which a CU's L1 gets its misses served, not by products, registers or waves.  Off by default.
+            const char *e_m16 = getenv("HIPATTN_MASK_M16");
+            const bool m16 = rows_eff <= 16 && p.nrows <= 16 && (e_m16 ? atoi(e_m16) : 0) != 0;
+            if constexpr (HID % 32 == 0) {
+                if (m16) {
+                    if (off32) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 7>), grid, block, 0, st, p, nsub, hpw);
+                    else hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 8>), grid, block, 0, st, p, nsub, hpw);
+                    HIPATTN_CHECK_HIP(hipGetLastError());
+                    return 0;
+                }
+            }
             if (off32) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 5>), grid, block, 0, st, p, nsub, hpw);
             else hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 4>), grid, block, 0, st, p, nsub, hpw);
             HIPATTN_CHECK_HIP(hipGetLastError());

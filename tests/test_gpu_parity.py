@@ -310,12 +310,16 @@ def test_single_token_scans_with_coalesced_row_fetch(layout, monkeypatch):
     assert torch.equal(meta0.mask_cache_statistics.access_counter, meta.mask_cache_statistics.access_counter)
 
 
+@pytest.mark.parametrize("m16", ["0", "1"])
 @pytest.mark.parametrize("paged", [0, 16])
-def test_prefill_scans_with_coalesced_row_fetch_on_a_small_launch(paged, monkeypatch):
+def test_prefill_scans_with_coalesced_row_fetch_on_a_small_launch(paged, m16, monkeypatch):
     """The coalesced fetch of the wide prefill launches (prescaled keys; 32-bit row offsets on a dense tensor, 64-bit
     ones on a paged cache), forced on a launch of a few hundred programs (HIPATTN_MASK_DMA=2): ragged candidate
     lists, a wave walking past the end of its chunk groups, statistics flags."""
-    _case(f"coalesced prefill scans on a small launch, paged={paged}")
+    _case(f"coalesced prefill scans on a small launch, paged={paged}, 16x16x32 products={m16}")
+    # m16: the products of 16-row programs on v_mfma_f32_16x16x32_bf16 with its groups of eight elements in the order
+    # of two 32x32x16 steps: the same bits
+    monkeypatch.setenv("HIPATTN_MASK_M16", m16)
     monkeypatch.setenv("HIP_ATTN_PRESCALE_K", "1")
     monkeypatch.setenv("HIPATTN_MASK_DENSE", "0")
     X = make_inputs(15, B=2, TQ=300, TK=8192, H=8, HKV=2, D=128, dtype="bf16")
