@@ -20,6 +20,7 @@ struct MaskParamsBase {
     float terminate;
     int ngroups;
     int group_reps;  // bf16 path: consecutive chunk groups walked by one wave (set by its launcher)
+    int share_first; // bf16 path, coalesced fetch: the four heads of a workgroup fetch the rows of a search's first round once
     long long total;
     float c_q, c_k;
     float *scores;

@@ -334,6 +334,8 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
     HIPATTN_CHECK_ARG(terminate_size >= 1, HIPATTN_E_ARG, "mask stage: terminate_size < 1");
     if (n == 0) return 0;
     MaskParams p;
+    p.group_reps = 1;
+    p.share_first = 0;
     rc = make_kv_view(kv, q->B, q->HID, q->dtype, &p.kv, &p.kx);
     if (rc) return rc;
     rc = make_rope_view(q, (1u << HIPATTN_EXTEND_RELATIVE) | (1u << HIPATTN_EXTEND_STREAMING) | (1u << HIPATTN_EXTEND_INFLLM) |

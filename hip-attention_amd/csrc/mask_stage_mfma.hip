@@ -111,7 +111,8 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     constexpr int NROWS = NB * 32;                // sampled rows per iteration of this wave
     constexpr int SWZ = (PPR < 16 ? PPR : 16) - 1;
     constexpr int SWZ_DIV = PPR < 16 ? 16 / PPR : 1;
-    __shared__ __align__(16) uint4 s_rows[VIA_LDS ? NROWS * PPR : DMA ? 4 * 32 * PPR : 1];  // DMA: one tile per wave (up to four)
+    constexpr bool SHAREABLE = DMA && PRESCALED && RMODE != 6;  // prefill variants: the first round's rows can be fetched once per workgroup
+    __shared__ __align__(16) uint4 s_rows[VIA_LDS ? NROWS * PPR : DMA ? (SHAREABLE ? 5 : 4) * 32 * PPR : 1];  // DMA: one tile per wave (up to four), one shared
     __shared__ int64_t s_off[VIA_LDS ? NROWS : 1];
     // a workgroup holds `hpw` waves = `hpw` query heads of one GQA group working on the same chunks:
     // their early-iteration samples coincide, so they share cache lines in the CU's L1
@@ -326,8 +327,16 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
         ptok[tb] = -1;
         pscore[tb] = 0.0f;
     }
+    // The first round of a search samples tokens that do not depend on the query: the four heads of a workgroup
+    // (same chunks, same keys) want the same 32 rows, so each wave fetches a quarter of them into a tile they all read
+    // (the vector-memory path of the CU is what holds these launches, and rows that hit L1 pass through it too).
+    // Every condition on the way here is the same for the waves of a workgroup, so they meet at the barriers.
+    bool first = true;
+    const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     while (width >= p.terminate) {
         width *= 0.5f;
+        bool share_now = false;
+        if constexpr (SHAREABLE) share_now = p.share_first != 0 && first;
         bool active[NB], reuse[NB], fresh[NB];
         int ctr[NB], tok[NB];
         float rscore[NB];
@@ -354,7 +363,7 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                     const int t = tok[tb];
                     if (t >= 0 && t < tsrc32) {
                         pieces[tb] = (int)(__umul24((uint32_t)t, piece_st) + piece_h);
-                        if (flag_row && hh == 0) flag_row[t] = 1;
+                        if (flag_row && hh == 0 && !(share_now && wv != 0)) flag_row[t] = 1;
                     }
                 }
             } else if (active[tb] && !reuse[tb]) {
@@ -392,6 +401,14 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
         }
         uint4 *my_tile = &s_rows[DMA ? (threadIdx.x >> 6) * 32 * PPR : 0];
         const uint32_t tile_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)my_tile);  // LDS address: low 32 bits
+        const uint4 *rd_tile = my_tile;   // where this round's fragments are read from
+        uint32_t dst_addr = tile_addr;
+        if constexpr (SHAREABLE) {
+            if (share_now) {
+                rd_tile = &s_rows[4 * 32 * PPR];
+                dst_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)rd_tile);
+            }
+        }
         if constexpr (DMA) {
             if (fresh[0]) {
                 // instruction i fetches rows 4i .. 4i+3: lane l takes slot l % 16 of row 4i + l / 16, which holds the
@@ -417,8 +434,10 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                         const int q = (lane % PPR) ^ (r & (PPR - 1));
                         so[i] = (uint32_t)(o[i] + q) << 4;
                     }
+                    if (share_now) __syncthreads();  // everyone is done with the shared tile of the search before
 #pragma unroll
-                    for (int i = 0; i < NI; i++) load_to_lds16_at_s(kb, so[i], tile_addr + i * 1024);
+                    for (int i = 0; i < NI; i++)
+                        if (!share_now || (i & 3) == wv) load_to_lds16_at_s(kb, so[i], dst_addr + i * 1024);
                 } else {
                     // Rows that are not sampled afresh come from a row of zeros, so that no load sits in a branch.
                     const uint4 *src[NI];
@@ -429,10 +448,13 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                         src[i] = o[i] >= 0 ? reinterpret_cast<const uint4 *>(p.kv.k) + ((int64_t)o[i] + q)
                                            : reinterpret_cast<const uint4 *>(g_scan_zero_row) + (lane % PPR);
                     }
+                    if (share_now) __syncthreads();
 #pragma unroll
-                    for (int i = 0; i < NI; i++) load_to_lds16_at(src[i], tile_addr + i * 1024);
+                    for (int i = 0; i < NI; i++)
+                        if (!share_now || (i & 3) == wv) load_to_lds16_at(src[i], dst_addr + i * 1024);
                 }
                 wait_vmcnt<0>();
+                if (share_now) __syncthreads();  // every wave's quarter has landed
             }
         }
         bool any_fresh = false;  // uniform over the wave, and the LDS path's workgroups are one wave
@@ -487,7 +509,7 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
 #pragma unroll
                         for (int j = 0; j < KS / 2; j++) {
                             const int piece = (kb & 1) * (PPR / 2) + 2 * j + (kb >> 1);
-                            kf16[j].q = my_tile[t * PPR + (piece ^ (t & (PPR - 1)))];
+                            kf16[j].q = rd_tile[t * PPR + (piece ^ (t & (PPR - 1)))];
                         }
 #pragma unroll
                         for (int j = 0; j < KS / 2; j++)
@@ -530,7 +552,7 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                 if constexpr (VIA_LDS) {
                     kf.q = s_rows[r * PPR + ((hh * (PPR / 2) + ks) ^ sw)];
                 } else if constexpr (DMA) {
-                    kf.q = my_tile[n * PPR + ((hh * (PPR / 2) + ks) ^ (n & (PPR - 1)))];
+                    kf.q = rd_tile[n * PPR + ((hh * (PPR / 2) + ks) ^ (n & (PPR - 1)))];
                     if constexpr (!PRESCALED) {  // the tile holds the rows as stored
 #pragma unroll
                         for (int e = 0; e < 4; e++) kf.u[e] = scale_pack(kf.u[e], p.c_k);
@@ -595,6 +617,7 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                 score[tb] = fmaxf(score[tb], win ? sL : sR);
             }
         }
+        first = false;
     }
     store_out();
     }
@@ -753,6 +776,9 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
     }
     p.group_reps = (!two && !dma) ? 1 : env_reps > 0 ? env_reps : dma ? 16 : (wide ? 8 : 1);
     if (p.group_reps > p.ngroups) p.group_reps = p.ngroups;
+    // HIPATTN_MASK_SHARE_FIRST=0: every head fetches the rows of a search's first round itself
+    const char *e_sf = getenv("HIPATTN_MASK_SHARE_FIRST");
+    p.share_first = (dma && hpw == 4 && p.G % 4 == 0 && p.hg == 1 && (e_sf ? atoi(e_sf) : 1) != 0) ? 1 : 0;
     const int groups_outer = (p.ngroups + p.group_reps - 1) / p.group_reps;
     p.total = (long long)p.B * p.kv.HKV * hblocks * p.BS * groups_outer * nsub;
     if (p.total >= 0x7fffffffLL) {
@@ -816,12 +842,12 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
             const bool off32 = !p.kv.paged && p.kv.k_stride_t >= 0 && p.kv.k_stride_h >= 0 && p.kv.k_stride_t % 8 == 0 &&
                                p.kv.k_stride_h % 8 == 0 && p.kv.k_stride_b % 8 == 0 && item_bytes < (1LL << 32) &&
                                p.kv.tsrc < (1LL << 24) && (p.kv.k_stride_t >> 3) < (1LL << 24);
-            // HIPATTN_MASK_M16=1: programs of up to 16 query rows take the 16x16x32 form of the products.  Same bits,
-            // half the matrix cycles, 86 registers instead of 126 (five waves per SIMD), and the same time to within
-            // 2% (cfg-2-like prefill: 2.08 / 2.62 against 2.05 / 2.59 ms): these launches are held by the rate at
-            // which a CU's L1 gets its misses served, not by products, registers or waves.  Off by default.
+            // Programs of up to 16 query rows take the 16x16x32 form of the products (HIPATTN_MASK_M16=0: the 32x32x16
+            // form).  Same bits, half the matrix cycles, 92 registers instead of 128, and the same time to within 2%
+            // (cfg-2-like prefill: 2.07 / 2.65 against 2.07 / 2.66 ms): these launches are held by the vector-memory
+            // path of a CU, not by products, registers or waves.
             const char *e_m16 = getenv("HIPATTN_MASK_M16");
-            const bool m16 = rows_eff <= 16 && p.nrows <= 16 && (e_m16 ? atoi(e_m16) : 0) != 0;
+            const bool m16 = rows_eff <= 16 && p.nrows <= 16 && (e_m16 ? atoi(e_m16) : 1) != 0;
             if constexpr (HID % 32 == 0) {
                 if (m16) {
                     if (off32) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 7>), grid, block, 0, st, p, nsub, hpw);
