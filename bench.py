@@ -38,10 +38,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 TRAFFIC_SOURCE = ("recorded: profiles/prefill_hbm_traffic_pmc.md (not measured in this run); FETCH_SIZE / WRITE_SIZE count bytes "
                   "between the L2 caches and the memory side, served by the 256 MB memory-side cache or by HBM")
 MEASURED_TRAFFIC_BYTES = {
-    "mask_stage[n=507,chunk=256,rows=16]": 2.0 * 5696929.1 * 1024 + 820468.3 * 1024,
-    "mask_stage[n=1024,chunk=32,rows=16]": 2.0 * 7232826.6 * 1024 + 629572.5 * 1024,
-    "mask_stage[n=1024,chunk=8,rows=64]": 2.0 * 2210617.5 * 1024 + 216533.0 * 1024,
-    "bsa_prefill": 2.0 * 1859619.9 * 1024 + 262144.4 * 1024,
+    "mask_stage[n=507,chunk=256,rows=16]": 2.0 * 5366948.4 * 1024 + 718949.5 * 1024,
+    "mask_stage[n=1024,chunk=32,rows=16]": 2.0 * 7033647.6 * 1024 + 564427.4 * 1024,
+    "mask_stage[n=1024,chunk=8,rows=64]": 2.0 * 2208493.8 * 1024 + 216630.1 * 1024,
+    "bsa_prefill": 2.0 * 1860808.6 * 1024 + 262144.2 * 1024,
 }
 
 
