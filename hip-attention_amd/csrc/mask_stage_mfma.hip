@@ -202,14 +202,17 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     (void)all_rows;
 
     const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
-    // OFF32 (dense keys, a batch item under 4 GB, no block cache): a row's place is a 32-bit number of 16-byte pieces
-    // from the item's first row, one 24-bit multiply per sample; the general routine's 64-bit products, its paged and
-    // cached branches and the scalar registers they pin (spilled and re-read in every iteration) stay out of the loop
-    const uint32_t piece_st = OFF32 ? (uint32_t)(p.kv.k_stride_t >> 3) : 0u;
-    const uint32_t piece_h = OFF32 ? (uint32_t)(((int64_t)kvh * p.kv.k_stride_h) >> 3) : 0u;
-    const int tsrc32 = OFF32 ? (int)p.kv.tsrc : 0;
+    // Coalesced variants (no block cache, the key buffer under 32 GiB): a row's place is a 32-bit number of 16-byte
+    // pieces, formed here with 32-bit products (one 24-bit multiply on OFF32's dense tensors); the general routine's
+    // 64-bit products, its cached branches and the scalar registers they pin (spilled and re-read in every iteration)
+    // stay out of the loop.  OFF32 counts pieces from the batch item's first row, the others from kv.k.
+    const uint32_t piece_st = DMA ? (uint32_t)(p.kv.k_stride_t >> 3) : 0u;
+    const uint32_t piece_sb = DMA ? (uint32_t)(p.kv.k_stride_b >> 3) : 0u;  // paged: pieces per page
+    const uint32_t piece_h = !DMA ? 0u
+                             : (uint32_t)(((int64_t)kvh * p.kv.k_stride_h + ((OFF32 || p.kv.paged) ? 0 : (int64_t)b * p.kv.k_stride_b)) >> 3);
+    const int tsrc32 = DMA ? (int)p.kv.tsrc : 0;
     int32_t *flag_row = nullptr;
-    if constexpr (OFF32) {
+    if constexpr (DMA) {
         if (kx->access_flags) flag_row = kx->access_flags + (int64_t)b * kx->flags_stride_b + (int64_t)kvh * kx->flags_stride_h;
     }
     // ---- a wave walks p.group_reps consecutive chunk groups of its (scan row, head) with the same Q^ fragments
@@ -357,13 +360,21 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
             }
             fresh[tb] = __any(active[tb] && !reuse[tb]) != 0;
             int64_t off = NO_ROW;
-            if constexpr (OFF32) {
+            if constexpr (DMA) {
                 pieces[tb] = -1;
                 if (active[tb] && !reuse[tb]) {
                     const int t = tok[tb];
-                    if (t >= 0 && t < tsrc32) {
-                        pieces[tb] = (int)(__umul24((uint32_t)t, piece_st) + piece_h);
-                        if (flag_row && hh == 0 && !(share_now && wv != 0)) flag_row[t] = 1;
+                    if (OFF32 || !p.kv.paged) {
+                        if (t >= 0 && t < tsrc32) {
+                            pieces[tb] = OFF32 ? (int)(__umul24((uint32_t)t, piece_st) + piece_h)
+                                               : (int)((uint32_t)t * piece_st + piece_h);
+                            if (flag_row && hh == 0 && !(share_now && wv != 0)) flag_row[t] = 1;
+                        }
+                    } else if (t >= 0) {
+                        // the block table's entry, or page 0 beyond the sequence (as the general routine reads it)
+                        const uint32_t page = (uint32_t)p.kv.page_of(b, t, seqlen);
+                        pieces[tb] = (int)(page * piece_sb + (uint32_t)(t & (p.kv.page_size - 1)) * piece_st + piece_h);
+                        if (flag_row && hh == 0 && !(share_now && wv != 0)) flag_row[page] = 1;
                     }
                 }
             } else if (active[tb] && !reuse[tb]) {
@@ -417,8 +428,7 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                 // (offsets are multiples of eight elements: they travel between lanes as 32-bit piece numbers)
                 // (OFF32: a lane without a fresh sample sends the first row of its kv head: any row will do, its
                 // products are not looked at, and no load needs a select or sits in a branch)
-                const int my_piece0 = OFF32 ? (pieces[0] < 0 ? (int)piece_h : pieces[0])
-                                            : offs[0] == NO_ROW ? -1 : (int)(offs[0] >> 3);
+                const int my_piece0 = OFF32 ? (pieces[0] < 0 ? (int)piece_h : pieces[0]) : pieces[0];
                 // all cross-lane reads first, then the loads back to back: the load statements keep their order, so a
                 // cross-lane read between two of them would be waited for there
                 constexpr int NI = 32 * PPR / 64;
