@@ -737,11 +737,11 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
                      !p.kx.cached && HID <= 128 && env_nb != 2 && !two;  // (64-row programs: 204 registers, 6.7 against 3.9 ms)
     // small chunks on wide launches: every token scored once per GQA group, searches replayed on the scores
     const bool dense = prescaled && p.rope.cos == nullptr && mask_stage_dense_applies(p, HID, rows_eff);
-    // HIPATTN_MASK_DMA_INLINE: launches with a single query token fetch their rows that way too, from keys as stored
-    // (1 = always, 0 = never, default: from 16384 waves on, e.g. a batch of sequences; a lone sequence's stages of
-    // small chunks are a few hundred workgroups whose searches share rows through L1)
+    // Launches with a single query token fetch their rows that way too, from keys as stored (HIPATTN_MASK_DMA_INLINE=0:
+    // never; 2: only from 16384 waves on, e.g. a batch of sequences).  1M-key decode: 63 / 11 / 11 us against 66 / 12 /
+    // 12 us for the three stages, 16 sequences: 582 against 622 us per refresh.
     const char *e_di = getenv("HIPATTN_MASK_DMA_INLINE");
-    const int di = e_di ? atoi(e_di) : 2;
+    const int di = e_di ? atoi(e_di) : 1;
     const long long waves_one_block = (long long)p.B * p.HEAD * p.BS * p.ngroups * (BC / 16);
     const bool dma_inline = dma_mode != 0 && !far_rows && di != 0 && !dense && p.TDST == 1 && !two &&
                             p.rope.cos == nullptr && !p.kx.kv8 && !p.kx.cached && HID <= 128 && env_nb != 2 &&
