@@ -336,3 +336,28 @@ def test_prefill_scans_with_coalesced_row_fetch_on_a_small_launch(paged, m16, mo
     ctx0, meta0 = run_product(X, A, require_cache_statistics=True)
     assert torch.equal(meta0.indices, meta.indices)
     assert torch.equal(meta0.mask_cache_statistics.access_counter, meta.mask_cache_statistics.access_counter)
+
+
+def test_key_buffers_reported_as_spanning_32_gib_take_the_plain_scans(monkeypatch):
+    """The flag that keeps launches off the coalesced variants (rows passed between lanes as 31-bit piece numbers)
+    when a key buffer is too large for them: forced here on a small problem, prefill and decode."""
+    _case("far rows flag")
+    from hip_attn import operator as op
+
+    monkeypatch.setenv("HIP_ATTN_PRESCALE_K", "1")
+    monkeypatch.setenv("HIPATTN_MASK_DMA", "2")
+    X = make_inputs(16, B=1, TQ=200, TK=8192, H=8, HKV=2, D=128, dtype="bf16")
+    A = O.OArgs(sliding_window_size=512)
+    octx, ometa = O.hip_attention_12(X, A)
+    ctx, meta = run_product(X, A, require_cache_statistics=True)
+    monkeypatch.setattr(op, "_spans_32_gib", lambda t: True)
+    ctx_far, meta_far = run_product(X, A, require_cache_statistics=True)
+    assert_metadata_equal(meta_far, ometa)
+    assert torch.equal(meta_far.indices, meta.indices)
+    assert torch.equal(meta_far.mask_cache_statistics.access_counter, meta.mask_cache_statistics.access_counter)
+    assert_context_close(ctx_far, octx, "bf16")
+    Xd = make_inputs(17, B=2, TQ=1, TK=4096, H=8, HKV=2, D=128, dtype="bf16", pos=np.array([[4095], [4095]]))
+    octx, ometa = O.hip_attention_12(Xd, A)
+    ctx_far, meta_far = run_product(Xd, A)
+    assert_metadata_equal(meta_far, ometa)
+    assert_context_close(ctx_far, octx, "bf16")
