@@ -188,22 +188,34 @@ def _kv_struct(args: HiPAttentionArgs, k: Optional[Tensor], v: Optional[Tensor],
 _ZERO_FLAG: dict = {}
 
 
-def _new_statistics(args: HiPAttentionArgs, B: int, head_kv: int, pages: int, device):
-    """Zeroed ``int32 [B, HEAD_KV, pages]`` access and miss flags (attention_extend.py:1994-2006).  Without an
-    offload cache nothing can miss: the miss flags are then a read-only view of one zero kept per device, which
-    saves clearing ``B * HEAD_KV * pages`` words per call."""
-    if not args.require_cache_statistics:
-        return HiPAttentionCacheAccessStatistics(None, None)
-    access = torch.zeros((B, head_kv, pages), dtype=torch.int32, device=device)
-    if args.offload_cache is not None:
-        return HiPAttentionCacheAccessStatistics(access, torch.zeros_like(access))
+def _zero_flag(device) -> Tensor:
+    """One int32 zero per device, the target of the read-only miss flags of calls without an offload cache."""
     key = (device.type, device.index)
     zero = _ZERO_FLAG.get(key)
     if zero is None:
         zero = torch.zeros((1, 1, 1), dtype=torch.int32, device=device)
         if not (device.type == "cuda" and torch.cuda.is_current_stream_capturing()):
             _ZERO_FLAG[key] = zero  # an allocation made during graph capture belongs to that graph: not kept
-    return HiPAttentionCacheAccessStatistics(access, zero.expand(B, head_kv, pages))
+    return zero
+
+
+def _new_statistics(args: HiPAttentionArgs, B: int, head_kv: int, pages: int, device, count: int = 1):
+    """Zeroed ``int32 [B, HEAD_KV, pages]`` access and miss flags (attention_extend.py:1994-2006).  Without an
+    offload cache nothing can miss: the miss flags are then a read-only view of one zero kept per device, which
+    saves clearing ``B * HEAD_KV * pages`` words per call.  ``count`` > 1 returns that many sets whose access flags
+    are cleared by one launch (a mask refresh needs one for the scan and one for the attention)."""
+    if count > 1:
+        if not args.require_cache_statistics or args.offload_cache is not None:
+            return [_new_statistics(args, B, head_kv, pages, device) for _ in range(count)]
+        both = torch.zeros((count, B, head_kv, pages), dtype=torch.int32, device=device)
+        miss = _zero_flag(device).expand(B, head_kv, pages)
+        return [HiPAttentionCacheAccessStatistics(both[i], miss) for i in range(count)]
+    if not args.require_cache_statistics:
+        return HiPAttentionCacheAccessStatistics(None, None)
+    access = torch.zeros((B, head_kv, pages), dtype=torch.int32, device=device)
+    if args.offload_cache is not None:
+        return HiPAttentionCacheAccessStatistics(access, torch.zeros_like(access))
+    return HiPAttentionCacheAccessStatistics(access, _zero_flag(device).expand(B, head_kv, pages))
 
 
 def _mask_kv(args: HiPAttentionArgs, k_mask: Optional[Tensor], max_tsrc: int, q: Tensor, programs_rows: int,
@@ -374,7 +386,11 @@ def dual_stage_quadratic_hip_attention(
     args.update_flags()
     MAX_PAGE = args.paged_cache_page_count if (k is None and args.using_paged_cache) else MAX_TSRC
     mask_stats = None
-    sa_stats = _new_statistics(args, BSZ, HEAD_KV, MAX_PAGE, device)
+    will_scan = (cached_metadata is None) or (cached_metadata.indices is None)
+    if will_scan:
+        sa_stats, mask_stats_new = _new_statistics(args, BSZ, HEAD_KV, MAX_PAGE, device, count=2)
+    else:
+        sa_stats = _new_statistics(args, BSZ, HEAD_KV, MAX_PAGE, device)
 
     qq = q if q.stride(-1) == 1 else q.contiguous()
     rope_tabs = _rope_tables(args, q.dtype) if (args.using_extend and args.need_apply_rope) else None
@@ -397,7 +413,7 @@ def dual_stage_quadratic_hip_attention(
 
         # Keys are scaled by c_k and re-rounded every time they are sampled.  When the scan will sample
         # far more rows than the key tensor holds (prefill), scale the whole tensor once instead.
-        mask_stats = _new_statistics(args, BSZ, HEAD_KV, MAX_PAGE, device)
+        mask_stats = mask_stats_new
         mask_kv, mask_kv_pre, keep_mask_kv, khat, k_side_delta = _mask_kv(
             args, k_mask, MAX_TSRC, q, BSZ * HEAD * BDST_SCAN, chunk_count, device, stats=mask_stats, rope_tabs=rope_tabs)
 
