@@ -119,7 +119,21 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
     long long m_ko = NO_ROW, m_vo = NO_ROW;
     int m_rp = 0;
     float m_bias = -INFINITY;
+    // The index entry of a slot is requested one resolve ahead of the resolve that uses it, and the plain build looks
+    // a token's page up once for K and V: a resolve then waits for one trip to memory (the page-table entry; none on
+    // a dense tensor) instead of three in a row (index entry, page for K, page for V).
+    long long pre_s64 = 0;
+    auto index_of = [&](int tile) -> long long {  // the index entry of this lane's slot of `tile`, 0 where it has none
+        const int o = o_begin + tile * DT + lane;
+        if (lane < DT && o < o_end && o < n_sel_tok) {
+            const int bi = bk_shift >= 0 ? (o >> bk_shift) : o / p.bk;
+            return p.indices[irow * p.BK + rs + bi];
+        }
+        return 0;
+    };
     auto resolve = [&](int tile) {  // lanes 0..31
+        const long long s64 = pre_s64;
+        pre_s64 = (tile + DWAVES < ntiles) ? index_of(tile + DWAVES) : 0;
         if (lane >= DT) return;
         const int o = o_begin + tile * DT + lane;
         int t = -1, win = 0;
@@ -133,7 +147,6 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
                     const int visits = bsa_seam_multiplicity(rs + bi, p.seam_blocks, p.seam_extra);
                     if (visits > 1) bias = __logf((float)visits);
                 }
-                const long long s64 = p.indices[irow * p.BK + rs + bi];
                 const int st = (s64 >= 0 && s64 < 0x7fffffffLL) ? (int)s64 : -0x40000000;
                 t = st + e;
                 if (!(t >= p.sink && t < tlimit)) t = -1;
@@ -153,8 +166,20 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
         if (t >= 0) {
             const bool att = win ? ((long long)t <= ppos && ppos < (long long)t + p.sw) : ((long long)t + p.sw <= ppos);
             // a staged but masked token still counts as an access; its rows are not needed
-            if (att) kv_rows<true, EXT>(p.kv, kx, b, t, kvh, seqlen, ko, vo, true);
-            else {
+            if (att) {
+                if constexpr (EXT) {
+                    kv_rows<true, EXT>(p.kv, kx, b, t, kvh, seqlen, ko, vo, true);
+                } else if (!p.kv.paged) {
+                    if (t < p.kv.tsrc) {
+                        ko = (int64_t)b * p.kv.k_stride_b + (int64_t)t * p.kv.k_stride_t + (int64_t)kvh * p.kv.k_stride_h;
+                        vo = (int64_t)b * p.kv.v_stride_b + (int64_t)t * p.kv.v_stride_t + (int64_t)kvh * p.kv.v_stride_h;
+                    }
+                } else {
+                    const int64_t page = p.kv.page_of(b, t, seqlen), inpage = t & (p.kv.page_size - 1);
+                    ko = page * p.kv.k_stride_b + inpage * p.kv.k_stride_t + (int64_t)kvh * p.kv.k_stride_h;
+                    vo = page * p.kv.v_stride_b + inpage * p.kv.v_stride_t + (int64_t)kvh * p.kv.v_stride_h;
+                }
+            } else {
                 if constexpr (EXT) kv_rows<false, EXT>(p.kv, kx, b, t, kvh, seqlen, ko, vo, true);
                 ko = NO_ROW;
                 vo = NO_ROW;
@@ -216,19 +241,23 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
 
     const int my_tiles = ntiles > wid ? (ntiles - wid + DWAVES - 1) / DWAVES : 0;
     if (my_tiles > 0) {
+        pre_s64 = index_of(wid);
         resolve(wid);
         post(0);
         wave_sync();
-        fetch(0);
+        // Slots are resolved before the rows of the tile ahead are requested, never after: a resolve waits for its
+        // index and page-table entries, vector-memory operations complete in order, and behind the row loads that
+        // wait would expose their whole latency ahead of the math that is meant to hide it.
         if (my_tiles > 1) resolve(wid + DWAVES);
+        fetch(0);
     }
     for (int it = 0; it < my_tiles; it++) {
         const int cur = it & 1;
         commit(cur);                                   // rows of tile `it` -> LDS
         if (it + 1 < my_tiles) post(cur ^ 1);          // slots of tile it + 1
         wave_sync();
-        if (it + 1 < my_tiles) fetch(cur ^ 1);         // rows of tile it + 1 fly during the math below
         if (it + 2 < my_tiles) resolve(wid + (it + 2) * DWAVES);
+        if (it + 1 < my_tiles) fetch(cur ^ 1);         // rows of tile it + 1 fly during the math below
 
         // ---- S^T = K^ Q^^T  (32 tokens x 32 columns, G of them live)
         f32x16 sacc;
