@@ -210,10 +210,157 @@ __global__ __launch_bounds__(SEL_THREADS) void select_stage_kernel(const float *
 
 // The same selection for launches of a few workgroups (decode: one per sequence), where the time is the length of the
 // dependent chain and not the work: 1024 threads hold ITEMS consecutive keys (and chunk edges) each in registers, so
-// the radix passes re-read nothing, the output ranks come from one block scan of packed counts, and every selected
-// entry is written by the thread that owns it.  Keys whose low 16 bits follow from their sign (scores that were
-// rounded to bf16) need two radix passes instead of four.
+// the radix passes re-read nothing, the output ranks come from one block scan of packed counts, and the trips to
+// memory are two: every load is requested before the first is used (no load sits in a branch: an entry past the end
+// reads the last one and is ignored), and the output is written by all threads at once from a list in LDS.  Keys whose
+// low 16 bits follow from their sign (scores that were rounded to bf16) need two radix passes instead of four.
 constexpr int FAST_THREADS = 1024;
+constexpr int FAST_MAX_K = 8192;  // selected entries a workgroup can list in LDS
+
+template <int ITEMS>
+constexpr int FAST_LIST = ITEMS * FAST_THREADS < FAST_MAX_K ? ITEMS * FAST_THREADS : FAST_MAX_K;
+
+// keys of entries c0 .. c0+ITEMS-1: the maximum over the heads of the group, as order-preserving integers
+template <int ITEMS>
+__device__ __forceinline__ void fast_load_keys(const float *srow, int nheads, int n, int c0, uint32_t (&key)[ITEMS],
+                                               bool *plain_low_out) {
+    float m[ITEMS];
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) m[i] = srow[c0 + i < n ? c0 + i : n - 1];
+    for (int hh = 1; hh < nheads; hh++) {
+        float x[ITEMS];
+#pragma unroll
+        for (int i = 0; i < ITEMS; i++) x[i] = srow[(int64_t)hh * n + (c0 + i < n ? c0 + i : n - 1)];
+#pragma unroll
+        for (int i = 0; i < ITEMS; i++) m[i] = fmaxf(m[i], x[i]);
+    }
+    bool plain_low = true;  // low 16 bits are all zero (positive) / all one (negative) in every key
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) {
+        key[i] = c0 + i < n ? score_key(m[i]) : 0u;
+        if (c0 + i < n) plain_low = plain_low && ((key[i] & 0xffffu) == ((key[i] >> 31) ? 0u : 0xffffu));
+    }
+    *plain_low_out = plain_low;
+}
+
+// The k-th largest key of the workgroup's n keys (k < n): on return an entry is above the threshold when
+// (key & mask) > prefix, and of those with (key & mask) == prefix the first `need` in position order are taken.
+template <int ITEMS>
+__device__ __forceinline__ void fast_threshold(const uint32_t (&key)[ITEMS], int c0, int n, int k, bool plain_low,
+                                               int *s_hist, int *s_misc, uint32_t *prefix_out, uint32_t *mask_out,
+                                               int *need_out) {
+    const int tid = threadIdx.x;
+    uint32_t prefix = 0, mask = 0;
+    int need = k;
+    const int last_shift = __syncthreads_and(plain_low ? 1 : 0) ? 16 : 0;
+    for (int shift = 24; shift >= last_shift; shift -= 8) {
+        if (tid < 256) s_hist[tid] = 0;
+        __syncthreads();
+        {
+            int cur = -1, cnt = 0;
+#pragma unroll
+            for (int i = 0; i < ITEMS; i++) {
+                if (c0 + i < n && (key[i] & mask) == prefix) {
+                    const int bin = (int)((key[i] >> shift) & 255u);
+                    if (bin == cur) {
+                        cnt++;
+                    } else {
+                        if (cnt) atomicAdd(&s_hist[cur], cnt);
+                        cur = bin;
+                        cnt = 1;
+                    }
+                }
+            }
+            if (cnt) atomicAdd(&s_hist[cur], cnt);
+        }
+        __syncthreads();
+        if (tid < 64) {  // lane l owns bins 255-4l .. 252-4l; a prefix sum from the top finds the need-th largest
+            int hv[4];
+            int mine = 0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                hv[j] = s_hist[255 - 4 * tid - j];
+                mine += hv[j];
+            }
+            int incl = mine;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const int up = __shfl_up(incl, off);
+                if (tid >= off) incl += up;
+            }
+            int cum = incl - mine;
+            if (cum < need && need <= incl) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    if (cum < need && need <= cum + hv[j]) {
+                        s_misc[0] = 255 - 4 * tid - j;
+                        s_misc[1] = need - cum;
+                    }
+                    cum += hv[j];
+                }
+            }
+        }
+        __syncthreads();
+        prefix |= ((uint32_t)s_misc[0]) << shift;
+        mask |= 255u << shift;
+        need = s_misc[1];
+    }
+    *prefix_out = prefix;
+    *mask_out = mask;
+    *need_out = need;
+}
+
+// block-wide exclusive sum of one packed pair of 16-bit counts per thread (1024 threads); *total: the sum over all
+__device__ __forceinline__ uint32_t fast_excl_scan(uint32_t packed, uint32_t *s_wave, uint32_t *total) {
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    uint32_t incl = packed;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t up = __shfl_up(incl, off);
+        if (lane >= off) incl += up;
+    }
+    if (lane == 63) s_wave[wid] = incl;
+    __syncthreads();
+    // the sixteen wave totals: lane w of every wave takes one, a scan over sixteen lanes gives base and total
+    uint32_t wt = lane < FAST_THREADS / 64 ? s_wave[lane] : 0u;
+    uint32_t winc = wt;
+#pragma unroll
+    for (int off = 1; off < FAST_THREADS / 64; off <<= 1) {
+        const uint32_t up = __shfl_up(winc, off);
+        if (lane >= off) winc += up;
+    }
+    const uint32_t base = __shfl(winc - wt, wid);
+    *total = __shfl(winc, FAST_THREADS / 64 - 1);
+    return base + incl - packed;
+}
+
+// Output rank of every selected entry of this thread (-1: not selected).  all: every entry is selected.
+template <int ITEMS>
+__device__ __forceinline__ void fast_ranks(const uint32_t (&key)[ITEMS], int c0, int n, bool all, uint32_t prefix,
+                                           uint32_t mask, int need, uint32_t *s_wave, int (&rank)[ITEMS]) {
+    uint32_t packed = 0;  // low half: entries above the threshold, high half: entries equal to it
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) {
+        if (c0 + i < n) {
+            const uint32_t mk = key[i] & mask;
+            packed += all ? 1u : ((mk > prefix ? 1u : 0u) + (mk == prefix ? 0x10000u : 0u));
+        }
+    }
+    uint32_t total;
+    const uint32_t before = fast_excl_scan(packed, s_wave, &total);
+    int gt_before = (int)(before & 0xffffu), eq_before = (int)(before >> 16);
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) {
+        rank[i] = -1;
+        if (c0 + i >= n) continue;
+        const uint32_t mk = key[i] & mask;
+        const bool gt = all || mk > prefix;
+        const bool eq = !all && mk == prefix;
+        if (gt || (eq && eq_before < need)) rank[i] = gt_before + (eq_before < need ? eq_before : need);
+        gt_before += gt ? 1 : 0;
+        eq_before += eq ? 1 : 0;
+    }
+}
 
 template <int ITEMS>
 __global__ __launch_bounds__(FAST_THREADS) void select_stage_fast_kernel(const float *scores, const int32_t *chunk_left,
@@ -224,8 +371,9 @@ __global__ __launch_bounds__(FAST_THREADS) void select_stage_fast_kernel(const f
     __shared__ int s_hist[256];
     __shared__ int s_misc[2];
     __shared__ uint32_t s_wave[FAST_THREADS / 64];
+    __shared__ int s_left[FAST_LIST<ITEMS>];  // left edges of the selected chunks in output order
 
-    const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+    const int tid = threadIdx.x;
     const int hgi = blockIdx.x % hg;
     const int o = (blockIdx.x / hg) % bs_out;
     const int b = blockIdx.x / (hg * bs_out);
@@ -235,125 +383,34 @@ __global__ __launch_bounds__(FAST_THREADS) void select_stage_fast_kernel(const f
     const int32_t *lrow = chunk_left + (((int64_t)b * bs_in + i_in) * hg + hgi) * n;
     const int64_t obase = (((int64_t)b * bs_out + o) * hg + hgi) * ((int64_t)k * splits);
 
-    uint32_t key[ITEMS];
-    int left[ITEMS];
     const int c0 = tid * ITEMS;
-    bool plain_low = true;  // low 16 bits are all zero (positive) / all one (negative) in every key
+    int left[ITEMS];
 #pragma unroll
-    for (int i = 0; i < ITEMS; i++) {
-        const int c = c0 + i;
-        key[i] = 0u;
-        left[i] = 0;
-        if (c < n) {
-            float m = srow[c];
-            for (int hh = 1; hh < nheads; hh++) m = fmaxf(m, srow[(int64_t)hh * n + c]);
-            key[i] = score_key(m);
-            left[i] = lrow[c];
-            plain_low = plain_low && ((key[i] & 0xffffu) == ((key[i] >> 31) ? 0u : 0xffffu));
-        }
-    }
+    for (int i = 0; i < ITEMS; i++) left[i] = lrow[c0 + i < n ? c0 + i : n - 1];
+    uint32_t key[ITEMS];
+    bool plain_low;
+    fast_load_keys<ITEMS>(srow, nheads, n, c0, key, &plain_low);
+
     uint32_t prefix = 0, mask = 0;
-    int need = k;
-    if (k < n) {
-        const int last_shift = __syncthreads_and(plain_low ? 1 : 0) ? 16 : 0;
-        for (int shift = 24; shift >= last_shift; shift -= 8) {
-            if (tid < 256) s_hist[tid] = 0;
-            __syncthreads();
-            {
-                int cur = -1, cnt = 0;
+    int need = 0;  // k >= n: everything is selected, no key equals the (empty) threshold
+    if (k < n) fast_threshold<ITEMS>(key, c0, n, k, plain_low, s_hist, s_misc, &prefix, &mask, &need);
+    int rank[ITEMS];
+    fast_ranks<ITEMS>(key, c0, n, k >= n, prefix, mask, need, s_wave, rank);
 #pragma unroll
-                for (int i = 0; i < ITEMS; i++) {
-                    if (c0 + i < n && (key[i] & mask) == prefix) {
-                        const int bin = (int)((key[i] >> shift) & 255u);
-                        if (bin == cur) {
-                            cnt++;
-                        } else {
-                            if (cnt) atomicAdd(&s_hist[cur], cnt);
-                            cur = bin;
-                            cnt = 1;
-                        }
-                    }
-                }
-                if (cnt) atomicAdd(&s_hist[cur], cnt);
-            }
-            __syncthreads();
-            if (tid < 64) {  // lane l owns bins 255-4l .. 252-4l; a prefix sum from the top finds the need-th largest
-                int hv[4];
-                int mine = 0;
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    hv[j] = s_hist[255 - 4 * tid - j];
-                    mine += hv[j];
-                }
-                int incl = mine;
-#pragma unroll
-                for (int off = 1; off < 64; off <<= 1) {
-                    const int up = __shfl_up(incl, off);
-                    if (tid >= off) incl += up;
-                }
-                int cum = incl - mine;
-                if (cum < need && need <= incl) {
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        if (cum < need && need <= cum + hv[j]) {
-                            s_misc[0] = 255 - 4 * tid - j;
-                            s_misc[1] = need - cum;
-                        }
-                        cum += hv[j];
-                    }
-                }
-            }
-            __syncthreads();
-            prefix |= ((uint32_t)s_misc[0]) << shift;
-            mask |= 255u << shift;
-            need = s_misc[1];
-        }
-    } else {
-        need = 0;  // everything is selected: no key equals the (empty) threshold, every key is above it
-    }
-    // ranks: entries above the threshold always, entries equal to it in position order until `need` are taken
-    const bool all = k >= n;
-    uint32_t packed = 0;  // low half: entries above the threshold, high half: entries equal to it
-#pragma unroll
-    for (int i = 0; i < ITEMS; i++) {
-        if (c0 + i < n) {
-            const uint32_t mk = key[i] & mask;
-            packed += all ? 1u : ((mk > prefix ? 1u : 0u) + (mk == prefix ? 0x10000u : 0u));
-        }
-    }
-    uint32_t incl = packed;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const uint32_t up = __shfl_up(incl, off);
-        if (lane >= off) incl += up;
-    }
-    if (lane == 63) s_wave[wid] = incl;
+    for (int i = 0; i < ITEMS; i++)
+        if (rank[i] >= 0) s_left[rank[i]] = left[i];
     __syncthreads();
-    uint32_t before = incl - packed;
-    for (int w = 0; w < wid; w++) before += s_wave[w];
-    int gt_before = (int)(before & 0xffffu), eq_before = (int)(before >> 16);
-#pragma unroll
-    for (int i = 0; i < ITEMS; i++) {
-        if (c0 + i >= n) continue;
-        const uint32_t mk = key[i] & mask;
-        const bool gt = all || mk > prefix;
-        const bool eq = !all && mk == prefix;
-        const bool sel = gt || (eq && eq_before < need);
-        if (sel) {
-            const int e = gt_before + (eq_before < need ? eq_before : need);
-            for (int j = 0; j < splits; j++) {
-                const int v = left[i] + j * sub_chunk;
-                const int64_t at = obase + (int64_t)e * splits + j;
-                next_left[at] = v;
-                if (next_scores) next_scores[at] = -INFINITY;
-                if (left64) {
-                    left64[at] = v;
-                    right64[at] = (int64_t)v + sub_chunk;
-                }
-            }
+    // exactly k entries are selected (k <= n): every thread emits sub-chunks of its own
+    const int total = k * splits;
+    for (int idx = tid; idx < total; idx += FAST_THREADS) {
+        const int e = idx / splits, j = idx - e * splits;
+        const int v = s_left[e] + j * sub_chunk;
+        next_left[obase + idx] = v;
+        if (next_scores) next_scores[obase + idx] = -INFINITY;  // the next stage's head-reduced scores start here
+        if (left64) {  // the same list as the next stage's cached inputs: int64 edges (left, left + chunk)
+            left64[obase + idx] = v;
+            right64[obase + idx] = (int64_t)v + sub_chunk;
         }
-        gt_before += gt ? 1 : 0;
-        eq_before += eq ? 1 : 0;
     }
 }
 
@@ -454,6 +511,92 @@ __global__ __launch_bounds__(SEL_THREADS) void finalize_kernel(const float *scor
     }
 }
 
+// The same layout for launches of a few query blocks (decode), one workgroup of 1024 threads per (batch, query
+// block, head): like select_stage_fast_kernel the selection runs on keys held in registers, the refined left edge of
+// every entry is requested together with its scores, and the row is deduplicated from a list in LDS, so that the
+// kernel makes two trips to memory.
+template <int ITEMS>
+__global__ __launch_bounds__(FAST_THREADS) void finalize_fast_kernel(const float *scores, const int32_t *left_out,
+                                                                    const int64_t *pos, int64_t pos_sb, int64_t pos_st,
+                                                                    int bs, int bdst, int scan_stride, int HEAD,
+                                                                    int score_heads, int hg, int n, int K, int chunk,
+                                                                    int bq, int64_t *indices, int64_t *ks,
+                                                                    int32_t *ks_start_end) {
+    __shared__ int s_hist[256];
+    __shared__ int s_misc[2];
+    __shared__ uint32_t s_wave[FAST_THREADS / 64];
+    __shared__ int s_val[ITEMS * FAST_THREADS];  // block-aligned left edges of the selected entries in output order
+
+    const int tid = threadIdx.x;
+    const int nheads = HEAD / hg;
+    const int hh = blockIdx.x % nheads;
+    const int wg = blockIdx.x / nheads;
+    const int hgi = wg % hg;
+    const int qb = (wg / hg) % bdst;
+    const int b = wg / (hg * bdst);
+    const int i_in = (qb + scan_stride * bs - bdst) / scan_stride;
+    const int nsh = score_heads / hg;
+    const int BK = K < n ? K : n;
+    const int h = hgi * nheads + hh;
+    const float *srow = scores + (((int64_t)b * bs + i_in) * score_heads + (int64_t)hgi * nsh) * n;
+    const int32_t *lrow = left_out + (((int64_t)b * bs + i_in) * HEAD + h) * n;
+    int64_t *irow = indices + (((int64_t)b * HEAD + h) * bdst + qb) * BK;
+
+    const int c0 = tid * ITEMS;
+    const int64_t first_pos = pos[(int64_t)b * pos_sb + (int64_t)qb * bq * pos_st];
+    int val[ITEMS];
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) val[i] = lrow[c0 + i < n ? c0 + i : n - 1];
+    uint32_t key[ITEMS];
+    bool plain_low;
+    fast_load_keys<ITEMS>(srow, nsh, n, c0, key, &plain_low);
+    const int64_t limit = first_pos + bq;
+
+    uint32_t prefix = 0, mask = 0;
+    int need = 0;
+    if (BK < n) fast_threshold<ITEMS>(key, c0, n, BK, plain_low, s_hist, s_misc, &prefix, &mask, &need);
+    int rank[ITEMS];
+    fast_ranks<ITEMS>(key, c0, n, BK >= n, prefix, mask, need, s_wave, rank);
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++)
+        if (rank[i] >= 0) s_val[rank[i]] = val[i] / chunk * chunk;  // aligned down to the block grid
+    __syncthreads();
+
+    // entries o0 .. o0+ITEMS-1 of the selected list: an entry is kept when it differs from the one before it
+    // (roll(1): entry 0 is compared with the last), and counts as active when it lies before the block's end
+    const int o0 = tid * ITEMS;
+    int v[ITEMS];
+    uint32_t packed = 0;  // low half: kept entries, high half: active ones
+    uint32_t keep = 0;
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) {
+        const int o = o0 + i;
+        v[i] = 0;
+        if (o < BK) {
+            v[i] = s_val[o];
+            const int prev = s_val[o == 0 ? BK - 1 : o - 1];
+            if (v[i] != prev) {
+                keep |= 1u << i;
+                packed += 1u + (((int64_t)v[i] < limit) ? 0x10000u : 0u);
+            }
+        }
+    }
+    uint32_t total;
+    const uint32_t before = fast_excl_scan(packed, s_wave, &total);
+    int at = (int)(before & 0xffffu);
+    const int tot_u = (int)(total & 0xffffu), tot_a = (int)(total >> 16);
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++)
+        if ((keep >> i) & 1u) irow[at++] = v[i];
+    for (int o = tot_u + tid; o < BK; o += FAST_THREADS) irow[o] = 0x7fffffffffffffffLL;
+    if (tid == 0) {
+        const int64_t r = ((int64_t)b * HEAD + h) * bdst + qb;
+        ks[r] = tot_a;
+        ks_start_end[r * 2 + 0] = 0;
+        ks_start_end[r * 2 + 1] = tot_a;
+    }
+}
+
 }  // namespace hipattn
 
 using namespace hipattn;
@@ -474,12 +617,10 @@ extern "C" int hipattn_select_stage(const float *scores, const int32_t *chunk_le
     HIPATTN_CHECK_ARG(bs_out <= row_rep * bs_in, HIPATTN_E_ARG, "select stage: bs_out > row_rep*bs_in");
     HIPATTN_CHECK_ARG(n <= SEL_MAX_N, HIPATTN_E_UNSUPPORTED, "select stage: %d chunks exceed the limit %d", n, SEL_MAX_N);
     dim3 grid((unsigned)(B * bs_out * hg)), block(SEL_THREADS);
-    static int fast = -1;  // HIPATTN_SELECT_FAST=0 keeps the throughput kernel everywhere (cross-checking aid)
-    if (fast < 0) {
-        const char *e = getenv("HIPATTN_SELECT_FAST");
-        fast = (e && e[0] == '0') ? 0 : 1;
-    }
-    if (fast && grid.x <= 64) {  // a few workgroups: the latency kernel
+    // HIPATTN_SELECT_FAST=0 keeps the throughput kernel everywhere (read on every call: tests switch it in one process)
+    const char *fast_env = getenv("HIPATTN_SELECT_FAST");
+    const bool fast = !(fast_env && fast_env[0] == '0');
+    if (fast && grid.x <= 64 && k <= FAST_MAX_K) {  // a few workgroups: the latency kernel
         dim3 fblock(FAST_THREADS);
 #define SEL_FAST(IT)                                                                                                  \
     hipLaunchKernelGGL(select_stage_fast_kernel<IT>, grid, fblock, 0, (hipStream_t)stream, scores, chunk_left, bs_in, \
@@ -514,9 +655,24 @@ extern "C" int hipattn_finalize_indices(const float *scores, const int32_t *left
                       "finalize: score_heads must be HEAD, or 1 with hg == 1");
     HIPATTN_CHECK_ARG(bdst <= scan_stride * bs, HIPATTN_E_ARG, "finalize: bdst > scan_stride*bs");
     HIPATTN_CHECK_ARG(n <= SEL_MAX_N, HIPATTN_E_UNSUPPORTED, "finalize: %d chunks exceed the limit %d", n, SEL_MAX_N);
-    // few query blocks (decode): slice each group's heads over several workgroups so that the chip is not idle
     const long long groups = (long long)B * bdst * hg;
     const int nheads = HEAD / hg;
+    // HIPATTN_SELECT_FAST=0 keeps the throughput kernel everywhere (read on every call: tests switch it in one process)
+    const char *fast_env = getenv("HIPATTN_SELECT_FAST");
+    const bool fast = !(fast_env && fast_env[0] == '0');
+    if (fast && groups * nheads <= 1024 && n <= 4 * FAST_THREADS) {  // few query blocks (decode): the latency kernel
+        dim3 fgrid((unsigned)(groups * nheads)), fblock(FAST_THREADS);
+#define FIN_FAST(IT)                                                                                                  \
+    hipLaunchKernelGGL(finalize_fast_kernel<IT>, fgrid, fblock, 0, (hipStream_t)stream, scores, left_out, pos,        \
+                       pos_stride_b, pos_stride_t, bs, bdst, scan_stride, HEAD, score_heads, hg, n, K, chunk_size, bq, \
+                       indices, ks, ks_start_end)
+        if (n <= FAST_THREADS) FIN_FAST(1);
+        else FIN_FAST(4);
+#undef FIN_FAST
+        HIPATTN_CHECK_HIP(hipGetLastError());
+        return 0;
+    }
+    // otherwise slice each group's heads over several workgroups while the launch is small
     int hsplit = 1;
     while (hsplit < nheads && groups * hsplit < 512) hsplit *= 2;
     if (hsplit > nheads) hsplit = nheads;
