@@ -346,6 +346,7 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
         uint4 raw[(VIA_LDS || DMA) ? 1 : NB][(VIA_LDS || DMA) ? 1 : KS];
         int64_t offs[NB];
         int pieces[NB];  // OFF32: the sampled row as a piece number, -1 = none
+        int mark[NB];    // coalesced fetch: the access flag (token or page) this lane sets for its sample, -1 = none
 #pragma unroll
         for (int tb = 0; tb < NB; tb++) {
             active[tb] = real[tb] && (cl[tb] < cr[tb]) && (cl[tb] <= lim) && (cl[tb] >= 0);
@@ -362,19 +363,20 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
             int64_t off = NO_ROW;
             if constexpr (DMA) {
                 pieces[tb] = -1;
+                mark[tb] = -1;
                 if (active[tb] && !reuse[tb]) {
                     const int t = tok[tb];
                     if (OFF32 || !p.kv.paged) {
                         if (t >= 0 && t < tsrc32) {
                             pieces[tb] = OFF32 ? (int)(__umul24((uint32_t)t, piece_st) + piece_h)
                                                : (int)((uint32_t)t * piece_st + piece_h);
-                            if (flag_row && hh == 0 && !(share_now && wv != 0)) flag_row[t] = 1;
+                            if (flag_row && hh == 0 && !(share_now && wv != 0)) mark[tb] = t;
                         }
                     } else if (t >= 0) {
                         // the block table's entry, or page 0 beyond the sequence (as the general routine reads it)
                         const uint32_t page = (uint32_t)p.kv.page_of(b, t, seqlen);
                         pieces[tb] = (int)(page * piece_sb + (uint32_t)(t & (p.kv.page_size - 1)) * piece_st + piece_h);
-                        if (flag_row && hh == 0 && !(share_now && wv != 0)) flag_row[page] = 1;
+                        if (flag_row && hh == 0 && !(share_now && wv != 0)) mark[tb] = (int)page;
                     }
                 }
             } else if (active[tb] && !reuse[tb]) {
@@ -465,6 +467,14 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                 }
                 wait_vmcnt<0>();
                 if (share_now) __syncthreads();  // every wave's quarter has landed
+            }
+            // the access flags of the round's samples are set once its rows have landed: vector-memory operations
+            // complete in order, so a store requested ahead of the rows would have to be acknowledged before the
+            // wait for them ends; from here the stores have the products of the round to complete behind
+            if (flag_row) {
+#pragma unroll
+                for (int tb = 0; tb < NB; tb++)
+                    if (mark[tb] >= 0) flag_row[mark[tb]] = 1;
             }
         }
         bool any_fresh = false;  // uniform over the wave, and the LDS path's workgroups are one wave
