@@ -325,10 +325,19 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     if constexpr (ROPE) cross_side = p.rope.backend != HIPATTN_EXTEND_RELATIVE;
     int ptok[NB];
     float pscore[NB];
+    // Paged keys, coalesced fetch: a round first needs its token's page-table entry, a trip to memory ahead of the
+    // trip for the row.  Which token a lane samples next depends only on which half wins this round, so both
+    // candidates' entries are requested now, ahead of this round's rows, and have arrived when the round ends.
+    int pf_tok[NB][2];       // the candidates (-1: none, or outside the sequence: page 0)
+    uint32_t pf_page[NB][2]; // their entries, not looked at before the next round
+    bool pf_in[NB][2];
 #pragma unroll
     for (int tb = 0; tb < NB; tb++) {
         ptok[tb] = -1;
         pscore[tb] = 0.0f;
+        pf_tok[tb][0] = pf_tok[tb][1] = -1;
+        pf_page[tb][0] = pf_page[tb][1] = 0u;
+        pf_in[tb][0] = pf_in[tb][1] = false;
     }
     // The first round of a search samples tokens that do not depend on the query: the four heads of a workgroup
     // (same chunks, same keys) want the same 32 rows, so each wave fetches a quarter of them into a tile they all read
@@ -374,9 +383,32 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                         }
                     } else if (t >= 0) {
                         // the block table's entry, or page 0 beyond the sequence (as the general routine reads it)
-                        const uint32_t page = (uint32_t)p.kv.page_of(b, t, seqlen);
+                        uint32_t page;
+                        if (t == pf_tok[tb][0]) page = pf_in[tb][0] ? pf_page[tb][0] : 0u;
+                        else if (t == pf_tok[tb][1]) page = pf_in[tb][1] ? pf_page[tb][1] : 0u;
+                        else page = (uint32_t)p.kv.page_of(b, t, seqlen);
                         pieces[tb] = (int)(page * piece_sb + (uint32_t)(t & (p.kv.page_size - 1)) * piece_st + piece_h);
                         if (flag_row && hh == 0 && !(share_now && wv != 0)) mark[tb] = (int)page;
+                    }
+                }
+                if constexpr (!OFF32 && RMODE != 4) {  // (the 32-row variant has no registers to spare for it)
+                    if (p.kv.paged) {
+                        // next round's token of this lane if the left half wins, and if the right half does
+                        const int ctr_l = (cl[tb] + ctr[tb]) >> 1, ctr_r = (ctr[tb] + cr[tb]) >> 1;
+                        const int cand[2] = {side ? ((ctr_l + ctr[tb]) >> 1) : ((cl[tb] + ctr_l) >> 1),
+                                             side ? ((ctr_r + cr[tb]) >> 1) : ((ctr[tb] + ctr_r) >> 1)};
+#pragma unroll
+                        for (int w = 0; w < 2; w++) {
+                            // no load in a branch: a token outside the sequence reads the entry of the sequence's
+                            // first token and is given page 0, as the general routine gives it
+                            const bool in_seq = cand[w] >= 0 && (int64_t)cand[w] < seqlen;
+                            const int64_t e = (int64_t)b * p.kv.bt_stride_b + (in_seq ? (cand[w] >> p.kv.page_shift) : 0);
+                            // the low word of an entry is the page number, in a table of either width
+                            const uint32_t entry = reinterpret_cast<const uint32_t *>(p.kv.block_table)[p.kv.bt_is64 ? 2 * e : e];
+                            pf_tok[tb][w] = cand[w];
+                            pf_page[tb][w] = entry;
+                            pf_in[tb][w] = in_seq;
+                        }
                     }
                 }
             } else if (active[tb] && !reuse[tb]) {
