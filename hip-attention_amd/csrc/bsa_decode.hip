@@ -413,6 +413,21 @@ extern "C" int hipattn_bsa_decode_partial(const hipattn_q_t *q, const hipattn_kv
 
 extern "C" int hipattn_bsa_decode_merge(const void *workspace, int32_t B, int32_t HEAD, int32_t HID, int32_t nsplits,
                                         int32_t dtype, void *out, int64_t out_stride_b, int64_t out_stride_h,
+                                        void *stream);
+
+extern "C" int hipattn_bsa_decode(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t *indices,
+                                  const int32_t *ks_start_end, int32_t idx_rows, int32_t BK, int32_t block_size_k,
+                                  int32_t sliding_window, int32_t sink, int32_t second_stage_k, int32_t nsplits,
+                                  void *workspace, void *out, int64_t out_stride_b, int64_t out_stride_h, void *stream) {
+    HIPATTN_CHECK_ARG(q && out, HIPATTN_E_ARG, "decode: null pointer");
+    const int rc = hipattn_bsa_decode_partial(q, kv, indices, ks_start_end, idx_rows, BK, block_size_k, sliding_window,
+                                              sink, second_stage_k, nsplits, workspace, stream);
+    if (rc) return rc;
+    return hipattn_bsa_decode_merge(workspace, q->B, q->HEAD, q->HID, nsplits, q->dtype, out, out_stride_b, out_stride_h, stream);
+}
+
+extern "C" int hipattn_bsa_decode_merge(const void *workspace, int32_t B, int32_t HEAD, int32_t HID, int32_t nsplits,
+                                        int32_t dtype, void *out, int64_t out_stride_b, int64_t out_stride_h,
                                         void *stream) {
     HIPATTN_CHECK_ARG(workspace && out, HIPATTN_E_ARG, "decode merge: null pointer");
     HIPATTN_CHECK_ARG(B > 0 && HEAD > 0 && nsplits > 0, HIPATTN_E_ARG, "decode merge: non-positive size");

@@ -109,7 +109,7 @@ def lib():
         L.hipattn_mask_stage_workspace_bytes.restype = ctypes.c_int64
         L.hipattn_bsa_decode_default_splits.restype = ctypes.c_int32
         for name in ("hipattn_mask_stage", "hipattn_prescale_k", "hipattn_select_stage", "hipattn_finalize_indices",
-                     "hipattn_bsa_prefill", "hipattn_bsa_decode_partial", "hipattn_bsa_decode_merge",
+                     "hipattn_bsa_prefill", "hipattn_bsa_decode_partial", "hipattn_bsa_decode_merge", "hipattn_bsa_decode",
                      "hipattn_bsa_decode_static",
                      "hipattn_cache_sizes", "hipattn_cache_create", "hipattn_cache_flush",
                      "hipattn_cache_lookup_and_schedule", "hipattn_cache_commit", "hipattn_cache_write_rows",
@@ -145,7 +145,15 @@ def storage_code(t: torch.Tensor) -> int:
     return FP8_E5M2 if t.dtype in _FP8_DTYPES else dtype_code(t)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr(device) -> ctypes.c_void_p:
+    """The current stream of ``device`` as the pointer the C ABI takes (the raw-handle query where torch has it: a
+    tenth of the cost of building a ``torch.cuda.Stream`` object, on a path that makes one per launch)."""
+    if _raw_stream is not None:
+        idx = getattr(device, "index", None)
+        return ctypes.c_void_p(_raw_stream(torch.cuda.current_device() if idx is None else idx))
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
@@ -397,16 +405,12 @@ def bsa_decode(qs, kvs, indices, ks_start_end, BK, bk, sw, sink, out, device, ns
     if workspace is None or workspace.numel() * workspace.element_size() < need:
         workspace = torch.empty(need // 4, dtype=torch.float32, device=out.device)
     with _timed("bsa_decode"):
-      rc = L.hipattn_bsa_decode_partial(
+      rc = L.hipattn_bsa_decode(
         ctypes.byref(qs), ctypes.byref(kvs), _p(indices), _p(ks_start_end), ctypes.c_int32(indices.shape[1]),
         ctypes.c_int32(BK), ctypes.c_int32(bk), ctypes.c_int32(sw), ctypes.c_int32(sink),
-        ctypes.c_int32(second_stage_k), ctypes.c_int32(nsplits), _p(workspace), stream_ptr(device))
-    check(rc, "hipattn_bsa_decode_partial")
-    rc = L.hipattn_bsa_decode_merge(
-        _p(workspace), ctypes.c_int32(B), ctypes.c_int32(HEAD), ctypes.c_int32(HID), ctypes.c_int32(nsplits),
-        ctypes.c_int32(qs.dtype), _p(out), ctypes.c_int64(out.stride(0)), ctypes.c_int64(out.stride(2)),
-        stream_ptr(device))
-    check(rc, "hipattn_bsa_decode_merge")
+        ctypes.c_int32(second_stage_k), ctypes.c_int32(nsplits), _p(workspace), _p(out),
+        ctypes.c_int64(out.stride(0)), ctypes.c_int64(out.stride(2)), stream_ptr(device))
+    check(rc, "hipattn_bsa_decode")
     return workspace
 
 

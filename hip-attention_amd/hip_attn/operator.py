@@ -610,7 +610,7 @@ def dual_stage_quadratic_hip_attention(
     seq_pos = position_ids[:, -q_bsa.shape[1]:]
     context = block_sparse_attention(
         q_bsa, k, v, seq_pos, indices, ks_start_end, args, MAX_TSRC, decode=use_decode, rows_shared=rows_shared,
-        khat=khat if (args.k_mask is None) else None, stats=sa_stats, rope_tables=rope_tabs,
+        khat=khat if (args.k_mask is None) else None, stats=sa_stats, rope_tables=rope_tabs, operands_checked=True,
     )
 
     metadata = HiPAttentionOutputMetadata(
@@ -644,7 +644,7 @@ def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], 
                            ks_start_end: Tensor, args: HiPAttentionArgs, max_tsrc: int, decode: bool = False,
                            impl: int = 0, rows_shared: bool = False, khat: Optional[Tensor] = None,
                            stats: Optional[HiPAttentionCacheAccessStatistics] = None,
-                           rope_tables=None) -> Tensor:
+                           rope_tables=None, operands_checked: bool = False) -> Tensor:
     """Sparse attention over (selected blocks, sink, sliding window) given the metadata tensors.
 
     ``position_ids`` are 0-based (the reference passes ``seq_lens = position_ids + 1``,
@@ -663,7 +663,8 @@ def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], 
     device = q.device
     if not q.is_cuda:
         raise N.HipAttnError("block_sparse_attention runs on the GPU only: q must be a device tensor")
-    _check_operands(q, k, v, args)
+    if not operands_checked:  # the operator above has looked at the same tensors already
+        _check_operands(q, k, v, args)
     qq = q if q.stride(-1) == 1 else q.contiguous()
     kvs, keep = _kv_struct(args, k, v, max_tsrc, masking=False, stats=stats)
     if position_ids.dtype != torch.int64:

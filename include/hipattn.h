@@ -256,6 +256,12 @@ int hipattn_bsa_decode_partial(const hipattn_q_t *q, const hipattn_kv_t *kv, con
 int hipattn_bsa_decode_merge(const void *workspace, int32_t B, int32_t HEAD, int32_t HID,
                              int32_t nsplits, int32_t dtype, void *out, int64_t out_stride_b,
                              int64_t out_stride_h, void *stream);
+/* The two calls above as one (two launches; the same decode_block_sparse_attention,
+ * attention_decode_bsa.py:1331-1435): for hosts on which a call into the library costs as much as a launch. */
+int hipattn_bsa_decode(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t *indices,
+                       const int32_t *ks_start_end, int32_t idx_rows, int32_t BK, int32_t block_size_k,
+                       int32_t sliding_window, int32_t sink, int32_t second_stage_k, int32_t nsplits,
+                       void *workspace, void *out, int64_t out_stride_b, int64_t out_stride_h, void *stream);
 
 /* Decode attention that allocates nothing and needs no workspace: hipattn_bsa_decode_partial followed by
  * hipattn_bsa_decode_merge with the split partials kept in a device array inside the library.  It has no

@@ -15,7 +15,7 @@ def _declared_functions():
 def test_header_declares_the_expected_surface():
     names = _declared_functions()
     for must in ("hipattn_mask_stage", "hipattn_select_stage", "hipattn_finalize_indices", "hipattn_bsa_prefill",
-                 "hipattn_bsa_decode_partial", "hipattn_bsa_decode_merge", "hipattn_version"):
+                 "hipattn_bsa_decode_partial", "hipattn_bsa_decode_merge", "hipattn_bsa_decode", "hipattn_version"):
         assert must in names
 
 
