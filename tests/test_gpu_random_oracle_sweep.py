@@ -53,3 +53,48 @@ def test_random_calls_match_the_oracle():
         assert_context_close(ctx, octx, dtype)
         ctx2, _ = run_product(X, A, cached=meta, require_cache_statistics=stats)
         assert_context_close(ctx2, octx, dtype)
+
+
+def test_random_calls_with_rotation_on_load_match_the_oracle():
+    """Thirty draws over the rotation rules of the scan (relative / streaming / infllm / dynamic_extend) and of the
+    attention (streaming / infllm / dynamic_extend), model context lengths below and above the key length, logit
+    soft-capping on / off, prefill and ragged paged decode.  (Eighty cases of the same draw found no difference.)"""
+    from helpers import tiny_args, with_rope
+
+    rng = random.Random(21)
+    for it in range(30):
+        D = rng.choice([64, 128])
+        HKV = rng.choice([1, 2])
+        H = HKV * rng.choice([1, 2, 4])
+        decode = rng.random() < 0.4
+        TK = rng.choice([1500, 2048, 3000, 4096])
+        TQ = 1 if decode else rng.choice([1, 40, 130, 200, 256])
+        B = rng.choice([1, 2])
+        paged = rng.choice([0, 1, 16]) if not decode else rng.choice([1, 16])
+        dtype = rng.choice(["bf16", "bf16", "f32"])
+        scan = rng.choice(["relative", "streaming", "infllm", "dynamic_extend"])
+        sa = rng.choice(["streaming", "infllm", "dynamic_extend"])
+        model_ctx = rng.choice([1024, 2048, 131072])
+        cap = rng.choice([None, None, 30.0])
+        if decode:
+            lens = np.array([rng.randint(TK // 2, TK) for _ in range(B)])
+            X = make_inputs(2000 + it, B=B, TQ=1, TK=TK, H=H, HKV=HKV, D=D, dtype=dtype, pos=(lens - 1)[:, None],
+                            scale=0.5)
+        else:
+            lens = None
+            X = make_inputs(2000 + it, B=B, TQ=TQ, TK=TK, H=H, HKV=HKV, D=D, dtype=dtype, scale=0.5)
+        kw = dict(using_extend=True, need_apply_rope=True, scan_extend_backend=scan, sa_extend_backend=sa,
+                  model_context_length=model_ctx)
+        if cap:
+            kw["logit_softcap"] = cap
+        if paged:
+            X = to_paged(X, paged, seed=it, seq_lens=lens) if decode else to_paged(X, paged, seed=it)
+            kw["extend_context_length"] = TK
+        X = with_rope(X, 8192)
+        print(f"[case {it}] {dtype} D={D} H={H}/{HKV} B={B} TQ={TQ} TK={TK} paged={paged} scan={scan} sa={sa} "
+              f"model_ctx={model_ctx} softcap={cap} decode={decode}", flush=True)
+        A = tiny_args(**kw)
+        octx, ometa = O.hip_attention_12(X, A)
+        ctx, meta = run_product(X, A)
+        assert_metadata_equal(meta, ometa)
+        assert_context_close(ctx, octx, dtype)
