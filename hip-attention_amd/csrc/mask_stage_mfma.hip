@@ -82,6 +82,7 @@ constexpr int mask_stage_waves(int HID, int MB, int NB, int RMODE) {
 // theirs (k-step 2j lower half, 2j upper half, 2j + 1 lower, 2j + 1 upper): the accumulation chain of a score, and
 // with it every bit of the result, is the same (compared on 2M products of adversarial inputs, while any other order
 // of the groups differs in a quarter of them), at half the matrix cycles, 24 registers fewer and no rows of zeros.
+// RMODE = 9: as 6, with the 32-bit row offsets of RMODE = 5 (a dense key tensor under 4 GB per batch item).
 // RMODE = 6: a single query token (as RMODE = 3) with the rows fetched as under RMODE = 4; keys prescaled or scaled
 // after the tile is read back.
 // RMODE = 3 (no rotation, one token block per wave, a single query token): the one valid program row is that token's
@@ -91,13 +92,13 @@ template <int HID, int MB, int NB, bool PRESCALED, bool VIA_LDS, bool EXT, int R
 __global__ __launch_bounds__(VIA_LDS ? 64 : 256) __attribute__((amdgpu_waves_per_eu(mask_stage_waves(HID, MB, NB, RMODE))))
 void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     constexpr bool ROPE = RMODE == 1;
-    constexpr bool QINL = RMODE == 3 || RMODE == 6;  // query rows scaled here instead of read from the prepared workspace
+    constexpr bool QINL = RMODE == 3 || RMODE == 6 || RMODE == 9;  // query rows scaled here instead of read from the prepared workspace
     static_assert(!QINL || NB == 1, "inline query rows: the one-token-block variants only");
-    constexpr bool DMA = RMODE >= 4 && RMODE <= 8;  // rows fetched coalesced, straight into a per-wave LDS tile
-    constexpr bool OFF32 = RMODE == 5 || RMODE == 7;  // their addresses: 32-bit byte offsets from the batch item's first key row
+    constexpr bool DMA = RMODE >= 4 && RMODE <= 9;  // rows fetched coalesced, straight into a per-wave LDS tile
+    constexpr bool OFF32 = RMODE == 5 || RMODE == 7 || RMODE == 9;  // their addresses: 32-bit byte offsets from the batch item's first key row
     constexpr bool M16 = RMODE == 7 || RMODE == 8;    // programs of up to 16 query rows on the 16x16x32 instruction
     static_assert(!DMA || (!VIA_LDS && NB == 1 && !KV8), "coalesced direct-to-LDS rows: one token block per wave, bf16 keys");
-    static_assert(!DMA || RMODE == 6 || PRESCALED, "coalesced rows on wide launches: prescaled keys");
+    static_assert(!DMA || RMODE == 6 || RMODE == 9 || PRESCALED, "coalesced rows on wide launches: prescaled keys");
     static_assert(!M16 || (MB == 1 && HID % 32 == 0), "16-row variant: one row block, head dim a multiple of 32");
     static_assert(!KV8 || (EXT && !PRESCALED), "fp8 keys: extended build, scaled in the kernel");
     static_assert(!ROPE || (EXT && !VIA_LDS && !PRESCALED), "rope variant: direct path of the extended build");
@@ -111,7 +112,7 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     constexpr int NROWS = NB * 32;                // sampled rows per iteration of this wave
     constexpr int SWZ = (PPR < 16 ? PPR : 16) - 1;
     constexpr int SWZ_DIV = PPR < 16 ? 16 / PPR : 1;
-    constexpr bool SHAREABLE = DMA && PRESCALED && RMODE != 6;  // prefill variants: the first round's rows can be fetched once per workgroup
+    constexpr bool SHAREABLE = DMA && PRESCALED && RMODE != 6 && RMODE != 9;  // prefill variants: the first round's rows can be fetched once per workgroup
     __shared__ __align__(16) uint4 s_rows[VIA_LDS ? NROWS * PPR : DMA ? (SHAREABLE ? 5 : 4) * 32 * PPR : 1];  // DMA: one tile per wave (up to four), one shared
     __shared__ int64_t s_off[VIA_LDS ? NROWS : 1];
     // a workgroup holds `hpw` waves = `hpw` query heads of one GQA group working on the same chunks:
@@ -887,13 +888,13 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
         set_error("mask stage: prescaled keys cannot be combined with fp8 key storage");
         return HIPATTN_E_ARG;
     }
+    // a dense key tensor whose batch items span less than 4 GB: row addresses as 32-bit offsets
+    const long long item_bytes = 2LL * ((p.kv.tsrc - 1) * p.kv.k_stride_t + (long long)(p.kv.HKV - 1) * p.kv.k_stride_h + HID);
+    const bool off32 = !p.kv.paged && p.kv.k_stride_t >= 0 && p.kv.k_stride_h >= 0 && p.kv.k_stride_t % 8 == 0 &&
+                       p.kv.k_stride_h % 8 == 0 && p.kv.k_stride_b % 8 == 0 && item_bytes < (1LL << 32) &&
+                       p.kv.tsrc < (1LL << 24) && (p.kv.k_stride_t >> 3) < (1LL << 24);
     if (dma && !q_inline) {
         if constexpr (HID <= 128) {
-            // a dense key tensor whose batch items span less than 4 GB: row addresses as 32-bit offsets
-            const long long item_bytes = 2LL * ((p.kv.tsrc - 1) * p.kv.k_stride_t + (long long)(p.kv.HKV - 1) * p.kv.k_stride_h + HID);
-            const bool off32 = !p.kv.paged && p.kv.k_stride_t >= 0 && p.kv.k_stride_h >= 0 && p.kv.k_stride_t % 8 == 0 &&
-                               p.kv.k_stride_h % 8 == 0 && p.kv.k_stride_b % 8 == 0 && item_bytes < (1LL << 32) &&
-                               p.kv.tsrc < (1LL << 24) && (p.kv.k_stride_t >> 3) < (1LL << 24);
             // Programs of up to 16 query rows take the 16x16x32 form of the products (HIPATTN_MASK_M16=0: the 32x32x16
             // form).  Same bits, half the matrix cycles, 92 registers instead of 128, and the same time to within 2%
             // (cfg-2-like prefill: 2.07 / 2.65 against 2.07 / 2.66 ms): these launches are held by the vector-memory
@@ -916,8 +917,14 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
     }
     if (dma_inline) {
         if constexpr (HID <= 128) {
-            if (prescaled) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 6>), grid, block, 0, st, p, nsub, hpw);
-            else hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, false, false, true, 6>), grid, block, 0, st, p, nsub, hpw);
+            if (off32) {
+                if (prescaled) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 9>), grid, block, 0, st, p, nsub, hpw);
+                else hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, false, false, true, 9>), grid, block, 0, st, p, nsub, hpw);
+            } else if (prescaled) {
+                hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, true, false, true, 6>), grid, block, 0, st, p, nsub, hpw);
+            } else {
+                hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, false, false, true, 6>), grid, block, 0, st, p, nsub, hpw);
+            }
             HIPATTN_CHECK_HIP(hipGetLastError());
             return 0;
         }
