@@ -152,7 +152,9 @@ def stream_ptr(device) -> ctypes.c_void_p:
     """The current stream of ``device`` as the pointer the C ABI takes (the raw-handle query where torch has it: a
     tenth of the cost of building a ``torch.cuda.Stream`` object, on a path that makes one per launch)."""
     if _raw_stream is not None:
-        idx = getattr(device, "index", None)
+        if not isinstance(device, torch.device):
+            device = torch.device(device)
+        idx = device.index
         return ctypes.c_void_p(_raw_stream(torch.cuda.current_device() if idx is None else idx))
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
