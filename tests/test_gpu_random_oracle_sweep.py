@@ -145,3 +145,49 @@ def test_random_calls_on_fp8_caches_match_the_oracle():
         ctx, meta = _run(XQ, A, kc, vc, as_bytes)
         assert_metadata_equal(meta, ometa)
         assert_context_close(ctx, octx, "bf16")
+
+
+def test_random_offload_caches_equal_resident_keys_and_the_oracle():
+    """Sixteen draws of an offloaded key pool behind device caches of random sizes (from far too small, so that blocks
+    are evicted in every step, to holding everything), block sizes 8 / 16 / 32, ragged batches, prefill and decode:
+    over four steps with a commit after each, masks must equal the oracle's and contexts the resident run's bit for
+    bit.  (Fifty cases of the same draw found no difference.)"""
+    import torch
+    from gpu_utils import to_torch
+    from hip_attn import HiPOffloadCache, hip_attention_12
+    from test_gpu_offload import _args, _bits, _fill, _offloaded_case
+
+    rng = random.Random(51)
+    for it in range(16):
+        D = rng.choice([64, 128])
+        HKV = rng.choice([1, 2, 4])
+        H = HKV * rng.choice([1, 2, 4])
+        B = rng.choice([1, 2, 3])
+        TK = rng.choice([1024, 2048, 3000, 4096])
+        TQ = rng.choice([1, 1, 1, 17, 64])
+        lens = np.array([rng.randint(max(TK // 2, 600), TK) for _ in range(B)])
+        mask_tokens = rng.choice([1 << 20, 4096, 1024, 256])
+        sa_tokens = rng.choice([1 << 20, 4096, 1024, 512])
+        block_tokens = rng.choice([16, 16, 8, 32])
+        print(f"[case {it}] D={D} H={H}/{HKV} B={B} TQ={TQ} TK={TK} lens={lens.tolist()} mask_tokens={mask_tokens} "
+              f"sa_tokens={sa_tokens} block_tokens={block_tokens}", flush=True)
+        X, XP = _offloaded_case(4000 + it, B, TK, H, HKV, D, lens, TQ)
+        A = O.OArgs(sliding_window_size=256, second_stage_k=512, extend_context_length=TK,
+                    stages=[O.OStage(64, 4, 64, None, 1), O.OStage(64, 4, 16, 1024, 1), O.OStage(64, 1, 8, 512, 1)])
+        octx, ometa = O.hip_attention_12(XP, A)
+        rows = XP.k_cache.shape[0]
+        cache = HiPOffloadCache(0, rows, mask_tokens, sa_tokens, HKV, D, torch.bfloat16, torch.device("cuda"),
+                                block_tokens=block_tokens)
+        _fill(cache, XP)
+        q = to_torch(X.q, "bf16")
+        res_args = _args(XP, A, k_cache=to_torch(XP.k_cache, "bf16"), v_cache=to_torch(XP.v_cache, "bf16"))
+        ctx_res, meta_res = hip_attention_12(q, None, None, res_args)
+        assert_metadata_equal(meta_res, ometa)
+        for step in range(4):
+            ctx, meta = hip_attention_12(q, None, None, _args(XP, A, offload_cache=cache))
+            torch.cuda.synchronize()
+            assert_metadata_equal(meta, ometa)
+            assert torch.equal(_bits(ctx), _bits(ctx_res)), f"case {it}, step {step}: offloaded context differs"
+            cache.handle_cache_miss(meta)
+        assert_context_close(ctx, octx, "bf16")
+        del cache
