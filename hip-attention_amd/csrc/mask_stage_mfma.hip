@@ -329,6 +329,7 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     // Paged keys, coalesced fetch: a round first needs its token's page-table entry, a trip to memory ahead of the
     // trip for the row.  Which token a lane samples next depends only on which half wins this round, so both
     // candidates' entries are requested now, ahead of this round's rows, and have arrived when the round ends.
+    int last_mark[NB];       // the access flag this lane stored last in this search (-1: none yet)
     int pf_tok[NB][2];       // the candidates (-1: none, or outside the sequence: page 0)
     uint32_t pf_page[NB][2]; // their entries, not looked at before the next round
     bool pf_in[NB][2];
@@ -336,6 +337,7 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     for (int tb = 0; tb < NB; tb++) {
         ptok[tb] = -1;
         pscore[tb] = 0.0f;
+        last_mark[tb] = -1;
         pf_tok[tb][0] = pf_tok[tb][1] = -1;
         pf_page[tb][0] = pf_page[tb][1] = 0u;
         pf_in[tb][0] = pf_in[tb][1] = false;
@@ -504,10 +506,14 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
             // the access flags of the round's samples are set once its rows have landed: vector-memory operations
             // complete in order, so a store requested ahead of the rows would have to be acknowledged before the
             // wait for them ends; from here the stores have the products of the round to complete behind
+            // (a search that has narrowed to a few tokens keeps sampling the same page: its flag is stored once)
             if (flag_row) {
 #pragma unroll
                 for (int tb = 0; tb < NB; tb++)
-                    if (mark[tb] >= 0) flag_row[mark[tb]] = 1;
+                    if (mark[tb] >= 0 && mark[tb] != last_mark[tb]) {
+                        flag_row[mark[tb]] = 1;
+                        last_mark[tb] = mark[tb];
+                    }
             }
         }
         bool any_fresh = false;  // uniform over the wave, and the LDS path's workgroups are one wave
