@@ -163,12 +163,22 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
             }
         }
         int64_t ko = NO_ROW, vo = NO_ROW;
+        // access flags of a paged cache are per page, and the slots of a tile are mostly runs of consecutive tokens:
+        // the first slot of a run inside a page stores the flag for the run (an offload cache keeps its own marks
+        // per block, which need not be pages: there every slot marks)
+        bool flag_leader = true;
+        if constexpr (EXT) {
+            const int t_before = __shfl_up(t, 1);
+            if (p.kv.paged && !kx->cached)
+                flag_leader = lane == 0 || t < 0 || t_before != t - 1 || (t & (p.kv.page_size - 1)) == 0 || (int64_t)t >= seqlen;
+        }
         if (t >= 0) {
             const bool att = win ? ((long long)t <= ppos && ppos < (long long)t + p.sw) : ((long long)t + p.sw <= ppos);
             // a staged but masked token still counts as an access; its rows are not needed
             if (att) {
                 if constexpr (EXT) {
-                    kv_rows<true, EXT>(p.kv, kx, b, t, kvh, seqlen, ko, vo, true);
+                    // (flags are stored without looking first: a look is a trip to memory in a chain of them)
+                    kv_rows<true, EXT, false>(p.kv, kx, b, t, kvh, seqlen, ko, vo, flag_leader);
                 } else if (!p.kv.paged) {
                     if (t < p.kv.tsrc) {
                         ko = (int64_t)b * p.kv.k_stride_b + (int64_t)t * p.kv.k_stride_t + (int64_t)kvh * p.kv.k_stride_h;
