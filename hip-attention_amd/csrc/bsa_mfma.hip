@@ -48,6 +48,173 @@ struct MfmaSmem {
 };
 static_assert(sizeof(MfmaSmem<256>) <= 160 * 1024, "LDS of a compute unit");
 
+
+// ---------------------------------------------------------------- the pipelined tile loop (head dim <= 128)
+// The matrix unit and the vector unit of a SIMD run side by side: while a 32x32x16 product occupies the matrix unit
+// for 32 cycles, the same wave can issue about six ordinary vector instructions for free.  A tile loop made of phases
+// (products, then softmax, then products) never offers the two units work at the same time, so the loop below is
+// software-pipelined by half tiles of 32 tokens: one step issues the products S^T(h+1) = K^ Q^^T and
+// O^T += V^T P^T(h-1) together with the softmax of S^T(h), none of which depends on another, and the compiler is
+// told to interleave them (sched_group_barrier).  K of tile i and V of tile i-1 are staged in the same iteration, so
+// that every iteration reads one K buffer and one V buffer and one barrier per tile still suffices.
+
+// One pipeline step: the products S^T(next half) = K^ Q^^T and O^T += V^T P^T(previous half) beside the online
+// softmax of the half in between.  kh: this lane's K^ fragment address in the half tile whose logits are produced
+// (k-step ks at + 16 * ks elements); vh: this lane's address for the transposing reads of the half tile whose P^T is
+// consumed (k-step u at + 16 * u rows, 32-row block db of O^T at + 32 * db elements, second four tokens 8 rows
+// further).  QK = false: the step after the last tile (no logits to produce).
+//
+// The softmax of a block of logits is cut in two.  Its head (mask, maximum, new reference point, the factor alpha
+// that the accumulator is due) runs in the tail of the step that produced the block, once the products have
+// delivered it; its body (exponentials, row sums, packing P) runs in the next step.  So a step opens with its first
+// product and every vector instruction of the loop sits in the shadow of a product.  State handed from step to step
+// with a block: its logits, minus its reference point (m_neg) and alpha.
+//
+// Element i of a lane's S^T block is token slot (i / 4) * 8 + hh * 4 + i % 4 of its half.  mask_next (wave-uniform):
+// a token t of the produced block is attended iff (unsigned)(t - att_lo) < att_span (empty slots hold -1); only the
+// masking itself sits in a branch, so that the accumulators have one home whichever way a step goes.
+// The order of the instructions is laid down here and fenced (sched_barrier): operands of a product are read from
+// LDS DEPTH products ahead and every product is followed by its share of the vector work.  chore(c), c = 0..15, is
+// called behind product c * NM / 16: the staging work of the loop (reading posted row addresses, storing the staged
+// rows of the next tile into LDS, issuing the loads of the tile after it) rides in the same shadow.
+#define PIN3(a, b, c) asm volatile("" : "+v"(a), "+v"(b), "+v"(c))  // keeps what computes a, b, c in front of it
+struct SoftmaxCarry {
+    float m_neg;   // minus the reference point of the block (0 while nothing has been seen)
+    float alpha;   // what raising the reference point to it costs the accumulator and the row sum
+};
+template <int HID, bool CAP, bool QK, typename Chore>
+__device__ __forceinline__ void pipe_step(const uint16_t *kh, const uint16_t *vh, const Frag (&qf)[HID / 16],
+                                          f32x16 (&oacc)[HID / 32], const Frag (&p_in)[2], f32x16 &s_out, f32x16 &s,
+                                          Frag (&pf)[2], const SoftmaxCarry cur, SoftmaxCarry &next, float &m_run,
+                                          float &l_run, bool mask_next, const int *tok_next, int hh, int att_lo,
+                                          unsigned att_span, float cap, float cap_k2, Chore &&chore) {
+    constexpr int KS = QK ? HID / 16 : 0, DB = HID / 32, VROW = HID + VPAD;
+    constexpr int NM = KS + 2 * DB;   // products of this step
+    constexpr int DEPTH = 4 < NM ? 4 : NM;  // operands in flight
+    constexpr int EPS = 16 / NM;      // exponentials per product
+    constexpr int MSPLIT = QK ? 10 * NM / 16 : NM;  // the produced block is complete before this product
+    static_assert(NM * EPS == 16, "the step spreads 16 logits over its products");
+    static_assert(!QK || MSPLIT >= KS + 1, "the head of the next softmax starts behind the last product that feeds it");
+    auto fetch = [&](int m) {
+        Frag a;
+        if (m < KS) {
+            a.q = *reinterpret_cast<const uint4 *>(kh + m * 16);
+        } else {
+            const int u = (m - KS) / DB, db = (m - KS) % DB;
+            a.d[0] = lds_read_tr16(vh + u * 16 * VROW + db * 32);
+            a.d[1] = lds_read_tr16(vh + (u * 16 + 8) * VROW + db * 32);
+        }
+        return a;
+    };
+    Frag ring[DEPTH];
+#pragma unroll
+    for (int m = 0; m < DEPTH; m++) ring[m] = fetch(m);
+    const float m_neg = cur.m_neg;
+    float lsum0 = 0.0f, lsum1 = 0.0f;
+    f32x16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[i] = 0.0f;
+    float mx = -INFINITY, m_use = m_run, alpha_n = 1.0f;
+    auto product = [&](int m) {
+        if (m < KS) {
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[m % DEPTH].v, qf[m < KS ? m : 0].v, acc, 0, 0, 0);
+        } else {
+            const int u = (m - KS) / DB, db = (m - KS) % DB;
+            oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[m % DEPTH].v, p_in[u].v, oacc[db], 0, 0, 0);
+        }
+        if (m + DEPTH < NM) ring[m % DEPTH] = fetch(m + DEPTH);
+    };
+    auto body = [&](int m) {  // exponentials of the block in hand
+#pragma unroll
+        for (int j = 0; j < EPS; j += 2) {
+            if constexpr (EPS >= 2) {
+                const int i = m * EPS + j;
+                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], LOG2E, m_neg));
+                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i + 1], LOG2E, m_neg));
+                lsum0 += p0;
+                lsum1 += p1;
+                pf[i / 8].u[(i % 8) / 2] = cvt_pk_bf16(p0, p1);
+                PIN3(lsum0, lsum1, pf[i / 8].u[(i % 8) / 2]);
+            }
+        }
+        if constexpr (EPS == 1) {
+            // one logit per product: the pair is packed behind every other one
+            const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[m], LOG2E, m_neg));
+            s[m] = pv;
+            if (m & 1) {
+                lsum0 += s[m - 1];
+                lsum1 += pv;
+                pf[m / 8].u[(m % 8) / 2] = cvt_pk_bf16(s[m - 1], pv);
+                PIN3(lsum0, lsum1, pf[m / 8].u[(m % 8) / 2]);
+            }
+        }
+    };
+    auto head = [&](int c) {  // head of the softmax of the produced block, in five pieces (c = 10 .. 14)
+        if (c == 10) {
+            mx = fmaxf(acc[0], acc[1]);
+#pragma unroll
+            for (int i = 2; i < 8; i += 2) mx = fmaxf(fmaxf(mx, acc[i]), acc[i + 1]);   // v_max3_f32
+        }
+        if (c == 11) {
+#pragma unroll
+            for (int i = 8; i < 16; i += 2) mx = fmaxf(fmaxf(mx, acc[i]), acc[i + 1]);
+        }
+        if (c == 12) mx = fmaxf(mx, swap_halves(mx)) * LOG2E;
+        if (c == 13) {
+            // raise the reference point only when the maximum grew noticeably
+            const bool raise = mx > m_run + RESCALE_STEP || m_run == -INFINITY;
+            m_use = raise ? fmaxf(m_run, mx) : m_run;
+            alpha_n = __builtin_amdgcn_exp2f(m_run - m_use);  // an unchanged point gives 1, a first one 0
+            PIN3(mx, m_use, alpha_n);
+        }
+        if (c == 14) {
+            next.alpha = (m_use == -INFINITY) ? 1.0f : alpha_n;   // nothing seen yet: -inf - -inf
+            next.m_neg = (m_use == -INFINITY) ? 0.0f : -m_use;
+            m_run = m_use;
+            PIN3(next.alpha, next.m_neg, m_run);
+        }
+    };
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int m = 0; m < MSPLIT; m++) {
+        product(m);
+        body(m);
+#pragma unroll
+        for (int c = m * 16 / NM; c < (m + 1) * 16 / NM; c++) chore(c);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (QK) {
+        if constexpr (CAP) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[i] = softcap_logit(acc[i], cap, cap_k2);
+        }
+        if (mask_next) {
+#pragma unroll
+            for (int i4 = 0; i4 < 4; i4++) {
+                const int4 tt = *reinterpret_cast<const int4 *>(tok_next + i4 * 8 + hh * 4);
+                const int ts[4] = {tt.x, tt.y, tt.z, tt.w};
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    acc[i4 * 4 + e] = ((unsigned)(ts[e] - att_lo) < att_span) ? acc[i4 * 4 + e] : -INFINITY;
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = MSPLIT; m < NM; m++) {
+            product(m);
+            body(m);
+#pragma unroll
+            for (int c = m * 16 / NM; c < (m + 1) * 16 / NM; c++) {
+                head(c);
+                chore(c);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    l_run = l_run * cur.alpha + (lsum0 + lsum1);
+    s_out = acc;
+}
+
 // ROPE = true (extended parameter block, unscaled keys): query rows and staged key rows are rotated on load.
 // A query lane holds both halves of its row (k-steps ks and ks + KS/2); the two halves of a staged key row are
 // fetched by lanes tid and tid ^ (HID/16) of one wave.
@@ -234,21 +401,21 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
             mt.all_valid = allv;
         }
     };
-    // tiles first .. first + HB - 1, spread over the waves
+    // tiles first .. first + HB - 1, spread over the waves; the two tiles past the end resolve to rows of zeros, so
+    // that the pipelined loop can stage ahead without asking where the list ends
     auto resolve_batch = [&](int first) {
-        for (int t = first + wid; t < first + HB && t < ntiles; t += NTHREADS / 64) resolve(t);
+        for (int t = first + wid; t < first + HB && t <= ntiles + 1; t += NTHREADS / 64) resolve(t);
     };
     uint4 kreg[CPT], vreg[CPT];
     uint4 creg[ROPE ? CPT : 1], sreg[ROPE ? CPT : 1];  // cos / sin pieces of the staged key rows
-    auto prefetch = [&](int tile) {
+    auto prefetch_k = [&](int tile) {
         const MfmaMeta &mt = sm.meta[tile & (2 * HB - 1)];
-        long long ka[CPT], va[CPT];
+        long long ka[CPT];
         int rp[CPT];
 #pragma unroll
         for (int j = 0; j < CPT; j++) {
             const int slot = (tid + NTHREADS * j) / (HID / 8);
             ka[j] = mt.ko[slot];
-            va[j] = mt.vo[slot];
             if constexpr (ROPE) rp[j] = mt.rp[slot];
         }
 #pragma unroll
@@ -259,11 +426,18 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
                 creg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr);
                 sreg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr);
             }
-            kreg[j] = load_kv_piece<KV8>((const void *)ka[j], piece * 8);
-            vreg[j] = load_kv_piece<KV8>((const void *)va[j], piece * 8);
+            kreg[j] = load_kv_piece_global<KV8>(ka[j], piece * 8);
         }
     };
-    auto commit = [&](int buf) {
+    auto prefetch_v = [&](int tile) {
+        const MfmaMeta &mt = sm.meta[tile & (2 * HB - 1)];
+        long long va[CPT];
+#pragma unroll
+        for (int j = 0; j < CPT; j++) va[j] = mt.vo[(tid + NTHREADS * j) / (HID / 8)];
+#pragma unroll
+        for (int j = 0; j < CPT; j++) vreg[j] = load_kv_piece_global<KV8>(va[j], ((tid + NTHREADS * j) % (HID / 8)) * 8);
+    };
+    auto commit_k = [&](int buf) {
 #pragma unroll
         for (int j = 0; j < CPT; j++) {
             const int c = tid + NTHREADS * j;
@@ -281,7 +455,13 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
                 kq.w = cvt_pk_bf16(__uint_as_float(kq.w << 16) * p.c_k, __uint_as_float(kq.w & 0xffff0000u) * p.c_k);
             }
             *reinterpret_cast<uint4 *>(&sm.k[buf][slot][piece * 8]) = kq;
-            *reinterpret_cast<uint4 *>(&sm.v[buf][slot][piece * 8]) = vreg[j];
+        }
+    };
+    auto commit_v = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < CPT; j++) {
+            const int c = tid + NTHREADS * j;
+            *reinterpret_cast<uint4 *>(&sm.v[buf][c / (HID / 8)][(c % (HID / 8)) * 8]) = vreg[j];
         }
     };
 
@@ -294,30 +474,180 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
     float m_run = -INFINITY;   // in log2 units, already multiplied by log2(e)
     float l_run = 0.0f;
 
+    // what the mask shortcut needs of a tile: is every (valid row, token) pair attended, and is it a window tile
+    auto tile_full = [&](int tile, bool &window) {
+        const MfmaMeta &mt = sm.meta[tile & (2 * HB - 1)];
+        const int tmin = __builtin_amdgcn_readfirstlane(mt.tmin), tmax = __builtin_amdgcn_readfirstlane(mt.tmax);
+        const bool all_valid = __builtin_amdgcn_readfirstlane(mt.all_valid) != 0;
+        window = tile >= tiles_sel + tiles_sink;
+        if (!window) return all_valid && ((long long)tmax + p.sw <= pmin_blk);
+        return all_valid && (tmax <= pmin_blk) && ((long long)pmax_blk < (long long)tmin + p.sw);
+    };
+
+    if constexpr (HID <= 128) {
+        // ---- pipelined loop (see pipe_step)
+        constexpr int KROW = HID + KPAD, VROW = HID + VPAD;
+        // the V buffer the first iteration multiplies by P = 0 must hold finite values
+        for (int c = tid; c < TN * VROW / 8; c += NTHREADS) reinterpret_cast<uint4 *>(&sm.v[1][0][0])[c] = make_uint4(0, 0, 0, 0);
+        const int k_off = col * KROW + hh * 8;
+        const int v_off = (hh * 4 + ((lane & 15) >> 2)) * VROW + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+        // attended token ranges of this lane's query row: far keys 0 <= t <= pq - sw, window keys
+        // max(0, pq - sw + 1) <= t <= pq; a row that does not exist attends nothing
+        const long long far_hi = (long long)pq - p.sw;
+        const unsigned far_span = far_hi >= 0 ? (unsigned)far_hi + 1u : 0u;
+        const int win_lo = far_hi + 1 > 0 ? (int)(far_hi + 1) : 0;
+        const unsigned win_span = pq >= win_lo ? (unsigned)(pq - win_lo) + 1u : 0u;
+        float cap = 0.0f, cap_k2 = 0.0f;
+        if constexpr (CAP) {
+            cap = p.softcap;
+            cap_k2 = 2.0f * LOG2E / p.softcap;
+        }
+        f32x16 s_a, s_b;   // logits of the first / second half of a tile
+        Frag p_a[2], p_b[2];
+#pragma unroll
+        for (int i = 0; i < 16; i++) { s_a[i] = -INFINITY; s_b[i] = -INFINITY; }
+#pragma unroll
+        for (int u = 0; u < 2; u++) { p_a[u].q = make_uint4(0, 0, 0, 0); p_b[u].q = make_uint4(0, 0, 0, 0); }
+        SoftmaxCarry c_a = {0.0f, 1.0f}, c_b = {0.0f, 1.0f};
+        auto rescale = [&](float alpha) {
+            if (__any(alpha != 1.0f)) {
+#pragma unroll
+                for (int db = 0; db < DB; db++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+            }
+        };
+        // posted row addresses of the rows this thread stages, read a step ahead of their loads, and the summary of
+        // the next tile
+        long long ka[CPT], va[CPT];
+        int rpk[ROPE ? CPT : 1];
+        int nx_tmin = 0, nx_tmax = -1, nx_allv = 0;
+        auto read_posted = [&](int i) {  // iteration i loads K of tile i + 2 and V of tile i + 1
+            const MfmaMeta &mk = sm.meta[(i + 2) & (2 * HB - 1)], &mv = sm.meta[(i + 1) & (2 * HB - 1)];
+#pragma unroll
+            for (int j = 0; j < CPT; j++) {
+                const int slot = (tid + NTHREADS * j) / (HID / 8);
+                ka[j] = mk.ko[slot];
+                va[j] = mv.vo[slot];
+                if constexpr (ROPE) rpk[j] = mk.rp[slot];
+            }
+            nx_tmin = mv.tmin;
+            nx_tmax = mv.tmax;
+            nx_allv = mv.all_valid;
+        };
+        auto issue_loads = [&]() {
+#pragma unroll
+            for (int j = 0; j < CPT; j++) {
+                const int piece = (tid + NTHREADS * j) % (HID / 8);
+                if constexpr (ROPE) {
+                    const int64_t tr = (int64_t)rpk[j] * p.rope.stride_t + (piece % (HID / 16)) * 8;
+                    creg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr);
+                    sreg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr);
+                }
+                kreg[j] = load_kv_piece_global<KV8>(ka[j], piece * 8);
+                vreg[j] = load_kv_piece_global<KV8>(va[j], piece * 8);
+            }
+        };
+        auto full_of = [&](int tile, int tmin, int tmax, int allv, bool &window) {
+            window = tile >= tiles_sel + tiles_sink;
+            if (!window) return allv != 0 && ((long long)tmax + p.sw <= pmin_blk);
+            return allv != 0 && (tmax <= pmin_blk) && ((long long)pmax_blk < (long long)tmin + p.sw);
+        };
+        if (ntiles > 0) {
+            // K of tile 0 into LDS, K of tile 1 and V of tile 0 on their way
+            resolve_batch(0);
+            __syncthreads();
+            prefetch_k(0);
+            commit_k(0);
+            prefetch_k(1);
+            prefetch_v(0);
+            bool window_cur;
+            bool full_cur = tile_full(0, window_cur);
+            if (!head_ok) {
+                // a wave without rows of its own stages its share of every tile and keeps the barriers company (a
+                // loop of its own: merged with the other as a branch, the staging registers of the two paths meet
+                // in copies at the end of every iteration, behind a wait for the loads in flight)
+                for (int i = 0; i < ntiles; i++) {
+                    __syncthreads();
+                    if (((i + 3) & (HB - 1)) == 0 && i + 3 <= ntiles + 1) resolve_batch(i + 3);
+                    read_posted(i);
+                    commit_k((i + 1) & 1);
+                    commit_v(i & 1);
+                    issue_loads();
+                }
+                __syncthreads();
+                return;
+            }
+            for (int i = 0; i < ntiles; i++) {
+                __syncthreads();  // K of tile i and V of tile i - 1 are in LDS (stored during the last iteration)
+                // the batch of tiles whose addresses are read three iterations from now
+                if (((i + 3) & (HB - 1)) == 0 && i + 3 <= ntiles + 1) resolve_batch(i + 3);
+                const uint16_t *kt = &sm.k[i & 1][0][0] + k_off;
+                const uint16_t *vt = &sm.v[(i - 1) & 1][0][0] + v_off;
+                const int *tok_cur = sm.meta[i & (2 * HB - 1)].tok;
+                // step A: logits of the first half of tile i, O += V P of the first half of tile i - 1, exponentials
+                // of the second half of tile i - 1
+                pipe_step<HID, CAP, true>(kt, vt, qf, oacc, p_a, s_a, s_b, p_b, c_b, c_a, m_run, l_run, !full_cur, tok_cur, hh,
+                                          window_cur ? win_lo : 0, window_cur ? win_span : far_span, cap, cap_k2,
+                                          [&](int c) { if (c == 1) read_posted(i); });
+                rescale(c_b.alpha);
+                // step B: logits of the second half of tile i, O += V P of the second half of tile i - 1,
+                // exponentials of the first half of tile i.  Beside it K of tile i + 1 and V of tile i go to LDS (their
+                // buffers were last read before this iteration's barrier) and the loads of the tile after are issued.
+                pipe_step<HID, CAP, true>(kt + 32 * KROW, vt + 32 * VROW, qf, oacc, p_b, s_b, s_a, p_a, c_a, c_b, m_run, l_run, !full_cur,
+                                          tok_cur + 32, hh, window_cur ? win_lo : 0, window_cur ? win_span : far_span, cap, cap_k2,
+                                          [&](int c) {
+                                              if (c == 1) commit_k((i + 1) & 1);
+                                              if (c == 3) commit_v(i & 1);
+                                              if (c == 6) issue_loads();
+                                          });
+                rescale(c_a.alpha);
+                full_cur = full_of(i + 1, __builtin_amdgcn_readfirstlane(nx_tmin), __builtin_amdgcn_readfirstlane(nx_tmax),
+                                   __builtin_amdgcn_readfirstlane(nx_allv), window_cur);
+            }
+            // drain: the softmax of the last tile's second half and its two products with V
+            __syncthreads();
+            {
+                const uint16_t *vt = &sm.v[(ntiles - 1) & 1][0][0] + v_off;
+                f32x16 s_none;
+                pipe_step<HID, CAP, false>(nullptr, vt, qf, oacc, p_a, s_none, s_b, p_b, c_b, c_a, m_run, l_run, false, nullptr, hh, 0, 0u,
+                                           cap, cap_k2, [](int) {});
+                rescale(c_b.alpha);
+#pragma unroll
+                for (int u = 0; u < 2; u++)
+#pragma unroll
+                    for (int db = 0; db < DB; db++) {
+                        Frag a;
+                        a.d[0] = lds_read_tr16(vt + (32 + u * 16) * VROW + db * 32);
+                        a.d[1] = lds_read_tr16(vt + (32 + u * 16 + 8) * VROW + db * 32);
+                        oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, p_b[u].v, oacc[db], 0, 0, 0);
+                    }
+            }
+        }
+    } else {
     if (ntiles > 0) {
         resolve_batch(0);
         __syncthreads();
-        prefetch(0);
+        prefetch_k(0);
+        prefetch_v(0);
     }
     for (int tile = 0; tile < ntiles; tile++) {
         const int buf = tile & 1;
-        commit(buf);
+        commit_k(buf);
+        commit_v(buf);
         __syncthreads();
-        if (tile + 1 < ntiles) prefetch(tile + 1);
+        if (tile + 1 < ntiles) {
+            prefetch_k(tile + 1);
+            prefetch_v(tile + 1);
+        }
         // the next batch of tiles: its half of the ring was last read a batch ago, and the barrier of the next
         // round stands between these writes and their first use
         if (((tile + 2) & (HB - 1)) == 0 && tile + 2 < ntiles) resolve_batch(tile + 2);
         const MfmaMeta &mt = sm.meta[tile & (2 * HB - 1)];
-        const bool window = tile >= tiles_sel + tiles_sink;
-
-        // tile summary (token range, all valid?) posted by wave 0
-        const int tmin = __builtin_amdgcn_readfirstlane(mt.tmin), tmax = __builtin_amdgcn_readfirstlane(mt.tmax);
-        const bool all_valid = __builtin_amdgcn_readfirstlane(mt.all_valid) != 0;
-        bool full;  // every (valid row, token) pair of the tile is attended
-        if (!window) full = all_valid && ((long long)tmax + p.sw <= pmin_blk);
-        else full = all_valid && (tmax <= pmin_blk) && ((long long)pmax_blk < (long long)tmin + p.sw);
+        bool window;
+        const bool full = tile_full(tile, window);
+        const int tmax = __builtin_amdgcn_readfirstlane(mt.tmax);
         if (tmax < 0 || !head_ok) continue;  // nothing valid in this tile, or an idle wave (both wave-uniform)
-
         // ---- S^T = K^ Q^^T
         f32x16 sacc[2];
 #pragma unroll
@@ -413,6 +743,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
                 oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pf[j].v, oacc[db], 0, 0, 0);
             }
         }
+    }
     }
 
     // ---- epilogue: O^T[d, m] / l -> out[b, m, h, d]

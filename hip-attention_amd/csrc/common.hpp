@@ -204,20 +204,35 @@ struct KVView {
 // uvm_gpu_cache.py:1043-1046); every value is widened to bf16 on load, which is exact.  Offsets stay in elements.
 typedef __attribute__((ext_vector_type(2))) float kv_f32x2;
 
+// eight fp8 (e5m2) bytes widened to four packed bf16 pairs (exact, so plain truncation packs the pairs)
+__device__ __forceinline__ uint4 widen_bf8x8(uint2 r) {
+    const kv_f32x2 a = __builtin_amdgcn_cvt_pk_f32_bf8((int)r.x, false), b = __builtin_amdgcn_cvt_pk_f32_bf8((int)r.x, true);
+    const kv_f32x2 c = __builtin_amdgcn_cvt_pk_f32_bf8((int)r.y, false), d = __builtin_amdgcn_cvt_pk_f32_bf8((int)r.y, true);
+    return make_uint4((__float_as_uint(a[0]) >> 16) | (__float_as_uint(a[1]) & 0xffff0000u),
+                      (__float_as_uint(b[0]) >> 16) | (__float_as_uint(b[1]) & 0xffff0000u),
+                      (__float_as_uint(c[0]) >> 16) | (__float_as_uint(c[1]) & 0xffff0000u),
+                      (__float_as_uint(d[0]) >> 16) | (__float_as_uint(d[1]) & 0xffff0000u));
+}
+
 // 8 consecutive elements as four packed bf16 pairs
 template <bool KV8>
 __device__ __forceinline__ uint4 load_kv_piece(const void *base, int64_t off) {
+    if constexpr (!KV8) return *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(base) + off);
+    else return widen_bf8x8(*reinterpret_cast<const uint2 *>(reinterpret_cast<const uint8_t *>(base) + off));
+}
+// The same from an address that went through memory as an integer (a posted row address): said to be global memory,
+// because a load through a generic pointer also counts as an LDS operation, and while one is in flight every wait for
+// an LDS read has to wait for all of them.
+typedef uint32_t kv_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t kv_u32x2 __attribute__((ext_vector_type(2)));
+template <bool KV8>
+__device__ __forceinline__ uint4 load_kv_piece_global(long long row_addr, int elem_off) {
     if constexpr (!KV8) {
-        return *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(base) + off);
+        const kv_u32x4 r = *(const kv_u32x4 __attribute__((address_space(1))) *)(uintptr_t)(row_addr + 2 * elem_off);
+        return make_uint4(r.x, r.y, r.z, r.w);
     } else {
-        const uint2 r = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint8_t *>(base) + off);
-        const kv_f32x2 a = __builtin_amdgcn_cvt_pk_f32_bf8((int)r.x, false), b = __builtin_amdgcn_cvt_pk_f32_bf8((int)r.x, true);
-        const kv_f32x2 c = __builtin_amdgcn_cvt_pk_f32_bf8((int)r.y, false), d = __builtin_amdgcn_cvt_pk_f32_bf8((int)r.y, true);
-        // widening is exact, so plain truncation packs the pairs
-        return make_uint4((__float_as_uint(a[0]) >> 16) | (__float_as_uint(a[1]) & 0xffff0000u),
-                          (__float_as_uint(b[0]) >> 16) | (__float_as_uint(b[1]) & 0xffff0000u),
-                          (__float_as_uint(c[0]) >> 16) | (__float_as_uint(c[1]) & 0xffff0000u),
-                          (__float_as_uint(d[0]) >> 16) | (__float_as_uint(d[1]) & 0xffff0000u));
+        const kv_u32x2 r = *(const kv_u32x2 __attribute__((address_space(1))) *)(uintptr_t)(row_addr + elem_off);
+        return widen_bf8x8(make_uint2(r.x, r.y));
     }
 }
 
