@@ -32,7 +32,7 @@ struct MfmaMeta {
     int tok[TN];               // token, -1 for an empty slot
     int rp[TN];                // row of the RoPE tables the key is rotated with
     int tmin, tmax, all_valid; // smallest / largest token of the tile (tmax < 0: empty tile), no empty slot
-    int pad_;
+    int full;                  // every (valid row, token) pair of the tile is attended: the mask can be skipped
 };
 
 // Tiles are resolved in batches of META_BATCH, one batch ahead of their use: the ring holds two batches.
@@ -399,6 +399,9 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
             mt.tmin = tmin;
             mt.tmax = tmax;
             mt.all_valid = allv;
+            // far keys need t + sw <= p for every row, window keys t <= p < t + sw
+            mt.full = allv && (kind != 2 ? ((long long)tmax + p.sw <= pmin_blk)
+                                         : (tmax <= pmin_blk && (long long)pmax_blk < (long long)tmin + p.sw));
         }
     };
     // tiles first .. first + HB - 1, spread over the waves; the two tiles past the end resolve to rows of zeros, so
@@ -521,7 +524,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
         // the next tile
         long long ka[CPT], va[CPT];
         int rpk[ROPE ? CPT : 1];
-        int nx_tmin = 0, nx_tmax = -1, nx_allv = 0;
+        int nx_full = 0;
         auto read_posted = [&](int i) {  // iteration i loads K of tile i + 2 and V of tile i + 1
             const MfmaMeta &mk = sm.meta[(i + 2) & (2 * HB - 1)], &mv = sm.meta[(i + 1) & (2 * HB - 1)];
 #pragma unroll
@@ -531,9 +534,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
                 va[j] = mv.vo[slot];
                 if constexpr (ROPE) rpk[j] = mk.rp[slot];
             }
-            nx_tmin = mv.tmin;
-            nx_tmax = mv.tmax;
-            nx_allv = mv.all_valid;
+            nx_full = mv.full;
         };
         auto issue_loads = [&]() {
 #pragma unroll
@@ -547,11 +548,6 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
                 kreg[j] = load_kv_piece_global<KV8>(ka[j], piece * 8);
                 vreg[j] = load_kv_piece_global<KV8>(va[j], piece * 8);
             }
-        };
-        auto full_of = [&](int tile, int tmin, int tmax, int allv, bool &window) {
-            window = tile >= tiles_sel + tiles_sink;
-            if (!window) return allv != 0 && ((long long)tmax + p.sw <= pmin_blk);
-            return allv != 0 && (tmax <= pmin_blk) && ((long long)pmax_blk < (long long)tmin + p.sw);
         };
         if (ntiles > 0) {
             // K of tile 0 into LDS, K of tile 1 and V of tile 0 on their way
@@ -602,8 +598,8 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
                                               if (c == 6) issue_loads();
                                           });
                 rescale(c_a.alpha);
-                full_cur = full_of(i + 1, __builtin_amdgcn_readfirstlane(nx_tmin), __builtin_amdgcn_readfirstlane(nx_tmax),
-                                   __builtin_amdgcn_readfirstlane(nx_allv), window_cur);
+                full_cur = __builtin_amdgcn_readfirstlane(nx_full) != 0;
+                window_cur = i + 1 >= tiles_sel + tiles_sink;
             }
             // drain: the softmax of the last tile's second half and its two products with V
             __syncthreads();
