@@ -231,6 +231,7 @@ template <typename T, int HID>
 __global__ __launch_bounds__(MERGE_THREADS) void bsa_decode_merge_kernel(const float *ws, int HEAD, int nsplits, T *out,
                                                                         int64_t o_sb, int64_t o_sh) {
     constexpr int ROW = HID + 4;
+    static_assert(MERGE_THREADS % HID == 0, "a part is a whole row of HID threads");
     constexpr int PARTS = MERGE_THREADS / HID;
     __shared__ float s_m[PARTS][HID], s_num[PARTS][HID], s_den[PARTS][HID];
     const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;

@@ -416,6 +416,19 @@ __device__ __forceinline__ uint4 rope_piece(uint4 w, uint4 o, uint4 c, uint4 s, 
                       rope_pair(w.z, o.z, c.z, s.z ^ sg), rope_pair(w.w, o.w, c.w, s.w ^ sg));
 }
 
+// Can a key row lie 32 GiB or more beyond view.k?  The scan variants that pass the places of rows between lanes as
+// 31-bit numbers of 16-byte pieces hold only below that.  A dense tensor's extent follows from its shape and strides
+// (`extra_elems`: a second copy of the keys that far behind the first, see RopeView::k_side_delta); a paged pool has
+// no page count in its description, so it counts as far unless the caller says otherwise.
+inline bool kv_rows_beyond_32gib(const KVView &kv, int B, int HID, int elem_bytes, int64_t extra_elems, bool pool_is_near) {
+    if (kv.paged) return !pool_is_near;
+    auto mag = [](int64_t x) { return x < 0 ? -x : x; };
+    const long double elems = (long double)(B > 0 ? B - 1 : 0) * mag(kv.k_stride_b) +
+                              (long double)(kv.tsrc > 0 ? kv.tsrc - 1 : 0) * mag(kv.k_stride_t) +
+                              (long double)(kv.HKV > 0 ? kv.HKV - 1 : 0) * mag(kv.k_stride_h) + HID + mag(extra_elems);
+    return elems * elem_bytes >= (long double)(1LL << 35);
+}
+
 // validates q->rope (may be NULL) and fills the view; `allowed` is a bit mask of HIPATTN_EXTEND_* values
 int make_rope_view(const hipattn_q_t *q, unsigned allowed, const char *who, RopeView *out);
 int make_kv_view(const hipattn_kv_t *kv, int B, int HID, int dtype, KVView *out, KVExt *ext);

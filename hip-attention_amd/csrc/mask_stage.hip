@@ -380,7 +380,7 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
         HIPATTN_CHECK_ARG(workspace && aligned16(workspace), HIPATTN_E_ARG,
                           "mask stage: bf16 inputs need a 16-byte aligned workspace (hipattn_mask_stage_workspace_bytes)");
         p.qhat = reinterpret_cast<const uint16_t *>(workspace);
-        return mask_stage_mfma_launch(p, q->HID, rows_eff, k_prescaled, st);  // bit 0: keys, bit 1: query rows ready, bit 2: rows beyond 32 GiB
+        return mask_stage_mfma_launch(p, q->HID, rows_eff, k_prescaled, st);  // bit 0: keys, bit 1: query rows ready, bit 2: paged pool under 32 GiB
     } else if (q->dtype == HIPATTN_F32) {
         HIPATTN_CHECK_ARG(!(k_prescaled & 1), HIPATTN_E_ARG, "mask stage: prescaled keys are a bf16-only option");
         if (p.reduce_heads == 1) {
@@ -397,6 +397,19 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
     }
     set_error("mask stage: head dim %d with dtype %d is not built", q->HID, q->dtype);
     return HIPATTN_E_UNSUPPORTED;
+}
+
+extern "C" int hipattn_kv_rows_beyond_32gib(const hipattn_kv_t *kv, int32_t B, int32_t HID, int32_t dtype) {
+    if (!kv || B < 0 || HID <= 0) return HIPATTN_E_ARG;
+    KVView v{};
+    v.paged = kv->paged;
+    v.k_stride_b = kv->k_stride_b;
+    v.k_stride_t = kv->k_stride_t;
+    v.k_stride_h = kv->k_stride_h;
+    v.tsrc = kv->tsrc;
+    v.HKV = kv->HKV;
+    const int esz = kv->fp8 ? 1 : dtype == HIPATTN_F32 ? 4 : 2;
+    return kv_rows_beyond_32gib(v, B, HID, esz, 0, false) ? 1 : 0;
 }
 
 extern "C" int64_t hipattn_mask_stage_workspace_bytes(int32_t dtype, int32_t B, int32_t bs, int32_t HEAD, int32_t HID,

@@ -764,8 +764,9 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
     const int prescaled = flags & 1;          // keys scaled (and rotated) ahead of the scan
     const bool q_ready = (flags & 2) != 0;    // the workspace holds this stage's query rows already
     // key rows may lie 32 GiB or more beyond kv.k: the coalesced variants, whose lanes exchange the rows' places as
-    // 31-bit numbers of 16-byte pieces, are not used
-    const bool far_rows = (flags & 4) != 0;
+    // 31-bit numbers of 16-byte pieces, are not used.  Worked out here for a dense tensor; for a paged pool the
+    // caller vouches for its size with bit 2.
+    const bool far_rows = kv_rows_beyond_32gib(p0.kv, p0.B, HID, p0.kx.kv8 ? 1 : 2, p0.rope.k_side_delta, (flags & 4) != 0);
     MaskParams p = p0;
     const int BC = p.block_chunk;
     const bool two = rows_eff > 32;
@@ -785,7 +786,7 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
     const bool dma = dma_mode != 0 && !far_rows && (wide || dma_mode == 2) && prescaled && p.rope.cos == nullptr && !p.kx.kv8 &&
                      !p.kx.cached && HID <= 128 && env_nb != 2 && !two;  // (64-row programs: 204 registers, 6.7 against 3.9 ms)
     // small chunks on wide launches: every token scored once per GQA group, searches replayed on the scores
-    const bool dense = prescaled && p.rope.cos == nullptr && mask_stage_dense_applies(p, HID, rows_eff);
+    const bool dense = prescaled && !far_rows && p.rope.cos == nullptr && mask_stage_dense_applies(p, HID, rows_eff);
     // Launches with a single query token fetch their rows that way too, from keys as stored (HIPATTN_MASK_DMA_INLINE=0:
     // never; 2: only from 16384 waves on, e.g. a batch of sequences).  1M-key decode: 63 / 11 / 11 us against 66 / 12 /
     // 12 us for the three stages, 16 sequences: 582 against 622 us per refresh.

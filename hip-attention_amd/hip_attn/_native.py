@@ -331,9 +331,10 @@ def prescale_k_rope(k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, posit
 
 def mask_stage(qs, kvs, chunk_left, hg, n, chunk, right_clamp, bs, bq, stride_q, block_chunk, scan_stride,
                sw_eff, terminate, scores, left_out, device, k_prescaled=False, reduce_heads=False, workspace=None,
-               far_rows=False):
+               near_pool=False):
     """``workspace``: the tensor an earlier call with the same query rows (same q, bs, bq, stride_q, scan_stride, no
-    rotation) returned; the rows it holds are used as they are.  ``far_rows``: the key buffer spans 32 GiB or more.
+    rotation) returned; the rows it holds are used as they are.  ``near_pool``: the keys are a paged pool that spans
+    less than 32 GiB (a dense tensor's extent is worked out by the library).
     Returns the workspace (None for f32)."""
     q_ready = workspace is not None
     if workspace is None:
@@ -346,7 +347,7 @@ def mask_stage(qs, kvs, chunk_left, hg, n, chunk, right_clamp, bs, bq, stride_q,
         ctypes.byref(qs), ctypes.byref(kvs), _p(chunk_left), ctypes.c_int32(hg), ctypes.c_int32(n),
         ctypes.c_int32(chunk), ctypes.c_int64(right_clamp), ctypes.c_int32(bs), ctypes.c_int32(bq),
         ctypes.c_int32(stride_q), ctypes.c_int32(block_chunk), ctypes.c_int32(scan_stride),
-        ctypes.c_int32(sw_eff), ctypes.c_int32(terminate), ctypes.c_int32(int(bool(k_prescaled)) | (2 if q_ready else 0) | (4 if far_rows else 0)),
+        ctypes.c_int32(sw_eff), ctypes.c_int32(terminate), ctypes.c_int32(int(bool(k_prescaled)) | (2 if q_ready else 0) | (4 if near_pool else 0)),
         ctypes.c_int32(int(reduce_heads)), _p(workspace),
         _p(scores),
         _p(left_out), stream_ptr(device))

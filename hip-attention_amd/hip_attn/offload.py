@@ -39,20 +39,25 @@ def concurrent_stream(device, tries: int = 6):
 
     A process has few hardware queues (four by default) and the runtime spreads its streams over them, so a new stream
     may share the current stream's queue; work on it then waits for everything enqueued there before it, and a fetch
-    on such a stream overlaps nothing.  The probe puts about a millisecond of copies on the current stream and a
-    small fill on the candidate: a candidate on a queue of its own finishes first.  Streams tried and rejected are
-    kept alive, so that later streams do not take their place on the queues.  Called once, at set-up."""
+    on such a stream overlaps nothing.  The probe puts about a millisecond of small launches on the current stream
+    and a small fill on the candidate: a candidate on a queue of its own finishes first.  Streams tried and rejected
+    are kept alive, so that later streams do not take their place on the queues; the process keeps at most
+    ``_MAX_REJECTED`` of them and probes those again once that many exist.  Called once per cache, at set-up."""
     device = torch.device(device)
     main = torch.cuda.current_stream(device)
-    big = torch.empty(64 << 20, dtype=torch.float32, device=device)
+    big = torch.empty(4 << 20, dtype=torch.float32, device=device)   # 16 MB: 128 passes take about a millisecond
     small = torch.empty(1024, dtype=torch.float32, device=device)
     cand = None
-    for _ in range(tries):
-        cand = torch.cuda.Stream(device=device)
-        _REJECTED_STREAMS.append(cand)
+    for attempt in range(tries):
+        fresh = len(_REJECTED_STREAMS) < _MAX_REJECTED
+        if fresh:
+            cand = torch.cuda.Stream(device=device)
+            _REJECTED_STREAMS.append(cand)
+        else:
+            cand = _REJECTED_STREAMS[attempt % len(_REJECTED_STREAMS)]
         torch.cuda.synchronize(device)
         done_main, done_side = torch.cuda.Event(), torch.cuda.Event()
-        for _ in range(8):
+        for _ in range(128):
             big.add_(1.0)
         done_main.record(main)
         with torch.cuda.stream(cand):
@@ -62,11 +67,12 @@ def concurrent_stream(device, tries: int = 6):
         beside = not done_main.query()
         torch.cuda.synchronize(device)
         if beside:
-            _REJECTED_STREAMS.pop()
+            _REJECTED_STREAMS.remove(cand)
             return cand, True
     return cand, False
 
 
+_MAX_REJECTED = 8
 _REJECTED_STREAMS = []
 
 
@@ -144,6 +150,7 @@ class GPUCache:
         # schedule + commit are about twenty small launches whose enqueueing costs more host time than the kernels
         # take when there is little to fetch: after a first eager run they are replayed from one HIP graph
         self._miss_graph: Optional[torch.cuda.CUDAGraph] = None
+        self._miss_graph_failed = False
         self._miss_calls = 0
         self.allocated_gpu_bytes = sum(t.numel() * t.element_size() for t in (
             self.bank, self.table, self.last_use, self.backref, self.miss, self.workspace))
@@ -188,23 +195,47 @@ class GPUCache:
             self._ready = torch.cuda.Event()
             self._ready.record(stream)
 
-    def _schedule_and_commit(self):
-        """Enqueue the lookup and the fetch on the current stream: eagerly the first time and inside a caller's own
-        graph capture, otherwise as one replay of a graph captured on the second call (the kernels take the cache's
-        arrays by address and read every count on the device, so one recording serves every later call)."""
-        capturing = torch.cuda.is_current_stream_capturing()
-        use_graph = os.getenv("HIP_ATTN_CACHE_MISS_GRAPH", "1") == "1" and not capturing
-        self._miss_calls += 1
-        if use_graph and self._miss_graph is None and self._miss_calls >= 2:
-            current = torch.cuda.current_stream(self.device)
+    def prepare_miss_graph(self, run_first: bool = True) -> bool:
+        """Record the lookup and the fetch into a HIP graph now (set-up time: a capture collects garbage and
+        synchronises the device).  Captured in thread-local mode, so that allocations or synchronisations of other host
+        threads do not break it; if the capture fails all the same, later calls launch eagerly.  ``run_first``: launch
+        the two calls once eagerly before recording them (an empty step when nothing has been read yet; it loads the
+        kernels outside the capture).  Returns whether a graph is in place."""
+        if self._miss_graph is not None:
+            return True
+        if self._miss_graph_failed or os.getenv("HIP_ATTN_CACHE_MISS_GRAPH", "1") != "1":
+            return False
+        if torch.cuda.is_current_stream_capturing():
+            return False
+        current = torch.cuda.current_stream(self.device)
+        try:
+            if run_first and self._miss_calls == 0:
+                N.cache_schedule(self.handle, self.device)
+                N.cache_commit(self.handle, self.device)
             graph = torch.cuda.CUDAGraph()
             cap = torch.cuda.Stream(device=self.device)
             cap.wait_stream(current)
-            with torch.cuda.graph(graph, stream=cap):
+            with torch.cuda.graph(graph, stream=cap, capture_error_mode="thread_local"):
                 N.cache_schedule(self.handle, self.device)
                 N.cache_commit(self.handle, self.device)
             current.wait_stream(cap)
             self._miss_graph = graph
+        except Exception:  # a failed capture must not take the serving path down with it
+            self._miss_graph_failed = True
+            torch.cuda.synchronize(self.device)
+            return False
+        return True
+
+    def _schedule_and_commit(self):
+        """Enqueue the lookup and the fetch on the current stream: as one replay of the graph ``prepare_miss_graph``
+        recorded (the kernels take the cache's arrays by address and read every count on the device, so one recording
+        serves every call), eagerly inside a caller's own graph capture or when there is no graph.  A cache whose
+        owner never called ``prepare_miss_graph`` records it on its second call."""
+        capturing = torch.cuda.is_current_stream_capturing()
+        use_graph = os.getenv("HIP_ATTN_CACHE_MISS_GRAPH", "1") == "1" and not capturing
+        self._miss_calls += 1
+        if use_graph and self._miss_graph is None and not self._miss_graph_failed and self._miss_calls >= 2:
+            self.prepare_miss_graph(run_first=False)
         if use_graph and self._miss_graph is not None:
             self._miss_graph.replay()
         else:
@@ -319,6 +350,9 @@ class HiPOffloadCache:
         """Fetch missed blocks on a side stream from now on (``miss_stream``); returns whether that stream was seen to
         run beside the current one (see ``concurrent_stream``)."""
         self.miss_stream, beside = concurrent_stream(self.device)
+        # set-up is also the time to record the fetch graphs (a capture synchronises the device)
+        self.mask_k_cache.prepare_miss_graph()
+        self.sa_kv_cache.prepare_miss_graph()
         return beside
 
     def _wait_pending_write(self, stream: Optional[torch.cuda.Stream] = None):

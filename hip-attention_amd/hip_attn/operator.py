@@ -531,7 +531,7 @@ def dual_stage_quadratic_hip_attention(
                                       right_clamp, bs, BLOCK_SIZE_Q, stage.stage_block_stride_q, BLOCK_CHUNK, STAGE_STRIDE,
                                       sw_eff, args.stage_early_terminate, scores, left_out, device, k_prescaled=use_pre,
                                       reduce_heads=reduce, workspace=query_rows.get(ws_key),
-                                      far_rows=_spans_32_gib(khat if use_pre else (k_mask if k_mask is not None else args.k_cache)))
+                                      near_pool=not _spans_32_gib(khat if use_pre else (k_mask if k_mask is not None else args.k_cache)))
                     if ws_key is not None and ws is not None:
                         query_rows[ws_key] = ws
             elif isinstance(stage, NopStage):

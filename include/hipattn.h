@@ -149,9 +149,13 @@ const char *hipattn_last_error(void);
  *   iteration count (:595-601,736-737).
  *   k_prescaled: bit 0: kv->k already holds bf16(K * c_k) (see hipattn_prescale_k); bit 1: the workspace already
  *   holds the query rows of this stage, left there by an earlier call with the same q, bs, bq, stride_q, scan_stride
- *   and no rotation (stages that differ only in their chunks share them); bit 2: key rows may lie 32 GiB or more
- *   beyond kv->k (a paged pool of that size; a dense tensor's extent is known from its strides): the launches that
- *   pass the places of rows between lanes as 31-bit numbers of 16-byte pieces are then not used.
+ *   and no rotation (stages that differ only in their chunks share them).  Only calls that average several query rows
+ *   per scan row (stride_q > 1) on more than one query token fill the workspace: the others scale their rows inside
+ *   the scan kernel and leave it unwritten, so bit 1 may only follow such a call.  Bit 2, paged pools only: the caller
+ *   states that every key row of the pool lies less than 32 GiB from kv->k, which admits the launches that pass the
+ *   places of rows between lanes as 31-bit numbers of 16-byte pieces.  Without it a paged pool is scanned by the
+ *   variants that form 64-bit addresses (the description of a pool carries no page count); for a dense tensor the
+ *   library works the extent out itself from B, tsrc, HKV and the strides (hipattn_kv_rows_beyond_32gib).
  *   workspace: device scratch of hipattn_mask_stage_workspace_bytes(...) bytes. */
 int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, const int32_t *chunk_left,
                        int32_t hg, int32_t n, int32_t chunk_size, int64_t right_clamp,
@@ -159,6 +163,12 @@ int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, const int32
                        int32_t scan_stride, int32_t sw_eff, int32_t terminate_size,
                        int32_t k_prescaled, int32_t reduce_heads, void *workspace, float *scores,
                        int32_t *left_out, void *stream);
+
+/* 1 when a key row of `kv` can lie 32 GiB or more beyond kv->k (a dense tensor: from B, tsrc, HKV and the strides; a
+ * paged pool: always, its size is not part of the description), 0 when not, negative on bad arguments.  The rule
+ * hipattn_mask_stage applies before it picks a launch; host arithmetic only.  No counterpart in the reference, whose
+ * Triton kernels form 64-bit offsets throughout (src/hip_attn/v1_2/uvm_gpu_cache.py:1034-1046). */
+int hipattn_kv_rows_beyond_32gib(const hipattn_kv_t *kv, int32_t B, int32_t HID, int32_t dtype);
 
 /* Bytes of caller-allocated scratch hipattn_mask_stage needs (bf16: the averaged, scaled query rows
  * of every scan program, [B, BS, HEAD, bq/stride_q, HID]; f32: 0, workspace may be NULL). */
@@ -234,7 +244,10 @@ int hipattn_bsa_prefill(const hipattn_q_t *q, const hipattn_kv_t *kv, const int6
 
 /* Decode (TDST == 1) split-KV attention.  Replaces decode_block_sparse_attention,
  * src/hip_attn/v1_2/attention_decode_bsa.py:1331-1435: _fwd_kernel_stage1 (:22-1045) writes
- * per-split partials, _fwd_kernel_stage2 (:1148-1226) merges them by log-sum-exp.
+ * per-split partials, _fwd_kernel_stage2 (:1148-1226) merges them by log-sum-exp.  The merge folds every
+ * (1024 / HID)-th split into a running (maximum, numerator, denominator) and then folds those parts, so its f32
+ * summation order depends on HID and is not the split order: outputs are held to the attention tolerance, not to
+ * bits, across builds and head dims (HID must divide 1024: 32, 64, 128, 256).
  *   workspace: f32, hipattn_bsa_decode_workspace_bytes(...) bytes, caller-allocated.
  *   nsplits: how many workgroups share one (sequence, kv head); hipattn_bsa_decode_default_splits picks one.
  *   second_stage_k: args.second_stage_k of the call being replaced, or 0.  The reference's launcher divides the

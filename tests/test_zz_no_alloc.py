@@ -79,3 +79,49 @@ def test_static_scratch_decode_refuses_what_does_not_fit():
     with pytest.raises(N.HipAttnError, match="scratch"):
         N.bsa_decode_static(P["qs"], P["kvs"], P["indices"], P["kse"], P["BK"], 8, 512, 256, out, dev, nsplits=too_many)
     torch.cuda.synchronize()
+
+
+def test_static_scratch_decode_under_graph_capture_allocates_nothing():
+    """What the entry point is for: after one eager call (which looks the array's address up) it is captured into a
+    HIP graph and replayed with new queries; device memory does not move across the calls."""
+    from hip_attn import _native as N
+
+    print("[case] decode without allocation: captured into a graph, replayed with new queries", flush=True)
+    P = _problem(307, B=2, lens=[4096, 3500], TK=4096, H=8, HKV=2, D=128, page=16)
+    dev = torch.device("cuda", torch.cuda.current_device())
+    A = P["A"]
+    q = P["keep"][0]
+    out = torch.empty(P["shape"], dtype=torch.bfloat16, device=dev)
+    want = torch.empty_like(out)
+
+    def static_call():
+        N.bsa_decode_static(P["qs"], P["kvs"], P["indices"], P["kse"], P["BK"], 8, 512, A.sink_token_size, out, dev,
+                            nsplits=0, second_stage_k=A.second_stage_k)
+
+    static_call()  # eager: address lookup, code objects loaded
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    torch_before = torch.cuda.memory_allocated()
+    static_call()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "the call changed the device's free memory"
+    assert torch.cuda.memory_allocated() == torch_before
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        static_call()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_call()
+    g = torch.Generator().manual_seed(11)
+    for rep in range(3):
+        q.copy_(torch.randn(q.shape, generator=g).to(torch.bfloat16))
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        N.bsa_decode(P["qs"], P["kvs"], P["indices"], P["kse"], P["BK"], 8, 512, A.sink_token_size, want, dev,
+                     nsplits=0, second_stage_k=A.second_stage_k)
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), want.view(torch.int16)), f"replay {rep} differs from the workspace path"
