@@ -25,6 +25,7 @@ struct BsaParamsBase {
     // each and number them from their first token rounded down to a multiple of the block size
     // (attention_decode_bsa.py:514-518, 740), so a token is rotated (share start % bk) positions lower; 0 = off.
     int sink_share;
+    int non_causal;  // no position tests in the mask (is_causal = False, attention_extend_bsa.py:511-523)
     int B, TDST, HEAD, G, NBQ;
     float c_q, c_k;
     void *out;

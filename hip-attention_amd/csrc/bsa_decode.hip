@@ -120,7 +120,7 @@ __global__ __launch_bounds__(256) void bsa_decode_partial_kernel(DecodeParamsT<E
                 rpos = t;
             }
         }
-        const bool att = valid && (kind == 0 ? (t + p.sw <= ppos) : (t <= ppos && ppos < t + p.sw));
+        const bool att = valid && (p.non_causal || (kind == 0 ? (t + p.sw <= ppos) : (t <= ppos && ppos < t + p.sw)));
         int64_t koff, voff;
         if (!att) {  // uniform inside the 16-lane group; shuffles below stay inside the group
             // staged but masked out: still an access as far as the statistics and the cache are concerned

@@ -173,7 +173,7 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
                 flag_leader = lane == 0 || t < 0 || t_before != t - 1 || (t & (p.kv.page_size - 1)) == 0 || (int64_t)t >= seqlen;
         }
         if (t >= 0) {
-            const bool att = win ? ((long long)t <= ppos && ppos < (long long)t + p.sw) : ((long long)t + p.sw <= ppos);
+            const bool att = p.non_causal || (win ? ((long long)t <= ppos && ppos < (long long)t + p.sw) : ((long long)t + p.sw <= ppos));
             // a staged but masked token still counts as an access; its rows are not needed
             if (att) {
                 if constexpr (EXT) {

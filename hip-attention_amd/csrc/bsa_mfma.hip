@@ -400,8 +400,8 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
             mt.tmax = tmax;
             mt.all_valid = allv;
             // far keys need t + sw <= p for every row, window keys t <= p < t + sw
-            mt.full = allv && (kind != 2 ? ((long long)tmax + p.sw <= pmin_blk)
-                                         : (tmax <= pmin_blk && (long long)pmax_blk < (long long)tmin + p.sw));
+            mt.full = allv && (p.non_causal || (kind != 2 ? ((long long)tmax + p.sw <= pmin_blk)
+                                                          : (tmax <= pmin_blk && (long long)pmax_blk < (long long)tmin + p.sw)));
         }
     };
     // tiles first .. first + HB - 1, spread over the waves; the two tiles past the end resolve to rows of zeros, so
@@ -483,6 +483,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
         const int tmin = __builtin_amdgcn_readfirstlane(mt.tmin), tmax = __builtin_amdgcn_readfirstlane(mt.tmax);
         const bool all_valid = __builtin_amdgcn_readfirstlane(mt.all_valid) != 0;
         window = tile >= tiles_sel + tiles_sink;
+        if (p.non_causal) return all_valid;
         if (!window) return all_valid && ((long long)tmax + p.sw <= pmin_blk);
         return all_valid && (tmax <= pmin_blk) && ((long long)pmax_blk < (long long)tmin + p.sw);
     };
@@ -497,9 +498,13 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
         // attended token ranges of this lane's query row: far keys 0 <= t <= pq - sw, window keys
         // max(0, pq - sw + 1) <= t <= pq; a row that does not exist attends nothing
         const long long far_hi = (long long)pq - p.sw;
-        const unsigned far_span = far_hi >= 0 ? (unsigned)far_hi + 1u : 0u;
-        const int win_lo = far_hi + 1 > 0 ? (int)(far_hi + 1) : 0;
-        const unsigned win_span = pq >= win_lo ? (unsigned)(pq - win_lo) + 1u : 0u;
+        unsigned far_span = far_hi >= 0 ? (unsigned)far_hi + 1u : 0u;
+        int win_lo = far_hi + 1 > 0 ? (int)(far_hi + 1) : 0;
+        unsigned win_span = pq >= win_lo ? (unsigned)(pq - win_lo) + 1u : 0u;
+        if (p.non_causal) {  // every valid token of an existing row
+            win_lo = 0;
+            far_span = win_span = row_ok ? 0x80000000u : 0u;
+        }
         float cap = 0.0f, cap_k2 = 0.0f;
         if constexpr (CAP) {
             cap = p.softcap;
@@ -685,7 +690,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
                         const int t = ts[e];
                         // branch-free: far keys need t + sw <= pq, window keys t <= pq < t + sw
                         const long long tsw = (long long)t + p.sw;
-                        const bool att = (t >= 0) & (window ? ((t <= pq) & ((long long)pq < tsw)) : (tsw <= (long long)pq));
+                        const bool att = (t >= 0) & (p.non_causal ? row_ok : window ? ((t <= pq) & ((long long)pq < tsw)) : (tsw <= (long long)pq));
                         const float s = att ? sacc[nb][i4 * 4 + e] : -INFINITY;
                         sacc[nb][i4 * 4 + e] = s;
                         mx = fmaxf(mx, s);

@@ -103,7 +103,7 @@ __global__ __launch_bounds__(256) void bsa_simple_kernel(BsaParams p) {
                 valid = true;
                 rpos = t;
             }
-            const bool att = valid && (kind == 0 ? (t + p.sw <= ppos) : (t <= ppos && ppos < t + p.sw));
+            const bool att = valid && (p.non_causal || (kind == 0 ? (t + p.sw <= ppos) : (t <= ppos && ppos < t + p.sw)));
             float logit = -INFINITY;
             int64_t voff = NO_ROW;
             if (valid && !att && j == wid && (p.kx.access_flags || p.kx.cached)) {
@@ -226,6 +226,7 @@ int bsa_fill_params(const hipattn_q_t *q, const hipattn_kv_t *kv, const int64_t 
     p->sw = sw; p->sink = sink; p->share_first_head = share_first_head;
     p->k_prescaled = 0;
     p->seam_blocks = 0; p->seam_extra = 0; p->sink_share = 0;
+    p->non_causal = q->non_causal != 0;
     p->B = q->B; p->TDST = q->TDST; p->HEAD = q->HEAD; p->G = q->HEAD / p->kv.HKV;
     p->NBQ = (q->TDST + bq - 1) / bq;
     HIPATTN_CHECK_ARG(p->NBQ <= idx_rows, HIPATTN_E_ARG, "bsa: %d query blocks but only %d index rows", p->NBQ, idx_rows);

@@ -387,6 +387,22 @@ __device__ __forceinline__ int64_t dynamic_extend_pos(int64_t t, int64_t pmin, i
     return pos > lowest ? pos : lowest;
 }
 
+// The SELF rule (attention_extend.py:275-289): keys older than 8192 positions are grouped by sixteen once the query
+// block reaches beyond the model's context; the quotient truncates toward zero, as the compiled kernel's does.
+__device__ __forceinline__ int64_t self_extend_pos(int64_t t, int64_t pmin, int64_t pmax, int64_t model_ctx) {
+    int64_t pos = t;
+    if (!(t >= pmax - 8192 || pmax <= model_ctx)) pos = (t - pmin) / 16 + pmin;
+    return pos > 0 ? pos : 0;
+}
+// rules under which a sampled key's rotated position follows its token (the table row is reloaded with every sample)
+__device__ __forceinline__ bool rope_follows_token(int backend) {
+    return backend == HIPATTN_EXTEND_DYNAMIC || backend == HIPATTN_EXTEND_SELF;
+}
+__device__ __forceinline__ int64_t token_extend_pos(const RopeView &r, int64_t t, int64_t pmin, int64_t pmax) {
+    return r.backend == HIPATTN_EXTEND_SELF ? self_extend_pos(t, pmin, pmax, r.model_ctx)
+                                            : dynamic_extend_pos(t, pmin, pmax, r.model_ctx);
+}
+
 // One element of a rotated row: x*c + o*s with `o` the partner element, already signed (-x[i + HID/2] in the
 // lower half, +x[i - HID/2] in the upper); both products and the sum are rounded to T, never fused.
 template <typename T>

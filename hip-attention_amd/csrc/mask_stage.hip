@@ -56,7 +56,7 @@ __device__ __forceinline__ float reduce16(const float (&part)[ROWS], int dl) {
 __device__ __forceinline__ int64_t mask_rope_qpos(const RopeView &r, long long pos, int n, int sw_eff) {
     if (r.backend == HIPATTN_EXTEND_RELATIVE) return 1 + (int64_t)sw_eff;
     if (r.backend == HIPATTN_EXTEND_INFLLM) return sw_eff;
-    if (r.backend == HIPATTN_EXTEND_DYNAMIC) return pos;
+    if (rope_follows_token(r.backend)) return pos;
     const long long cap = (long long)n + sw_eff;
     return pos < cap ? pos : cap;
 }
@@ -64,7 +64,7 @@ __device__ __forceinline__ int64_t mask_rope_qpos(const RopeView &r, long long p
 __device__ __forceinline__ int64_t mask_rope_kpos(const RopeView &r, int c, int side, int t, int64_t pmin, int64_t pmax) {
     if (r.backend == HIPATTN_EXTEND_RELATIVE) return side;
     if (r.backend == HIPATTN_EXTEND_STREAMING) return c;
-    if (r.backend == HIPATTN_EXTEND_DYNAMIC) return dynamic_extend_pos(t, pmin, pmax, r.model_ctx);
+    if (rope_follows_token(r.backend)) return token_extend_pos(r, t, pmin, pmax);
     return 0;
 }
 
@@ -339,7 +339,7 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
     rc = make_kv_view(kv, q->B, q->HID, q->dtype, &p.kv, &p.kx);
     if (rc) return rc;
     rc = make_rope_view(q, (1u << HIPATTN_EXTEND_RELATIVE) | (1u << HIPATTN_EXTEND_STREAMING) | (1u << HIPATTN_EXTEND_INFLLM) |
-                               (1u << HIPATTN_EXTEND_DYNAMIC),
+                               (1u << HIPATTN_EXTEND_DYNAMIC) | (1u << HIPATTN_EXTEND_SELF),
                         "mask stage", &p.rope);
     if (rc) return rc;
     HIPATTN_CHECK_ARG(k_prescaled >= 0 && k_prescaled <= 7, HIPATTN_E_ARG, "mask stage: k_prescaled %d not in 0..7", k_prescaled);

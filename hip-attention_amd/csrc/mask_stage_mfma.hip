@@ -48,7 +48,7 @@ __device__ __forceinline__ uint32_t scale_pack(uint32_t w, float c) {
 __device__ __forceinline__ int64_t rope_qpos(const RopeView &r, long long pos, int n, int sw_eff) {
     if (r.backend == HIPATTN_EXTEND_RELATIVE) return 1 + (int64_t)sw_eff;
     if (r.backend == HIPATTN_EXTEND_INFLLM) return sw_eff;
-    if (r.backend == HIPATTN_EXTEND_DYNAMIC) return pos;
+    if (rope_follows_token(r.backend)) return pos;
     const long long cap = (long long)n + sw_eff;
     return pos < cap ? pos : cap;
 }
@@ -423,8 +423,8 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                     if (side && off != NO_ROW) off += p.rope.k_side_delta;
                 }
                 if constexpr (ROPE) {
-                    if (p.rope.backend == HIPATTN_EXTEND_DYNAMIC) {
-                        const int64_t tr = p.rope.row(dynamic_extend_pos(t, pmin, pmin + __popcll(rowmask), p.rope.model_ctx));
+                    if (rope_follows_token(p.rope.backend)) {
+                        const int64_t tr = p.rope.row(token_extend_pos(p.rope, t, pmin, pmin + __popcll(rowmask)));
 #pragma unroll
                         for (int ks = 0; ks < KS; ks++) {
                             rcos[tb][ks] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr + ks * 8);

@@ -33,6 +33,7 @@ class QStruct(ctypes.Structure):
         ("dtype", ctypes.c_int32),
         ("rope", ctypes.c_void_p),
         ("logit_softcap", ctypes.c_float),
+        ("non_causal", ctypes.c_int32),
     ]
 
 
@@ -46,7 +47,7 @@ class RopeStruct(ctypes.Structure):
     ]
 
 
-EXTEND_BACKENDS = {"relative": 1, "streaming": 2, "infllm": 3, "dynamic_extend": 4}
+EXTEND_BACKENDS = {"relative": 1, "streaming": 2, "infllm": 3, "dynamic_extend": 4, "self_extend": 5}
 
 
 class KVStruct(ctypes.Structure):
@@ -167,7 +168,8 @@ def make_rope(cos: torch.Tensor, sin: torch.Tensor, backend: str, k_side_delta: 
               model_context_length: int = 0, attention: bool = False) -> RopeStruct:
     """Describe RoPE tables ``[len, >= HID/2]`` (q's dtype, unit inner stride) and the rotation rule of one call.
     ``attention`` marks a call of block sparse attention, which knows fewer rules than the mask stage."""
-    built = [b for b in EXTEND_BACKENDS if not (attention and b == "relative")]
+    # the reference's attention kernels know neither "relative" nor "self_extend" (attention_extend_bsa.py:62-63)
+    built = [b for b in EXTEND_BACKENDS if not (attention and b in ("relative", "self_extend"))]
     if backend not in built:
         where = "block sparse attention" if attention else "the mask stage"
         raise NotImplementedError(f"extend backend {backend!r} is not built for {where} (built: {sorted(built)})")
@@ -183,11 +185,13 @@ def make_rope(cos: torch.Tensor, sin: torch.Tensor, backend: str, k_side_delta: 
 
 
 def make_q(q: torch.Tensor, pos: torch.Tensor, rope: Optional[RopeStruct] = None,
-           logit_softcap: Optional[float] = None) -> QStruct:
+           logit_softcap: Optional[float] = None, non_causal: bool = False) -> QStruct:
     assert q.ndim == 4 and q.stride(3) == 1
     assert pos.dtype == torch.int64 and pos.ndim == 2
     s = QStruct()
     s.logit_softcap = float(logit_softcap or 0.0)
+    s.non_causal = int(bool(non_causal))
+    s._pos_keep = pos  # the struct holds a bare pointer to it
     if rope is not None:
         s._rope_keep = rope  # the struct holds a bare pointer to it
         s.rope = ctypes.addressof(rope)

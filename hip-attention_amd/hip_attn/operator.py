@@ -51,8 +51,6 @@ def _reject_unsupported(args: HiPAttentionArgs):
                                   "store q and k without RoPE and pass need_apply_rope=True")
     if args.logit_softcap is not None and not (args.logit_softcap > 0):
         raise ValueError("logit_softcap must be positive (or None)")
-    if not args.is_causal:
-        raise NotImplementedError("is_causal=False is not built")
     if args.sliding_window_indices is not None:
         raise NotImplementedError("sliding_window_indices is a research switch and is not built")
     if args.online_update_cache:
@@ -671,7 +669,12 @@ def block_sparse_attention(q: Tensor, k: Optional[Tensor], v: Optional[Tensor], 
         position_ids = position_ids.to(torch.int64)
     rope = (N.make_rope(*rope_tables, args.sa_extend_backend, 0, args.model_context_length, attention=True)
             if rope_tables is not None else None)
-    qs = N.make_q(qq, position_ids, rope, args.logit_softcap)
+    non_causal = not args.is_causal
+    if non_causal and not decode:
+        # the reference's query-block kernel takes MAX_TSRC for every row's position when the mask is not causal
+        # (attention_extend_bsa.py:743-752); its decode kernel keeps the true ones
+        position_ids = torch.full_like(position_ids, max_tsrc - 1)
+    qs = N.make_q(qq, position_ids, rope, args.logit_softcap, non_causal)
     if rope is not None or args.logit_softcap is not None:
         khat = None
     if not indices.is_contiguous():

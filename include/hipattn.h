@@ -52,12 +52,20 @@ extern "C" {
  *                the mask-stage formula above gives for their token (pmin = smallest position of the query block,
  *                pmax = pmin + its valid rows; decode: pmax = pmin + 1); both products and the sum are rounded to
  *                the element type.  Served by the portable attention kernels.
- * Positions are clamped into [0, len).  The reference's "self_extend" rule and the mode that re-rotates keys stored
- * WITH rotation (need_apply_rope = False) are not built. */
+ *   SELF, mask stage only (attention_extend.py:275-289, :637-638): the query at its own position; the sampled key at
+ *                token t keeps position t when t >= pmax - 8192 or pmax <= model_context_length, else it moves to
+ *                (t - pmin) / 16 + pmin with the quotient truncated toward zero (what the compiled kernel's int32
+ *                division does; the reference's CPU interpreter floors instead, so no execution of it on a CPU
+ *                pins this rule: parity unpinned by execution, pinned by the closed form), then max(0, .).  The
+ *                reference's attention kernels raise on this rule (attention_extend_bsa.py:62-63), and so does the
+ *                attention entry here.
+ * Positions are clamped into [0, len).  The mode that re-rotates keys stored WITH rotation (need_apply_rope = False)
+ * is not built. */
 #define HIPATTN_EXTEND_RELATIVE 1
 #define HIPATTN_EXTEND_STREAMING 2
 #define HIPATTN_EXTEND_INFLLM 3
 #define HIPATTN_EXTEND_DYNAMIC 4
+#define HIPATTN_EXTEND_SELF 5
 
 typedef struct hipattn_rope {
     const void *cos; /* [len, >= HID/2], q's dtype, 16-byte aligned rows; column i = frequency i */
@@ -69,8 +77,8 @@ typedef struct hipattn_rope {
      * and scaled (hipattn_prescale_k_rope), and the copy rotated to position 1, which the right-hand samples
      * read, starts this many elements behind it.  INFLLM needs the position-0 copy only.  Unused otherwise. */
     int64_t k_side_delta;
-    /* HiPAttentionArgs.model_context_length (attention_extend.py:250); read by the DYNAMIC rule only, which needs
-     * at least 512 */
+    /* HiPAttentionArgs.model_context_length (attention_extend.py:250); read by the DYNAMIC rule, which needs at
+     * least 512, and by the SELF rule */
     int64_t model_context_length;
 } hipattn_rope_t;
 
@@ -89,6 +97,12 @@ typedef struct hipattn_q {
      * softmax (src/hip_attn/v1_2/attention_extend_bsa.py:507-508).  Read by the bsa entry points only; the mask
      * stage scores are never capped (the reference's scan kernel has no such option). */
     float logit_softcap;
+    /* HiPAttentionArgs.is_causal == False (src/hip_attn/v1_2/attention_extend_bsa.py:511-523, :743-752; read by the
+     * bsa entry points only): != 0 drops the position tests of the attention mask, so every valid sink, selected
+     * and window key the kernels walk is attended (a key that is both selected and in the window counts twice, as in
+     * the reference).  The reference's query-block kernel then also takes MAX_TSRC for every row's position; the
+     * caller passes such positions in `pos` (max_tsrc - 1), the decode kernel keeps the true ones (:118). */
+    int32_t non_causal;
 } hipattn_q_t;
 
 /* Key/value storage: dense k,v[B, TSRC, HKV, HID] or a paged cache [pages, page_size, HKV, HID]

@@ -60,10 +60,11 @@ class _Tensors(ctypes.Structure):
         ("sa_backend", ctypes.c_int),
         ("logit_softcap", ctypes.c_float),
         ("model_context_length", ctypes.c_int64),
+        ("non_causal", ctypes.c_int),
     ]
 
 
-EXTEND_BACKENDS = {None: 0, "relative": 1, "streaming": 2, "infllm": 3, "dynamic_extend": 4}
+EXTEND_BACKENDS = {None: 0, "relative": 1, "streaming": 2, "infllm": 3, "dynamic_extend": 4, "self_extend": 5}
 
 
 def build(force: bool = False) -> str:
@@ -144,6 +145,7 @@ class OArgs:
     block_sparse_block_size_q: Optional[int] = 64
     stage_early_terminate: int = 1
     disable_flashdecode: bool = False
+    is_causal: bool = True  # attention_metadata.py:189; read by block sparse attention only
     head_reduce: bool = True  # env HIP_HEAD_REDUCE, default on (attention_extend.py:2566)
     mask_only: bool = False
     # RoPE applied on load (attention_metadata.py:191-198); only using_extend with need_apply_rope is modelled
@@ -172,6 +174,7 @@ class OInputs:
     scan_backend: Optional[str] = None  # rotation rule of the mask stage / of sparse attention; None = no RoPE
     sa_backend: Optional[str] = None
     logit_softcap: float = 0.0
+    non_causal: int = 0  # block sparse attention only: 1 = query-block kernel's form, 2 = decode kernel's (hipo_bsa)
 
     def c_struct(self, max_tsrc: int):
         np_t = np.uint16 if self.dtype == "bf16" else np.float32
@@ -210,6 +213,7 @@ class OInputs:
         S.MAX_TSRC = max_tsrc
         S.logit_softcap = float(self.logit_softcap or 0.0)
         S.model_context_length = int(self.model_context_length)
+        S.non_causal = int(self.non_causal)
         if self.access is not None:
             assert self.access.dtype == np.int32 and self.access.flags.c_contiguous and self.access.ndim == 3
             S.access = self.access.ctypes.data
@@ -533,6 +537,7 @@ def hip_attention_12(X: OInputs, A: OArgs, cached: Optional[OMetadata] = None):
     X.access = sa_access
     user_cap = X.logit_softcap
     X.logit_softcap = float(A.logit_softcap or 0.0)
+    X.non_causal = 0 if A.is_causal else (2 if decode else 1)  # attention only; the scan knows no such switch
     try:
         seams = decode_seams(A.second_stage_k, sink, sw_bsa, block_size_k, indices.shape[-1]) if decode else (0, 0)
         sink_share = decode_sink_share(A.second_stage_k, sink, sw_bsa) if decode else 0
@@ -541,6 +546,7 @@ def hip_attention_12(X: OInputs, A: OArgs, cached: Optional[OMetadata] = None):
     finally:
         X.access = user_access
         X.logit_softcap = user_cap
+        X.non_causal = 0
         X.scan_backend, X.sa_backend = user_backends
     meta = OMetadata(indices=indices, ks=ks, ks_count=ks_count, ks_start_end=ks_start_end,
                      stage_caches=stage_caches, mask_access=mask_access, sa_access=sa_access)

@@ -53,6 +53,7 @@
 #define HIPO_EXT_STREAMING 2
 #define HIPO_EXT_INFLLM 3
 #define HIPO_EXT_DYNAMIC 4
+#define HIPO_EXT_SELF 5
 
 typedef struct {
     int dtype;               /* HIPO_F32 / HIPO_BF16 (q, k, v, caches all share it) */
@@ -84,11 +85,17 @@ typedef struct {
     int sa_backend;          /* HIPO_EXT_* for block sparse attention */
     float logit_softcap;     /* 0 = off; attention logits become tanh(qk / cap) * cap (attention_extend_bsa.py:507-508) */
     int64_t model_context_length; /* HiPAttentionArgs.model_context_length (the "dynamic_extend" rule needs it) */
+    /* HiPAttentionArgs.is_causal == False, block sparse attention only.  0: causal.  1: the query-block kernel's form
+     * (attention_extend_bsa.py:743-752, :511-523): every valid row takes MAX_TSRC as its position + 1 and the mask
+     * keeps nothing but validity.  2: the decode kernel's form (attention_decode_bsa.py: positions stay, the mask
+     * keeps nothing but validity). */
+    int non_causal;
 } hipo_tensors_t;
 
 /* ---------------------------------------------------------------- scalar helpers */
 
 static int64_t dynamic_extend_pos(int64_t t, int64_t pmin, int64_t pmax, int64_t model_ctx);
+static int64_t self_extend_pos(int64_t t, int64_t pmin, int64_t pmax, int64_t model_ctx);
 
 static inline float bf16_bits_to_f32(uint16_t h) {
     uint32_t u = (uint32_t)h << 16;
@@ -379,7 +386,7 @@ int hipo_mask_stage(const hipo_tensors_t *X, int64_t *left, int64_t *right, floa
                     int64_t p = X->pos[(int64_t)b * TDST + it];
                     if (X->scan_backend == HIPO_EXT_RELATIVE) qpos = 1 + (int64_t)sw_eff;
                     else if (X->scan_backend == HIPO_EXT_INFLLM) qpos = sw_eff;
-                    else if (X->scan_backend == HIPO_EXT_DYNAMIC) qpos = p; /* :635-636 */
+                    else if (X->scan_backend == HIPO_EXT_DYNAMIC || X->scan_backend == HIPO_EXT_SELF) qpos = p; /* :635-638 */
                     else qpos = p < (int64_t)n + sw_eff ? p : (int64_t)n + sw_eff;
                 }
                 for (int o = 0; o < stride_q; o++) {
@@ -432,7 +439,10 @@ int hipo_mask_stage(const hipo_tensors_t *X, int64_t *left, int64_t *right, floa
                         int64_t kposL = 0, kposR = 0;
                         if (X->scan_backend == HIPO_EXT_RELATIVE) kposR = 1;
                         else if (X->scan_backend == HIPO_EXT_STREAMING) kposL = kposR = c;
-                        else if (X->scan_backend == HIPO_EXT_DYNAMIC) {
+                        else if (X->scan_backend == HIPO_EXT_SELF) {
+                            kposL = self_extend_pos(tl_, pmin, pmin + nvalid, X->model_context_length);
+                            kposR = self_extend_pos(tr_, pmin, pmin + nvalid, X->model_context_length);
+                        } else if (X->scan_backend == HIPO_EXT_DYNAMIC) {
                             kposL = dynamic_extend_pos(tl_, pmin, pmin + nvalid, X->model_context_length);
                             kposR = dynamic_extend_pos(tr_, pmin, pmin + nvalid, X->model_context_length);
                         }
@@ -486,12 +496,26 @@ static int64_t dynamic_extend_pos(int64_t t, int64_t pmin, int64_t pmax, int64_t
     return pos > floor_ ? pos : floor_;
 }
 
+/* Rotated position of a sampled key under the "self_extend" rule (attention_extend.py:275-289): once the query block
+ * reaches beyond the model's context, keys older than 8192 positions are grouped by sixteen around the block's first
+ * position.  `//` in the kernel is an int32 division: the compiled kernel truncates toward zero (sampled keys lie
+ * below pmin, so the numerator is negative and the two roundings differ); the reference's CPU interpreter floors.
+ * This follows the compiled kernel: parity unpinned by execution here, pinned by the closed form in the tests. */
+static int64_t self_extend_pos(int64_t t, int64_t pmin, int64_t pmax, int64_t model_ctx) {
+    int64_t pos = t;
+    if (!(t >= pmax - 8192 || pmax <= model_ctx)) pos = (t - pmin) / 16 + pmin; /* C division truncates */
+    return pos > 0 ? pos : 0;
+}
+
 /* ---------------------------------------------------------------- block sparse attention
  * Attended set of a query row at position p inside a query block whose largest position+1
  * is CURR (attention_extend_bsa.py:511-523,881-891,1137,1371-1379):
  *   selected blocks j < min(BK, ks_end): tokens t with 0<=t<MAX_TSRC, sink<=t<CURR, t+sw<=p
  *   sink:   t < min(CURR, sink), t+sw<=p
  *   window: max(0,CURR-sw-BQ) <= t < CURR,  t<=p<t+sw
+ * With X->non_causal the position tests t+sw<=p / t<=p<t+sw fall away (the lists stay as they are, so a token that
+ * is both selected and inside the window is attended twice, as the reference's loops do), and form 1 puts every
+ * valid row at position MAX_TSRC - 1.
  * Softmax in base 2 over f32 logits, probabilities rounded to T before the value product
  * (:531-558).  Rows with an empty set give 0 (l stays at its initial 1.0, :764,1625).
  * share_first_head != 0 uses, for every head of a GQA group, the index row of the group's
@@ -557,7 +581,7 @@ int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_
                 int64_t it = (int64_t)qb * block_size_q + j;
                 if (it < TDST) {
                     nvalid++;
-                    int64_t sl = X->pos[(int64_t)b * TDST + it] + 1;
+                    int64_t sl = (X->non_causal == 1 ? MAXT - 1 : X->pos[(int64_t)b * TDST + it]) + 1;
                     if (sl > curr) curr = sl;
                     if (sl - 1 < pos_min) pos_min = sl - 1;
                 }
@@ -610,7 +634,7 @@ int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_
             for (int j = 0; j < block_size_q; j++) {
                 int64_t it = (int64_t)qb * block_size_q + j;
                 if (it >= TDST) continue;
-                int64_t p = X->pos[(int64_t)b * TDST + it];
+                int64_t p = X->non_causal == 1 ? MAXT - 1 : X->pos[(int64_t)b * TDST + it];
                 int64_t qoff = (((int64_t)b * TDST + it) * HEAD + h) * HID;
                 for (int d = 0; d < HID; d++) qhat[d] = load_T(X->q, qoff + d, X->dtype);
                 if (X->rope_cos) rope_rotate(X, qhat, p); /* :796-852: the query keeps its true position */
@@ -618,7 +642,7 @@ int hipo_bsa(const hipo_tensors_t *X, const int64_t *indices, const int32_t *ks_
                 float m = -INFINITY;
                 for (int i = 0; i < nt; i++) {
                     int64_t t = tok[i];
-                    int att = kind[i] == 0 ? (t + sw <= p) : (t <= p && p < t + sw);
+                    int att = X->non_causal ? 1 : kind[i] == 0 ? (t + sw <= p) : (t <= p && p < t + sw);
                     if (!att) { logit[i] = -INFINITY; continue; }
                     float qk = hipo_dot(qhat, khat + (size_t)i * HID, HID);
                     if (X->logit_softcap != 0.0f) qk = tanhf(qk / X->logit_softcap) * X->logit_softcap;

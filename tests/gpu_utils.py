@@ -32,7 +32,7 @@ def product_args(A: O.OArgs, X: O.OInputs, device="cuda", **extra):
                 for s in A.stages],
         model_context_length=A.model_context_length, extend_context_length=A.extend_context_length,
         block_sparse_block_size_q=A.block_sparse_block_size_q, stage_early_terminate=A.stage_early_terminate,
-        disable_flashdecode=A.disable_flashdecode, mask_only=A.mask_only,
+        disable_flashdecode=A.disable_flashdecode, mask_only=A.mask_only, is_causal=A.is_causal,
         position_ids=torch.from_numpy(np.ascontiguousarray(X.pos)).to(device),
     )
     if X.k is None:

@@ -11,7 +11,8 @@ from test_oracle_bsa import random_indices
 pytestmark = pytest.mark.gpu
 
 
-def _run(X, max_tsrc, idx, kse, bq, bk, sw, sink, impl, share=False, decode=False, softcap=None, second_k=0):
+def _run(X, max_tsrc, idx, kse, bq, bk, sw, sink, impl, share=False, decode=False, softcap=None, second_k=0,
+         causal=True):
     from hip_attn import HiPAttentionArgs12
     from hip_attn.operator import block_sparse_attention
 
@@ -22,7 +23,7 @@ def _run(X, max_tsrc, idx, kse, bq, bk, sw, sink, impl, share=False, decode=Fals
         kw = dict(k_cache=to_torch(X.k_cache, X.dtype, dev), v_cache=to_torch(X.v_cache, X.dtype, dev),
                   block_table=torch.from_numpy(X.block_table).to(dev),
                   cache_seq_lens=torch.from_numpy(X.cache_seq_lens).to(dev))
-    args = HiPAttentionArgs12(sink_token_size=sink, sliding_window_size=sw, logit_softcap=softcap, **kw)
+    args = HiPAttentionArgs12(sink_token_size=sink, sliding_window_size=sw, logit_softcap=softcap, is_causal=causal, **kw)
     args.block_size_q, args.block_size_k = bq, bk
     args.second_stage_k = second_k  # decode only: sizes the reference's own split of the index row
     out = block_sparse_attention(q, to_torch(X.k, X.dtype, dev), to_torch(X.v, X.dtype, dev),
@@ -123,3 +124,42 @@ def test_logit_softcap_in_every_attention_kernel(dtype, D):
     idx, ks, kse = random_indices(rng, 2, H, 1, BK, bk, TK, same_heads=True)
     ref = O.bsa(Xd, TK, idx, kse, 1, bk, sw, sink, share_first_head=True)
     assert_context_close(_run(Xd, TK, idx, kse, 1, bk, sw, sink, impl=0, decode=True, softcap=3.0), ref, dtype)
+
+
+@pytest.mark.parametrize("dtype,D", [("bf16", 64), ("bf16", 128), ("bf16", 256), ("f32", 64)])
+def test_non_causal_attention_in_every_kernel(dtype, D):
+    """is_causal = False (attention_extend_bsa.py:511-523, :743-752): the mask keeps validity only; the query-block
+    kernels put every row at the end of the keys, the decode kernels keep the row's position.  Blocks selected inside
+    the last window are attended twice, by the kernels as by the oracle."""
+    print(f"[case] bsa non-causal {dtype} D={D}", flush=True)
+    rng = np.random.default_rng(D)
+    TK, TQ, H, HKV, bq, bk, BK, sw, sink = 1536, 200, 8, 2, 64, 8, 24, 100, 24
+    X = make_inputs(15, B=2, TQ=TQ, TK=TK, H=H, HKV=HKV, D=D, dtype=dtype, scale=0.5)
+    nbq = O.cdiv(TQ, bq)
+    idx, ks, kse = random_indices(rng, 2, H, nbq, BK, bk, TK, same_heads=True)
+    idx[:, :, 0] = 64  # one early block, and one inside the last sw + bq tokens
+    idx[:, :, 1] = TK - 96
+    idx[:, :, 2:] = O.INT64_MAX
+    kse[..., 1] = 2
+    X.non_causal = 1
+    ref = O.bsa(X, TK, idx, kse, bq, bk, sw, sink)
+    X.non_causal = 0
+    assert np.abs(widen_any(ref, dtype) - widen_any(O.bsa(X, TK, idx, kse, bq, bk, sw, sink), dtype)).max() > 1e-2
+    impls = (2, 1) if dtype == "bf16" else (1,)
+    for impl in impls:
+        out = _run(X, TK, idx, kse, bq, bk, sw, sink, impl=impl, share=True, causal=False)
+        assert_context_close(out, ref, dtype)
+    # decode: one query token per sequence, true positions kept
+    lens = np.array([TK, 1000])
+    XD = make_inputs(16, B=2, TQ=1, TK=TK, H=H, HKV=HKV, D=D, dtype=dtype, pos=(lens - 1)[:, None], scale=0.5)
+    XP = to_paged(XD, 16, seed=3, seq_lens=lens)
+    idx, ks, kse = random_indices(rng, 2, H, 1, BK, bk, 900, same_heads=True)
+    XP.non_causal = 2
+    ref = O.bsa(XP, 2048, idx, kse, 1, bk, sw, sink, share_first_head=True)
+    XP.non_causal = 0
+    out = _run(XP, 2048, idx, kse, 1, bk, sw, sink, impl=0, decode=True, causal=False)
+    assert_context_close(out, ref, dtype)
+
+
+def widen_any(a, dtype):
+    return O.bf16_bits_to_f32(a) if dtype == "bf16" else a

@@ -361,3 +361,27 @@ def test_key_buffers_reported_as_spanning_32_gib_take_the_plain_scans(monkeypatc
     ctx_far, meta_far = run_product(Xd, A)
     assert_metadata_equal(meta_far, ometa)
     assert_context_close(ctx_far, octx, "bf16")
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_non_causal_operator_prefill_and_decode(dtype):
+    """is_causal = False end to end: mask estimation is unchanged (the scan knows no such switch), attention drops its
+    position tests."""
+    print(f"[case] operator non-causal {dtype}", flush=True)
+    X = make_inputs(71, B=2, TQ=200, TK=2048, H=4, HKV=2, D=64, dtype=dtype, scale=0.5)
+    A = tiny_args(is_causal=False)
+    octx, ometa = O.hip_attention_12(X, A)
+    ctx, meta = run_product(X, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, dtype)
+    cctx, _ = O.hip_attention_12(X, tiny_args())
+    wid = (lambda a: O.bf16_bits_to_f32(a)) if dtype == "bf16" else (lambda a: a)
+    assert np.abs(wid(cctx) - wid(octx)).max() > 1e-2
+    lens = np.array([2048, 1500])
+    XD = make_inputs(72, B=2, TQ=1, TK=2048, H=4, HKV=2, D=64, dtype=dtype, pos=(lens - 1)[:, None], scale=0.5)
+    XP = to_paged(XD, 16, seed=4, seq_lens=lens)
+    A = tiny_args(is_causal=False, extend_context_length=2048)
+    octx, ometa = O.hip_attention_12(XP, A)
+    ctx, meta = run_product(XP, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, dtype)

@@ -1,5 +1,5 @@
 """GPU parity of RoPE applied on load (the "extend" modes): mask stage rules relative / streaming / infllm /
-dynamic_extend, sparse
+dynamic_extend / self_extend, sparse
 attention rules streaming / infllm, through every kernel that loads query or key rows (scan on the matrix cores and
 portable scan, tile kernel, portable attention kernel, decode kernel).
 
@@ -165,12 +165,41 @@ def test_dynamic_extend_inside_attention_prefill_and_paged_decode(dtype, D, mode
     assert_context_close(ctx, octx, dtype)
 
 
+@pytest.mark.parametrize("dtype,D", [("f32", 64), ("bf16", 64), ("bf16", 128)])
+@pytest.mark.parametrize("model_ctx", [4096, 131072])
+def test_self_extend_scan_prefill_and_paged_decode(dtype, D, model_ctx):
+    """The self_extend rule of the scan (attention_extend.py:275-289): once a query block reaches beyond the model's
+    context (4096 against 9000 keys), keys older than 8192 positions are grouped by sixteen; below it (131072) every
+    key keeps its own position.  Parity unpinned by execution of the reference (its CPU interpreter floors the
+    quotient the compiled kernel truncates); the oracle's rule is pinned by the closed form in
+    tests/test_oracle_rope.py."""
+    print(f"[case] rope self_extend {dtype} D={D} model_ctx={model_ctx}", flush=True)
+    X = with_rope(make_inputs(61, B=1, TQ=200, TK=9000, H=4, HKV=2, D=D, dtype=dtype, scale=0.5), 9216)
+    A = _ext(scan_extend_backend="self_extend", sa_extend_backend="streaming", model_context_length=model_ctx)
+    octx, ometa = O.hip_attention_12(X, A)
+    ctx, meta = run_product(X, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, dtype)
+    if model_ctx == 4096:  # the grouping really changes what is selected
+        _, plain = O.hip_attention_12(X, _ext(scan_extend_backend="self_extend", sa_extend_backend="streaming"))
+        assert not np.array_equal(plain.indices, ometa.indices)
+    lens = np.array([9000, 8800])
+    XD = make_inputs(62, B=2, TQ=1, TK=9000, H=4, HKV=2, D=D, dtype=dtype, pos=(lens - 1)[:, None], scale=0.5)
+    XP = with_rope(to_paged(XD, 16, seed=5, seq_lens=lens), 9216)
+    A = _ext(scan_extend_backend="self_extend", sa_extend_backend="infllm", model_context_length=model_ctx,
+             extend_context_length=9008)
+    octx, ometa = O.hip_attention_12(XP, A)
+    ctx, meta = run_product(XP, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, dtype)
+
+
 def test_unbuilt_rules_fail_loudly():
     from hip_attn import _native as N
     print("[case] rope unbuilt rules", flush=True)
     X = with_rope(make_inputs(36, B=1, TQ=32, TK=512, H=2, HKV=1, D=32, dtype="f32"), 1024)
-    with pytest.raises(NotImplementedError):
-        run_product(X, _ext(scan_extend_backend="self_extend"))
+    with pytest.raises(NotImplementedError):  # the reference's attention kernels raise on these two as well
+        run_product(X, _ext(sa_extend_backend="self_extend"))
     with pytest.raises(NotImplementedError):
         run_product(X, _ext(sa_extend_backend="relative"))
     with pytest.raises(N.HipAttnError):  # the squeeze divides by pmin - model_context_length / 4: tiny lengths are refused

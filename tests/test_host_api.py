@@ -87,7 +87,7 @@ def test_unsupported_options_fail_loudly():
     from hip_attn import HiPAttentionArgs12
     from hip_attn.operator import _reject_unsupported
 
-    for kw in (dict(using_extend=True), dict(is_causal=False),
+    for kw in (dict(using_extend=True),
                dict(online_update_cache=True), dict(sliding_window_indices=torch.zeros(1))):
         with pytest.raises(NotImplementedError):
             _reject_unsupported(HiPAttentionArgs12(**kw))

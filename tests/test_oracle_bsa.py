@@ -242,3 +242,73 @@ def test_sink_numbering_of_the_decode_programs_equals_a_walk_of_their_loops():
         assert np.array_equal(slot, t - ((t // share) * share) % bk), (bk, sink, second_k, sw)
         slipped += int((slot != t).any())
     assert slipped > 20
+
+
+def _non_causal_reference(X, indices, ks, bq, bk, sw, sink, max_tsrc, decode):
+    """is_causal = False written from its description (attention_extend_bsa.py:511-523, :743-752): the mask keeps
+    nothing but validity.  Query-block form: every row sits at position max_tsrc - 1, so all rows of a block attend
+    the same multiset: the tokens of their selected blocks (at or above the sink), the sink, and the last
+    sw + bq tokens; a token that is selected and in that window counts twice.  Decode form: the same with the row's
+    true position in place of max_tsrc - 1.  float64."""
+    B, TQ, H, D = X.q.shape
+    k = widen(X.k, X.dtype).astype(np.float64)
+    v = widen(X.v, X.dtype).astype(np.float64)
+    TK = k.shape[1]
+    G = H // k.shape[2]
+    cq, ck = O.scale_constants(D, X.dtype)
+    f32 = lambda a: a.astype(np.float32).astype(np.float64)
+    qh, kh = f32(widen(X.q, X.dtype) * np.float32(cq)), f32(widen(X.k, X.dtype) * np.float32(ck))
+    out = np.zeros((B, TQ, H, D))
+    for b in range(B):
+        for h in range(H):
+            for qb in range(O.cdiv(TQ, bq)):
+                rows = np.arange(qb * bq, min(TQ, (qb + 1) * bq))
+                curr = (int(X.pos[b, rows].max()) + 1) if decode else max_tsrc
+                count = np.zeros(TK)
+                for j in range(int(ks[b * H + h, qb])):
+                    st = int(indices[b * H + h, qb, j])
+                    for t in range(st, st + bk):
+                        if 0 <= t < min(TK, max_tsrc) and sink <= t < curr:
+                            count[t] += 1
+                count[:min(sink, curr)] += 1
+                if sw > 0:
+                    count[max(0, curr - sw - bq):curr] += 1
+                logits = np.where(count[None, :] > 0, qh[b, rows, h] @ kh[b, :, h // G].T, -np.inf)
+                pr = np.exp(logits - logits.max(axis=1, keepdims=True)) * count[None, :]
+                out[b, rows, h] = (pr / pr.sum(axis=1, keepdims=True)) @ v[b, :, h // G]
+    return out
+
+
+@pytest.mark.parametrize("decode", [False, True])
+def test_non_causal_mask_keeps_validity_only(decode):
+    rng = np.random.default_rng(5)
+    TK, H, HKV, D, bk, BK, sw, sink = 192, 4, 2, 32, 4, 12, 24, 8
+    bq, TQ = (1, 1) if decode else (16, 40)
+    pos = np.array([[150], [99]]) if decode else None
+    X = make_inputs(14, B=2, TQ=TQ, TK=TK, H=H, HKV=HKV, D=D, dtype="f32", scale=0.3, pos=pos)
+    nbq = O.cdiv(TQ, bq)
+    idx, ks, kse = random_indices(rng, 2, H, nbq, BK, bk, TK, same_heads=False)
+    idx[0, 0, :3] = [TK - 40, TK - 24, TK - 8]  # blocks inside the last sw + bq tokens: attended twice
+    idx[0, 0, 3:] = O.INT64_MAX
+    ks[0, 0] = 3; kse[0, 0, 1] = 3
+    X.non_causal = 2 if decode else 1
+    got = O.bsa(X, TK, idx, kse, bq, bk, sw, sink)
+    ref = _non_causal_reference(X, idx, ks, bq, bk, sw, sink, TK, decode)
+    assert np.abs(got - ref).max() < 2e-5
+    X.non_causal = 0
+    causal = O.bsa(X, TK, idx, kse, bq, bk, sw, sink)
+    assert np.abs(causal - got).max() > 1e-3  # the switch really changes the result
+
+
+def test_non_causal_with_a_huge_window_is_plain_bidirectional_attention():
+    TK, TQ, H, D = 96, 96, 2, 64
+    X = make_inputs(8, B=1, TQ=TQ, TK=TK, H=H, HKV=1, D=D, dtype="f32", scale=0.3)
+    idx = np.full((H, 6, 2), O.INT64_MAX, dtype=np.int64)
+    kse = np.zeros((H, 6, 2), dtype=np.int32)
+    X.non_causal = 1
+    got = O.bsa(X, TK, idx, kse, 16, 2, 4096, 0)
+    q = torch.from_numpy(X.q).permute(0, 2, 1, 3).double()
+    k = torch.from_numpy(X.k).permute(0, 2, 1, 3).double().repeat(1, 2, 1, 1)
+    v = torch.from_numpy(X.v).permute(0, 2, 1, 3).double().repeat(1, 2, 1, 1)
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=False, scale=1.0)
+    assert np.abs(got - ref.permute(0, 2, 1, 3).numpy()).max() < 2e-5

@@ -48,25 +48,34 @@ def _stage0(TK, sink, sw_eff, chunk, B, BS, H):
     return left, right, scores
 
 
-@pytest.mark.parametrize("backend", ["relative", "streaming", "infllm", "dynamic_extend", "dynamic_extend squeezed"])
+@pytest.mark.parametrize("backend", ["relative", "streaming", "infllm", "dynamic_extend", "dynamic_extend squeezed",
+                                     "self_extend", "self_extend grouped"])
 def test_mask_stage_chunk_size_one_scores(backend):
     # Chunks of one token: the scan evaluates token t once as the "left" and once as the "right" candidate and
     # keeps the larger score.  relative: key at 0 (left) or 1 (right), query at 1 + window; streaming: key at its
     # chunk number, query at min(position, chunks + window); infllm: key at 0, query at the window; dynamic_extend:
     # every query row at its own position, and the key at its own token while the block ends inside the model's
     # context -- plain rotary scores -- or, beyond it (model context 32 against positions 48..63), keys older than
-    # a quarter of that context squeezed linearly into the rest (attention_extend.py:249-274).
+    # a quarter of that context squeezed linearly into the rest (attention_extend.py:249-274).  self_extend: like
+    # dynamic_extend, except that beyond the model's context a key older than 8192 positions moves to
+    # pmin + trunc((t - pmin) / 16): sixteen neighbours share a position (attention_extend.py:275-289; the quotient
+    # of the negative numerator truncates toward zero, as the compiled kernel's int32 division does).  8192 is fixed
+    # in the reference, so the grouped case needs positions beyond it.
     D, BQ, sink, sw_eff = 32, 8, 4, 6
-    X = make_inputs(11, B=1, TQ=16, TK=64, H=2, HKV=1, D=D, dtype="f32")
     squeezed = backend.endswith("squeezed")
+    grouped = backend.endswith("grouped")
     backend = backend.split()[0]
-    X = with_rope(X, 256, scan_backend=backend)
+    TK = 8400 if grouped else 64
+    X = make_inputs(11, B=1, TQ=16, TK=TK, H=2, HKV=1, D=D, dtype="f32")
+    X = with_rope(X, TK + 64 if grouped else 256, scan_backend=backend)
     if squeezed:
         X.model_context_length = 32
-    left, right, scores = _stage0(64, sink, sw_eff, 1, 1, 2, 2)
+    if grouped:
+        X.model_context_length = 4096
+    left, right, scores = _stage0(TK, sink, sw_eff, 1, 1, 2, 2)
     l_in = left.copy()
     n = left.shape[-1]
-    O.mask_stage(X, 64, left, right, scores, BS=2, BQ=BQ, stride_q=1, block_chunk=16, scan_stride=1, sw_eff=sw_eff)
+    O.mask_stage(X, TK, left, right, scores, BS=2, BQ=BQ, stride_q=1, block_chunk=16, scan_stride=1, sw_eff=sw_eff)
     cq, ck = O.scale_constants(D, "f32")
     q = widen(X.q, "f32").astype(np.float64)
     k = widen(X.k, "f32").astype(np.float64)
@@ -87,6 +96,12 @@ def test_mask_stage_chunk_size_one_scores(backend):
                     moved = int((np.float32(t) - np.float32(pmin - w)) * (np.float32(ctx - w) / np.float32(pmin - w)))
                     return (max(pmax - ctx, moved + pmin - w),) * 2
                 qpos = p
+            elif backend == "self_extend":
+                def kpos(c, t, pmin=int(p.min()), pmax=int(p.min()) + BQ, ctx=int(X.model_context_length)):
+                    if t >= pmax - 8192 or pmax <= ctx:
+                        return (t, t)
+                    return (max(0, pmin - (pmin - t) // 16),) * 2  # t < pmin: truncation of (t - pmin) / 16
+                qpos = p
             else:
                 qpos, kpos = np.minimum(p, n + sw_eff), (lambda c: (c, c))
             qr = _rot(q[0, rows, h], qpos, D) * cq
@@ -95,9 +110,14 @@ def test_mask_stage_chunk_size_one_scores(backend):
                 if t > p.min() - sw_eff:
                     assert scores[0, qb, h, c] == -32000.0
                     continue
-                kps = kpos(c, t) if backend == "dynamic_extend" else kpos(c)
+                if grouped and 300 < t < TK - 300:
+                    continue  # the grouped case checks both ends of the key range, not all 8400 tokens
+                kps = kpos(c, t) if backend in ("dynamic_extend", "self_extend") else kpos(c)
                 if squeezed and t < 40:
                     assert kps[0] != t  # the squeeze really moves these keys
+                if grouped and t < 190:
+                    assert kps[0] != t
+                    assert int(p.min()) - kps[0] == (int(p.min()) - t) // 16  # sixteen keys share a position
                 best = max(float((qr @ (_rot(k[0, t, 0], kp, D) * ck)).max()) for kp in kps)
                 assert abs(scores[0, qb, h, c] - best) <= 2e-5 * max(1.0, abs(best)), (backend, h, qb, c)
                 checked += 1
