@@ -33,16 +33,63 @@ HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 # HBM bytes per launch of the prefill kernels, from two rocprofv3 --pmc runs of this file (FETCH_SIZE, then
-# WRITE_SIZE, KiB per dispatch).  A 268 435 456-byte device copy reads 131 095 KiB of FETCH_SIZE and 262 144 KiB of
-# WRITE_SIZE in the same runs, so FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0.
+# WRITE_SIZE, KiB per dispatch; `python bench.py --traffic-from <fetch run dir> <write run dir>` prints this table from
+# their output).  A 268 435 456-byte device copy reads 131 095 KiB of FETCH_SIZE and 262 144 KiB of WRITE_SIZE in the
+# same runs, so FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0.  The figures belong to the kernel sources they were
+# taken on: TRAFFIC_SOURCES_SHA256 is the digest of those sources, and when the sources at hand differ the bench
+# reports no traffic instead of a stale one.
 TRAFFIC_SOURCE = ("recorded: profiles/prefill_hbm_traffic_pmc.md (not measured in this run); FETCH_SIZE / WRITE_SIZE count bytes "
                   "between the L2 caches and the memory side, served by the 256 MB memory-side cache or by HBM")
+TRAFFIC_SOURCES_SHA256 = "unrecorded"
 MEASURED_TRAFFIC_BYTES = {
     "mask_stage[n=507,chunk=256,rows=16]": 2.0 * 5366948.4 * 1024 + 718949.5 * 1024,
     "mask_stage[n=1024,chunk=32,rows=16]": 2.0 * 7033647.6 * 1024 + 564427.4 * 1024,
     "mask_stage[n=1024,chunk=8,rows=64]": 2.0 * 2208493.8 * 1024 + 216630.1 * 1024,
     "bsa_prefill": 2.0 * 1860808.6 * 1024 + 262144.2 * 1024,
 }
+
+
+def kernel_sources_sha256():
+    """Digest of the kernel sources the library is built from (names and contents, in name order)."""
+    import hashlib
+
+    d = os.path.join(ROOT, "hip-attention_amd", "csrc")
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(d)):
+        if name.endswith((".hip", ".hpp")) or name == "Makefile":
+            h.update(name.encode())
+            h.update(open(os.path.join(d, name), "rb").read())
+    return h.hexdigest()
+
+
+def recorded_traffic(name):
+    """(bytes or None, where the figure comes from): None once the kernel sources have changed since the record."""
+    now = kernel_sources_sha256()
+    if now != TRAFFIC_SOURCES_SHA256:
+        return None, (f"none: the kernel sources have changed since the counters were taken "
+                      f"(recorded on {TRAFFIC_SOURCES_SHA256[:12]}, now {now[:12]}); see profiles/prefill_hbm_traffic_pmc.md "
+                      "for the last record")
+    return MEASURED_TRAFFIC_BYTES.get(name), TRAFFIC_SOURCE
+
+
+def print_traffic_table(fetch_dir, write_dir):
+    """The table above from the output directories of the two counter runs (rocprofv3 ... -d <dir>)."""
+    import glob
+    import sqlite3
+
+    def per_kernel(d, counter):
+        db = sorted(glob.glob(os.path.join(d, "**", "*.db"), recursive=True))[-1]
+        c = sqlite3.connect(db)
+        q = ("select kernel_name, grid_size, avg(value), count(*) from counters_collection where counter_name = ? "
+             "group by kernel_name, grid_size order by min(dispatch_id)")
+        return [(n.split("(")[0], g, v, k) for n, g, v, k in c.execute(q, (counter,))]
+
+    fetch, write = per_kernel(fetch_dir, "FETCH_SIZE"), per_kernel(write_dir, "WRITE_SIZE")
+    wmap = {(n, g): v for n, g, v, _ in write}
+    print(f'TRAFFIC_SOURCES_SHA256 = "{kernel_sources_sha256()}"')
+    for n, g, v, k in fetch:
+        if any(t in n for t in ("mask_stage", "bsa_mfma", "qhat", "copyBuffer", "prescale")):
+            print(f"{n[-70:]:70s} grid {g:>10} dispatches {k:>3}  FETCH_SIZE {v:14.1f} KiB  WRITE_SIZE {wmap.get((n, g), float('nan')):14.1f} KiB")
 
 
 SAMPLE_QUERIES = 512  # the last queries of the prefill workload that the CPU oracle recomputes
@@ -120,10 +167,10 @@ def run_prefill(args, device):
             # re-read by every query block), so the rows it reads per second are reported as what they are, logical
             # bytes, with no roof; the fraction of the HBM peak is taken from the recorded HBM counters.
             gbs = by / (kern[nm] * 1e-3) / 1e9
-            traffic = MEASURED_TRAFFIC_BYTES.get(nm)
+            traffic, traffic_source = recorded_traffic(nm)
             hbm_gbs = traffic / (kern[nm] * 1e-3) / 1e9 if traffic else None
             rooflines.append({"kernel": nm, "bound": "l2-gather", "achieved": gbs, "peak": None, "unit": "GB/s",
-                              "frac": None, "logical_GBps": gbs, "traffic": traffic, "traffic_source": TRAFFIC_SOURCE,
+                              "frac": None, "logical_GBps": gbs, "traffic": traffic, "traffic_source": traffic_source,
                               "hbm_counter_GBps": hbm_gbs,
                               "frac_hbm_counter": hbm_gbs / HBM_PEAK_GBS if hbm_gbs else None,
                               "ms": kern[nm], "algorithmic_bytes": by})
@@ -131,7 +178,7 @@ def run_prefill(args, device):
         tf = bsa_flops / (kern["bsa_prefill"] * 1e-3) / 1e12
         rooflines.append({"kernel": "bsa_prefill", "bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS,
                           "unit": "TFLOP/s", "frac": tf / MFMA_BF16_PEAK_TFLOPS,
-                          "traffic": MEASURED_TRAFFIC_BYTES.get("bsa_prefill"), "traffic_source": TRAFFIC_SOURCE,
+                          "traffic": recorded_traffic("bsa_prefill")[0], "traffic_source": recorded_traffic("bsa_prefill")[1],
                           "ms": kern["bsa_prefill"], "algorithmic_flops": bsa_flops})
     # headline: the kernel of this step that sits under a hardware roof, the sparse attention kernel (matrix cores)
     roofed = [r for r in rooflines if r["frac"] is not None]
@@ -763,7 +810,13 @@ def main():
                     help="profiling aid: prefill without the access-statistics flags the default arguments ask for")
     ap.add_argument("--only", choices=["prefill", "decode", "batched_decode", "offload", "cpu"], default=None,
                     help="profiling aid: run one part; the other fields of the JSON line are null")
+    ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"), default=None,
+                    help="no GPU work: print the recorded-traffic table from the output directories of the two "
+                         "rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of this file")
     args = ap.parse_args()
+    if args.traffic_from:
+        print_traffic_table(*args.traffic_from)
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; every figure is one MI355X's throughput (--gpus 1).",
               file=sys.stderr)
