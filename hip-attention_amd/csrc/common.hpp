@@ -149,7 +149,7 @@ struct CacheView {
 // same rows many times); CHECK = false stores blindly (right for one pass over mostly distinct rows).
 // Racing lanes store the same value; a stale read only repeats the store.
 template <bool CHECK = true>
-__device__ __forceinline__ void mark_flag(int32_t *f) {
+__device__ __forceinline__ void mark_flag(uint8_t *f) {
     if (!CHECK || *f == 0) *f = 1;
 }
 
@@ -280,7 +280,7 @@ __device__ __forceinline__ float load_kv_elem(const void *base, int64_t off) {
 struct KVExt {
     int cached;
     CacheView cache;
-    int32_t *access_flags, *miss_flags;
+    uint8_t *access_flags, *miss_flags;  // one byte per page (a quarter of the words to clear and to keep in cache)
     int64_t flags_stride_b, flags_stride_h;
     int kv8;  // host: K / V are stored as fp8 (e5m2) bytes, kernels are launched in their KV8 builds
     // host: does a launch need the EXT build of its kernel

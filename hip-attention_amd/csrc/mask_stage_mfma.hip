@@ -212,7 +212,7 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     const uint32_t piece_h = !DMA ? 0u
                              : (uint32_t)(((int64_t)kvh * p.kv.k_stride_h + ((OFF32 || p.kv.paged) ? 0 : (int64_t)b * p.kv.k_stride_b)) >> 3);
     const int tsrc32 = DMA ? (int)p.kv.tsrc : 0;
-    int32_t *flag_row = nullptr;
+    uint8_t *flag_row = nullptr;
     if constexpr (DMA) {
         if (kx->access_flags) flag_row = kx->access_flags + (int64_t)b * kx->flags_stride_b + (int64_t)kvh * kx->flags_stride_h;
     }

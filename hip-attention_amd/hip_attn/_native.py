@@ -219,14 +219,15 @@ def make_kv_dense(k: torch.Tensor, v: torch.Tensor) -> KVStruct:
 
 
 def set_flags(s: KVStruct, access: Optional[torch.Tensor], miss: Optional[torch.Tensor]) -> KVStruct:
-    """Attach ``int32 [B, HKV, pages]`` access / miss flag tensors to a KV description (returns a copy)."""
+    """Attach ``uint8 [B, HKV, pages]`` access / miss flag tensors to a KV description (returns a copy)."""
     out = KVStruct.from_buffer_copy(s)
     if access is not None:
-        assert access.dtype == torch.int32 and access.ndim == 3 and access.stride(2) == 1
+        assert access.dtype == torch.uint8 and access.ndim == 3 and access.stride(2) == 1, \
+            "statistics flags are bytes until a counter has been read; a call needs fresh ones"
         out.access_flags = access.data_ptr()
         out.flags_stride_b, out.flags_stride_h = access.stride(0), access.stride(1)
         if miss is not None:
-            assert miss.shape == access.shape and miss.stride() == access.stride() and miss.dtype == torch.int32
+            assert miss.shape == access.shape and miss.stride() == access.stride() and miss.dtype == torch.uint8
             out.miss_flags = miss.data_ptr()
     return out
 

@@ -178,8 +178,9 @@ def _kv_struct(args: HiPAttentionArgs, k: Optional[Tensor], v: Optional[Tensor],
             assert args.k_cache is not None and args.v_cache is not None, "paged mode needs k_cache and v_cache"
             assert args.k_cache.ndim == 4 and args.v_cache.ndim == 4
             st, keep = N.make_kv_paged(args.k_cache, args.v_cache, bt, sl, max_tsrc), (bt, sl)
-    if stats is not None and stats.access_counter is not None:
-        st = N.set_flags(st, stats.access_counter, stats.cache_miss_counter if st.cache else None)
+    if stats is not None and stats.flags()[0] is not None:
+        access, miss = stats.flags()
+        st = N.set_flags(st, access, miss if st.cache else None)
     return st, keep
 
 
@@ -187,30 +188,31 @@ _ZERO_FLAG: dict = {}
 
 
 def _zero_flag(device) -> Tensor:
-    """One int32 zero per device, the target of the read-only miss flags of calls without an offload cache."""
+    """One zero byte per device, the target of the read-only miss flags of calls without an offload cache."""
     key = (device.type, device.index)
     zero = _ZERO_FLAG.get(key)
     if zero is None:
-        zero = torch.zeros((1, 1, 1), dtype=torch.int32, device=device)
+        zero = torch.zeros((1, 1, 1), dtype=torch.uint8, device=device)
         if not (device.type == "cuda" and torch.cuda.is_current_stream_capturing()):
             _ZERO_FLAG[key] = zero  # an allocation made during graph capture belongs to that graph: not kept
     return zero
 
 
 def _new_statistics(args: HiPAttentionArgs, B: int, head_kv: int, pages: int, device, count: int = 1):
-    """Zeroed ``int32 [B, HEAD_KV, pages]`` access and miss flags (attention_extend.py:1994-2006).  Without an
+    """Zeroed ``[B, HEAD_KV, pages]`` access and miss flags (attention_extend.py:1994-2006), one byte per page as the
+    kernels keep them (``HiPAttentionCacheAccessStatistics`` widens them to int32 when they are read).  Without an
     offload cache nothing can miss: the miss flags are then a read-only view of one zero kept per device, which
     saves clearing ``B * HEAD_KV * pages`` words per call.  ``count`` > 1 returns that many sets whose access flags
     are cleared by one launch (a mask refresh needs one for the scan and one for the attention)."""
     if count > 1:
         if not args.require_cache_statistics or args.offload_cache is not None:
             return [_new_statistics(args, B, head_kv, pages, device) for _ in range(count)]
-        both = torch.zeros((count, B, head_kv, pages), dtype=torch.int32, device=device)
+        both = torch.zeros((count, B, head_kv, pages), dtype=torch.uint8, device=device)
         miss = _zero_flag(device).expand(B, head_kv, pages)
         return [HiPAttentionCacheAccessStatistics(both[i], miss) for i in range(count)]
     if not args.require_cache_statistics:
         return HiPAttentionCacheAccessStatistics(None, None)
-    access = torch.zeros((B, head_kv, pages), dtype=torch.int32, device=device)
+    access = torch.zeros((B, head_kv, pages), dtype=torch.uint8, device=device)
     if args.offload_cache is not None:
         return HiPAttentionCacheAccessStatistics(access, torch.zeros_like(access))
     return HiPAttentionCacheAccessStatistics(access, _zero_flag(device).expand(B, head_kv, pages))

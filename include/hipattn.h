@@ -130,12 +130,14 @@ typedef struct hipattn_kv {
      * memory (see hipattn_cache_create).  Requires paged != 0. */
     const struct hipattn_cache *cache;
     /* Access statistics (HiPAttentionCacheAccessStatistics, src/hip_attn/v1_2/attention_metadata.py:76-81,
-     * stores at src/hip_attn/v1_2/uvm_gpu_cache.py:845-862,1365-1372): NULL, or int32 [B, HKV, pages]
+     * stores at src/hip_attn/v1_2/uvm_gpu_cache.py:845-862,1365-1372): NULL, or uint8 [B, HKV, pages]
      * (pages = tsrc when dense) where every page whose key row was loaded is set to 1, and the same
      * for loads the offload cache could not serve.  Only hipattn_mask_stage and the bsa entry points
-     * write them. */
-    int32_t *access_flags;
-    int32_t *miss_flags;
+     * write them.  The reference keeps int32 counters that only ever hold 0 or 1; a byte per page is what a decode
+     * step at 1M keys can afford to clear (two tensors of 8 MB instead of 32 MB) and leaves more of the memory-side
+     * cache to the key rows.  The host widens them to the reference's int32 layout when a caller reads them. */
+    uint8_t *access_flags;
+    uint8_t *miss_flags;
     int64_t flags_stride_b, flags_stride_h;
     /* fp8 != 0: k and v hold one byte per element, the uint8 view of a float8_e5m2 paged cache
      * (src/hip_attn/v1_2/paged_hip.py:409-418, src/hip_attn/v1_2/uvm_gpu_cache.py:1043-1046); every loaded value is
