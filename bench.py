@@ -201,8 +201,10 @@ def run_prefill(args, device):
     }
 
 
-def _time_decode(step, steps, refresh_every):
-    """Times a decode loop given ``step(meta_or_None) -> (out, meta)``: eager calls, then HIP-graph replay."""
+def _time_decode(step, steps, refresh_every, step_prescaled=None):
+    """Times a decode loop given ``step(meta_or_None) -> (out, meta)``: eager calls, then HIP-graph replay.
+    ``step_prescaled``: the same refresh step reading a caller-kept pre-scaled key copy (the opt-in
+    ``HiPAttentionArgs.k_prescaled``), timed beside the plain one."""
     import torch
     from hip_attn import _native as N
 
@@ -314,6 +316,23 @@ def _time_decode(step, steps, refresh_every):
         return median(ts)
 
     us_refresh_cold, us_plain_cold, us_cached_cold = cold(g_refresh), cold(g_plain), cold(g_cached)
+    prescaled = None
+    if step_prescaled is not None:
+        with torch.cuda.stream(side):
+            step_prescaled(None)
+        torch.cuda.synchronize()
+        g_pre = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g_pre, pool=g_refresh.pool()):
+            out_pre, meta_pre = step_prescaled(None)
+        torch.cuda.synchronize()
+        us_pre = median([timed(16, lambda i: g_pre.replay()) for _ in range(9)])
+        us_pre_cold = cold(g_pre)
+        prescaled = {"us_per_step_refresh": us_pre, "cold_us_per_step_refresh": us_pre_cold,
+                     "indices_equal_plain_step": bool(torch.equal(meta_pre.indices, meta_r.indices)),
+                     "context_equal_plain_step": bool(torch.equal(out_pre.view(torch.int16), out_r.view(torch.int16))),
+                     "what": "opt-in HiPAttentionArgs.k_prescaled: the scans read bf16(K * c_k) from a copy the caller "
+                             "keeps (twice the key memory) instead of scaling every sampled row; with statistics"}
+        del g_pre, out_pre, meta_pre
     del g_plain, out_p, evict
     N.profile_begin()
     _, meta_last = step(None)
@@ -329,6 +348,7 @@ def _time_decode(step, steps, refresh_every):
                         "us_per_step_cached": us_cached_cold,
                         "how": "1 GiB of other data read and written before every replay, each replay timed on its own"},
         "graph_replay_matches_eager": graph_matches,
+        "prescaled_keys": prescaled,
         "eager": {"us_per_step_mixed": eager_mixed, "us_per_step_refresh": eager_refresh,
                   "us_per_step_cached": eager_cached, "wall_us_per_step_mixed": eager_wall},
         "refresh_kernels_us": [(n, round(ms * 1e3, 1)) for n, ms in prof],
@@ -358,6 +378,10 @@ def _with_rooflines(res, refresh_bytes, attn_bytes):
     cold["hbm_frac_refresh_without_statistics"] = (
         refresh_bytes / (cold["us_per_step_refresh_without_statistics"] * 1e-6) / 1e9 / HBM_PEAK_GBS)
     cold["hbm_frac_cached"] = attn_bytes / (cold["us_per_step_cached"] * 1e-6) / 1e9 / HBM_PEAK_GBS
+    pre = res.get("prescaled_keys")
+    if pre:
+        pre["hbm_frac_refresh"] = refresh_bytes / (pre["us_per_step_refresh"] * 1e-6) / 1e9 / HBM_PEAK_GBS
+        pre["cold_hbm_frac_refresh"] = refresh_bytes / (pre["cold_us_per_step_refresh"] * 1e-6) / 1e9 / HBM_PEAK_GBS
     res.update({"refresh_algorithmic_bytes": refresh_bytes, "cached_algorithmic_bytes": attn_bytes,
                 "hbm_frac_refresh": gbs_refresh / HBM_PEAK_GBS, "hbm_frac_cached": gbs_cached / HBM_PEAK_GBS,
                 "refresh_GBps": gbs_refresh, "cached_GBps": gbs_cached})
@@ -413,7 +437,17 @@ def run_decode(args, device, TK=1 << 20, steps=64, refresh_every=8, needles=64):
                                require_cache_statistics=(meta_in is None) if stats is None else stats)
         return hip_attention_12(q, k, v, a, cached_metadata=meta_in)
 
-    res, meta = _time_decode(step, steps, refresh_every)
+    from hip_attn import prescale_keys
+
+    khat = prescale_keys(k)
+
+    def step_prescaled(meta_in):
+        a = HiPAttentionArgs12(sliding_window_size=1024, position_ids=pos, require_cache_statistics=meta_in is None,
+                               k_prescaled=khat)
+        return hip_attention_12(q, k, v, a, cached_metadata=meta_in)
+
+    res, meta = _time_decode(step, steps, refresh_every, step_prescaled)
+    del khat
     # needle recall: a needle counts as found when its 8-token block is among the selected blocks of a head
     idx = meta.indices[:, 0, :]  # [H, BK]
     found = (idx[:, :, None] == starts.to(device)[None, None, :]).any(dim=1).float()  # [H, needles]
@@ -481,7 +515,18 @@ def run_batched_decode(args, device, B=16, steps=64, refresh_every=8):
                                require_cache_statistics=(meta_in is None) if stats is None else stats)
         return hip_attention_12(q, None, None, a, cached_metadata=meta_in)
 
-    res, meta = _time_decode(step, steps, refresh_every)
+    from hip_attn import prescale_keys
+
+    khat = prescale_keys(kc)
+
+    def step_prescaled(meta_in):
+        a = HiPAttentionArgs12(sliding_window_size=1024, position_ids=pos, k_cache=kc, v_cache=vc, block_table=bt,
+                               cache_seq_lens=sl, extend_context_length=MAXLEN,
+                               require_cache_statistics=meta_in is None, k_prescaled=khat)
+        return hip_attention_12(q, None, None, a, cached_metadata=meta_in)
+
+    res, meta = _time_decode(step, steps, refresh_every, step_prescaled)
+    del khat
     if not args.skip_cpu:
         # the oracle on the shortest and the longest sequence of the batch, same paged cache and block table
         import numpy as np

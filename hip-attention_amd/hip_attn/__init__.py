@@ -16,6 +16,18 @@ from .offload import HiPOffloadCache
 from .memory_pool import HiPMetadataCachePool, cuda_graph_capture_configs
 from .model_offload import HiPModelOffloadCache
 
+
+
+def prescale_keys(k, head_major: bool = True, rows=None):
+    """``bf16(k * c_k)`` for a whole bf16 key tensor (dense ``[B, T, HKV, D]`` or a paged cache
+    ``[pages, page, HKV, D]``): the copy ``HiPAttentionArgs.k_prescaled`` takes.  ``head_major`` lays the copy out
+    with the kv head outermost in memory (same logical shape), which keeps the rows a search samples close together.
+    No counterpart in the reference (an extension; see ``HiPAttentionArgs.k_prescaled``)."""
+    from . import _native
+
+    return _native.prescale_k(k, k.device, head_major=head_major)
+
+
 hip_attention = hip_attention_12
 HiPAttentionArgs = HiPAttentionArgs12
 HiPAttentionOutputMetadata = HiPAttentionOutputMetadata12
@@ -39,4 +51,5 @@ __all__ = [
     "HiPMetadataCachePool",
     "HiPModelOffloadCache",
     "cuda_graph_capture_configs",
+    "prescale_keys",
 ]

@@ -234,9 +234,16 @@ def _mask_kv(args: HiPAttentionArgs, k_mask: Optional[Tensor], max_tsrc: int, q:
         if src is not None and src.dtype == torch.bfloat16 and src.ndim == 4 and src.stride(-1) == 1:
             rows_total = src.shape[0] * src.shape[1] * src.shape[2]
             force = os.getenv("HIP_ATTN_PRESCALE_K", "")  # "0" / "1" override the heuristic (testing)
-            if force == "1" or (force != "0" and sampled_rows >= 4 * rows_total):
+            given = args.k_prescaled if rope_tabs is None else None  # a copy the caller keeps up to date
+            if given is not None:
+                if given.shape != src.shape or given.dtype != torch.bfloat16 or given.stride(-1) != 1 or given.device != src.device:
+                    raise ValueError("k_prescaled must be a bf16 device tensor with the shape of the key storage "
+                                     f"({tuple(src.shape)}), got {tuple(given.shape)} {given.dtype}")
+            if given is not None or force == "1" or (force != "0" and sampled_rows >= 4 * rows_total):
                 delta = 0
-                if rope_tabs is None:
+                if given is not None:
+                    khat = khat0 = given
+                elif rope_tabs is None:
                     # the copy is laid out with the kv head outermost: the rows a search samples then lie within a
                     # few KB instead of spreading over HKV times as much (cfg-2-like prefill: the 256- and 32-token
                     # stages 4.13 -> 3.77 and 5.19 -> 4.82 ms, the same from a page-16 cache)

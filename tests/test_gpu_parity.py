@@ -11,7 +11,7 @@ import torch
 
 from oracle import hip12 as O
 from helpers import make_inputs, tiny_args, to_paged
-from gpu_utils import assert_context_close, assert_metadata_equal, run_product
+from gpu_utils import assert_context_close, assert_metadata_equal, run_product, to_torch
 
 pytestmark = pytest.mark.gpu
 
@@ -385,3 +385,36 @@ def test_non_causal_operator_prefill_and_decode(dtype):
     ctx, meta = run_product(XP, A)
     assert_metadata_equal(meta, ometa)
     assert_context_close(ctx, octx, dtype)
+
+
+def test_caller_kept_prescaled_keys_change_nothing_but_the_time():
+    """``HiPAttentionArgs.k_prescaled`` (an extension): mask estimation reads bf16(K * c_k) from a copy the caller keeps
+    instead of scaling every sampled row; indices, flags and context must be what they are without it.  Decode on a
+    dense tensor and on a paged cache, and a prefill."""
+    from hip_attn import prescale_keys
+
+    print("[case] caller-kept prescaled keys", flush=True)
+    lens = np.array([4096, 3000])
+    XD = make_inputs(81, B=2, TQ=1, TK=4096, H=8, HKV=2, D=128, dtype="bf16", pos=(lens - 1)[:, None])
+    A = O.OArgs(sliding_window_size=512)
+    octx, ometa = O.hip_attention_12(XD, A)
+    for head_major in (True, False):
+        khat = prescale_keys(to_torch(XD.k, "bf16"), head_major=head_major)
+        ctx, meta = run_product(XD, A, k_prescaled=khat)
+        assert_metadata_equal(meta, ometa)
+        assert_context_close(ctx, octx, "bf16")
+    XP = to_paged(XD, 16, seed=6, seq_lens=lens)
+    A = O.OArgs(sliding_window_size=512, extend_context_length=4096)
+    octx, ometa = O.hip_attention_12(XP, A)
+    khat = prescale_keys(to_torch(XP.k_cache, "bf16"))
+    ctx, meta = run_product(XP, A, k_prescaled=khat)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, "bf16")
+    X = make_inputs(82, B=1, TQ=256, TK=4096, H=8, HKV=2, D=128, dtype="bf16")
+    A = O.OArgs(sliding_window_size=512)
+    octx, ometa = O.hip_attention_12(X, A)
+    ctx, meta = run_product(X, A, k_prescaled=prescale_keys(to_torch(X.k, "bf16")))
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, "bf16")
+    with pytest.raises(ValueError):
+        run_product(X, A, k_prescaled=prescale_keys(to_torch(X.k, "bf16"))[:, :100])
