@@ -1,4 +1,4 @@
-// MFMA tile kernel for block-sparse attention (bf16, head dim 64 / 128, query block <= 64 rows).
+// MFMA tile kernel for block-sparse attention (bf16, head dim 64 / 128 / 256, query block <= 64 rows).
 //
 // One workgroup = one (batch, kv head, query block) and up to four query heads of the GQA group;
 // a wavefront owns one head and one 32-row half of the query block, so every gathered K/V tile in
@@ -38,6 +38,14 @@ struct MfmaMeta {
 // Tiles are resolved in batches of META_BATCH, one batch ahead of their use: the ring holds two batches.
 template <int HID>
 constexpr int META_BATCH = HID <= 128 ? 16 : 4;
+
+// Columns of V, and of the output, that one wave works on.  Head dim 256 is served in two passes of 128 columns by
+// two waves, each forming all of the logits of its 32 rows: with 256 columns a wave would need 128 accumulator
+// registers beside 64 of query fragments and 32 of logits, and spilled about 110; half again as many products
+// cost less than that.  The passes of a head sit in one workgroup (which then serves two heads instead of four) and
+// share its K and V tiles.
+template <int HID>
+constexpr int V_COLS = HID <= 128 ? HID : 128;
 
 template <int HID>
 struct MfmaSmem {
@@ -228,7 +236,8 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
     const KVExt *kx = nullptr;
     if constexpr (EXT) kx = &p.kx;
     constexpr int KS = HID / 16;   // k-steps of the first product
-    constexpr int DB = HID / 32;   // 32-row blocks of O^T
+    constexpr int DV = V_COLS<HID>, NPASS = HID / DV;
+    constexpr int DB = DV / 32;    // 32-row blocks of O^T
     constexpr int CPT = TN * (HID / 8) / NTHREADS;  // 16-byte chunks per thread per tile
     extern __shared__ __align__(16) unsigned char smem_raw[];
     MfmaSmem<HID> &sm = *reinterpret_cast<MfmaSmem<HID> *>(smem_raw);
@@ -237,7 +246,9 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
     // scalar unit instead of under execution masks
     const int tid = threadIdx.x, lane = tid & 63, wid = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, hh = lane >> 5;
-    const int whead = wid >> 1, half = wid & 1;
+    const int half = wid & 1;
+    const int whead = (wid >> 1) / NPASS;            // head slot of the workgroup
+    const int dv0 = ((wid >> 1) % NPASS) * DV;       // first output column of this wave
 
     long long L = xcd_remap((long long)blockIdx.x, total_wg);
     const int qb = (int)(L % p.NBQ);
@@ -411,6 +422,10 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
     };
     uint4 kreg[CPT], vreg[CPT];
     uint4 creg[ROPE ? CPT : 1], sreg[ROPE ? CPT : 1];  // cos / sin pieces of the staged key rows
+    // head dim 256: the table pieces are requested late in a tile (prefetch_rope), when the key fragments of its
+    // logits are dead, instead of together with the rows; 32 registers less while the logits are formed
+    constexpr bool LATE_ROPE = ROPE && HID > 128;
+    int rp_late[LATE_ROPE ? CPT : 1];
     auto prefetch_k = [&](int tile) {
         const MfmaMeta &mt = sm.meta[tile & (2 * HB - 1)];
         long long ka[CPT];
@@ -424,12 +439,24 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
 #pragma unroll
         for (int j = 0; j < CPT; j++) {
             const int piece = (tid + NTHREADS * j) % (HID / 8);
-            if constexpr (ROPE) {
+            if constexpr (ROPE && !LATE_ROPE) {
                 const int64_t tr = (int64_t)rp[j] * p.rope.stride_t + (piece % (HID / 16)) * 8;
                 creg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr);
                 sreg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr);
             }
+            if constexpr (LATE_ROPE) rp_late[j] = rp[j];
             kreg[j] = load_kv_piece_global<KV8>(ka[j], piece * 8);
+        }
+    };
+    auto prefetch_rope = [&]() {
+        if constexpr (LATE_ROPE) {
+#pragma unroll
+            for (int j = 0; j < CPT; j++) {
+                const int piece = (tid + NTHREADS * j) % (HID / 8);
+                const int64_t tr = (int64_t)rp_late[j] * p.rope.stride_t + (piece % (HID / 16)) * 8;
+                creg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr);
+                sreg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr);
+            }
         }
     };
     auto prefetch_v = [&](int tile) {
@@ -630,6 +657,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
         resolve_batch(0);
         __syncthreads();
         prefetch_k(0);
+        prefetch_rope();
         prefetch_v(0);
     }
     for (int tile = 0; tile < ntiles; tile++) {
@@ -648,39 +676,40 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
         bool window;
         const bool full = tile_full(tile, window);
         const int tmax = __builtin_amdgcn_readfirstlane(mt.tmax);
-        if (tmax < 0 || !head_ok) continue;  // nothing valid in this tile, or an idle wave (both wave-uniform)
-        // ---- S^T = K^ Q^^T
-        f32x16 sacc[2];
-#pragma unroll
-        for (int nb = 0; nb < 2; nb++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) sacc[nb][i] = 0.0f;
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            Frag a0, a1;
-            a0.q = *reinterpret_cast<const uint4 *>(&sm.k[buf][col][ks * 16 + hh * 8]);
-            a1.q = *reinterpret_cast<const uint4 *>(&sm.k[buf][32 + col][ks * 16 + hh * 8]);
-            sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0.v, qf[ks].v, sacc[0], 0, 0, 0);
-            sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1.v, qf[ks].v, sacc[1], 0, 0, 0);
+        if (tmax < 0 || !head_ok) {  // nothing valid in this tile, or an idle wave (both wave-uniform)
+            prefetch_rope();
+            continue;
         }
-        if constexpr (CAP) {
-            const float k2 = 2.0f * LOG2E / p.softcap;
+        // a half tile of 32 tokens at a time (logits, softmax, products with V): one block of logits and one of P
+        // live beside the accumulators and the query fragments
 #pragma unroll
-            for (int nb = 0; nb < 2; nb++)
+        for (int nb = 0; nb < 2; nb++) {
+            // ---- S^T = K^ Q^^T
+            f32x16 sacc;
 #pragma unroll
-                for (int i = 0; i < 16; i++) sacc[nb][i] = softcap_logit(sacc[nb][i], p.softcap, k2);
-        }
+            for (int i = 0; i < 16; i++) sacc[i] = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                Frag a0;
+                a0.q = *reinterpret_cast<const uint4 *>(&sm.k[buf][nb * 32 + col][ks * 16 + hh * 8]);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0.v, qf[ks].v, sacc, 0, 0, 0);
+                // keeps the fragment reads of at most four k-steps in flight (left alone the scheduler hoists all
+                // sixteen and spills the accumulators)
+                if ((ks & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+            }
+            if (nb == 1) prefetch_rope();
+            if constexpr (CAP) {
+                const float k2 = 2.0f * LOG2E / p.softcap;
+#pragma unroll
+                for (int i = 0; i < 16; i++) sacc[i] = softcap_logit(sacc[i], p.softcap, k2);
+            }
 
-        // ---- mask + online softmax; element (nb, i) of a lane is token slot nb*32 + (i/4)*8 + hh*4 + i%4
-        float mx = -INFINITY;
-        if (full) {
+            // ---- mask + online softmax; element i of a lane is token slot nb*32 + (i/4)*8 + hh*4 + i%4
+            float mx = -INFINITY;
+            if (full) {
 #pragma unroll
-            for (int nb = 0; nb < 2; nb++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[nb][i]);
-        } else {
-#pragma unroll
-            for (int nb = 0; nb < 2; nb++)
+                for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[i]);
+            } else {
 #pragma unroll
                 for (int i4 = 0; i4 < 4; i4++) {
                     const int4 tt = *reinterpret_cast<const int4 *>(&mt.tok[nb * 32 + i4 * 8 + hh * 4]);
@@ -691,57 +720,57 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
                         // branch-free: far keys need t + sw <= pq, window keys t <= pq < t + sw
                         const long long tsw = (long long)t + p.sw;
                         const bool att = (t >= 0) & (p.non_causal ? row_ok : window ? ((t <= pq) & ((long long)pq < tsw)) : (tsw <= (long long)pq));
-                        const float s = att ? sacc[nb][i4 * 4 + e] : -INFINITY;
-                        sacc[nb][i4 * 4 + e] = s;
+                        const float s = att ? sacc[i4 * 4 + e] : -INFINITY;
+                        sacc[i4 * 4 + e] = s;
                         mx = fmaxf(mx, s);
                     }
                 }
-        }
-        mx = fmaxf(mx, swap_halves(mx)) * LOG2E;
-        // raise the reference point only when the maximum grew noticeably
-        float m_use = m_run;
-        float alpha = 1.0f;
-        if (mx > m_run + RESCALE_STEP || m_run == -INFINITY) {
-            m_use = fmaxf(m_run, mx);
-            alpha = (m_use == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_use);  // m_run = -inf -> 0
-        }
-        const float m_sub = (m_use == -INFINITY) ? 0.0f : m_use;
-        Frag pf[4];
-        float lsum = 0.0f;
-#pragma unroll
-        for (int nb = 0; nb < 2; nb++)
+            }
+            mx = fmaxf(mx, swap_halves(mx)) * LOG2E;
+            // raise the reference point only when the maximum grew noticeably
+            float m_use = m_run;
+            float alpha = 1.0f;
+            if (mx > m_run + RESCALE_STEP || m_run == -INFINITY) {
+                m_use = fmaxf(m_run, mx);
+                alpha = (m_use == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_use);  // m_run = -inf -> 0
+            }
+            const float m_sub = (m_use == -INFINITY) ? 0.0f : m_use;
+            Frag pf[2];
+            float lsum = 0.0f;
 #pragma unroll
             for (int u = 0; u < 2; u++)
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[nb][u * 8 + 2 * e], LOG2E, -m_sub));
-                    const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[nb][u * 8 + 2 * e + 1], LOG2E, -m_sub));
+                    const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[u * 8 + 2 * e], LOG2E, -m_sub));
+                    const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[u * 8 + 2 * e + 1], LOG2E, -m_sub));
                     lsum += p0 + p1;
-                    pf[nb * 2 + u].u[e] = cvt_pk_bf16(p0, p1);
+                    pf[u].u[e] = cvt_pk_bf16(p0, p1);
                 }
-        l_run = l_run * alpha + lsum;
-        m_run = m_use;
-        // ---- O^T += V^T P^T
-        if (__any(alpha != 1.0f)) {
+            l_run = l_run * alpha + lsum;
+            m_run = m_use;
+            // ---- O^T += V^T P^T
+            if (__any(alpha != 1.0f)) {
 #pragma unroll
-            for (int db = 0; db < DB; db++)
+                for (int db = 0; db < DB; db++)
 #pragma unroll
-                for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
-        }
+                    for (int i = 0; i < 16; i++) oacc[db][i] *= alpha;
+            }
 #pragma unroll
-        for (int db = 0; db < DB; db++) {
+            for (int db = 0; db < DB; db++) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                // V^T fragments straight from the row-major tile: a transposing LDS read hands lane l of a 16-lane
-                // group column l % 4 of the four rows addressed by lanes l / 4, l / 4 + 4, + 8, + 12 of the group, so
-                // with source lane s pointing at (token T0 + s / 4, d = D0 + 4 * (s % 4)) lane l receives tokens
-                // T0 .. T0 + 3 at d = D0 + l.
-                Frag a;
-                const int trow = j * 16 + hh * 4 + ((lane & 15) >> 2);
-                const int tcol = db * 32 + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
-                a.d[0] = lds_read_tr16(&sm.v[buf][trow][tcol]);
-                a.d[1] = lds_read_tr16(&sm.v[buf][trow + 8][tcol]);
-                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pf[j].v, oacc[db], 0, 0, 0);
+                for (int u = 0; u < 2; u++) {
+                    // V^T fragments straight from the row-major tile: a transposing LDS read hands lane l of a
+                    // 16-lane group column l % 4 of the four rows addressed by lanes l / 4, l / 4 + 4, + 8, + 12 of the
+                    // group, so with source lane s pointing at (token T0 + s / 4, d = D0 + 4 * (s % 4)) lane l
+                    // receives tokens T0 .. T0 + 3 at d = D0 + l.
+                    Frag a;
+                    const int trow = nb * 32 + u * 16 + hh * 4 + ((lane & 15) >> 2);
+                    const int tcol = dv0 + db * 32 + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+                    a.d[0] = lds_read_tr16(&sm.v[buf][trow][tcol]);
+                    a.d[1] = lds_read_tr16(&sm.v[buf][trow + 8][tcol]);
+                    oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pf[u].v, oacc[db], 0, 0, 0);
+                }
+                if (db & 1) __builtin_amdgcn_sched_barrier(0);
             }
         }
     }
@@ -757,7 +786,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
     for (int db = 0; db < DB; db++)
 #pragma unroll
         for (int i4 = 0; i4 < 4; i4++) {
-            const int d = db * 32 + i4 * 8 + hh * 4;
+            const int d = dv0 + db * 32 + i4 * 8 + hh * 4;
             uint2 o;
             o.x = cvt_pk_bf16(oacc[db][i4 * 4 + 0] * inv, oacc[db][i4 * 4 + 1] * inv);
             o.y = cvt_pk_bf16(oacc[db][i4 * 4 + 2] * inv, oacc[db][i4 * 4 + 3] * inv);
@@ -816,7 +845,7 @@ __global__ __launch_bounds__(256) void bsa_mark_kernel(BsaParams p, int hgroups,
 
 template <int HID, bool KSCALED, bool EXT, bool ROPE = false, bool CAP = false, bool KV8 = false>
 static int launch_mfma(const BsaParams &p, hipStream_t st) {
-    const int hpw = p.share_first_head ? 4 : 1;  // per-head index rows: one head per workgroup
+    const int hpw = p.share_first_head ? 4 / (HID / V_COLS<HID>) : 1;  // per-head index rows: one head per workgroup
     const int hgroups = (p.G + hpw - 1) / hpw;
     const long long total = (long long)p.B * p.kv.HKV * hgroups * p.NBQ;
     if (total >= 0x7fffffffLL) return HIPATTN_E_UNSUPPORTED;
