@@ -22,6 +22,7 @@ struct DecWaveSmem {
     long long ko[2][DT], vo[2][DT];  // row offsets (NO_ROW: zero row)
     float bias[2][DT];               // added to the slot's logit: 0, log of the visit count, -inf: empty or masked
     int rp[2][DT];                   // row of the RoPE tables
+    int rp2[2][DT];                  // dynamic rule: the second row a far key's tables are blended from, -1 = no blend
 };
 
 struct DecodeMfmaParams {
@@ -117,8 +118,10 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
     // page-table loads in flight), posted one tile ahead, and the K / V rows of the next tile are in flight while the
     // current tile is multiplied
     long long m_ko = NO_ROW, m_vo = NO_ROW;
-    int m_rp = 0;
+    int m_rp = 0, m_rp2 = -1;
     float m_bias = -INFINITY;
+    bool dyn = false;  // the "dynamic_extend" rule: sink and selected keys rotated with a blend of two table rows
+    if constexpr (ROPE) dyn = p.rope.backend == HIPATTN_EXTEND_DYNAMIC;
     // The index entry of a slot is requested one resolve ahead of the resolve that uses it, and the plain build looks
     // a token's page up once for K and V: a resolve then waits for one trip to memory (the page-table entry; none on
     // a dense tensor) instead of three in a row (index entry, page for K, page for V).
@@ -199,14 +202,21 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
         m_ko = ko;
         m_vo = vo;
         m_bias = t >= 0 ? bias : -INFINITY;
-        if constexpr (ROPE) m_rp = (int)p.rope.clamp(rpos);
+        if constexpr (ROPE) {
+            m_rp = (int)p.rope.clamp(rpos);
+            // one query row: pmax = its position + 1 (attention_decode_bsa.py, as in the query-block kernel)
+            m_rp2 = (dyn && !win && t >= 0) ? (int)p.rope.clamp(dynamic_extend_pos(t, ppos, ppos + 1, p.rope.model_ctx)) : -1;
+        }
     };
     auto post = [&](int slot2) {  // lanes 0..31 -> meta buffer slot2 (0 / 1)
         if (lane >= DT) return;
         sm.ko[slot2][lane] = m_ko;
         sm.vo[slot2][lane] = m_vo;
         sm.bias[slot2][lane] = m_bias;
-        if constexpr (ROPE) sm.rp[slot2][lane] = m_rp;
+        if constexpr (ROPE) {
+            sm.rp[slot2][lane] = m_rp;
+            sm.rp2[slot2][lane] = m_rp2;
+        }
     };
     auto wave_sync = [&]() {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -234,8 +244,17 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
             uint4 kq = kreg[j];
             if constexpr (ROPE) {
                 const int64_t tr = (int64_t)sm.rp[slot2][slot] * p.rope.stride_t + (piece % (PPR / 2)) * 8;
-                const uint4 cc = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr);
-                const uint4 sn = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr);
+                uint4 cc = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr);
+                uint4 sn = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr);
+                if (dyn) {  // wave-uniform
+                    const int r2 = sm.rp2[slot2][slot];
+                    const int64_t tr2 = (int64_t)(r2 < 0 ? 0 : r2) * p.rope.stride_t + (piece % (PPR / 2)) * 8;
+                    const uint4 c2 = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr2);
+                    const uint4 s2 = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr2);
+                    const float wa = r2 >= 0 ? 0.75f : 1.0f, wb = r2 >= 0 ? 0.25f : 0.0f;
+                    cc = rope_blend_piece(cc, c2, wa, wb);
+                    sn = rope_blend_piece(sn, s2, wa, wb);
+                }
                 const uint4 oth = make_uint4(__shfl_xor(kq.x, PPR / 2), __shfl_xor(kq.y, PPR / 2), __shfl_xor(kq.z, PPR / 2),
                                              __shfl_xor(kq.w, PPR / 2));
                 kq = rope_piece(kq, oth, cc, sn, piece < PPR / 2);
@@ -417,8 +436,6 @@ static int pick_dec(const DecodeMfmaParams &dp, hipStream_t st) {
 
 int bsa_decode_mfma_launch(const BsaParams &p, int dtype, int HID, int nsplits, float *ws, hipStream_t st) {
     if (dtype != HIPATTN_BF16 || p.G > 8) return HIPATTN_E_UNSUPPORTED;
-    // the dynamic rule blends two table rows per key: served by the vector-unit kernel
-    if (p.rope.cos && p.rope.backend == HIPATTN_EXTEND_DYNAMIC) return HIPATTN_E_UNSUPPORTED;
     DecodeMfmaParams dp;
     dp.a = p;
     dp.nsplits = nsplits;

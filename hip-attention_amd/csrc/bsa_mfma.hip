@@ -27,10 +27,12 @@ constexpr int NTHREADS = 512;
 constexpr int MAX_LDS_IDX = 1024;  // selected-block starts kept in LDS
 
 // what wave 0 posts about the 64 token slots of a tile
+template <int HID>
 struct MfmaMeta {
     long long ko[TN], vo[TN];  // addresses of the K / V rows (an empty slot: the row of zeros)
     int tok[TN];               // token, -1 for an empty slot
     int rp[TN];                // row of the RoPE tables the key is rotated with
+    int rp2[HID <= 128 ? TN : 1];  // dynamic rule: the second row a far key's tables are blended from, -1 = no blend
     int tmin, tmax, all_valid; // smallest / largest token of the tile (tmax < 0: empty tile), no empty slot
     int full;                  // every (valid row, token) pair of the tile is attended: the mask can be skipped
 };
@@ -51,7 +53,7 @@ template <int HID>
 struct MfmaSmem {
     uint16_t k[2][TN][HID + KPAD];
     uint16_t v[2][TN][HID + VPAD];
-    MfmaMeta meta[2 * META_BATCH<HID>];
+    MfmaMeta<HID> meta[2 * META_BATCH<HID>];
     int idx[MAX_LDS_IDX];
 };
 static_assert(sizeof(MfmaSmem<256>) <= 160 * 1024, "LDS of a compute unit");
@@ -228,11 +230,13 @@ __device__ __forceinline__ void pipe_step(const uint16_t *kh, const uint16_t *vh
 // fetched by lanes tid and tid ^ (HID/16) of one wave.
 // CAP = true (extended parameter block): logits are soft-capped before the softmax.
 // KV8 = true (extended parameter block): K / V rows are fp8 (e5m2) bytes, widened on load.
-template <int HID, bool KSCALED, bool EXT, bool ROPE = false, bool CAP = false, bool KV8 = false>
+// DYN = true (rope variant, head dim <= 128): the "dynamic_extend" rule, far keys rotated with a blend of two table rows.
+template <int HID, bool KSCALED, bool EXT, bool ROPE = false, bool CAP = false, bool KV8 = false, bool DYN = false>
 __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p, int hgroups, int hpw, long long total_wg) {
     static_assert(!ROPE || (EXT && !KSCALED), "rope variant: extended parameter block, keys scaled in the kernel");
     static_assert(!CAP || EXT, "softcap variant: extended parameter block");
     static_assert(!KV8 || (EXT && !KSCALED), "fp8 storage: extended parameter block, keys scaled in the kernel");
+    static_assert(!DYN || (ROPE && HID <= 128), "dynamic rule: a rope variant of the pipelined loop");
     const KVExt *kx = nullptr;
     if constexpr (EXT) kx = &p.kx;
     constexpr int KS = HID / 16;   // k-steps of the first product
@@ -396,12 +400,20 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
         }
         int64_t ko = NO_ROW, vo = NO_ROW;
         if (t >= 0) kv_rows<true, EXT>(p.kv, kx, b, t, kvh, seqlen, ko, vo, true);
-        MfmaMeta &mt = sm.meta[tile & (2 * HB - 1)];
+        MfmaMeta<HID> &mt = sm.meta[tile & (2 * HB - 1)];
         constexpr int ESZ = KV8 ? 1 : 2;
         mt.ko[lane] = ko != NO_ROW ? (long long)(reinterpret_cast<const char *>(p.kv.k) + ko * ESZ) : (long long)g_zero_row;
         mt.vo[lane] = vo != NO_ROW ? (long long)(reinterpret_cast<const char *>(p.kv.v) + vo * ESZ) : (long long)g_zero_row;
         mt.tok[lane] = t;
         if constexpr (ROPE) mt.rp[lane] = (int)p.rope.clamp(rpos);
+        if constexpr (DYN) {
+            // sink and selected keys: second row = the key's own position squeezed into the model's context, with
+            // pmax = pmin + the block's valid rows (attention_extend_bsa.py:271-292)
+            const long long nvalid = (long long)p.TDST - (long long)qb * p.bq < p.bq ? (long long)p.TDST - (long long)qb * p.bq : p.bq;
+            mt.rp2[lane] = (kind != 2 && t >= 0)
+                               ? (int)p.rope.clamp(dynamic_extend_pos(t, pmin_blk, pmin_blk + nvalid, p.rope.model_ctx))
+                               : -1;
+        }
         // tile summary for the mask shortcut, once for the whole workgroup
         const int tmin = wave_min_i(t < 0 ? 0x7fffffff : t);
         const int tmax = wave_max_i(t);
@@ -426,16 +438,21 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
     // logits are dead, instead of together with the rows; 32 registers less while the logits are formed
     constexpr bool LATE_ROPE = ROPE && HID > 128;
     int rp_late[LATE_ROPE ? CPT : 1];
+    // dynamic rule: the pieces of the second table row and, per staged piece, whether it takes the blend
+    uint4 creg2[DYN ? CPT : 1], sreg2[DYN ? CPT : 1];
+    unsigned blend_bits = 0;
     auto prefetch_k = [&](int tile) {
-        const MfmaMeta &mt = sm.meta[tile & (2 * HB - 1)];
+        const MfmaMeta<HID> &mt = sm.meta[tile & (2 * HB - 1)];
         long long ka[CPT];
-        int rp[CPT];
+        int rp[CPT], rp2[DYN ? CPT : 1];
 #pragma unroll
         for (int j = 0; j < CPT; j++) {
             const int slot = (tid + NTHREADS * j) / (HID / 8);
             ka[j] = mt.ko[slot];
             if constexpr (ROPE) rp[j] = mt.rp[slot];
+            if constexpr (DYN) rp2[j] = mt.rp2[slot];
         }
+        if constexpr (DYN) blend_bits = 0;
 #pragma unroll
         for (int j = 0; j < CPT; j++) {
             const int piece = (tid + NTHREADS * j) % (HID / 8);
@@ -445,6 +462,12 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
                 sreg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr);
             }
             if constexpr (LATE_ROPE) rp_late[j] = rp[j];
+            if constexpr (DYN) {
+                const int64_t tr2 = (int64_t)(rp2[j] < 0 ? 0 : rp2[j]) * p.rope.stride_t + (piece % (HID / 16)) * 8;
+                creg2[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr2);
+                sreg2[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr2);
+                blend_bits |= (rp2[j] >= 0 ? 1u : 0u) << j;
+            }
             kreg[j] = load_kv_piece_global<KV8>(ka[j], piece * 8);
         }
     };
@@ -460,7 +483,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
         }
     };
     auto prefetch_v = [&](int tile) {
-        const MfmaMeta &mt = sm.meta[tile & (2 * HB - 1)];
+        const MfmaMeta<HID> &mt = sm.meta[tile & (2 * HB - 1)];
         long long va[CPT];
 #pragma unroll
         for (int j = 0; j < CPT; j++) va[j] = mt.vo[(tid + NTHREADS * j) / (HID / 8)];
@@ -476,7 +499,14 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
             if constexpr (ROPE) {
                 const uint4 oth = make_uint4(__shfl_xor(kq.x, HID / 16), __shfl_xor(kq.y, HID / 16),
                                              __shfl_xor(kq.z, HID / 16), __shfl_xor(kq.w, HID / 16));
-                kq = rope_piece(kq, oth, creg[j], sreg[j], piece < HID / 16);
+                uint4 cc = creg[j], sn = sreg[j];
+                if constexpr (DYN) {
+                    const bool bl = (blend_bits >> j) & 1u;
+                    const float wa = bl ? 0.75f : 1.0f, wb = bl ? 0.25f : 0.0f;
+                    cc = rope_blend_piece(cc, creg2[j], wa, wb);
+                    sn = rope_blend_piece(sn, sreg2[j], wa, wb);
+                }
+                kq = rope_piece(kq, oth, cc, sn, piece < HID / 16);
             }
             if (!KSCALED) {
                 kq.x = cvt_pk_bf16(__uint_as_float(kq.x << 16) * p.c_k, __uint_as_float(kq.x & 0xffff0000u) * p.c_k);
@@ -506,7 +536,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
 
     // what the mask shortcut needs of a tile: is every (valid row, token) pair attended, and is it a window tile
     auto tile_full = [&](int tile, bool &window) {
-        const MfmaMeta &mt = sm.meta[tile & (2 * HB - 1)];
+        const MfmaMeta<HID> &mt = sm.meta[tile & (2 * HB - 1)];
         const int tmin = __builtin_amdgcn_readfirstlane(mt.tmin), tmax = __builtin_amdgcn_readfirstlane(mt.tmax);
         const bool all_valid = __builtin_amdgcn_readfirstlane(mt.all_valid) != 0;
         window = tile >= tiles_sel + tiles_sink;
@@ -555,20 +585,22 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
         // posted row addresses of the rows this thread stages, read a step ahead of their loads, and the summary of
         // the next tile
         long long ka[CPT], va[CPT];
-        int rpk[ROPE ? CPT : 1];
+        int rpk[ROPE ? CPT : 1], rp2k[DYN ? CPT : 1];
         int nx_full = 0;
         auto read_posted = [&](int i) {  // iteration i loads K of tile i + 2 and V of tile i + 1
-            const MfmaMeta &mk = sm.meta[(i + 2) & (2 * HB - 1)], &mv = sm.meta[(i + 1) & (2 * HB - 1)];
+            const MfmaMeta<HID> &mk = sm.meta[(i + 2) & (2 * HB - 1)], &mv = sm.meta[(i + 1) & (2 * HB - 1)];
 #pragma unroll
             for (int j = 0; j < CPT; j++) {
                 const int slot = (tid + NTHREADS * j) / (HID / 8);
                 ka[j] = mk.ko[slot];
                 va[j] = mv.vo[slot];
                 if constexpr (ROPE) rpk[j] = mk.rp[slot];
+                if constexpr (DYN) rp2k[j] = mk.rp2[slot];
             }
             nx_full = mv.full;
         };
         auto issue_loads = [&]() {
+            if constexpr (DYN) blend_bits = 0;
 #pragma unroll
             for (int j = 0; j < CPT; j++) {
                 const int piece = (tid + NTHREADS * j) % (HID / 8);
@@ -576,6 +608,12 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
                     const int64_t tr = (int64_t)rpk[j] * p.rope.stride_t + (piece % (HID / 16)) * 8;
                     creg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr);
                     sreg[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr);
+                }
+                if constexpr (DYN) {
+                    const int64_t tr2 = (int64_t)(rp2k[j] < 0 ? 0 : rp2k[j]) * p.rope.stride_t + (piece % (HID / 16)) * 8;
+                    creg2[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr2);
+                    sreg2[j] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr2);
+                    blend_bits |= (rp2k[j] >= 0 ? 1u : 0u) << j;
                 }
                 kreg[j] = load_kv_piece_global<KV8>(ka[j], piece * 8);
                 vreg[j] = load_kv_piece_global<KV8>(va[j], piece * 8);
@@ -672,7 +710,7 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
         // the next batch of tiles: its half of the ring was last read a batch ago, and the barrier of the next
         // round stands between these writes and their first use
         if (((tile + 2) & (HB - 1)) == 0 && tile + 2 < ntiles) resolve_batch(tile + 2);
-        const MfmaMeta &mt = sm.meta[tile & (2 * HB - 1)];
+        const MfmaMeta<HID> &mt = sm.meta[tile & (2 * HB - 1)];
         bool window;
         const bool full = tile_full(tile, window);
         const int tmax = __builtin_amdgcn_readfirstlane(mt.tmax);
@@ -843,7 +881,7 @@ __global__ __launch_bounds__(256) void bsa_mark_kernel(BsaParams p, int hgroups,
     }
 }
 
-template <int HID, bool KSCALED, bool EXT, bool ROPE = false, bool CAP = false, bool KV8 = false>
+template <int HID, bool KSCALED, bool EXT, bool ROPE = false, bool CAP = false, bool KV8 = false, bool DYN = false>
 static int launch_mfma(const BsaParams &p, hipStream_t st) {
     const int hpw = p.share_first_head ? 4 / (HID / V_COLS<HID>) : 1;  // per-head index rows: one head per workgroup
     const int hgroups = (p.G + hpw - 1) / hpw;
@@ -852,12 +890,12 @@ static int launch_mfma(const BsaParams &p, hipStream_t st) {
     const size_t smem = sizeof(MfmaSmem<HID>);
     static bool attr_set = false;
     if (!attr_set) {
-        HIPATTN_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&bsa_mfma_kernel<HID, KSCALED, EXT, ROPE, CAP, KV8>),
+        HIPATTN_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&bsa_mfma_kernel<HID, KSCALED, EXT, ROPE, CAP, KV8, DYN>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
     const BsaParamsFor<EXT> &pk = p;  // the plain kernel takes the block without the extras
-    hipLaunchKernelGGL((bsa_mfma_kernel<HID, KSCALED, EXT, ROPE, CAP, KV8>), dim3((unsigned)total), dim3(NTHREADS), smem, st, pk, hgroups,
+    hipLaunchKernelGGL((bsa_mfma_kernel<HID, KSCALED, EXT, ROPE, CAP, KV8, DYN>), dim3((unsigned)total), dim3(NTHREADS), smem, st, pk, hgroups,
                        hpw, total);
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
@@ -866,8 +904,9 @@ static int launch_mfma(const BsaParams &p, hipStream_t st) {
 int bsa_mfma_launch(const BsaParams &p, int dtype, int HID, hipStream_t st) {
     if (dtype != HIPATTN_BF16) return HIPATTN_E_UNSUPPORTED;
     if (p.bq > 64) return HIPATTN_E_UNSUPPORTED;
-    // the dynamic rule blends two table rows per key: served by the portable kernel
-    if (p.rope.cos && p.rope.backend == HIPATTN_EXTEND_DYNAMIC) return HIPATTN_E_UNSUPPORTED;
+    // the dynamic rule blends two table rows per key: variants of the pipelined loop (head dim 256: the portable kernel)
+    const bool dyn = p.rope.cos && p.rope.backend == HIPATTN_EXTEND_DYNAMIC;
+    if (dyn && HID > 128) return HIPATTN_E_UNSUPPORTED;
     if ((p.o_st % 4) != 0 || (p.o_sh % 4) != 0 || (p.o_sb % 4) != 0) return HIPATTN_E_UNSUPPORTED;
     bool ext = p.kx.extended();
     BsaParams plain;
@@ -906,6 +945,22 @@ int bsa_mfma_launch(const BsaParams &p, int dtype, int HID, hipStream_t st) {
         if (p.rope.cos) return launch_mfma<H, false, true, true>(p, st);             \
         if (p.k_prescaled) return ext ? launch_mfma<H, true, true>(p, st) : launch_mfma<H, true, false>(p, st); \
         return ext ? launch_mfma<H, false, true>(p, st) : launch_mfma<H, false, false>(p, st);
+#define BSA_PICK_DYN(H)                                                                         \
+    case H:                                                                                     \
+        if (p.k_prescaled) return HIPATTN_E_UNSUPPORTED;                                        \
+        if (p.kx.kv8)                                                                           \
+            return p.softcap != 0.0f ? launch_mfma<H, false, true, true, true, true, true>(p, st)   \
+                                     : launch_mfma<H, false, true, true, false, true, true>(p, st); \
+        return p.softcap != 0.0f ? launch_mfma<H, false, true, true, true, false, true>(p, st)      \
+                                 : launch_mfma<H, false, true, true, false, false, true>(p, st);
+    if (dyn) {
+        switch (HID) {
+            BSA_PICK_DYN(64)
+            BSA_PICK_DYN(128)
+        }
+        return HIPATTN_E_UNSUPPORTED;
+    }
+#undef BSA_PICK_DYN
     switch (HID) {
         BSA_PICK(64)
         BSA_PICK(128)

@@ -426,6 +426,19 @@ __device__ __forceinline__ uint32_t rope_pair(uint32_t w, uint32_t o, uint32_t c
     return rope_pk(__fadd_rn(__uint_as_float(a << 16), __uint_as_float(b << 16)),
                    __fadd_rn(__uint_as_float(a & 0xffff0000u), __uint_as_float(b & 0xffff0000u)));
 }
+// Blend of two packed table pairs, T(T(a * wa) + T(b * wb)) per element: the "dynamic_extend" rule of attention
+// rotates a far key with 0.75 of the table row of its packed position and 0.25 of the row of its own squeezed
+// position (attention_extend_bsa.py:323-357); weights (1, 0) hand back `a` unchanged.
+__device__ __forceinline__ uint32_t rope_blend_pair(uint32_t a, uint32_t b, float wa, float wb) {
+    const uint32_t x = rope_pk(__fmul_rn(__uint_as_float(a << 16), wa), __fmul_rn(__uint_as_float(a & 0xffff0000u), wa));
+    const uint32_t y = rope_pk(__fmul_rn(__uint_as_float(b << 16), wb), __fmul_rn(__uint_as_float(b & 0xffff0000u), wb));
+    return rope_pk(__fadd_rn(__uint_as_float(x << 16), __uint_as_float(y << 16)),
+                   __fadd_rn(__uint_as_float(x & 0xffff0000u), __uint_as_float(y & 0xffff0000u)));
+}
+__device__ __forceinline__ uint4 rope_blend_piece(uint4 a, uint4 b, float wa, float wb) {
+    return make_uint4(rope_blend_pair(a.x, b.x, wa, wb), rope_blend_pair(a.y, b.y, wa, wb),
+                      rope_blend_pair(a.z, b.z, wa, wb), rope_blend_pair(a.w, b.w, wa, wb));
+}
 __device__ __forceinline__ uint4 rope_piece(uint4 w, uint4 o, uint4 c, uint4 s, bool lower) {
     const uint32_t sg = lower ? 0x80008000u : 0u;
     return make_uint4(rope_pair(w.x, o.x, c.x, s.x ^ sg), rope_pair(w.y, o.y, c.y, s.y ^ sg),
