@@ -35,41 +35,46 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the prefill kernels, from two rocprofv3 --pmc runs of this file (FETCH_SIZE, then
 # WRITE_SIZE, KiB per dispatch; `python bench.py --traffic-from <fetch run dir> <write run dir>` prints this table from
 # their output).  A 268 435 456-byte device copy reads 131 095 KiB of FETCH_SIZE and 262 144 KiB of WRITE_SIZE in the
-# same runs, so FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0.  The figures belong to the kernel sources they were
-# taken on: TRAFFIC_SOURCES_SHA256 is the digest of those sources, and when the sources at hand differ the bench
-# reports no traffic instead of a stale one.
+# same runs, so FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0.  A figure belongs to the sources its kernel was
+# built from when the counters were taken: every entry carries the digest of those files, and when the files at hand
+# differ the bench reports no traffic for that kernel instead of a stale one.
 TRAFFIC_SOURCE = ("recorded: profiles/prefill_hbm_traffic_pmc.md (not measured in this run); FETCH_SIZE / WRITE_SIZE count bytes "
                   "between the L2 caches and the memory side, served by the 256 MB memory-side cache or by HBM")
-TRAFFIC_SOURCES_SHA256 = "unrecorded"
-MEASURED_TRAFFIC_BYTES = {
-    "mask_stage[n=507,chunk=256,rows=16]": 2.0 * 5366948.4 * 1024 + 718949.5 * 1024,
-    "mask_stage[n=1024,chunk=32,rows=16]": 2.0 * 7033647.6 * 1024 + 564427.4 * 1024,
-    "mask_stage[n=1024,chunk=8,rows=64]": 2.0 * 2208493.8 * 1024 + 216630.1 * 1024,
-    "bsa_prefill": 2.0 * 1860808.6 * 1024 + 262144.2 * 1024,
+SCAN_SOURCES = ("Makefile", "common.hpp", "mask_common.hpp", "mask_stage_mfma.hip", "mask_stage_dense.hip")
+ATTENTION_SOURCES = ("Makefile", "common.hpp", "bsa.hpp", "bsa_mfma.hip")
+# name -> (bytes per launch, the files the kernel is built from, their digest when the counters were taken)
+SCAN_DIGEST = "168670e784822dc287e6e25afb5bee47f3b262759556e5da23048b17726c4ce8"
+ATTENTION_DIGEST = "6d3b7d60022d55e2d547cb28ae7f8124f245f72978a205032011740408fa003e"
+MEASURED_TRAFFIC = {
+    "mask_stage[n=507,chunk=256,rows=16]": (2.0 * 4992539.5 * 1024 + 127148.2 * 1024, SCAN_SOURCES, SCAN_DIGEST),
+    "mask_stage[n=1024,chunk=32,rows=16]": (2.0 * 6834764.3 * 1024 + 175526.4 * 1024, SCAN_SOURCES, SCAN_DIGEST),
+    "mask_stage[n=1024,chunk=8,rows=64]": (2.0 * 2239531.2 * 1024 + 157019.5 * 1024, SCAN_SOURCES, SCAN_DIGEST),
+    "bsa_prefill": (2.0 * 1835641.9 * 1024 + 262144.0 * 1024, ATTENTION_SOURCES, ATTENTION_DIGEST),
 }
 
 
-def kernel_sources_sha256():
-    """Digest of the kernel sources the library is built from (names and contents, in name order)."""
+def kernel_sources_sha256(names):
+    """Digest of the named kernel source files (names and contents, in the order given)."""
     import hashlib
 
     d = os.path.join(ROOT, "hip-attention_amd", "csrc")
     h = hashlib.sha256()
-    for name in sorted(os.listdir(d)):
-        if name.endswith((".hip", ".hpp")) or name == "Makefile":
-            h.update(name.encode())
-            h.update(open(os.path.join(d, name), "rb").read())
+    for name in names:
+        h.update(name.encode())
+        h.update(open(os.path.join(d, name), "rb").read())
     return h.hexdigest()
 
 
 def recorded_traffic(name):
-    """(bytes or None, where the figure comes from): None once the kernel sources have changed since the record."""
-    now = kernel_sources_sha256()
-    if now != TRAFFIC_SOURCES_SHA256:
-        return None, (f"none: the kernel sources have changed since the counters were taken "
-                      f"(recorded on {TRAFFIC_SOURCES_SHA256[:12]}, now {now[:12]}); see profiles/prefill_hbm_traffic_pmc.md "
-                      "for the last record")
-    return MEASURED_TRAFFIC_BYTES.get(name), TRAFFIC_SOURCE
+    """(bytes or None, where the figure comes from): None once the kernel's sources have changed since the record."""
+    if name not in MEASURED_TRAFFIC:
+        return None, "none recorded for this launch"
+    nbytes, sources, digest = MEASURED_TRAFFIC[name]
+    now = kernel_sources_sha256(sources)
+    if now != digest:
+        return None, (f"none: the kernel's sources ({', '.join(sources)}) have changed since the counters were taken "
+                      f"(recorded on {digest[:12]}, now {now[:12]}); see profiles/prefill_hbm_traffic_pmc.md for the last record")
+    return nbytes, TRAFFIC_SOURCE
 
 
 def print_traffic_table(fetch_dir, write_dir):
@@ -84,12 +89,23 @@ def print_traffic_table(fetch_dir, write_dir):
              "group by kernel_name, grid_size order by min(dispatch_id)")
         return [(n.split("(")[0], g, v, k) for n, g, v, k in c.execute(q, (counter,))]
 
+    def per_dispatch(d, counter, sub):  # launches of one kernel in launch order (two stages share the sampling kernel)
+        db = sorted(glob.glob(os.path.join(d, "**", "*.db"), recursive=True))[-1]
+        q = "select value from counters_collection where counter_name = ? and kernel_name like ? order by dispatch_id"
+        return [v for (v,) in sqlite3.connect(db).execute(q, (counter, f"%{sub}%"))]
+
     fetch, write = per_kernel(fetch_dir, "FETCH_SIZE"), per_kernel(write_dir, "WRITE_SIZE")
     wmap = {(n, g): v for n, g, v, _ in write}
-    print(f'TRAFFIC_SOURCES_SHA256 = "{kernel_sources_sha256()}"')
+    print(f'digest of SCAN_SOURCES      = "{kernel_sources_sha256(SCAN_SOURCES)}"')
+    print(f'digest of ATTENTION_SOURCES = "{kernel_sources_sha256(ATTENTION_SOURCES)}"')
     for n, g, v, k in fetch:
         if any(t in n for t in ("mask_stage", "bsa_mfma", "qhat", "copyBuffer", "prescale")):
             print(f"{n[-70:]:70s} grid {g:>10} dispatches {k:>3}  FETCH_SIZE {v:14.1f} KiB  WRITE_SIZE {wmap.get((n, g), float('nan')):14.1f} KiB")
+    f, w = per_dispatch(fetch_dir, "FETCH_SIZE", "mask_stage_mfma"), per_dispatch(write_dir, "WRITE_SIZE", "mask_stage_mfma")
+    for i in range(2):  # launches alternate between the stages of a call
+        if f[i::2] and w[i::2]:
+            print(f"mask_stage_mfma_kernel, launch {i} of every call: FETCH_SIZE {sum(f[i::2]) / len(f[i::2]):14.1f} KiB  "
+                  f"WRITE_SIZE {sum(w[i::2]) / len(w[i::2]):14.1f} KiB  ({len(f[i::2])} dispatches)")
 
 
 SAMPLE_QUERIES = 512  # the last queries of the prefill workload that the CPU oracle recomputes
