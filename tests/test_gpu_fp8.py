@@ -84,6 +84,32 @@ def test_fp8_cache_with_rope_on_load_and_softcap():
         assert_context_close(ctx, octx, "bf16")
 
 
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("cap", [None, 20.0])
+def test_fp8_cache_with_the_dynamic_rule_inside_attention(D, cap):
+    """dynamic_extend inside attention on an fp8 cache (the tile kernel's and the decode kernel's variants that blend
+    two table rows while they stage widened key rows), prefill and ragged decode, with and without soft-capping."""
+    print(f"[case] fp8 + dynamic_extend attention D={D} softcap={cap}", flush=True)
+    kw = dict(extend_context_length=3000, using_extend=True, need_apply_rope=True, scan_extend_backend="relative",
+              sa_extend_backend="dynamic_extend", model_context_length=1024)
+    if cap:
+        kw["logit_softcap"] = cap
+    X = make_inputs(57, B=2, TQ=100, TK=3000, H=4, HKV=2, D=D, dtype="bf16", scale=0.5)
+    XQ, kc, vc = _quantise(with_rope(to_paged(X, 16, seed=12), 4096))
+    A = tiny_args(**kw)
+    octx, ometa = O.hip_attention_12(XQ, A)
+    ctx, meta = _run(XQ, A, kc, vc, True)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, "bf16")
+    lens = np.array([3000, 1700])
+    Xd = make_inputs(58, B=2, TQ=1, TK=3000, H=4, HKV=2, D=D, dtype="bf16", pos=(lens - 1)[:, None], scale=0.5)
+    XQ, kc, vc = _quantise(with_rope(to_paged(Xd, 8, seed=13, seq_lens=lens), 4096))
+    octx, ometa = O.hip_attention_12(XQ, A)
+    ctx, meta = _run(XQ, A, kc, vc, False)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, "bf16")
+
+
 def test_portable_attention_kernel_on_fp8_cache():
     from hip_attn import HiPAttentionArgs12
     from hip_attn.operator import block_sparse_attention
