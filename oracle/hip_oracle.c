@@ -34,7 +34,11 @@
  * selection, both attention kernels, decode, RoPE on load (relative, streaming, infllm, and dynamic_extend in
  * the mask stage, whose squeeze branch the reference_*_rope_dynamic vectors exercise).  Parity unpinned against the running
  * reference: bfloat16 arithmetic (the interpreter has no bfloat16; the order of accumulation here is
- * MI355X's, not NVIDIA's) and logit_softcap (the interpreter cannot call libdevice.tanh).
+ * MI355X's, not NVIDIA's), logit_softcap (the interpreter cannot call libdevice.tanh), the self_extend rule of the
+ * mask stage (self_extend_pos: PARITY UNPINNED by execution, because the interpreter floors the quotient the compiled
+ * kernel truncates; pinned by the closed form in tests/test_oracle_rope.py).  Non-causal attention is pinned by two executions of the reference
+ * (reference_f32_prefill_non_causal.npz, reference_f32_decode_non_causal.npz) and by float64 dense softmax references
+ * in tests/test_oracle_bsa.py.
  */
 #include <math.h>
 #include <stdint.h>

@@ -103,11 +103,11 @@ def access_flags(md, suffix):
 
 def make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, dtype=torch.float32,
               lens=None, page_size=0, extend=None, softcap=None, block_size_k=64, replay=False, exact=False,
-              model_ctx=None, early=None):
+              model_ctx=None, early=None, causal=True):
     """One call of the reference operator; ``lens`` (decode: TQ == 1) places each sequence's query at lens[b] - 1;
     ``page_size`` > 0 moves K/V into a paged cache behind a shuffled block table; ``extend`` = (scan rule, sa rule)
     turns on RoPE applied on load; ``model_ctx`` sets model_context_length (the dynamic_extend rule reads it);
-    ``early`` sets stage_early_terminate."""
+    ``early`` sets stage_early_terminate; ``causal=False`` passes ``is_causal=False`` (attention kernels only)."""
     g = torch.Generator().manual_seed(seed)
     # values with 8 significant bits, so that the files can hold q, k, v as 16-bit patterns
     short = lambda t: t.to(torch.bfloat16).to(dtype)  # noqa: E731
@@ -143,6 +143,9 @@ def make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, sec
     if early is not None:
         kw.update(stage_early_terminate=early)
         extra.update(stage_early_terminate=early)
+    if not causal:
+        kw.update(is_causal=False)
+        extra.update(is_causal=0)
     if page_size > 0:
         per = -(-TK // page_size)
         npages = B * per + 4
@@ -331,6 +334,10 @@ def main():
                                         dict(extend=("relative", "dynamic_extend"), model_ctx=1024)),
         "f32_decode_sa_rope_dynamic": (13, 2, 1, 2048, 4, 2, 32, tiny, 16, 256, 512, 32,
                                        dict(lens=[2048, 1400], page_size=4, extend=("streaming", "dynamic_extend"), model_ctx=512)),
+        # is_causal=False: the attention kernels drop the key <= query test (the scan is not told)
+        "f32_prefill_non_causal": (14, 2, 96, 1536, 4, 2, 32, tiny, 16, 256, 512, 32, dict(causal=False)),
+        "f32_decode_non_causal": (15, 2, 1, 2048, 4, 2, 32, tiny, 16, 256, 512, 32,
+                                  dict(lens=[2048, 1300], page_size=8, causal=False)),
         # Not generated: Triton's interpreter has no bfloat16 constants (``get_bf16``) and cannot call
         # ``libdevice.tanh`` (logit_softcap) outside a compiled kernel, so bfloat16 inputs and soft-capped logits
         # have no vectors from the reference.

@@ -46,6 +46,8 @@ def load_case(path):
         kw["logit_softcap"] = float(d["softcap"])
     if "stage_early_terminate" in d.files:
         kw["stage_early_terminate"] = int(d["stage_early_terminate"])
+    if "is_causal" in d.files:
+        kw["is_causal"] = bool(int(d["is_causal"]))
     return d, X, O.OArgs(**kw), dtype
 
 
@@ -63,7 +65,8 @@ def test_fixtures_are_present():
             "reference_f32_decode_rope_infllm.npz", "reference_f32_prefill_stride_d64.npz",
             "reference_f32_prefill_rope_dynamic.npz", "reference_f32_decode_rope_dynamic.npz",
             "reference_f32_decode_default_stages.npz", "reference_f32_paged_api_prefill.npz",
-            "reference_f32_smallest_benchmark_prefill.npz",
+            "reference_f32_smallest_benchmark_prefill.npz", "reference_f32_prefill_non_causal.npz",
+            "reference_f32_decode_non_causal.npz",
             "reference_f32_paged_api_decode_rope.npz"} <= names
 
 
