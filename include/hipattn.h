@@ -51,12 +51,11 @@ extern "C" {
  *                two table rows, 0.75 of the row of their STREAMING position and 0.25 of the row of the position
  *                the mask-stage formula above gives for their token (pmin = smallest position of the query block,
  *                pmax = pmin + its valid rows; decode: pmax = pmin + 1); both products and the sum are rounded to
- *                the element type.  Served by the portable attention kernels.
+ *                the element type.  (bf16, head dim 64 / 128: the matrix-core kernels; other shapes: the portable ones.)
  *   SELF, mask stage only (attention_extend.py:275-289, :637-638): the query at its own position; the sampled key at
  *                token t keeps position t when t >= pmax - 8192 or pmax <= model_context_length, else it moves to
- *                (t - pmin) / 16 + pmin with the quotient truncated toward zero (what the compiled kernel's int32
- *                division does; the reference's CPU interpreter floors instead, so no execution of it on a CPU
- *                pins this rule: parity unpinned by execution, pinned by the closed form), then max(0, .).  The
+ *                (t - pmin) / 16 + pmin with the quotient truncated toward zero (the kernel's int32 division;
+ *                moved keys lie below pmin, so flooring would give another position), then max(0, .).  The
  *                reference's attention kernels raise on this rule (attention_extend_bsa.py:62-63), and so does the
  *                attention entry here.
  * Positions are clamped into [0, len).  The mode that re-rotates keys stored WITH rotation (need_apply_rope = False)

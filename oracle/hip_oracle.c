@@ -34,11 +34,10 @@
  * selection, both attention kernels, decode, RoPE on load (relative, streaming, infllm, and dynamic_extend in
  * the mask stage, whose squeeze branch the reference_*_rope_dynamic vectors exercise).  Parity unpinned against the running
  * reference: bfloat16 arithmetic (the interpreter has no bfloat16; the order of accumulation here is
- * MI355X's, not NVIDIA's), logit_softcap (the interpreter cannot call libdevice.tanh), the self_extend rule of the
- * mask stage (self_extend_pos: PARITY UNPINNED by execution, because the interpreter floors the quotient the compiled
- * kernel truncates; pinned by the closed form in tests/test_oracle_rope.py).  Non-causal attention is pinned by two executions of the reference
- * (reference_f32_prefill_non_causal.npz, reference_f32_decode_non_causal.npz) and by float64 dense softmax references
- * in tests/test_oracle_bsa.py.
+ * MI355X's, not NVIDIA's) and logit_softcap (the interpreter cannot call libdevice.tanh).  The self_extend rule of the
+ * mask stage (reference_f32_prefill_rope_self_extend.npz) and non-causal attention
+ * (reference_f32_prefill_non_causal.npz, reference_f32_decode_non_causal.npz; also float64 dense softmax references
+ * in tests/test_oracle_bsa.py) are pinned by executions of the reference as well.
  */
 #include <math.h>
 #include <stdint.h>
@@ -502,9 +501,9 @@ static int64_t dynamic_extend_pos(int64_t t, int64_t pmin, int64_t pmax, int64_t
 
 /* Rotated position of a sampled key under the "self_extend" rule (attention_extend.py:275-289): once the query block
  * reaches beyond the model's context, keys older than 8192 positions are grouped by sixteen around the block's first
- * position.  `//` in the kernel is an int32 division: the compiled kernel truncates toward zero (sampled keys lie
- * below pmin, so the numerator is negative and the two roundings differ); the reference's CPU interpreter floors.
- * This follows the compiled kernel: parity unpinned by execution here, pinned by the closed form in the tests. */
+ * position.  `//` in the kernel is an int32 division that truncates toward zero (sampled keys lie below pmin, so the
+ * numerator is negative and flooring would give another position).  Pinned by the closed form in the tests and by an
+ * execution of the reference, reference_f32_prefill_rope_self_extend.npz, which a floored quotient does not reproduce. */
 static int64_t self_extend_pos(int64_t t, int64_t pmin, int64_t pmax, int64_t model_ctx) {
     int64_t pos = t;
     if (!(t >= pmax - 8192 || pmax <= model_ctx)) pos = (t - pmin) / 16 + pmin; /* C division truncates */

@@ -103,7 +103,7 @@ def access_flags(md, suffix):
 
 def make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, second_k, bsbq, dtype=torch.float32,
               lens=None, page_size=0, extend=None, softcap=None, block_size_k=64, replay=False, exact=False,
-              model_ctx=None, early=None, causal=True):
+              model_ctx=None, early=None, causal=True, rope_len=None):
     """One call of the reference operator; ``lens`` (decode: TQ == 1) places each sequence's query at lens[b] - 1;
     ``page_size`` > 0 moves K/V into a paged cache behind a shuffled block table; ``extend`` = (scan rule, sa rule)
     turns on RoPE applied on load; ``model_ctx`` sets model_context_length (the dynamic_extend rule reads it);
@@ -129,7 +129,7 @@ def make_case(ext, meta, name, seed, B, TQ, TK, H, HKV, D, stages, sink, sw, sec
               require_cache_statistics=True, position_ids=pos, block_size_k=block_size_k)
     extra = {}
     if extend is not None:
-        cos, sin = rope_tables(2 * TK, D)
+        cos, sin = rope_tables(rope_len or 2 * TK, D)
         kw.update(using_extend=True, need_apply_rope=True, rope_cos=cos.to(dtype), rope_sin=sin.to(dtype),
                   scan_extend_backend=extend[0], sa_extend_backend=extend[1])
         extra.update(rope_cos=cos.to(dtype).float().numpy(), rope_sin=sin.to(dtype).float().numpy(),
@@ -334,6 +334,11 @@ def main():
                                         dict(extend=("relative", "dynamic_extend"), model_ctx=1024)),
         "f32_decode_sa_rope_dynamic": (13, 2, 1, 2048, 4, 2, 32, tiny, 16, 256, 512, 32,
                                        dict(lens=[2048, 1400], page_size=4, extend=("streaming", "dynamic_extend"), model_ctx=512)),
+        # self_extend in the scan: keys older than 8192 positions are grouped by sixteen once the block reaches beyond
+        # the model's context (the quotient of the negative distance is truncated toward zero, by the interpreter too)
+        # (one case, and tables just long enough: 9216 keys make this the largest vector)
+        "f32_prefill_rope_self_extend": (16, 1, 64, 9216, 2, 1, 32, tiny, 16, 256, 512, 32,
+                                         dict(extend=("self_extend", "streaming"), model_ctx=4096, rope_len=9216 + 64)),
         # is_causal=False: the attention kernels drop the key <= query test (the scan is not told)
         "f32_prefill_non_causal": (14, 2, 96, 1536, 4, 2, 32, tiny, 16, 256, 512, 32, dict(causal=False)),
         "f32_decode_non_causal": (15, 2, 1, 2048, 4, 2, 32, tiny, 16, 256, 512, 32,

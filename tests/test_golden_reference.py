@@ -66,7 +66,7 @@ def test_fixtures_are_present():
             "reference_f32_prefill_rope_dynamic.npz", "reference_f32_decode_rope_dynamic.npz",
             "reference_f32_decode_default_stages.npz", "reference_f32_paged_api_prefill.npz",
             "reference_f32_smallest_benchmark_prefill.npz", "reference_f32_prefill_non_causal.npz",
-            "reference_f32_decode_non_causal.npz",
+            "reference_f32_decode_non_causal.npz", "reference_f32_prefill_rope_self_extend.npz",
             "reference_f32_paged_api_decode_rope.npz"} <= names
 
 

@@ -170,9 +170,8 @@ def test_dynamic_extend_inside_attention_prefill_and_paged_decode(dtype, D, mode
 def test_self_extend_scan_prefill_and_paged_decode(dtype, D, model_ctx):
     """The self_extend rule of the scan (attention_extend.py:275-289): once a query block reaches beyond the model's
     context (4096 against 9000 keys), keys older than 8192 positions are grouped by sixteen; below it (131072) every
-    key keeps its own position.  Parity unpinned by execution of the reference (its CPU interpreter floors the
-    quotient the compiled kernel truncates); the oracle's rule is pinned by the closed form in
-    tests/test_oracle_rope.py."""
+    key keeps its own position.  The oracle's rule is pinned by the closed form in tests/test_oracle_rope.py and by
+    an execution of the reference (tests/golden/reference_f32_prefill_rope_self_extend.npz)."""
     print(f"[case] rope self_extend {dtype} D={D} model_ctx={model_ctx}", flush=True)
     X = with_rope(make_inputs(61, B=1, TQ=200, TK=9000, H=4, HKV=2, D=D, dtype=dtype, scale=0.5), 9216)
     A = _ext(scan_extend_backend="self_extend", sa_extend_backend="streaming", model_context_length=model_ctx)
