@@ -212,6 +212,9 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     const uint32_t piece_h = !DMA ? 0u
                              : (uint32_t)(((int64_t)kvh * p.kv.k_stride_h + ((OFF32 || p.kv.paged) ? 0 : (int64_t)b * p.kv.k_stride_b)) >> 3);
     const int tsrc32 = DMA ? (int)p.kv.tsrc : 0;
+    // keys rotated ahead, one copy per sample side (the relative rule): this lane's samples come from its side's copy
+    uint32_t side_pieces = 0u;
+    if constexpr (DMA && EXT) side_pieces = side ? (uint32_t)(p.rope.k_side_delta >> 3) : 0u;
     uint8_t *flag_row = nullptr;
     if constexpr (DMA) {
         if (kx->access_flags) flag_row = kx->access_flags + (int64_t)b * kx->flags_stride_b + (int64_t)kvh * kx->flags_stride_h;
@@ -324,6 +327,7 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     // rotated ahead per side) the rotation follows the side, so only the lane's own side counts there.
     bool cross_side = RMODE != 2;
     if constexpr (ROPE) cross_side = p.rope.backend != HIPATTN_EXTEND_RELATIVE;
+    if constexpr (DMA && EXT) cross_side = p.rope.k_side_delta == 0;
     int ptok[NB];
     float pscore[NB];
     // Paged keys, coalesced fetch: a round first needs its token's page-table entry, a trip to memory ahead of the
@@ -380,8 +384,8 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                     const int t = tok[tb];
                     if (OFF32 || !p.kv.paged) {
                         if (t >= 0 && t < tsrc32) {
-                            pieces[tb] = OFF32 ? (int)(__umul24((uint32_t)t, piece_st) + piece_h)
-                                               : (int)((uint32_t)t * piece_st + piece_h);
+                            pieces[tb] = OFF32 ? (int)(__umul24((uint32_t)t, piece_st) + piece_h + side_pieces)
+                                               : (int)((uint32_t)t * piece_st + piece_h + side_pieces);
                             if (flag_row && hh == 0 && !(share_now && wv != 0)) mark[tb] = t;
                         }
                     } else if (t >= 0) {
@@ -390,7 +394,7 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                         if (t == pf_tok[tb][0]) page = pf_in[tb][0] ? pf_page[tb][0] : 0u;
                         else if (t == pf_tok[tb][1]) page = pf_in[tb][1] ? pf_page[tb][1] : 0u;
                         else page = (uint32_t)p.kv.page_of(b, t, seqlen);
-                        pieces[tb] = (int)(page * piece_sb + (uint32_t)(t & (p.kv.page_size - 1)) * piece_st + piece_h);
+                        pieces[tb] = (int)(page * piece_sb + (uint32_t)(t & (p.kv.page_size - 1)) * piece_st + piece_h + side_pieces);
                         if (flag_row && hh == 0 && !(share_now && wv != 0)) mark[tb] = (int)page;
                     }
                 }
@@ -783,7 +787,9 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
     // (2 = on every launch the variant can serve, however small: testing)
     const char *e_dma = getenv("HIPATTN_MASK_DMA");
     const int dma_mode = e_dma ? atoi(e_dma) : 1;
-    const bool dma = dma_mode != 0 && !far_rows && (wide || dma_mode == 2) && prescaled && p.rope.cos == nullptr && !p.kx.kv8 &&
+    // (keys rotated ahead under the relative / infllm rules are prescaled keys like any other: the kernel takes a
+    // right-hand sample from the second copy)
+    const bool dma = dma_mode != 0 && !far_rows && (wide || dma_mode == 2) && prescaled && p.rope.k_side_delta >= 0 && !p.kx.kv8 &&
                      !p.kx.cached && HID <= 128 && env_nb != 2 && !two;  // (64-row programs: 204 registers, 6.7 against 3.9 ms)
     // small chunks on wide launches: every token scored once per GQA group, searches replayed on the scores
     const bool dense = prescaled && !far_rows && p.rope.cos == nullptr && mask_stage_dense_applies(p, HID, rows_eff);
@@ -896,7 +902,8 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
         return HIPATTN_E_ARG;
     }
     // a dense key tensor whose batch items span less than 4 GB: row addresses as 32-bit offsets
-    const long long item_bytes = 2LL * ((p.kv.tsrc - 1) * p.kv.k_stride_t + (long long)(p.kv.HKV - 1) * p.kv.k_stride_h + HID);
+    const long long item_bytes = 2LL * ((p.kv.tsrc - 1) * p.kv.k_stride_t + (long long)(p.kv.HKV - 1) * p.kv.k_stride_h + HID +
+                                        (p.rope.k_side_delta > 0 ? p.rope.k_side_delta : 0));
     const bool off32 = !p.kv.paged && p.kv.k_stride_t >= 0 && p.kv.k_stride_h >= 0 && p.kv.k_stride_t % 8 == 0 &&
                        p.kv.k_stride_h % 8 == 0 && p.kv.k_stride_b % 8 == 0 && item_bytes < (1LL << 32) &&
                        p.kv.tsrc < (1LL << 24) && (p.kv.k_stride_t >> 3) < (1LL << 24);

@@ -338,6 +338,41 @@ def test_prefill_scans_with_coalesced_row_fetch_on_a_small_launch(paged, m16, mo
     assert torch.equal(meta0.mask_cache_statistics.access_counter, meta.mask_cache_statistics.access_counter)
 
 
+@pytest.mark.parametrize("scan", ["relative", "infllm"])
+@pytest.mark.parametrize("paged", [0, 16])
+def test_coalesced_prefill_scans_on_keys_rotated_ahead(paged, scan, monkeypatch):
+    """RoPE on load under the rules with fixed key positions: the keys are rotated and scaled ahead of the scan, one
+    copy per sample side under ``relative``, and the coalesced fetch takes a right-hand sample from the second copy
+    (forced on a small launch, both widths of the matrix instruction).  A score then belongs to (token, side): a lane
+    may not take a repeated token's score from its partner of the other side."""
+    from helpers import with_rope
+
+    _case(f"coalesced prefill scans on keys rotated ahead, scan={scan}, paged={paged}")
+    monkeypatch.setenv("HIP_ATTN_PRESCALE_K", "1")
+    monkeypatch.setenv("HIPATTN_MASK_DENSE", "0")
+    X = make_inputs(17, B=2, TQ=300, TK=8192, H=8, HKV=2, D=128, dtype="bf16", scale=0.5)
+    kw = dict(sliding_window_size=512, using_extend=True, need_apply_rope=True, scan_extend_backend=scan,
+              sa_extend_backend="streaming")
+    if paged:
+        X = to_paged(X, paged, seed=14)
+        kw["extend_context_length"] = 8192
+    X = with_rope(X, 16384)
+    A = O.OArgs(**kw)
+    octx, ometa = O.hip_attention_12(X, A)
+    res = {}
+    for m16 in ("0", "1"):
+        monkeypatch.setenv("HIPATTN_MASK_M16", m16)
+        monkeypatch.setenv("HIPATTN_MASK_DMA", "2")
+        ctx, meta = run_product(X, A, require_cache_statistics=True)
+        assert_metadata_equal(meta, ometa)
+        assert_context_close(ctx, octx, "bf16")
+        res[m16] = meta
+    monkeypatch.setenv("HIPATTN_MASK_DMA", "0")
+    ctx0, meta0 = run_product(X, A, require_cache_statistics=True)
+    assert torch.equal(meta0.indices, res["0"].indices)
+    assert torch.equal(meta0.mask_cache_statistics.access_counter, res["1"].mask_cache_statistics.access_counter)
+
+
 def test_key_buffers_reported_as_spanning_32_gib_take_the_plain_scans(monkeypatch):
     """The flag that keeps launches off the coalesced variants (rows passed between lanes as 31-bit piece numbers)
     when a key buffer is too large for them: forced here on a small problem, prefill and decode."""
