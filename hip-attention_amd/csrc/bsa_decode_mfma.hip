@@ -255,8 +255,8 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
                     cc = rope_blend_piece(cc, c2, wa, wb);
                     sn = rope_blend_piece(sn, s2, wa, wb);
                 }
-                const uint4 oth = make_uint4(__shfl_xor(kq.x, PPR / 2), __shfl_xor(kq.y, PPR / 2), __shfl_xor(kq.z, PPR / 2),
-                                             __shfl_xor(kq.w, PPR / 2));
+                const uint4 oth = make_uint4(lane_xor<PPR / 2>(kq.x), lane_xor<PPR / 2>(kq.y), lane_xor<PPR / 2>(kq.z),
+                                             lane_xor<PPR / 2>(kq.w));
                 kq = rope_piece(kq, oth, cc, sn, piece < PPR / 2);
             }
             kq.x = cvt_pk_bf16(__uint_as_float(kq.x << 16) * p.c_k, __uint_as_float(kq.x & 0xffff0000u) * p.c_k);

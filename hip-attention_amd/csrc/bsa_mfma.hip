@@ -497,8 +497,8 @@ __global__ __launch_bounds__(NTHREADS) void bsa_mfma_kernel(BsaParamsFor<EXT> p,
             const int slot = c / (HID / 8), piece = c % (HID / 8);
             uint4 kq = kreg[j];
             if constexpr (ROPE) {
-                const uint4 oth = make_uint4(__shfl_xor(kq.x, HID / 16), __shfl_xor(kq.y, HID / 16),
-                                             __shfl_xor(kq.z, HID / 16), __shfl_xor(kq.w, HID / 16));
+                const uint4 oth = make_uint4(lane_xor<HID / 16>(kq.x), lane_xor<HID / 16>(kq.y), lane_xor<HID / 16>(kq.z),
+                                             lane_xor<HID / 16>(kq.w));
                 uint4 cc = creg[j], sn = sreg[j];
                 if constexpr (DYN) {
                     const bool bl = (blend_bits >> j) & 1u;

@@ -503,6 +503,14 @@ __device__ __forceinline__ uint32_t swap_halves(uint32_t x) {
     return (threadIdx.x & 32) ? r[0] : r[1];
 }
 __device__ __forceinline__ float swap_halves(float x) { return __uint_as_float(swap_halves(__float_as_uint(x))); }
+// The value held by lane ^ N.  N = 8 is a rotation of every row of 16 lanes by eight places, which the data-parallel
+// path does in one vector instruction; the general exchange goes through the LDS crossbar and has to be waited for.
+template <int N>
+__device__ __forceinline__ uint32_t lane_xor(uint32_t x) {
+    if constexpr (N == 8) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x128 /* row_ror:8 */, 0xf, 0xf, false);
+    else if constexpr (N == 32) return swap_halves(x);
+    else return (uint32_t)__shfl_xor((int)x, N);
+}
 
 // ---------------------------------------------------------------- direct global -> LDS loads
 // 16 bytes per lane from global memory straight into LDS (global_load_lds_dwordx4): lane i's piece lands at
