@@ -236,35 +236,64 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
             if (vo != NO_ROW) vreg[j] = load_kv_piece<KV8>(p.kv.v, vo + piece * 8);
         }
     };
+    auto scale_store_k = [&](uint4 kq, int slot, int piece) {
+        kq.x = cvt_pk_bf16(__uint_as_float(kq.x << 16) * p.c_k, __uint_as_float(kq.x & 0xffff0000u) * p.c_k);
+        kq.y = cvt_pk_bf16(__uint_as_float(kq.y << 16) * p.c_k, __uint_as_float(kq.y & 0xffff0000u) * p.c_k);
+        kq.z = cvt_pk_bf16(__uint_as_float(kq.z << 16) * p.c_k, __uint_as_float(kq.z & 0xffff0000u) * p.c_k);
+        kq.w = cvt_pk_bf16(__uint_as_float(kq.w << 16) * p.c_k, __uint_as_float(kq.w & 0xffff0000u) * p.c_k);
+        *reinterpret_cast<uint4 *>(&sm.k[slot][piece * 8]) = kq;
+    };
     auto commit = [&](int slot2) {
+        if constexpr (!ROPE) {
 #pragma unroll
-        for (int j = 0; j < CPT; j++) {
-            const int c = lane + 64 * j;
-            const int slot = c / PPR, piece = c % PPR;
-            uint4 kq = kreg[j];
-            if constexpr (ROPE) {
-                const int64_t tr = (int64_t)sm.rp[slot2][slot] * p.rope.stride_t + (piece % (PPR / 2)) * 8;
-                uint4 cc = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr);
-                uint4 sn = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr);
-                if (dyn) {  // wave-uniform
-                    const int r2 = sm.rp2[slot2][slot];
-                    const int64_t tr2 = (int64_t)(r2 < 0 ? 0 : r2) * p.rope.stride_t + (piece % (PPR / 2)) * 8;
-                    const uint4 c2 = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr2);
-                    const uint4 s2 = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr2);
-                    const float wa = r2 >= 0 ? 0.75f : 1.0f, wb = r2 >= 0 ? 0.25f : 0.0f;
-                    cc = rope_blend_piece(cc, c2, wa, wb);
-                    sn = rope_blend_piece(sn, s2, wa, wb);
-                }
-                const uint4 oth = make_uint4(lane_xor<PPR / 2>(kq.x), lane_xor<PPR / 2>(kq.y), lane_xor<PPR / 2>(kq.z),
-                                             lane_xor<PPR / 2>(kq.w));
-                kq = rope_piece(kq, oth, cc, sn, piece < PPR / 2);
+            for (int j = 0; j < CPT; j++) {
+                const int c = lane + 64 * j;
+                const int slot = c / PPR, piece = c % PPR;
+                scale_store_k(kreg[j], slot, piece);
+                *reinterpret_cast<uint4 *>(&sm.v[slot][piece * 8]) = vreg[j];
             }
-            kq.x = cvt_pk_bf16(__uint_as_float(kq.x << 16) * p.c_k, __uint_as_float(kq.x & 0xffff0000u) * p.c_k);
-            kq.y = cvt_pk_bf16(__uint_as_float(kq.y << 16) * p.c_k, __uint_as_float(kq.y & 0xffff0000u) * p.c_k);
-            kq.z = cvt_pk_bf16(__uint_as_float(kq.z << 16) * p.c_k, __uint_as_float(kq.z & 0xffff0000u) * p.c_k);
-            kq.w = cvt_pk_bf16(__uint_as_float(kq.w << 16) * p.c_k, __uint_as_float(kq.w & 0xffff0000u) * p.c_k);
-            *reinterpret_cast<uint4 *>(&sm.k[slot][piece * 8]) = kq;
-            *reinterpret_cast<uint4 *>(&sm.v[slot][piece * 8]) = vreg[j];
+        } else {
+            // V first: its registers then hold the table pieces.  The table pieces of half the tile's K pieces are
+            // requested back to back and used after one wait: left to the register allocator, which has nothing to
+            // spare here, each piece's two loads were requested and waited for on their own, eight trips per tile.
+#pragma unroll
+            for (int j = 0; j < CPT; j++) {
+                const int c = lane + 64 * j;
+                *reinterpret_cast<uint4 *>(&sm.v[c / PPR][(c % PPR) * 8]) = vreg[j];
+            }
+            constexpr int HB = CPT / 2 > 0 ? CPT / 2 : 1;
+#pragma unroll
+            for (int j0 = 0; j0 < CPT; j0 += HB) {
+                uint4 cc[HB], sn[HB];
+#pragma unroll
+                for (int jj = 0; jj < HB; jj++) {
+                    const int c = lane + 64 * (j0 + jj);
+                    const int slot = c / PPR, piece = c % PPR;
+                    const int64_t tr = (int64_t)sm.rp[slot2][slot] * p.rope.stride_t + (piece % (PPR / 2)) * 8;
+                    cc[jj] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr);
+                    sn[jj] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int jj = 0; jj < HB; jj++) {
+                    const int c = lane + 64 * (j0 + jj);
+                    const int slot = c / PPR, piece = c % PPR;
+                    uint4 kq = kreg[j0 + jj];
+                    if (dyn) {  // wave-uniform
+                        const int r2 = sm.rp2[slot2][slot];
+                        const int64_t tr2 = (int64_t)(r2 < 0 ? 0 : r2) * p.rope.stride_t + (piece % (PPR / 2)) * 8;
+                        const uint4 c2 = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + tr2);
+                        const uint4 s2 = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + tr2);
+                        const float wa = r2 >= 0 ? 0.75f : 1.0f, wb = r2 >= 0 ? 0.25f : 0.0f;
+                        cc[jj] = rope_blend_piece(cc[jj], c2, wa, wb);
+                        sn[jj] = rope_blend_piece(sn[jj], s2, wa, wb);
+                    }
+                    const uint4 oth = make_uint4(lane_xor<PPR / 2>(kq.x), lane_xor<PPR / 2>(kq.y), lane_xor<PPR / 2>(kq.z),
+                                                 lane_xor<PPR / 2>(kq.w));
+                    scale_store_k(rope_piece(kq, oth, cc[jj], sn[jj], piece < PPR / 2), slot, piece);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
     };
 
