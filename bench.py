@@ -43,13 +43,13 @@ TRAFFIC_SOURCE = ("recorded: profiles/prefill_hbm_traffic_pmc.md (not measured i
 SCAN_SOURCES = ("Makefile", "common.hpp", "mask_common.hpp", "mask_stage_mfma.hip", "mask_stage_dense.hip")
 ATTENTION_SOURCES = ("Makefile", "common.hpp", "bsa.hpp", "bsa_mfma.hip")
 # name -> (bytes per launch, the files the kernel is built from, their digest when the counters were taken)
-SCAN_DIGEST = "168670e784822dc287e6e25afb5bee47f3b262759556e5da23048b17726c4ce8"
-ATTENTION_DIGEST = "6d3b7d60022d55e2d547cb28ae7f8124f245f72978a205032011740408fa003e"
+SCAN_DIGEST = "c017b7d7056aefdb48d4cd6b645a5208f25cf38e68c75a2079cd5c49e01b28a1"
+ATTENTION_DIGEST = "68ef186b308074c4728ae362ad811730369e437ae3e5f2b42c7e293748f442dc"
 MEASURED_TRAFFIC = {
-    "mask_stage[n=507,chunk=256,rows=16]": (2.0 * 4992539.5 * 1024 + 127148.2 * 1024, SCAN_SOURCES, SCAN_DIGEST),
-    "mask_stage[n=1024,chunk=32,rows=16]": (2.0 * 6834764.3 * 1024 + 175526.4 * 1024, SCAN_SOURCES, SCAN_DIGEST),
-    "mask_stage[n=1024,chunk=8,rows=64]": (2.0 * 2239531.2 * 1024 + 157019.5 * 1024, SCAN_SOURCES, SCAN_DIGEST),
-    "bsa_prefill": (2.0 * 1835641.9 * 1024 + 262144.0 * 1024, ATTENTION_SOURCES, ATTENTION_DIGEST),
+    "mask_stage[n=507,chunk=256,rows=16]": (2.0 * 4943837.0 * 1024 + 125223.4 * 1024, SCAN_SOURCES, SCAN_DIGEST),
+    "mask_stage[n=1024,chunk=32,rows=16]": (2.0 * 6845521.0 * 1024 + 176161.9 * 1024, SCAN_SOURCES, SCAN_DIGEST),
+    "mask_stage[n=1024,chunk=8,rows=64]": (2.0 * 2234678.8 * 1024 + 156947.9 * 1024, SCAN_SOURCES, SCAN_DIGEST),
+    "bsa_prefill": (2.0 * 1834612.2 * 1024 + 262144.0 * 1024, ATTENTION_SOURCES, ATTENTION_DIGEST),
 }
 
 
