@@ -61,8 +61,11 @@ __device__ __forceinline__ int64_t rope_kpos(const RopeView &r, int c, int side)
 // Waves per SIMD the register allocator is held to: the scans are chains of dependent round trips (token logic, row
 // loads, products, compares) that only other waves can fill, so a variant that drifts a few registers over the
 // boundary of its class loses a quarter of its throughput (the coalesced variant had grown to 144 registers).
+template <int HID>
+constexpr bool PPR_OK = HID / 8 <= 16;
 constexpr int mask_stage_waves(int HID, int MB, int NB, int RMODE) {
-    const int w = RMODE == 1 ? (MB == 2 ? 1 : 2) : (MB == 1 && NB == 1) ? 4 : (MB == 1 || (NB == 1 && RMODE == 3)) ? 3 : 2;
+    const int w = RMODE == 1 ? (MB == 2 ? 1 : 2) : (RMODE == 10 || RMODE == 11) ? 3
+                : (MB == 1 && NB == 1) ? 4 : (MB == 1 || (NB == 1 && RMODE == 3)) ? 3 : 2;
     return HID > 128 ? (w + 1) / 2 : w;  // 256-element rows: twice the fragments
 }
 // RMODE = 1 (direct path, one token block per wave, extended parameter block): every sampled key row is rotated
@@ -85,6 +88,14 @@ constexpr int mask_stage_waves(int HID, int MB, int NB, int RMODE) {
 // RMODE = 9: as 6, with the 32-bit row offsets of RMODE = 5 (a dense key tensor under 4 GB per batch item).
 // RMODE = 6: a single query token (as RMODE = 3) with the rows fetched as under RMODE = 4; keys prescaled or scaled
 // after the tile is read back.
+// RMODE = 10 / 11 (as 7 / 8 on keys as stored, rotation on load under the RELATIVE rule): left-hand samples sit at
+// position 0 and right-hand samples at position 1, so the wave's tile holds the sixteen left-hand rows first and the
+// sixteen right-hand rows behind them, and the products of the 16-token halves are formed one after the other:
+// only the second half's fragments are rotated (with the one table row of position 1, kept in registers; the partner
+// piece of a fragment is read from the same tile row), and a rotation to position 0 changes nothing as long as the
+// table's first row is (1, 0), which every wave checks for itself (a table that is scaled there takes the slow way:
+// the first half is rotated too).  Half the rotation work of RMODE = 1 and its load shape exchanged for the
+// coalesced one.
 // RMODE = 3 (no rotation, one token block per wave, a single query token): the one valid program row is that token's
 // row, which the kernel scales itself; no preparation launch is needed.
 // KV8 = true (extended parameter block, unscaled keys): key rows are fp8 (e5m2) bytes, widened on load.
@@ -94,11 +105,13 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     constexpr bool ROPE = RMODE == 1;
     constexpr bool QINL = RMODE == 3 || RMODE == 6 || RMODE == 9;  // query rows scaled here instead of read from the prepared workspace
     static_assert(!QINL || NB == 1, "inline query rows: the one-token-block variants only");
-    constexpr bool DMA = RMODE >= 4 && RMODE <= 9;  // rows fetched coalesced, straight into a per-wave LDS tile
-    constexpr bool OFF32 = RMODE == 5 || RMODE == 7 || RMODE == 9;  // their addresses: 32-bit byte offsets from the batch item's first key row
-    constexpr bool M16 = RMODE == 7 || RMODE == 8;    // programs of up to 16 query rows on the 16x16x32 instruction
+    constexpr bool DMA = RMODE >= 4 && RMODE <= 11;  // rows fetched coalesced, straight into a per-wave LDS tile
+    constexpr bool OFF32 = RMODE == 5 || RMODE == 7 || RMODE == 9 || RMODE == 10;  // their addresses: 32-bit byte offsets from the batch item's first key row
+    constexpr bool M16 = RMODE == 7 || RMODE == 8 || RMODE == 10 || RMODE == 11;    // programs of up to 16 query rows on the 16x16x32 instruction
+    constexpr bool SPLIT = RMODE == 10 || RMODE == 11;  // RELATIVE rule on keys as stored: tile rows ordered by sample side
     static_assert(!DMA || (!VIA_LDS && NB == 1 && !KV8), "coalesced direct-to-LDS rows: one token block per wave, bf16 keys");
-    static_assert(!DMA || RMODE == 6 || RMODE == 9 || PRESCALED, "coalesced rows on wide launches: prescaled keys");
+    static_assert(!DMA || RMODE == 6 || RMODE == 9 || SPLIT || PRESCALED, "coalesced rows on wide launches: prescaled keys");
+    static_assert(!SPLIT || (EXT && !PRESCALED && PPR_OK<HID>), "side-split variant: extended build, keys as stored, sixteen pieces per row at most");
     static_assert(!M16 || (MB == 1 && HID % 32 == 0), "16-row variant: one row block, head dim a multiple of 32");
     static_assert(!KV8 || (EXT && !PRESCALED), "fp8 keys: extended build, scaled in the kernel");
     static_assert(!ROPE || (EXT && !VIA_LDS && !PRESCALED), "rope variant: direct path of the extended build");
@@ -328,6 +341,27 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
     bool cross_side = RMODE != 2;
     if constexpr (ROPE) cross_side = p.rope.backend != HIPATTN_EXTEND_RELATIVE;
     if constexpr (DMA && EXT) cross_side = p.rope.k_side_delta == 0;
+    if constexpr (SPLIT) cross_side = false;  // a score belongs to (token, side)
+    // SPLIT: the table row of position 1 for this lane's fragments (k-step 2j + kb / 2 of the half kb % 2), and whether
+    // the row of position 0 leaves a key as it is
+    uint4 cos1[SPLIT ? KS / 2 : 1], sin1[SPLIT ? KS / 2 : 1];
+    bool left_plain = true;
+    if constexpr (SPLIT) {
+        const int kb = lane >> 4;
+        const uint16_t *ct = reinterpret_cast<const uint16_t *>(p.rope.cos), *st = reinterpret_cast<const uint16_t *>(p.rope.sin);
+        const int64_t r0 = p.rope.row(0), r1 = p.rope.row(1);
+        bool ok = true;
+#pragma unroll
+        for (int j = 0; j < KS / 2; j++) {
+            const int col = (2 * j + (kb >> 1)) * 8;
+            cos1[j] = *reinterpret_cast<const uint4 *>(ct + r1 + col);
+            sin1[j] = *reinterpret_cast<const uint4 *>(st + r1 + col);
+            const uint4 c0 = *reinterpret_cast<const uint4 *>(ct + r0 + col), s0 = *reinterpret_cast<const uint4 *>(st + r0 + col);
+            ok = ok && c0.x == 0x3f803f80u && c0.y == 0x3f803f80u && c0.z == 0x3f803f80u && c0.w == 0x3f803f80u &&
+                 (s0.x & 0x7fff7fffu) == 0u && (s0.y & 0x7fff7fffu) == 0u && (s0.z & 0x7fff7fffu) == 0u && (s0.w & 0x7fff7fffu) == 0u;
+        }
+        left_plain = __all(ok) != 0;
+    }
     int ptok[NB];
     float pscore[NB];
     // Paged keys, coalesced fetch: a round first needs its token's page-table entry, a trip to memory ahead of the
@@ -475,7 +509,10 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                 constexpr int NI = 32 * PPR / 64;
                 int o[NI];
 #pragma unroll
-                for (int i = 0; i < NI; i++) o[i] = __shfl(my_piece0, i * (64 / PPR) + lane / PPR);
+                for (int i = 0; i < NI; i++) {
+                    const int r = i * (64 / PPR) + lane / PPR;  // tile row; SPLIT: row side * 16 + c is the sample of lane 2 c + side
+                    o[i] = __shfl(my_piece0, SPLIT ? (((r & 15) << 1) | (r >> 4)) : r);
+                }
                 if constexpr (OFF32) {
                     const uint16_t *kb = reinterpret_cast<const uint16_t *>(p.kv.k) + (int64_t)b * p.kv.k_stride_b;
                     uint32_t so[NI];
@@ -573,6 +610,23 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                         for (int j = 0; j < KS / 2; j++) {
                             const int piece = (kb & 1) * (PPR / 2) + 2 * j + (kb >> 1);
                             kf16[j].q = rd_tile[t * PPR + (piece ^ (t & (PPR - 1)))];
+                            if constexpr (SPLIT) {
+                                // rows as stored: the right-hand half is rotated to position 1 (the partner piece is
+                                // the same columns of the row's other half), then every row is scaled
+                                if (half == 1 || !left_plain) {
+                                    const uint4 oth = rd_tile[t * PPR + ((piece ^ (PPR / 2)) ^ (t & (PPR - 1)))];
+                                    uint4 cc = cos1[j], sn = sin1[j];
+                                    if (half == 0) {  // a table whose first row is not (1, 0): rotate to position 0 as well
+                                        const int64_t r0 = p.rope.row(0);
+                                        const int colx = (2 * j + (kb >> 1)) * 8;
+                                        cc = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.cos) + r0 + colx);
+                                        sn = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.rope.sin) + r0 + colx);
+                                    }
+                                    kf16[j].q = rope_piece(kf16[j].q, oth, cc, sn, (kb & 1) == 0);
+                                }
+#pragma unroll
+                                for (int e = 0; e < 4; e++) kf16[j].u[e] = scale_pack(kf16[j].u[e], p.c_k);
+                            }
                         }
 #pragma unroll
                         for (int j = 0; j < KS / 2; j++)
@@ -597,6 +651,7 @@ void mask_stage_mfma_kernel(MaskParamsFor<EXT> p, int nsub, int hpw) {
                     v = fmaxf(keep, __shfl_xor(send, 16));
                     v = fmaxf(v, __shfl_xor(v, 32));
                     v = round_bf16(v);
+                    if constexpr (SPLIT) v = __shfl(v, ((n & 1) << 4) | (n >> 1));  // from the lane of this lane's tile row
                     if constexpr (OFF32) {
                         if (pieces[tb] < 0) v = 0.0f;
                     }
@@ -959,6 +1014,19 @@ static int launch_mfma_hid(const MaskParams &p0, int rows_eff, int flags, hipStr
 #undef MS_INLINE
         HIPATTN_CHECK_HIP(hipGetLastError());
         return 0;
+    }
+    // rotation on load under the relative rule, programs of up to 16 rows (decode above all): coalesced rows with the
+    // tile ordered by sample side, so that only the right-hand half is rotated (HIPATTN_MASK_DMA=0: the variant below)
+    if constexpr (HID <= 128 && HID % 32 == 0) {
+        // (rows_eff: the valid rows of a program are its first ones; a stage of 64-row programs under a single query
+        // token has one)
+        if (rope && p.rope.backend == HIPATTN_EXTEND_RELATIVE && dma_mode != 0 && !far_rows && !two && rows_eff <= 16 &&
+            !p.kx.kv8 && !p.kx.cached && nb == 1) {
+            if (off32) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, false, false, true, 10>), grid, block, 0, st, p, nsub, hpw);
+            else hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 1, 1, false, false, true, 11>), grid, block, 0, st, p, nsub, hpw);
+            HIPATTN_CHECK_HIP(hipGetLastError());
+            return 0;
+        }
     }
     if (rope && p.kx.kv8) {
         if (two) hipLaunchKernelGGL((mask_stage_mfma_kernel<HID, 2, 1, false, false, true, 1, true>), grid, block, 0, st, p, nsub, hpw);
