@@ -343,9 +343,12 @@ extern "C" int hipattn_mask_stage(const hipattn_q_t *q, const hipattn_kv_t *kv, 
                         "mask stage", &p.rope);
     if (rc) return rc;
     HIPATTN_CHECK_ARG(k_prescaled >= 0 && k_prescaled <= 7, HIPATTN_E_ARG, "mask stage: k_prescaled %d not in 0..7", k_prescaled);
+    // (STREAMING: the caller vouches that every key row was rotated to the place of its chunk in THIS stage's list,
+    // hipattn_prescale_k_rope_chunks; that holds for a first stage, whose list is every chunk in order)
     HIPATTN_CHECK_ARG(!(p.rope.cos && (k_prescaled & 1)) || p.rope.backend == HIPATTN_EXTEND_RELATIVE ||
-                          p.rope.backend == HIPATTN_EXTEND_INFLLM,
-                      HIPATTN_E_ARG, "mask stage: prescaled keys need a rule with fixed key positions (relative, infllm)");
+                          p.rope.backend == HIPATTN_EXTEND_INFLLM || p.rope.backend == HIPATTN_EXTEND_STREAMING,
+                      HIPATTN_E_ARG, "mask stage: prescaled keys need a rule with key positions known ahead (relative, infllm, "
+                                     "streaming on a first stage)");
     if (p.rope.backend != HIPATTN_EXTEND_RELATIVE || !(k_prescaled & 1)) p.rope.k_side_delta = 0;
     HIPATTN_CHECK_ARG(p.rope.k_side_delta % 8 == 0, HIPATTN_E_ALIGN, "mask stage: k_side_delta must keep 16-byte alignment");
     HIPATTN_CHECK_ARG(q->HEAD % p.kv.HKV == 0, HIPATTN_E_ARG, "mask stage: HEAD %% HKV != 0");

@@ -1072,10 +1072,12 @@ __global__ void prescale_k_kernel(const uint16_t *in, uint16_t *out, long long r
     *reinterpret_cast<uint4 *>(out + r * hid + piece * 8) = o;
 }
 
-// the same after rotating every row to one fixed position (table rows cos_row / sin_row)
+// the same after rotating every row to one fixed position (table rows cos_row / sin_row), or, with chunk > 0, row
+// (., t, .) to position (t - first) / chunk, clamped into the tables: the place of token t's chunk in the list of a
+// scan's first stage (chunk c starts at first + c * chunk)
 __global__ void prescale_k_rope_kernel(const uint16_t *in, uint16_t *out, long long rows, int hid, int64_t s0, int64_t s1,
                                        int64_t s2, int d1, int d2, float c_k, const uint16_t *cos_row,
-                                       const uint16_t *sin_row) {
+                                       const uint16_t *sin_row, int64_t table_stride, int64_t table_len, int first, int chunk) {
     const int per_row = hid / 8;
     const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (gid >= rows * per_row) return;
@@ -1086,6 +1088,12 @@ __global__ void prescale_k_rope_kernel(const uint16_t *in, uint16_t *out, long l
     const uint16_t *row = in + i0 * s0 + i1 * s1 + i2 * s2;
     const uint4 raw = *reinterpret_cast<const uint4 *>(row + piece * 8);
     const uint4 oth = *reinterpret_cast<const uint4 *>(row + ppiece * 8);
+    if (chunk > 0) {
+        long long pos = i1 >= first ? (i1 - first) / chunk : 0;
+        pos = pos < table_len ? pos : table_len - 1;
+        cos_row += pos * table_stride;
+        sin_row += pos * table_stride;
+    }
     const uint4 c = *reinterpret_cast<const uint4 *>(cos_row + (piece % (per_row / 2)) * 8);
     const uint4 sn = *reinterpret_cast<const uint4 *>(sin_row + (piece % (per_row / 2)) * 8);
     const uint4 rot = rope_piece(raw, oth, c, sn, piece < per_row / 2);
@@ -1119,7 +1127,33 @@ extern "C" int hipattn_prescale_k_rope(const void *k, int64_t stride0, int64_t s
     hipLaunchKernelGGL(prescale_k_rope_kernel, dim3((unsigned)blocks), dim3(threads), 0, (hipStream_t)stream,
                        reinterpret_cast<const uint16_t *>(k), reinterpret_cast<uint16_t *>(out), rows, HID, stride0,
                        stride1, stride2, n1, n2, c_k, reinterpret_cast<const uint16_t *>(cos_row),
-                       reinterpret_cast<const uint16_t *>(sin_row));
+                       reinterpret_cast<const uint16_t *>(sin_row), (int64_t)0, (int64_t)1, 0, 0);
+    HIPATTN_CHECK_HIP(hipGetLastError());
+    return 0;
+}
+
+extern "C" int hipattn_prescale_k_rope_chunks(const void *k, int64_t stride_b, int64_t stride_t, int64_t stride_h, int64_t B,
+                                              int32_t T, int32_t HKV, int32_t HID, const void *cos, const void *sin,
+                                              int64_t table_stride, int64_t table_len, int32_t first, int32_t chunk,
+                                              void *out, void *stream) {
+    HIPATTN_CHECK_ARG(k && out && cos && sin, HIPATTN_E_ARG, "prescale: null pointer");
+    HIPATTN_CHECK_ARG(B > 0 && T > 0 && HKV > 0 && HID > 0 && HID % 32 == 0, HIPATTN_E_ARG, "prescale: bad sizes");
+    HIPATTN_CHECK_ARG(chunk > 0 && first >= 0 && table_len > 0 && table_stride >= HID / 2, HIPATTN_E_ARG,
+                      "prescale: bad chunk list or table description");
+    HIPATTN_CHECK_ARG(aligned16(k) && aligned16(out) && aligned16(cos) && aligned16(sin) && stride_b % 8 == 0 &&
+                          stride_t % 8 == 0 && stride_h % 8 == 0 && table_stride % 8 == 0,
+                      HIPATTN_E_ALIGN, "prescale: pointers, strides and table rows must be 16-byte aligned");
+    float c_q, c_k;
+    scale_constants(HID, HIPATTN_BF16, &c_q, &c_k);
+    const long long rows = (long long)B * T * HKV;
+    const long long work = rows * (HID / 8);
+    const int threads = 256;
+    const long long blocks = (work + threads - 1) / threads;
+    HIPATTN_CHECK_ARG(blocks < 0x7fffffffLL, HIPATTN_E_UNSUPPORTED, "prescale: tensor too large");
+    hipLaunchKernelGGL(prescale_k_rope_kernel, dim3((unsigned)blocks), dim3(threads), 0, (hipStream_t)stream,
+                       reinterpret_cast<const uint16_t *>(k), reinterpret_cast<uint16_t *>(out), rows, HID, stride_b,
+                       stride_t, stride_h, T, HKV, c_k, reinterpret_cast<const uint16_t *>(cos),
+                       reinterpret_cast<const uint16_t *>(sin), table_stride, table_len, first, chunk);
     HIPATTN_CHECK_HIP(hipGetLastError());
     return 0;
 }

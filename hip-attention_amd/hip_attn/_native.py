@@ -334,6 +334,23 @@ def prescale_k_rope(k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, posit
     return out
 
 
+def prescale_k_rope_chunks(k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, first: int, chunk: int, device) -> torch.Tensor:
+    """``bf16(rot(k[b, t, h], (t - first) // chunk) * c_k)`` for a dense ``[B, T, HKV, D]`` bf16 key tensor: every key
+    rotated to the place of its chunk in a first stage's list (the streaming rule there) and scaled."""
+    assert k.ndim == 4 and k.dtype == torch.bfloat16 and k.stride(3) == 1
+    assert cos.dtype == torch.bfloat16 and sin.dtype == torch.bfloat16 and cos.stride(1) == 1 and sin.stride(1) == 1
+    assert cos.stride(0) == sin.stride(0) and cos.shape[0] == sin.shape[0]
+    out = torch.empty(tuple(k.shape), dtype=k.dtype, device=k.device)
+    with _timed("prescale_k"):
+        rc = lib().hipattn_prescale_k_rope_chunks(
+            _p(k), ctypes.c_int64(k.stride(0)), ctypes.c_int64(k.stride(1)), ctypes.c_int64(k.stride(2)),
+            ctypes.c_int64(k.shape[0]), ctypes.c_int32(k.shape[1]), ctypes.c_int32(k.shape[2]),
+            ctypes.c_int32(k.shape[3]), _p(cos), _p(sin), ctypes.c_int64(cos.stride(0)), ctypes.c_int64(cos.shape[0]),
+            ctypes.c_int32(first), ctypes.c_int32(chunk), _p(out), stream_ptr(device))
+    check(rc, "hipattn_prescale_k_rope_chunks")
+    return out
+
+
 def mask_stage(qs, kvs, chunk_left, hg, n, chunk, right_clamp, bs, bq, stride_q, block_chunk, scan_stride,
                sw_eff, terminate, scores, left_out, device, k_prescaled=False, reduce_heads=False, workspace=None,
                near_pool=False):

@@ -219,11 +219,14 @@ def _new_statistics(args: HiPAttentionArgs, B: int, head_kv: int, pages: int, de
 
 
 def _mask_kv(args: HiPAttentionArgs, k_mask: Optional[Tensor], max_tsrc: int, q: Tensor, programs_rows: int,
-             chunk_count: int, device, stats=None, rope_tabs=None):
-    """KV descriptions for the scan kernels: ``(plain, prescaled or None, keepalive, khat, k_side_delta)``.
+             chunk_count: int, device, stats=None, rope_tabs=None, backends=(), first_stage_list=None):
+    """KV descriptions for the scan kernels: ``(plain, prescaled or None, keepalive, khat, k_side_delta, first or None)``.
 
     ``prescaled`` describes keys scaled (and, with RoPE on load under the relative / infllm rules, rotated) once for
-    the whole tensor; it is built when the scan will sample far more rows than the key tensor holds.
+    the whole tensor; it is built when the scan will sample far more rows than the key tensor holds.  ``backends``:
+    the rotation rules of the stages that will run; ``first_stage_list`` = ``(sink, chunk size)`` when the first of
+    them scans the initial list of a dense key tensor under the streaming rule: there a key's rotated position is the
+    place of its chunk, whatever the query, and ``first`` describes a copy rotated that way.
     """
     stage0 = args.stages[0]
     iters = max(1, int(stage0.stage_chunk_size).bit_length())
@@ -241,6 +244,14 @@ def _mask_kv(args: HiPAttentionArgs, k_mask: Optional[Tensor], max_tsrc: int, q:
                                      f"({tuple(src.shape)}), got {tuple(given.shape)} {given.dtype}")
             if given is not None or force == "1" or (force != "0" and sampled_rows >= 4 * rows_total):
                 delta = 0
+                first = None
+                if rope_tabs is not None and first_stage_list is not None and k_mask is not None:
+                    kfirst = N.prescale_k_rope_chunks(src, rope_tabs[0], rope_tabs[1], first_stage_list[0],
+                                                      first_stage_list[1], device)
+                    st0, keep0 = _kv_struct(args, kfirst, kfirst, max_tsrc, masking=True, stats=stats)
+                    first = (st0, (keep0, kfirst))
+                if rope_tabs is not None and not any(b in ("relative", "infllm") for b in backends):
+                    return plain, None, keep, None, 0, first  # no stage reads keys rotated to a fixed position
                 if given is not None:
                     khat = khat0 = given
                 elif rope_tabs is None:
@@ -258,8 +269,8 @@ def _mask_kv(args: HiPAttentionArgs, k_mask: Optional[Tensor], max_tsrc: int, q:
                     a2 = args.clone()
                     a2.k_cache, a2.v_cache = khat0, khat0
                     st, keep2 = _kv_struct(a2, None, None, max_tsrc, masking=True, stats=stats)
-                return plain, st, (keep, keep2, khat), (khat if rope_tabs is None else None), delta
-    return plain, None, keep, None, 0
+                return plain, st, (keep, keep2, khat), (khat if rope_tabs is None else None), delta, first
+    return plain, None, keep, None, 0, None
 
 
 def _spans_32_gib(t: Optional[Tensor]) -> bool:
@@ -421,14 +432,20 @@ def dual_stage_quadratic_hip_attention(
         # Keys are scaled by c_k and re-rounded every time they are sampled.  When the scan will sample
         # far more rows than the key tensor holds (prefill), scale the whole tensor once instead.
         mask_stats = mask_stats_new
-        mask_kv, mask_kv_pre, keep_mask_kv, khat, k_side_delta = _mask_kv(
-            args, k_mask, MAX_TSRC, q, BSZ * HEAD * BDST_SCAN, chunk_count, device, stats=mask_stats, rope_tabs=rope_tabs)
+        n_cached = len(stage_caches) if stage_caches is not None else 0
+        stage_backends = [(st.stage_extend_backend or args.scan_extend_backend) if isinstance(st, ScanStage) else None
+                          for i, st in enumerate(stages) if i >= n_cached - 1]
+        first_list = None
+        if fresh and rope_tabs is not None and stage_backends and stage_backends[0] == "streaming":
+            first_list = (sink, chunk_size)
+        mask_kv, mask_kv_pre, keep_mask_kv, khat, k_side_delta, mask_kv_first = _mask_kv(
+            args, k_mask, MAX_TSRC, q, BSZ * HEAD * BDST_SCAN, chunk_count, device, stats=mask_stats, rope_tabs=rope_tabs,
+            backends=stage_backends, first_stage_list=first_list)
 
         scores = None
         left_out = None
         prev_n = None
         left64 = right64 = None
-        n_cached = len(stage_caches) if stage_caches is not None else 0
         query_rows = {}
         for i_stage, stage in enumerate(stages):
             prefilled_scores = None
@@ -524,17 +541,21 @@ def dual_stage_quadratic_hip_attention(
                 if chunk_count > 0:
                     rope = None
                     use_pre = mask_kv_pre is not None
+                    kv_pre = mask_kv_pre
                     if rope_tabs is not None:  # :2200-2204
                         backend = stage.stage_extend_backend or args.scan_extend_backend
                         use_pre = use_pre and backend in ("relative", "infllm")  # key positions fixed per sample side
-                        rope = N.make_rope(*rope_tabs, backend, k_side_delta if use_pre else 0, args.model_context_length)
+                        if i_stage == 0 and fresh and mask_kv_first is not None and backend == "streaming":
+                            use_pre, kv_pre = True, mask_kv_first[0]  # keys rotated to the place of their chunk
+                        rope = N.make_rope(*rope_tabs, backend, k_side_delta if (use_pre and backend == "relative") else 0,
+                                           args.model_context_length)
                     qs = N.make_q(qq, position_ids, rope)
                     # Stages that differ only in their chunks share their averaged, scaled query rows.  Only where a
                     # row is a mean of several query rows: otherwise a kernel may scale its rows itself and leave the
                     # workspace unwritten.
                     shared = rope is None and stage.stage_block_stride_q > 1 and TDST > 1
                     ws_key = (bs, BLOCK_SIZE_Q, stage.stage_block_stride_q, STAGE_STRIDE) if shared else None
-                    ws = N.mask_stage(qs, mask_kv_pre if use_pre else mask_kv, chunk_left, hg, chunk_count, chunk_size,
+                    ws = N.mask_stage(qs, kv_pre if use_pre else mask_kv, chunk_left, hg, chunk_count, chunk_size,
                                       right_clamp, bs, BLOCK_SIZE_Q, stage.stage_block_stride_q, BLOCK_CHUNK, STAGE_STRIDE,
                                       sw_eff, args.stage_early_terminate, scores, left_out, device, k_prescaled=use_pre,
                                       reduce_heads=reduce, workspace=query_rows.get(ws_key),

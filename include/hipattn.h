@@ -74,7 +74,8 @@ typedef struct hipattn_rope {
     int32_t backend;  /* HIPATTN_EXTEND_* for this call */
     /* hipattn_mask_stage with k_prescaled != 0 and the RELATIVE rule: kv->k holds the keys rotated to position 0
      * and scaled (hipattn_prescale_k_rope), and the copy rotated to position 1, which the right-hand samples
-     * read, starts this many elements behind it.  INFLLM needs the position-0 copy only.  Unused otherwise. */
+     * read, starts this many elements behind it.  INFLLM needs the position-0 copy only; STREAMING on a first stage
+     * takes the copy hipattn_prescale_k_rope_chunks makes.  Unused otherwise. */
     int64_t k_side_delta;
     /* HiPAttentionArgs.model_context_length (attention_extend.py:250); read by the DYNAMIC rule, which needs at
      * least 512, and by the SELF rule */
@@ -204,6 +205,18 @@ int hipattn_prescale_k(const void *k, int64_t stride0, int64_t stride1, int64_t 
 int hipattn_prescale_k_rope(const void *k, int64_t stride0, int64_t stride1, int64_t stride2, int64_t n0,
                             int32_t n1, int32_t n2, int32_t HID, const void *cos_row, const void *sin_row,
                             void *out, void *stream);
+
+/* The same for the STREAMING rule on the FIRST stage of a scan (attention_extend.py:289-298: a sampled key is rotated
+ * to the place of its chunk in the stage's list): a first stage's list is every chunk in order, chunk c starting at
+ * token `first + c * chunk`, so the position of token t is (t - first) / chunk whatever the query, and
+ * out[b, t, h] = bf16(rot(K[b, t, h], min((t - first) / chunk, table_len - 1)) * c_k) (tokens below `first` are never
+ * sampled there and are rotated to position 0).  K is a dense [B, T, HKV, HID] tensor with the element strides given,
+ * `out` contiguous; cos / sin are the whole tables ([table_len, >= HID/2], table_stride elements between rows).
+ * hipattn_mask_stage takes `out` as kv->k with k_prescaled = 1 and the STREAMING rule. */
+int hipattn_prescale_k_rope_chunks(const void *k, int64_t stride_b, int64_t stride_t, int64_t stride_h, int64_t B,
+                                   int32_t T, int32_t HKV, int32_t HID, const void *cos, const void *sin,
+                                   int64_t table_stride, int64_t table_len, int32_t first, int32_t chunk, void *out,
+                                   void *stream);
 
 /* Between two stages: max over heads, top-k under (score desc, position asc), realign, split.
  * Replaces the ATen glue at src/hip_attn/v1_2/attention_extend.py:2566-2570 (head reduce),

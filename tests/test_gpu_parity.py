@@ -338,13 +338,15 @@ def test_prefill_scans_with_coalesced_row_fetch_on_a_small_launch(paged, m16, mo
     assert torch.equal(meta0.mask_cache_statistics.access_counter, meta.mask_cache_statistics.access_counter)
 
 
-@pytest.mark.parametrize("scan", ["relative", "infllm"])
+@pytest.mark.parametrize("scan", ["relative", "infllm", "streaming"])
 @pytest.mark.parametrize("paged", [0, 16])
 def test_coalesced_prefill_scans_on_keys_rotated_ahead(paged, scan, monkeypatch):
     """RoPE on load under the rules with fixed key positions: the keys are rotated and scaled ahead of the scan, one
     copy per sample side under ``relative``, and the coalesced fetch takes a right-hand sample from the second copy
     (forced on a small launch, both widths of the matrix instruction).  A score then belongs to (token, side): a lane
-    may not take a repeated token's score from its partner of the other side."""
+    may not take a repeated token's score from its partner of the other side.  Under ``streaming`` a key's position is
+    the place of its chunk in the stage's list, which for the first stage of a dense tensor is known ahead too: that
+    stage reads a copy rotated per token (a paged cache keeps the rotation in the kernel)."""
     from helpers import with_rope
 
     _case(f"coalesced prefill scans on keys rotated ahead, scan={scan}, paged={paged}")
