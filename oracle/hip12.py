@@ -265,6 +265,8 @@ def mask_stage(X: OInputs, max_tsrc, left, right, scores, BS, BQ, stride_q, bloc
 def rope_row(X: OInputs, row: np.ndarray, pos: int) -> np.ndarray:
     """One row (float32 values of X's dtype) rotated to ``pos`` with X's tables."""
     S, keep = X.c_struct(0)
+    if not S.rope_cos:
+        raise ValueError("rope_row needs X's tables: give X a scan_backend or sa_backend")
     out = np.ascontiguousarray(row, dtype=np.float32).copy()
     lib().hipo_rope_row(ctypes.byref(S), ctypes.c_void_p(out.ctypes.data), ctypes.c_int64(pos))
     del keep

@@ -224,3 +224,32 @@ def test_keys_rotated_and_scaled_ahead_give_identical_masks(scan, force, monkeyp
         ctx, meta = run_product(XX, AA)
         assert np.array_equal(meta.indices.cpu().numpy(), ometa.indices)
         assert_context_close(ctx, octx, "bf16")
+
+
+def test_keys_rotated_to_the_place_of_their_chunk():
+    """hipattn_prescale_k_rope_chunks: every key row rotated to (t - first) // chunk, clamped into the tables, and
+    scaled, against the oracle's row rotation followed by its scaling."""
+    import torch
+    from hip_attn import _native as N
+    from gpu_utils import to_torch
+
+    print("[case] keys rotated to the place of their chunk", flush=True)
+    B, T, HKV, D, first, chunk, table_len = 2, 300, 2, 64, 16, 64, 4
+    X = with_rope(make_inputs(71, B=B, TQ=8, TK=T, H=HKV, HKV=HKV, D=D, dtype="bf16", scale=0.7), table_len,
+                  scan_backend="relative")
+    k = to_torch(X.k, "bf16")
+    cos = torch.from_numpy(X.rope_cos).to(torch.bfloat16).cuda().contiguous()
+    sin = torch.from_numpy(X.rope_sin).to(torch.bfloat16).cuda().contiguous()
+    out = N.prescale_k_rope_chunks(k, cos, sin, first, chunk, k.device)
+    torch.cuda.synchronize()
+    got = out.view(torch.int16).cpu().numpy().view(np.uint16)
+    _, ck = O.scale_constants(D, "bf16")
+    kf = O.bf16_bits_to_f32(X.k)
+    for b in range(B):
+        for t in (0, 15, 16, 79, 80, 143, 271, 272, 299):   # below `first`, chunk edges, beyond the table (clamped)
+            pos = min((t - first) // chunk if t >= first else 0, table_len - 1)
+            for h in range(HKV):
+                rot = O.rope_row(X, kf[b, t, h], pos)
+                want = O.f32_to_bf16_bits((rot * np.float32(ck)).astype(np.float32))
+                assert np.array_equal(got[b, t, h], want), (b, t, h)
+
