@@ -349,6 +349,48 @@ def _time_decode(step, steps, refresh_every, step_prescaled=None):
                      "what": "opt-in HiPAttentionArgs.k_prescaled: the scans read bf16(K * c_k) from a copy the caller "
                              "keeps (twice the key memory) instead of scaling every sampled row; with statistics"}
         del g_pre, out_pre, meta_pre
+    # The reference's serving loop does not redo the whole hierarchy at every refresh: its default intervals are
+    # (32, 16, 8) decode steps for the three stages (hip_config.py:89-95, mask_refresh_interval.py:9-30), i.e. in 32
+    # steps one full estimation, one that resumes at the second stage from the first stage's cached output, two
+    # that resume at the third, and 28 steps on the kept mask.  A resumed step gets the stage inputs the full step
+    # left behind (metadata.stage_caches cut to the stages kept) and no finished mask.
+    from hip_attn import HiPAttentionOutputMetadata
+
+    def resumed_from(n_kept):
+        return HiPAttentionOutputMetadata(indices=None, ks=None, ks_count=None, ks_start_end=None,
+                                          mask_cache_statistics=None, sa_cache_statistics=None,
+                                          stage_caches=list(meta_r.stage_caches[:n_kept + 1]))
+
+    staged = None
+    if meta_r.stage_caches is not None and len(meta_r.stage_caches) == 3:
+        graphs, same = {}, True
+        for n_kept in (1, 2):
+            with torch.cuda.stream(side):
+                step(resumed_from(n_kept))
+            torch.cuda.synchronize()
+            graphs[n_kept] = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graphs[n_kept], pool=g_refresh.pool()):
+                out_s, meta_s = step(resumed_from(n_kept))
+            graphs[n_kept].replay()
+            torch.cuda.synchronize()
+            same = same and bool(torch.equal(meta_s.indices, meta_r.indices)) and bool(
+                torch.equal(out_s.view(torch.int16), out_r.view(torch.int16)))
+        us_from1 = median([timed(16, lambda i: graphs[1].replay()) for _ in range(9)])
+        us_from2 = median([timed(16, lambda i: graphs[2].replay()) for _ in range(9)])
+        cold_from1, cold_from2 = cold(graphs[1]), cold(graphs[2])
+        per32 = lambda full, s1, s2, kept: (full + s1 + 2 * s2 + 28 * kept) / 32
+        staged = {"intervals": [32, 16, 8], "us_per_step_resumed_at_stage_1": us_from1,
+                  "us_per_step_resumed_at_stage_2": us_from2,
+                  "us_per_step_over_32_steps": per32(us_refresh, us_from1, us_from2, us_cached),
+                  "cold_caches": {"us_per_step_resumed_at_stage_1": cold_from1,
+                                  "us_per_step_resumed_at_stage_2": cold_from2,
+                                  "us_per_step_over_32_steps": per32(us_refresh_cold, cold_from1, cold_from2,
+                                                                     us_cached_cold)},
+                  "resumed_steps_equal_full_step": same,
+                  "what": "the reference's default refresh intervals: of 32 steps one full estimation, one resumed "
+                          "at the second stage, two at the third, 28 on the kept mask; each kind replayed from its "
+                          "own HIP graph, the average formed from the four step times"}
+        del graphs, out_s, meta_s
     del g_plain, out_p, evict
     N.profile_begin()
     _, meta_last = step(None)
@@ -365,6 +407,7 @@ def _time_decode(step, steps, refresh_every, step_prescaled=None):
                         "how": "1 GiB of other data read and written before every replay, each replay timed on its own"},
         "graph_replay_matches_eager": graph_matches,
         "prescaled_keys": prescaled,
+        "staged_refresh": staged,
         "eager": {"us_per_step_mixed": eager_mixed, "us_per_step_refresh": eager_refresh,
                   "us_per_step_cached": eager_cached, "wall_us_per_step_mixed": eager_wall},
         "refresh_kernels_us": [(n, round(ms * 1e3, 1)) for n, ms in prof],
@@ -450,7 +493,7 @@ def run_decode(args, device, TK=1 << 20, steps=64, refresh_every=8, needles=64):
     def step(meta_in, stats=None):
         # statistics only when the mask is estimated, as the serving entry point asks for them (paged_hip.py:400-406)
         a = HiPAttentionArgs12(sliding_window_size=1024, position_ids=pos,
-                               require_cache_statistics=(meta_in is None) if stats is None else stats)
+                               require_cache_statistics=(meta_in is None or meta_in.indices is None) if stats is None else stats)
         return hip_attention_12(q, k, v, a, cached_metadata=meta_in)
 
     from hip_attn import prescale_keys
@@ -528,7 +571,7 @@ def run_batched_decode(args, device, B=16, steps=64, refresh_every=8):
     def step(meta_in, stats=None):
         a = HiPAttentionArgs12(sliding_window_size=1024, position_ids=pos, k_cache=kc, v_cache=vc, block_table=bt,
                                cache_seq_lens=sl, extend_context_length=MAXLEN,
-                               require_cache_statistics=(meta_in is None) if stats is None else stats)
+                               require_cache_statistics=(meta_in is None or meta_in.indices is None) if stats is None else stats)
         return hip_attention_12(q, None, None, a, cached_metadata=meta_in)
 
     from hip_attn import prescale_keys
