@@ -74,35 +74,53 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
 
     // ---- Q^ fragments: column = head of the group (B operand of the first product)
     Frag qf[KS];
-    {
+    if constexpr (!ROPE) {
         const bool ok = col < G;
         const uint16_t *qrow = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_sb + (int64_t)(h0 + (ok ? col : 0)) * p.q_sh;
-        uint4 qraw[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
-            qraw[ks] = make_uint4(0, 0, 0, 0);
-            if (ok) qraw[ks] = *reinterpret_cast<const uint4 *>(qrow + ks * 16 + hh * 8);
-        }
-        if constexpr (ROPE) {
-            if (ok) {  // the query keeps its own position (attention_decode_bsa.py:135-262)
-                const uint16_t *ct = reinterpret_cast<const uint16_t *>(p.rope.cos) + p.rope.row(ppos);
-                const uint16_t *st = reinterpret_cast<const uint16_t *>(p.rope.sin) + p.rope.row(ppos);
-#pragma unroll
-                for (int ks = 0; ks < KS / 2; ks++) {
-                    const uint4 c = *reinterpret_cast<const uint4 *>(ct + ks * 16 + hh * 8);
-                    const uint4 sn = *reinterpret_cast<const uint4 *>(st + ks * 16 + hh * 8);
-                    const uint4 lo = qraw[ks], hi = qraw[ks + KS / 2];
-                    qraw[ks] = rope_piece(lo, hi, c, sn, true);
-                    qraw[ks + KS / 2] = rope_piece(hi, lo, c, sn, false);
-                }
-            }
-        }
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            const uint32_t w[4] = {qraw[ks].x, qraw[ks].y, qraw[ks].z, qraw[ks].w};
+            uint4 qraw = make_uint4(0, 0, 0, 0);
+            if (ok) qraw = *reinterpret_cast<const uint4 *>(qrow + ks * 16 + hh * 8);
+            const uint32_t w[4] = {qraw.x, qraw.y, qraw.z, qraw.w};
 #pragma unroll
             for (int e = 0; e < 4; e++)
                 qf[ks].u[e] = cvt_pk_bf16(__uint_as_float(w[e] << 16) * p.c_q, __uint_as_float(w[e] & 0xffff0000u) * p.c_q);
+        }
+    } else {
+        // The query keeps its own position (attention_decode_bsa.py:135-262).  A wave is one tile deep in a chain of
+        // trips to memory here, so every instruction of this prologue is paid in full: instead of the G lanes that
+        // own a column rotating their whole row (8 pieces of 100 instructions), every lane rotates and scales one
+        // 16-byte piece (column c of its half-wave: head c % GP, k-step c / GP; the partner piece of the rotation is
+        // KS / 2 k-steps away, i.e. 16 lanes) and the owners collect their KS pieces from their half-wave.
+        constexpr int GP = 32 / KS;  // heads per pass
+        const uint16_t *ct = reinterpret_cast<const uint16_t *>(p.rope.cos) + p.rope.row(ppos);
+        const uint16_t *st = reinterpret_cast<const uint16_t *>(p.rope.sin) + p.rope.row(ppos);
+        const int pks = col / GP, pg = col % GP;
+        const uint4 tc = *reinterpret_cast<const uint4 *>(ct + (pks % (KS / 2)) * 16 + hh * 8);
+        const uint4 ts = *reinterpret_cast<const uint4 *>(st + (pks % (KS / 2)) * 16 + hh * 8);
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) qf[ks].q = make_uint4(0, 0, 0, 0);
+        for (int g0 = 0; g0 < G; g0 += GP) {  // one pass unless the group has more heads than a pass holds
+            const bool have = g0 + pg < G;
+            const uint16_t *qrow = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_sb + (int64_t)(h0 + (have ? g0 + pg : 0)) * p.q_sh;
+            const uint4 own = *reinterpret_cast<const uint4 *>(qrow + pks * 16 + hh * 8);
+            const uint4 oth = make_uint4(lane_xor<16>(own.x), lane_xor<16>(own.y), lane_xor<16>(own.z), lane_xor<16>(own.w));
+            const uint4 rot = rope_piece(own, oth, tc, ts, pks < KS / 2);
+            const uint32_t w[4] = {rot.x, rot.y, rot.z, rot.w};
+            uint32_t sc[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                sc[e] = cvt_pk_bf16(__uint_as_float(w[e] << 16) * p.c_q, __uint_as_float(w[e] & 0xffff0000u) * p.c_q);
+            const bool mine = col >= g0 && col < g0 + GP && col < G;  // this lane owns column col, served by this pass
+            const int src0 = mine ? ((lane & 32) | (col - g0)) : (lane & 32);
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const uint32_t got = (uint32_t)__shfl((int)sc[e], src0 + GP * ks);
+                    if (mine) qf[ks].u[e] = got;
+                }
+            }
         }
     }
 
@@ -459,6 +477,8 @@ static int pick_dec(const DecodeMfmaParams &dp, hipStream_t st) {
         if (rope) return cap ? launch_dec<HID, true, true, true, true>(dp, st) : launch_dec<HID, true, true, false, true>(dp, st);
         return cap ? launch_dec<HID, true, false, true, true>(dp, st) : launch_dec<HID, true, false, false, true>(dp, st);
     }
+    // rotation without any other option is every cached step of a serving loop that rotates: it gets the plain build
+    if (rope && !cap && !ext) return launch_dec<HID, false, true, false, false>(dp, st);
     if (rope) return cap ? launch_dec<HID, true, true, true, false>(dp, st) : launch_dec<HID, true, true, false, false>(dp, st);
     return launch_dec<HID, true, false, true, false>(dp, st);
 }
