@@ -1,7 +1,8 @@
 // Decode (one query token per sequence) split-KV attention on the matrix cores (bf16, head dim 64 / 128).
 //
 // A workgroup owns one (sequence, kv head, split); its four waves walk the split's token list independently, 32
-// tokens at a time, each in a private LDS region, so nothing inside the loop synchronises across waves.  The G query
+// tokens at a time (16 or 8 when the split is too short to give every wave a tile), each in a private LDS region, so
+// nothing inside the loop synchronises across waves.  The G query
 // heads of the GQA group play the role of query rows: S^T[token, head] = K^ . Q^^T and O^T[d, head] += V^T . P^T
 // use v_mfma_f32_32x32x16_bf16 with G of the 32 columns occupied.  The matrix unit is mostly idle by design; what the
 // layout buys is that a gathered K / V row is fetched once, coalesced (16 lanes per row), and that the per-token
@@ -37,6 +38,7 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
     constexpr int DB = HID / 32;
     constexpr int PPR = HID / 8;            // 16-byte pieces per row
     constexpr int CPT = DT * PPR / 64;      // pieces per lane per tile
+    constexpr int SPJ = 64 / PPR;           // token slots covered by one piece per lane
     const BsaParams &p = dp.a;
     const KVExt *kx = &p.kx;
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -67,7 +69,12 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
     per = (per + DT - 1) / DT * DT;
     const int o_begin = split * per;
     const int o_end = o_begin + per < total ? o_begin + per : total;
-    const int ntiles = o_end > o_begin ? (o_end - o_begin + DT - 1) / DT : 0;
+    // A split shorter than the four waves' tiles together is cut into tiles of 16 or 8 tokens, so that every wave has
+    // one: a wave walks a chain of trips to memory with the staging arithmetic of its tile in between, and four
+    // quarter-filled tiles side by side are a shorter chain than one or two full ones.  Slots from dte on stay empty.
+    int dte = DT;
+    while (dte > 8 && (o_end - o_begin + dte - 1) / dte * 2 <= DWAVES) dte >>= 1;
+    const int ntiles = o_end > o_begin ? (o_end - o_begin + dte - 1) / dte : 0;
     const int bk_shift = (p.bk & (p.bk - 1)) == 0 ? __builtin_ctz(p.bk) : -1;
     const int tlimit = (int)(p.kv.max_tsrc < curr ? p.kv.max_tsrc : curr);
     const int64_t seqlen = p.kv.paged ? p.kv.seq_len(b) : 0;
@@ -145,8 +152,8 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
     // a dense tensor) instead of three in a row (index entry, page for K, page for V).
     long long pre_s64 = 0;
     auto index_of = [&](int tile) -> long long {  // the index entry of this lane's slot of `tile`, 0 where it has none
-        const int o = o_begin + tile * DT + lane;
-        if (lane < DT && o < o_end && o < n_sel_tok) {
+        const int o = o_begin + tile * dte + lane;
+        if (lane < dte && o < o_end && o < n_sel_tok) {
             const int bi = bk_shift >= 0 ? (o >> bk_shift) : o / p.bk;
             return p.indices[irow * p.BK + rs + bi];
         }
@@ -156,11 +163,11 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
         const long long s64 = pre_s64;
         pre_s64 = (tile + DWAVES < ntiles) ? index_of(tile + DWAVES) : 0;
         if (lane >= DT) return;
-        const int o = o_begin + tile * DT + lane;
+        const int o = o_begin + tile * dte + lane;
         int t = -1, win = 0;
         long long rpos = 0;
         float bias = 0.0f;
-        if (o < o_end) {
+        if (lane < dte && o < o_end) {
             if (o < n_sel_tok) {
                 const int bi = bk_shift >= 0 ? (o >> bk_shift) : o / p.bk;
                 const int e = o - bi * p.bk;
@@ -245,6 +252,7 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
     auto fetch = [&](int slot2) {  // piece c = lane + 64 j is 16-byte piece c % PPR of slot c / PPR
 #pragma unroll
         for (int j = 0; j < CPT; j++) {
+            if (j * SPJ >= dte) break;  // (wave-uniform) slots from dte on are empty
             const int c = lane + 64 * j;
             const int slot = c / PPR, piece = c % PPR;
             const long long ko = sm.ko[slot2][slot], vo = sm.vo[slot2][slot];
@@ -265,6 +273,7 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
         if constexpr (!ROPE) {
 #pragma unroll
             for (int j = 0; j < CPT; j++) {
+                if (j * SPJ >= dte) break;
                 const int c = lane + 64 * j;
                 const int slot = c / PPR, piece = c % PPR;
                 scale_store_k(kreg[j], slot, piece);
@@ -276,15 +285,18 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
             // spare here, each piece's two loads were requested and waited for on their own, eight trips per tile.
 #pragma unroll
             for (int j = 0; j < CPT; j++) {
+                if (j * SPJ >= dte) break;
                 const int c = lane + 64 * j;
                 *reinterpret_cast<uint4 *>(&sm.v[c / PPR][(c % PPR) * 8]) = vreg[j];
             }
             constexpr int HB = CPT / 2 > 0 ? CPT / 2 : 1;
 #pragma unroll
             for (int j0 = 0; j0 < CPT; j0 += HB) {
+                if (j0 * SPJ >= dte) break;
                 uint4 cc[HB], sn[HB];
 #pragma unroll
                 for (int jj = 0; jj < HB; jj++) {
+                    if ((j0 + jj) * SPJ >= dte) break;
                     const int c = lane + 64 * (j0 + jj);
                     const int slot = c / PPR, piece = c % PPR;
                     const int64_t tr = (int64_t)sm.rp[slot2][slot] * p.rope.stride_t + (piece % (PPR / 2)) * 8;
@@ -294,6 +306,7 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int jj = 0; jj < HB; jj++) {
+                    if ((j0 + jj) * SPJ >= dte) break;
                     const int c = lane + 64 * (j0 + jj);
                     const int slot = c / PPR, piece = c % PPR;
                     uint4 kq = kreg[j0 + jj];
@@ -316,6 +329,15 @@ __global__ __launch_bounds__(DWAVES * 64, 2) void bsa_decode_mfma_kernel(DecodeM
     };
 
     const int my_tiles = ntiles > wid ? (ntiles - wid + DWAVES - 1) / DWAVES : 0;
+    if (my_tiles > 0 && dte < DT) {  // rows of the slots that never get a token: read by the products, so zero
+#pragma unroll
+        for (int j = 0; j < CPT; j++) {
+            if (j * SPJ < dte) continue;
+            const int c = lane + 64 * j;
+            *reinterpret_cast<uint4 *>(&sm.k[c / PPR][(c % PPR) * 8]) = make_uint4(0, 0, 0, 0);
+            *reinterpret_cast<uint4 *>(&sm.v[c / PPR][(c % PPR) * 8]) = make_uint4(0, 0, 0, 0);
+        }
+    }
     if (my_tiles > 0) {
         pre_s64 = index_of(wid);
         resolve(wid);
