@@ -414,6 +414,64 @@ def _time_decode(step, steps, refresh_every, step_prescaled=None):
     }, meta_last
 
 
+def _time_decode_rotated(q, k, v, pos, device, table_len=131072):
+    """The same decode steps with keys and query rotated as they are loaded (``using_extend``), as the reference's
+    serving configuration runs them (hip_config.py:68-81: the scans under the "relative" rule on 27 of 32 layers and
+    under "streaming" on the dense ones, attention under "streaming"), each step kind replayed from a HIP graph."""
+    import torch
+    from hip_attn import HiPAttentionArgs12, hip_attention_12
+
+    D = q.shape[-1]
+    inv = 10000.0 ** (-torch.arange(0, D, 2, dtype=torch.float64) / D)
+    ang = torch.arange(table_len, dtype=torch.float64)[:, None] * inv[None]
+    cos = torch.cat([ang.cos(), ang.cos()], 1).to(torch.bfloat16).to(device)
+    sin = torch.cat([ang.sin(), ang.sin()], 1).to(torch.bfloat16).to(device)
+
+    def timed(n, fn):
+        s_ev = torch.cuda.Event(enable_timing=True)
+        e_ev = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        s_ev.record()
+        for _ in range(n):
+            fn()
+        e_ev.record()
+        torch.cuda.synchronize()
+        return s_ev.elapsed_time(e_ev) * 1e3 / n
+
+    def median(xs):
+        xs = sorted(xs)
+        return xs[len(xs) // 2]
+
+    out = {"what": "using_extend with a 131072-row table, attention under the streaming rule; warm loop, HIP graphs"}
+    for scan in ("relative", "streaming"):
+        def step(meta_in):
+            a = HiPAttentionArgs12(sliding_window_size=1024, position_ids=pos, require_cache_statistics=meta_in is None,
+                                   using_extend=True, need_apply_rope=True, rope_cos=cos, rope_sin=sin,
+                                   scan_extend_backend=scan, sa_extend_backend="streaming",
+                                   model_context_length=table_len)
+            return hip_attention_12(q, k, v, a, cached_metadata=meta_in)
+
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            _, m_warm = step(None)
+            step(m_warm)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g_refresh = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g_refresh):
+            out_r, meta_r = step(None)
+        g_cached16 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g_cached16, pool=g_refresh.pool()):
+            for _ in range(16):
+                out_c, _ = step(meta_r)
+        torch.cuda.synchronize()
+        out[scan] = {"us_per_step_refresh": median([timed(16, g_refresh.replay) for _ in range(9)]),
+                     "us_per_step_cached": median([timed(4, g_cached16.replay) / 16 for _ in range(9)])}
+        del g_refresh, g_cached16, out_r, out_c, meta_r
+    return out
+
+
 def _decode_bytes(lens, H, HKV, D):
     """Algorithmic bytes of a refresh step and of a cached step, summed over the batch (default stages)."""
     sink, sw = 256, 1024
@@ -507,6 +565,7 @@ def run_decode(args, device, TK=1 << 20, steps=64, refresh_every=8, needles=64):
 
     res, meta = _time_decode(step, steps, refresh_every, step_prescaled)
     del khat
+    res["rotation_on_load"] = _time_decode_rotated(q, k, v, pos, device)
     # needle recall: a needle counts as found when its 8-token block is among the selected blocks of a head
     idx = meta.indices[:, 0, :]  # [H, BK]
     found = (idx[:, :, None] == starts.to(device)[None, None, :]).any(dim=1).float()  # [H, needles]
