@@ -502,7 +502,12 @@ def _with_rooflines(res, refresh_bytes, attn_bytes):
     res.update({"refresh_algorithmic_bytes": refresh_bytes, "cached_algorithmic_bytes": attn_bytes,
                 "hbm_frac_refresh": gbs_refresh / HBM_PEAK_GBS, "hbm_frac_cached": gbs_cached / HBM_PEAK_GBS,
                 "refresh_GBps": gbs_refresh, "cached_GBps": gbs_cached})
-    return res
+    # The fraction of the HBM peak that stands for this workload is the cold one: in the warm loop much of what a
+    # step reads comes from the memory-side cache, so its rate is not a rate of the memory.
+    headline = {"condition": "refresh step with statistics behind cold caches (every replay timed on its own)",
+                "us_per_step_refresh": cold["us_per_step_refresh"], "hbm_frac_refresh": cold["hbm_frac_refresh"],
+                "warm_loop_hbm_frac_refresh": res["hbm_frac_refresh"]}
+    return {"headline": headline, **res}
 
 
 def run_decode(args, device, TK=1 << 20, steps=64, refresh_every=8, needles=64):
