@@ -55,6 +55,10 @@ def concurrent_stream(device, tries: int = 6):
             _REJECTED_STREAMS.append(cand)
         else:
             cand = _REJECTED_STREAMS[attempt % len(_REJECTED_STREAMS)]
+        # the first launch on a stream sets its queue up and takes longer than the whole probe: a stream that has
+        # never run anything always looks as if it waited for the main stream
+        with torch.cuda.stream(cand):
+            small.zero_()
         torch.cuda.synchronize(device)
         done_main, done_side = torch.cuda.Event(), torch.cuda.Event()
         for _ in range(128):
