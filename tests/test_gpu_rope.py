@@ -93,6 +93,25 @@ def test_batched_paged_decode_with_rope(dtype, sa):
     assert_context_close(ctx2, octx2, dtype)
 
 
+@pytest.mark.parametrize("D,G", [(128, 8), (128, 6), (64, 8), (128, 3)])
+def test_decode_with_rope_and_wide_groups(D, G):
+    """Groups of more heads than one pass of the decode kernel's query preparation holds (head dim 128: four), of as
+    many (head dim 64: eight), and of a number that does not divide a pass."""
+    print(f"[case] rope decode D={D} G={G}", flush=True)
+    B, TK, HKV = 2, 2500, 2
+    lens = np.array([2500, 1300])
+    X = make_inputs(37, B=B, TQ=1, TK=TK, H=HKV * G, HKV=HKV, D=D, dtype="bf16", pos=(lens - 1)[:, None], scale=0.5)
+    XP = with_rope(to_paged(X, 16, seed=6, seq_lens=lens), 4096)
+    A = _ext(scan_extend_backend="relative", sa_extend_backend="streaming", extend_context_length=3072)
+    octx, ometa = O.hip_attention_12(XP, A)
+    ctx, meta = run_product(XP, A)
+    assert_metadata_equal(meta, ometa)
+    assert_context_close(ctx, octx, "bf16")
+    octx2, _ = O.hip_attention_12(XP, A, cached=O.OMetadata(ometa.indices, ometa.ks, ometa.ks_count, ometa.ks_start_end, None))
+    ctx2, _ = run_product(XP, A, cached=meta)
+    assert_context_close(ctx2, octx2, "bf16")
+
+
 def _run_bsa(X, max_tsrc, idx, kse, bq, bk, sw, sink, impl, backend, share=True, decode=False):
     from hip_attn import HiPAttentionArgs12
     from hip_attn.operator import block_sparse_attention
