@@ -550,11 +550,17 @@ def dual_stage_quadratic_hip_attention(
                         rope = N.make_rope(*rope_tabs, backend, k_side_delta if (use_pre and backend == "relative") else 0,
                                            args.model_context_length)
                     qs = N.make_q(qq, position_ids, rope)
-                    # Stages that differ only in their chunks share their averaged, scaled query rows.  Only where a
-                    # row is a mean of several query rows: otherwise a kernel may scale its rows itself and leave the
-                    # workspace unwritten.
-                    shared = rope is None and stage.stage_block_stride_q > 1 and TDST > 1
-                    ws_key = (bs, BLOCK_SIZE_Q, stage.stage_block_stride_q, STAGE_STRIDE) if shared else None
+                    # Stages that differ only in their chunks share their averaged, scaled query rows.  Without
+                    # rotation only where a row is a mean of several query rows: otherwise a kernel may scale its
+                    # rows itself and leave the workspace unwritten.  Rotated rows are always prepared into the
+                    # workspace, and only the streaming rule places a query by the stage's chunk count
+                    # (attention_extend.py:632-647).
+                    if rope is None:
+                        shared = stage.stage_block_stride_q > 1 and TDST > 1
+                    else:
+                        shared = backend != "streaming"
+                    ws_key = ((bs, BLOCK_SIZE_Q, stage.stage_block_stride_q, STAGE_STRIDE, backend if rope is not None else None)
+                              if shared else None)
                     ws = N.mask_stage(qs, kv_pre if use_pre else mask_kv, chunk_left, hg, chunk_count, chunk_size,
                                       right_clamp, bs, BLOCK_SIZE_Q, stage.stage_block_stride_q, BLOCK_CHUNK, STAGE_STRIDE,
                                       sw_eff, args.stage_early_terminate, scores, left_out, device, k_prescaled=use_pre,
