@@ -43,13 +43,13 @@ TRAFFIC_SOURCE = ("recorded: profiles/prefill_hbm_traffic_pmc.md (not measured i
 SCAN_SOURCES = ("Makefile", "common.hpp", "mask_common.hpp", "mask_stage_mfma.hip", "mask_stage_dense.hip")
 ATTENTION_SOURCES = ("Makefile", "common.hpp", "bsa.hpp", "bsa_mfma.hip")
 # name -> (bytes per launch, the files the kernel is built from, their digest when the counters were taken)
-SCAN_DIGEST = "c92b7b126b13acbf0791949758e83366d7cbcd432769b343070737296b652b92"
-ATTENTION_DIGEST = "68ef186b308074c4728ae362ad811730369e437ae3e5f2b42c7e293748f442dc"
+SCAN_DIGEST = "17fbb8212ff65dfd911820b963777a5f511aaa756f51ac3821f2937df275c576"
+ATTENTION_DIGEST = "8fb61ffc807bd4feee4241ba9f37cdd01b1cd48daad2fd8b7378b65521e02454"
 MEASURED_TRAFFIC = {
-    "mask_stage[n=507,chunk=256,rows=16]": (2.0 * 5017418.2 * 1024 + 129685.5 * 1024, SCAN_SOURCES, SCAN_DIGEST),
-    "mask_stage[n=1024,chunk=32,rows=16]": (2.0 * 6852381.9 * 1024 + 176718.2 * 1024, SCAN_SOURCES, SCAN_DIGEST),
-    "mask_stage[n=1024,chunk=8,rows=64]": (2.0 * 2246729.7 * 1024 + 157324.9 * 1024, SCAN_SOURCES, SCAN_DIGEST),
-    "bsa_prefill": (2.0 * 1834612.2 * 1024 + 262144.0 * 1024, ATTENTION_SOURCES, ATTENTION_DIGEST),
+    "mask_stage[n=507,chunk=256,rows=16]": (2.0 * 4989936.7 * 1024 + 129282.6 * 1024, SCAN_SOURCES, SCAN_DIGEST),
+    "mask_stage[n=1024,chunk=32,rows=16]": (2.0 * 6861823.0 * 1024 + 176098.1 * 1024, SCAN_SOURCES, SCAN_DIGEST),
+    "mask_stage[n=1024,chunk=8,rows=64]": (2.0 * 2235225.8 * 1024 + 157139.8 * 1024, SCAN_SOURCES, SCAN_DIGEST),
+    "bsa_prefill": (2.0 * 1834016.9 * 1024 + 262144.1 * 1024, ATTENTION_SOURCES, ATTENTION_DIGEST),
 }
 
 
@@ -204,11 +204,35 @@ def run_prefill(args, device):
     sample = {"indices": meta.indices[:, -nb:].cpu().numpy(), "ks": meta.ks[:, -nb:].cpu().numpy(),
               "ks_start_end": meta.ks_start_end[:, -nb:].cpu().numpy(),
               "context": ctx[:, -SAMPLE_QUERIES:].float().cpu().numpy()}
-    del q, k, v, ctx, meta
+    del ctx, meta
+    # The same call with keys and queries rotated as they are loaded (`using_extend`), as the reference's serving
+    # configuration runs its layers (hip_config.py:68-81: scans under "relative" on 27 of 32 layers, under "streaming"
+    # on the dense ones, attention under "streaming"); not part of `value`, which is BASELINE's workload.
+    rotated = None
+    if args.only is None and not args.skip_decode and not args.skip_rotation:  # full runs only: profiling commands time BASELINE's workload alone
+        inv = 10000.0 ** (-torch.arange(0, D, 2, dtype=torch.float64) / D)
+        ang = torch.arange(TK + 1024, dtype=torch.float64)[:, None] * inv[None]
+        cos = torch.cat([ang.cos(), ang.cos()], 1).to(torch.bfloat16).to(device)
+        sin = torch.cat([ang.sin(), ang.sin()], 1).to(torch.bfloat16).to(device)
+        rotated = {"what": "using_extend, attention under the streaming rule, eager calls, ms per call by scan rule"}
+        for scan in ("relative", "streaming"):
+            rargs = HiPAttentionArgs12(sliding_window_size=1024, require_cache_statistics=not args.no_statistics,
+                                       using_extend=True, need_apply_rope=True, rope_cos=cos, rope_sin=sin,
+                                       scan_extend_backend=scan, sa_extend_backend="streaming")
+            hip_attention_12(q, k, v, rargs)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(3):
+                hip_attention_12(q, k, v, rargs)
+            torch.cuda.synchronize()
+            rotated[scan] = (time.perf_counter() - t0) * 1e3 / 3
+        del cos, sin
+    del q, k, v
     torch.cuda.empty_cache()
     return {
         "sample": sample,
         "ms_per_step": ms_per_step,
+        "rotation_on_load_ms": rotated,
         "tok_per_s": TQ / (ms_per_step * 1e-3),
         "kernels_ms": kern,
         "launches_per_step": launches_per_step,
@@ -972,6 +996,7 @@ def main():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--skip-decode", action="store_true")
+    ap.add_argument("--skip-rotation", action="store_true", help="leave out the prefill calls with rotation on load")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-offload", action="store_true")
     ap.add_argument("--no-statistics", action="store_true",
@@ -1021,6 +1046,7 @@ def main():
             "kernel": dom.get("kernel")},
         "roofline_all": pre["rooflines"],
         "kernels_ms": pre["kernels_ms"],
+        "prefill_rotation_on_load_ms": pre.get("rotation_on_load_ms"),
         "decode": dec,
         "batched_decode": bdec,
         "offload": off,

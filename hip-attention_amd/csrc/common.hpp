@@ -290,10 +290,13 @@ struct KVExt {
 // Element offsets (from kv.k and kv.v) of the rows of token t, kv head h; NO_ROW = "zero row".
 // WANT_V = false skips the V side.  EXT = true also records the access and consults the block cache through
 // `kx` (ignored otherwise).  Several lanes usually fetch pieces of one row: `leader` is true for the one that
-// records the access.
-template <bool WANT_V, bool EXT, bool CHECK = true>
+// records the access.  DEFER = true: the access flag is not touched here; `*mark_out` receives its index in the
+// (batch item, kv head) row of flags (token or page; untouched when there is nothing to record), and the caller
+// marks it once its row loads are on their way: a look at the flag is a trip to memory, and ahead of the row loads
+// it is a trip of its own.
+template <bool WANT_V, bool EXT, bool CHECK = true, bool DEFER = false>
 __device__ __forceinline__ void kv_rows(const KVView &kv, const KVExt *kx, int b, int64_t t, int h, int64_t seqlen,
-                                        int64_t &ko, int64_t &vo, bool leader = true) {
+                                        int64_t &ko, int64_t &vo, bool leader = true, int64_t *mark_out = nullptr) {
     if constexpr (!EXT) {
         // Plain path: K and V offsets as two independent selects.  Sharing the range test and the page lookup
         // between them reads better but made the attention tile kernel 18% slower (the compiler then keeps both
@@ -307,8 +310,10 @@ __device__ __forceinline__ void kv_rows(const KVView &kv, const KVExt *kx, int b
     if (!kv.paged) {
         if (t < 0 || t >= kv.tsrc) return;
         if constexpr (EXT) {
-            if (kx->access_flags && leader)
-                mark_flag<CHECK>(kx->access_flags + (int64_t)b * kx->flags_stride_b + (int64_t)h * kx->flags_stride_h + t);
+            if (kx->access_flags && leader) {
+                if constexpr (DEFER) *mark_out = t;
+                else mark_flag<CHECK>(kx->access_flags + (int64_t)b * kx->flags_stride_b + (int64_t)h * kx->flags_stride_h + t);
+            }
         }
         ko = (int64_t)b * kv.k_stride_b + t * kv.k_stride_t + (int64_t)h * kv.k_stride_h;
         if (WANT_V) vo = (int64_t)b * kv.v_stride_b + t * kv.v_stride_t + (int64_t)h * kv.v_stride_h;
@@ -318,8 +323,10 @@ __device__ __forceinline__ void kv_rows(const KVView &kv, const KVExt *kx, int b
     const int64_t page = kv.page_of(b, t, seqlen);
     const int64_t inpage = t & (kv.page_size - 1);
     if constexpr (EXT) {
-        if (kx->access_flags && leader)
-            mark_flag<CHECK>(kx->access_flags + (int64_t)b * kx->flags_stride_b + (int64_t)h * kx->flags_stride_h + page);
+        if (kx->access_flags && leader) {
+            if constexpr (DEFER) *mark_out = page;
+            else mark_flag<CHECK>(kx->access_flags + (int64_t)b * kx->flags_stride_b + (int64_t)h * kx->flags_stride_h + page);
+        }
         if (kx->cached) {
             const CacheView &c = kx->cache;
             const int64_t row = (page << kv.page_shift) + inpage;
@@ -348,11 +355,11 @@ __device__ __forceinline__ void kv_rows(const KVView &kv, const KVExt *kx, int b
     if (WANT_V) vo = page * kv.v_stride_b + inpage * kv.v_stride_t + (int64_t)h * kv.v_stride_h;
 }
 
-template <bool EXT, bool CHECK = true>
+template <bool EXT, bool CHECK = true, bool DEFER = false>
 __device__ __forceinline__ int64_t kv_k_row(const KVView &kv, const KVExt *kx, int b, int64_t t, int h,
-                                            int64_t seqlen, bool leader = true) {
+                                            int64_t seqlen, bool leader = true, int64_t *mark_out = nullptr) {
     int64_t ko, vo;
-    kv_rows<false, EXT, CHECK>(kv, kx, b, t, h, seqlen, ko, vo, leader);
+    kv_rows<false, EXT, CHECK, DEFER>(kv, kx, b, t, h, seqlen, ko, vo, leader, mark_out);
     return ko;
 }
 
